@@ -1,0 +1,189 @@
+/*
+ * mi355attn -- C ABI of the MI355X (gfx950) attention library.
+ *
+ * This is the boundary a host language binds with its FFI (Julia `ccall`, Python
+ * `ctypes`, ...).  Plain pointers and sizes only.  It replaces, for device arrays,
+ * the following pieces of NNlib.jl (paths relative to the NNlib.jl source tree):
+ *
+ *   dot_product_attention / _dot_product_attention      src/attention.jl:40-101
+ *   dot_product_attention_scores                        src/attention.jl:112-127
+ *   apply_attn_bias / apply_attn_mask                   src/attention.jl:129-138
+ *   make_causal_mask                                    src/attention.jl:149-153
+ *   softmax / softmax! / _softmax! (dims = 1)           src/softmax.jl:56-79
+ *   batched_mul! -> _batched_gemm! backend hook         src/batched/batchedmul.jl:238-298
+ *   batched_gemm! (CPU backend being replaced)          src/gemm.jl:89-188
+ *   rocBLAS hook of the AMDGPU extension                ext/NNlibAMDGPUExt/batched_mul.jl:11-24
+ *
+ * Conventions
+ *   - Every array is column-major (Julia layout).  A (E, L, B) array stores element
+ *     (d, i, b) at d + i*E + b*E*L.  Heads are feature slices: head h owns features
+ *     [h*D, (h+1)*D), D = E / H  (split_heads, src/attention.jl:158).
+ *   - All pointers passed to op entry points are DEVICE pointers owned by the caller.
+ *     Op entry points never allocate or free device memory and are asynchronous on
+ *     the given stream (NULL = the default stream).
+ *   - Every function returns an int32 status; 0 = MI_OK.  No exception crosses the
+ *     boundary.  mi_last_error_string() gives a thread-local message for the last
+ *     non-zero status returned on the calling thread.
+ */
+#ifndef MI355ATTN_H
+#define MI355ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355ATTN_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* ---- status codes ---------------------------------------------------------------- */
+enum {
+    MI_OK = 0,
+    MI_EINVAL = 1,       /* null pointer, negative size, bad flag                       */
+    MI_EDTYPE = 2,       /* dtype not one of MI_F32 / MI_F16 / MI_BF16                  */
+    MI_ESHAPE = 3,       /* sizes inconsistent (the reference throws ArgumentError /    */
+                         /* DimensionMismatch for the same conditions)                  */
+    MI_EHIP = 4,         /* a HIP runtime call failed; message carries hipGetErrorString */
+    MI_ENOMEM = 5,       /* device allocation failed (mi_malloc only)                   */
+    MI_EWORKSPACE = 6    /* workspace missing or smaller than mi_attention_workspace_size */
+};
+
+/* ---- element types --------------------------------------------------------------- */
+enum { MI_F32 = 0, MI_F16 = 1, MI_BF16 = 2 };
+
+typedef void *mi_stream; /* a hipStream_t */
+typedef void *mi_event;  /* a hipEvent_t  */
+
+/* ---- runtime: device memory, streams, events ------------------------------------- */
+/* The reference has no counterpart: its CPU path uses Julia's GC'd Arrays.  These exist
+ * so that a host language without a HIP binding can own device buffers. */
+int32_t mi_version(void);
+const char *mi_last_error_string(void);
+int32_t mi_init(int32_t device); /* select device, verify it is gfx950; idempotent */
+int32_t mi_device_count(int32_t *count);
+int32_t mi_device_name(char *buf, size_t buflen);
+int32_t mi_malloc(void **ptr, size_t bytes);
+int32_t mi_free(void *ptr);
+int32_t mi_memcpy_h2d(void *dst, const void *src, size_t bytes, mi_stream stream);
+int32_t mi_memcpy_d2h(void *dst, const void *src, size_t bytes, mi_stream stream);
+int32_t mi_memcpy_d2d(void *dst, const void *src, size_t bytes, mi_stream stream);
+int32_t mi_fill_zero(void *ptr, size_t bytes, mi_stream stream); /* fill kernel, graph-capture safe */
+int32_t mi_stream_create(mi_stream *stream);
+int32_t mi_stream_destroy(mi_stream stream);
+int32_t mi_stream_sync(mi_stream stream);
+int32_t mi_device_sync(void);
+int32_t mi_event_create(mi_event *event);
+int32_t mi_event_destroy(mi_event event);
+int32_t mi_event_record(mi_event event, mi_stream stream);
+int32_t mi_event_sync(mi_event event);
+int32_t mi_event_elapsed_ms(mi_event start, mi_event stop, float *ms);
+
+/* ---- attention ------------------------------------------------------------------- */
+
+/* Which kernel family mi_attention_fwd picked (reported by mi_attention_plan). */
+enum {
+    MI_ATTN_KERNEL_GENERIC = 0,  /* any shape / dtype, scalar FMA                        */
+    MI_ATTN_KERNEL_FLASH16 = 1,  /* f16 / bf16 MFMA flash forward, head dim 64 or 128    */
+    MI_ATTN_KERNEL_FLASH32 = 2,  /* f32 MFMA flash forward, head dim 64 or 128           */
+    MI_ATTN_KERNEL_DECODE = 3    /* split-kv bandwidth-bound path for short queries      */
+};
+
+/* flags */
+#define MI_ATTN_FORCE_GENERIC 1u /* use the generic kernel regardless of shape (testing) */
+
+/*
+ * One call of dot_product_attention(q, k, v, bias; mask, nheads) with fdrop = identity
+ * (src/attention.jl:52-84), or of dot_product_attention_scores when `out` is NULL
+ * (src/attention.jl:112-127; the 4-D (D, H, L, B) inputs of that function have the
+ * same memory layout as the 3-D (D*H, L, B) ones).
+ *
+ *   q   (E,  Lq,  B)       k (E, Lkv, B)       v (Ev, Lkv, B)      all of `dtype`
+ *   out (Ev, Lq,  B) of `dtype`, or NULL to compute weights only (then v may be NULL)
+ *   weights (Lkv, Lq, H, B) of `weights_dtype`, or NULL to not materialise them
+ *   bias   : NULL, or `dtype` array with element strides for the (kv, q, head, batch)
+ *            dims of the score tensor; stride 0 = broadcast along that dim
+ *            (apply_attn_bias, src/attention.jl:131: logits .+ bias)
+ *   mask   : NULL, or uint8 array (0 = drop, non-zero = keep) with strides as for bias
+ *            (apply_attn_mask, src/attention.jl:133-138: dropped logits become -Inf)
+ *   causal : non-zero = additionally apply make_causal_mask's pattern
+ *            keep(kv, q) = kv <= q (src/attention.jl:145) without reading a mask array;
+ *            requires Lq == Lkv as a (len, len) mask would.
+ *
+ * Scores are sum_d k[d]*(q[d]/sqrt(D)) + bias, masked, softmax over kv, as the
+ * reference orders them (bias before mask).  A query whose kv positions are all
+ * dropped yields NaN weights and NaN output, as the reference's softmax does.
+ *
+ * weights_dtype must be `dtype` or MI_F32.
+ * workspace: device scratch of at least mi_attention_workspace_size() bytes (may be
+ * NULL when that size is 0).
+ */
+typedef struct mi_attn_desc {
+    int32_t struct_size; /* = sizeof(mi_attn_desc); guards against ABI drift */
+    int32_t dtype;
+    int32_t weights_dtype;
+    int32_t causal;
+    uint32_t flags;
+    int32_t reserved;
+    int64_t E, Ev, Lq, Lkv, H, B;
+    const void *q;
+    const void *k;
+    const void *v;
+    void *out;
+    void *weights;
+    const void *bias;
+    int64_t bias_strides[4];
+    const uint8_t *mask;
+    int64_t mask_strides[4];
+    void *workspace;
+    size_t workspace_bytes;
+} mi_attn_desc;
+
+/* Validates shapes the way src/attention.jl:55-78 does (MI_ESHAPE on failure) and
+ * reports the kernel family and workspace need without touching the device. */
+int32_t mi_attention_plan(const mi_attn_desc *desc, int32_t *kernel, size_t *workspace_bytes);
+int32_t mi_attention_workspace_size(const mi_attn_desc *desc, size_t *bytes);
+int32_t mi_attention_fwd(const mi_attn_desc *desc, mi_stream stream);
+
+/* make_causal_mask (src/attention.jl:149-153): m (len, len) uint8, m[i,j] = (i <= j). */
+int32_t mi_make_causal_mask(uint8_t *m, int64_t len, mi_stream stream);
+
+/* ---- softmax over the first dimension -------------------------------------------- */
+/* y[:, c] = softmax(x[:, c]) for a (rows, cols) column-major matrix; y may alias x
+ * (softmax!(x), src/softmax.jl:64).  Arithmetic in fp32; +-Inf / NaN rules of
+ * src/softmax.jl:69-79 (a +Inf maximum turns the column into an indicator of its
+ * +Inf entries, normalised; NaN poisons its column; an all -Inf column is NaN). */
+int32_t mi_softmax_dim1(int32_t dtype, const void *x, void *y, int64_t rows, int64_t cols,
+                        mi_stream stream);
+
+/* ---- batched GEMM ---------------------------------------------------------------- */
+/* C[:,:,b] = alpha * op(A[:,:,b]) * op(B[:,:,b]) + beta * C[:,:,b],  b in [0, batch).
+ * The signature follows the backend hook NNlib._batched_gemm!(transA, transB, alpha,
+ * A, B, beta, C) (src/batched/batchedmul.jl:298) flattened to BLAS-style arguments as
+ * src/gemm.jl:141-149 passes them: trans flags are the characters 'N' or 'T' ('C' is
+ * accepted as 'T': all supported element types are real); op(A) is m x k, op(B) is
+ * k x n; lda/ldb/ldc are column strides in elements; strideA/strideB = 0 broadcasts a
+ * single slice over the batch (src/gemm.jl:117-118).  beta == 0 overwrites C without
+ * reading it.  Accumulation is fp32 for every dtype. */
+int32_t mi_batched_gemm(int32_t dtype, char transA, char transB, int64_t m, int64_t n, int64_t k,
+                        float alpha, const void *A, int64_t lda, int64_t strideA, const void *B,
+                        int64_t ldb, int64_t strideB, float beta, void *C, int64_t ldc,
+                        int64_t strideC, int64_t batch, mi_stream stream);
+
+/* ---- reproducible inputs --------------------------------------------------------- */
+/* ptr[i] = dtype(scale * z_i), z_i ~ N(0,1) from a counter-based generator keyed by
+ * (seed, stream_id, i); the same call always produces the same bits.  No counterpart
+ * in the reference (its tests use Julia's rand/randn). */
+int32_t mi_randn_fill(void *ptr, int32_t dtype, int64_t n, uint64_t seed, uint64_t stream_id,
+                      float scale, mi_stream stream);
+/* mask[i] = (u_i < keep_prob) as uint8, same generator. */
+int32_t mi_bernoulli_fill(uint8_t *mask, int64_t n, uint64_t seed, uint64_t stream_id,
+                          float keep_prob, mi_stream stream);
+/* dst[i] = dtype_dst(src[i]) with round-to-nearest-even. */
+int32_t mi_convert(void *dst, int32_t dtype_dst, const void *src, int32_t dtype_src, int64_t n,
+                   mi_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355ATTN_H */

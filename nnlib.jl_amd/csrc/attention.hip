@@ -1,0 +1,125 @@
+// mi_attention_fwd: validation (mirrors the reference's argument checks) and kernel selection.
+#include "common.h"
+#include "attention_params.h"
+
+int32_t launch_flash16_bf16_d64(const AttnParams &, hipStream_t);
+int32_t launch_flash16_bf16_d128(const AttnParams &, hipStream_t);
+int32_t launch_flash16_f16_d64(const AttnParams &, hipStream_t);
+int32_t launch_flash16_f16_d128(const AttnParams &, hipStream_t);
+
+static inline bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
+
+bool attention_flash16_supports(const AttnParams &p) {
+    if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
+    if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
+    if (!aligned16(p.q) || !aligned16(p.k) || (p.out && (!aligned16(p.v) || !aligned16(p.out)))) return false;
+    // one workgroup per (query tile, head, batch) in a 1-D grid
+    const int64_t tiles = (p.Lq + 127) / 128;
+    if (tiles * p.H * p.B > 2147483647LL) return false;
+    return true;
+}
+
+int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
+    if (p.dtype == MI_BF16) return p.D == 64 ? launch_flash16_bf16_d64(p, st) : launch_flash16_bf16_d128(p, st);
+    return p.D == 64 ? launch_flash16_f16_d64(p, st) : launch_flash16_f16_d128(p, st);
+}
+
+// Validation.  The first four conditions are the reference's ArgumentErrors
+// (src/attention.jl:55-78); with (E, L, B) sizes passed as scalars, "batch dimensions equal",
+// "qk feature dims equal" and "kv lengths equal" hold by construction, which leaves divisibility.
+static int32_t validate(const mi_attn_desc *d, AttnParams *out) {
+    if (!d) return mi_set_error(MI_EINVAL, "mi_attention: desc is NULL");
+    if (d->struct_size != (int32_t)sizeof(mi_attn_desc))
+        return mi_set_error(MI_EINVAL, "mi_attention: desc.struct_size is %d, library expects %zu", d->struct_size,
+                            sizeof(mi_attn_desc));
+    if (!mi_dtype_ok(d->dtype)) return mi_set_error(MI_EDTYPE, "mi_attention: unknown dtype %d", d->dtype);
+    if (d->E < 0 || d->Ev < 0 || d->Lq < 0 || d->Lkv < 0 || d->B < 0)
+        return mi_set_error(MI_ESHAPE, "mi_attention: negative size");
+    if (d->H < 1) return mi_set_error(MI_ESHAPE, "mi_attention: nheads must be at least 1 (got %lld)", (long long)d->H);
+    if (d->E % d->H != 0 || d->Ev % d->H != 0)
+        return mi_set_error(MI_ESHAPE,
+                            "First dimension in query, key and value must be divisible by `nheads`. Instead: "
+                            "size(q,1) = size(k,1) = %lld, size(v,1) = %lld, nheads = %lld",
+                            (long long)d->E, (long long)d->Ev, (long long)d->H);
+    if (d->causal && d->Lq != d->Lkv)
+        return mi_set_error(MI_ESHAPE, "mi_attention: a causal (len, len) mask needs Lq == Lkv (got %lld, %lld)",
+                            (long long)d->Lq, (long long)d->Lkv);
+    if (!d->out && !d->weights) return mi_set_error(MI_EINVAL, "mi_attention: both out and weights are NULL");
+    if (d->weights && d->weights_dtype != d->dtype && d->weights_dtype != MI_F32)
+        return mi_set_error(MI_EDTYPE, "mi_attention: weights_dtype must equal dtype or be MI_F32");
+    const bool empty = d->Lq == 0 || d->B == 0 || (d->E == 0 && d->Ev == 0);
+    if (!empty) {
+        if (d->Lkv > 0 && d->E > 0 && (!d->q || !d->k)) return mi_set_error(MI_EINVAL, "mi_attention: q or k is NULL");
+        if (d->out && d->Lkv > 0 && d->Ev > 0 && !d->v) return mi_set_error(MI_EINVAL, "mi_attention: v is NULL but out is not");
+    }
+    for (int i = 0; i < 4; i++) {
+        if (d->bias && d->bias_strides[i] < 0) return mi_set_error(MI_ESHAPE, "mi_attention: negative bias stride");
+        if (d->mask && d->mask_strides[i] < 0) return mi_set_error(MI_ESHAPE, "mi_attention: negative mask stride");
+    }
+    AttnParams p;
+    p.q = d->q; p.k = d->k; p.v = d->v; p.out = d->out; p.weights = d->weights;
+    p.bias = d->bias; p.mask = d->mask; p.workspace = d->workspace;
+    for (int i = 0; i < 4; i++) {
+        p.bias_strides[i] = d->bias ? d->bias_strides[i] : 0;
+        p.mask_strides[i] = d->mask ? d->mask_strides[i] : 0;
+    }
+    p.E = d->E; p.Ev = d->Ev; p.Lq = d->Lq; p.Lkv = d->Lkv; p.H = d->H; p.B = d->B;
+    p.D = d->E / d->H; p.Dv = d->Ev / d->H;
+    p.dtype = d->dtype;
+    p.weights_dtype = d->weights ? d->weights_dtype : d->dtype;
+    p.causal = d->causal != 0;
+    *out = p;
+    return MI_OK;
+}
+
+static int32_t choose(const mi_attn_desc *d, const AttnParams &p, size_t *ws) {
+    *ws = 0;
+    if (d->flags & MI_ATTN_FORCE_GENERIC) return MI_ATTN_KERNEL_GENERIC;
+    if (attention_decode_supports(p)) {
+        *ws = attention_decode_workspace(p);
+        return MI_ATTN_KERNEL_DECODE;
+    }
+    if (attention_flash16_supports(p)) return MI_ATTN_KERNEL_FLASH16;
+    if (attention_flash32_supports(p)) return MI_ATTN_KERNEL_FLASH32;
+    return MI_ATTN_KERNEL_GENERIC;
+}
+
+MI_API int32_t mi_attention_plan(const mi_attn_desc *d, int32_t *kernel, size_t *workspace_bytes) {
+    AttnParams p;
+    int32_t rc = validate(d, &p);
+    if (rc != MI_OK) return rc;
+    size_t ws = 0;
+    int32_t k = choose(d, p, &ws);
+    if (kernel) *kernel = k;
+    if (workspace_bytes) *workspace_bytes = ws;
+    return MI_OK;
+}
+
+MI_API int32_t mi_attention_workspace_size(const mi_attn_desc *d, size_t *bytes) {
+    if (!bytes) return mi_set_error(MI_EINVAL, "mi_attention_workspace_size: bytes is NULL");
+    return mi_attention_plan(d, nullptr, bytes);
+}
+
+MI_API int32_t mi_attention_fwd(const mi_attn_desc *d, mi_stream s) {
+    AttnParams p;
+    int32_t rc = validate(d, &p);
+    if (rc != MI_OK) return rc;
+    hipStream_t st = (hipStream_t)s;
+    if (p.Lq == 0 || p.B == 0) return MI_OK;  // empty outputs
+    if (p.Lkv == 0) {
+        // softmax over an empty column has no entries; the product with the (Dv x 0) values is all zeros
+        if (p.out) return mi_fill_zero(p.out, (size_t)(p.Ev * p.Lq * p.B) * mi_dtype_size(p.dtype), s);
+        return MI_OK;
+    }
+    size_t ws = 0;
+    const int32_t kernel = choose(d, p, &ws);
+    if (ws > 0 && (!d->workspace || d->workspace_bytes < ws))
+        return mi_set_error(MI_EWORKSPACE, "mi_attention_fwd: workspace of %zu bytes required, %zu given", ws,
+                            d->workspace ? d->workspace_bytes : (size_t)0);
+    switch (kernel) {
+    case MI_ATTN_KERNEL_DECODE: return launch_attention_decode(p, st);
+    case MI_ATTN_KERNEL_FLASH16: return launch_attention_flash16(p, st);
+    case MI_ATTN_KERNEL_FLASH32: return launch_attention_flash32(p, st);
+    default: return launch_attention_generic(p, st);
+    }
+}

@@ -1,0 +1,23 @@
+// Kernel-side view of one attention call (validated copy of mi_attn_desc).
+#pragma once
+#include "common.h"
+
+struct AttnParams {
+    const void *q, *k, *v;
+    void *out, *weights;
+    const void *bias;
+    const uint8_t *mask;
+    void *workspace;
+    int64_t bias_strides[4], mask_strides[4];
+    int64_t E, Ev, Lq, Lkv, H, B, D, Dv;
+    int32_t dtype, weights_dtype, causal;
+};
+
+int32_t launch_attention_generic(const AttnParams &p, hipStream_t st);
+int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st);
+int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st);
+int32_t launch_attention_decode(const AttnParams &p, hipStream_t st);
+size_t attention_decode_workspace(const AttnParams &p);
+bool attention_flash16_supports(const AttnParams &p);
+bool attention_flash32_supports(const AttnParams &p);
+bool attention_decode_supports(const AttnParams &p);

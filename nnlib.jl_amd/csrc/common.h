@@ -1,0 +1,100 @@
+// Shared host/device helpers for the gfx950 attention library.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <math.h>
+
+#include "../../include/mi355attn.h"
+
+#define MI_API extern "C" __attribute__((visibility("default")))
+
+// ---- error reporting ---------------------------------------------------------------
+int32_t mi_set_error(int32_t code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define MI_HIP_CHECK(expr)                                                                  \
+    do {                                                                                    \
+        hipError_t _e = (expr);                                                             \
+        if (_e != hipSuccess)                                                               \
+            return mi_set_error(MI_EHIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), \
+                                __FILE__, __LINE__);                                        \
+    } while (0)
+
+#define MI_LAUNCH_CHECK()                                                                   \
+    do {                                                                                    \
+        hipError_t _e = hipGetLastError();                                                  \
+        if (_e != hipSuccess)                                                               \
+            return mi_set_error(MI_EHIP, "kernel launch failed: %s (%s:%d)",                \
+                                hipGetErrorString(_e), __FILE__, __LINE__);                 \
+    } while (0)
+
+static inline size_t mi_dtype_size(int32_t dt) { return dt == MI_F32 ? 4 : 2; }
+static inline bool mi_dtype_ok(int32_t dt) { return dt == MI_F32 || dt == MI_F16 || dt == MI_BF16; }
+
+// ---- vector types ------------------------------------------------------------------
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 f16x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
+
+// ---- element traits ----------------------------------------------------------------
+struct F32 {
+    typedef float type;
+    static constexpr int id = MI_F32;
+    __device__ static inline float to_f32(float x) { return x; }
+    __device__ static inline float from_f32(float x) { return x; }
+};
+struct F16 {
+    typedef _Float16 type;
+    typedef f16x8_t vec8;
+    typedef f16x4_t vec4;
+    static constexpr int id = MI_F16;
+    __device__ static inline float to_f32(_Float16 x) { return (float)x; }
+    __device__ static inline _Float16 from_f32(float x) { return (_Float16)x; }
+    __device__ static inline floatx16_t mfma32(vec8 a, vec8 b, floatx16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+struct BF16 {
+    typedef __bf16 type;
+    typedef bf16x8_t vec8;
+    typedef bf16x4_t vec4;
+    static constexpr int id = MI_BF16;
+    __device__ static inline float to_f32(__bf16 x) { return (float)x; }
+    __device__ static inline __bf16 from_f32(float x) { return (__bf16)x; }
+    __device__ static inline floatx16_t mfma32(vec8 a, vec8 b, floatx16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+#define MI_NEG_INF (-__builtin_huge_valf())
+#define MI_POS_INF (__builtin_huge_valf())
+#define MI_LOG2E 1.44269504088896340736f
+
+// exchange a value between lane l and lane l^32 of a 64-wide wavefront
+__device__ static inline float mi_swap32(float x) {
+    return __shfl_xor(x, 32, 64);
+}
+
+__device__ static inline float mi_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// wavefront (64 lanes) reductions
+__device__ static inline float mi_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ static inline float mi_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}

@@ -1,0 +1,117 @@
+// Reproducible input generators, dtype conversion and make_causal_mask.
+#include "common.h"
+
+__device__ static inline uint64_t mix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+__device__ static inline uint64_t counter_bits(uint64_t seed, uint64_t stream_id, uint64_t i) {
+    return mix64(mix64(seed ^ (stream_id * 0xD1342543DE82EF95ull)) + i * 0x9E3779B97F4A7C15ull);
+}
+
+template <typename T>
+__global__ void randn_kernel(typename T::type *p, int64_t n, uint64_t seed, uint64_t stream_id, float scale) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        uint64_t r = counter_bits(seed, stream_id, (uint64_t)i);
+        // two uniforms in (0,1]: 24 bits each
+        float u1 = ((float)((r >> 40) & 0xFFFFFF) + 1.0f) * (1.0f / 16777216.0f);
+        float u2 = ((float)((r >> 8) & 0xFFFFFF) + 1.0f) * (1.0f / 16777216.0f);
+        float z = sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2);
+        p[i] = T::from_f32(scale * z);
+    }
+}
+
+__global__ void bernoulli_kernel(uint8_t *p, int64_t n, uint64_t seed, uint64_t stream_id, float keep) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        uint64_t r = counter_bits(seed, stream_id, (uint64_t)i);
+        float u = (float)((r >> 40) & 0xFFFFFF) * (1.0f / 16777216.0f);
+        p[i] = (uint8_t)(u < keep);
+    }
+}
+
+template <typename TD, typename TS>
+__global__ void convert_kernel(typename TD::type *d, const typename TS::type *s, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) d[i] = TD::from_f32(TS::to_f32(s[i]));
+}
+
+// m[i + j*len] = (i <= j): reference src/attention.jl:145,149-153
+__global__ void causal_mask_kernel(uint8_t *m, int64_t len) {
+    int64_t n = len * len;
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; idx < n; idx += stride) {
+        int64_t i = idx % len, j = idx / len;
+        m[idx] = (uint8_t)(i <= j);
+    }
+}
+
+static inline int grid_for(int64_t n) {
+    int64_t b = (n + 255) / 256;
+    return (int)(b < 1 ? 1 : (b > 16384 ? 16384 : b));
+}
+
+MI_API int32_t mi_randn_fill(void *ptr, int32_t dtype, int64_t n, uint64_t seed, uint64_t stream_id,
+                             float scale, mi_stream s) {
+    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_randn_fill: unknown dtype %d", dtype);
+    if (n < 0) return mi_set_error(MI_EINVAL, "mi_randn_fill: negative length");
+    if (n == 0) return MI_OK;
+    if (!ptr) return mi_set_error(MI_EINVAL, "mi_randn_fill: null pointer");
+    dim3 g(grid_for(n)), b(256);
+    hipStream_t st = (hipStream_t)s;
+    if (dtype == MI_F32) hipLaunchKernelGGL(randn_kernel<F32>, g, b, 0, st, (float *)ptr, n, seed, stream_id, scale);
+    else if (dtype == MI_F16) hipLaunchKernelGGL(randn_kernel<F16>, g, b, 0, st, (_Float16 *)ptr, n, seed, stream_id, scale);
+    else hipLaunchKernelGGL(randn_kernel<BF16>, g, b, 0, st, (__bf16 *)ptr, n, seed, stream_id, scale);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+MI_API int32_t mi_bernoulli_fill(uint8_t *mask, int64_t n, uint64_t seed, uint64_t stream_id, float keep_prob,
+                                 mi_stream s) {
+    if (n < 0) return mi_set_error(MI_EINVAL, "mi_bernoulli_fill: negative length");
+    if (n == 0) return MI_OK;
+    if (!mask) return mi_set_error(MI_EINVAL, "mi_bernoulli_fill: null pointer");
+    hipLaunchKernelGGL(bernoulli_kernel, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)s, mask, n, seed, stream_id,
+                       keep_prob);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+template <typename TD>
+static void launch_convert_from(void *d, const void *src, int32_t ds, int64_t n, hipStream_t st) {
+    dim3 g(grid_for(n)), b(256);
+    typedef typename TD::type td;
+    if (ds == MI_F32) hipLaunchKernelGGL((convert_kernel<TD, F32>), g, b, 0, st, (td *)d, (const float *)src, n);
+    else if (ds == MI_F16) hipLaunchKernelGGL((convert_kernel<TD, F16>), g, b, 0, st, (td *)d, (const _Float16 *)src, n);
+    else hipLaunchKernelGGL((convert_kernel<TD, BF16>), g, b, 0, st, (td *)d, (const __bf16 *)src, n);
+}
+
+MI_API int32_t mi_convert(void *dst, int32_t dd, const void *src, int32_t ds, int64_t n, mi_stream s) {
+    if (!mi_dtype_ok(dd) || !mi_dtype_ok(ds)) return mi_set_error(MI_EDTYPE, "mi_convert: unknown dtype");
+    if (n < 0) return mi_set_error(MI_EINVAL, "mi_convert: negative length");
+    if (n == 0) return MI_OK;
+    if (!dst || !src) return mi_set_error(MI_EINVAL, "mi_convert: null pointer");
+    hipStream_t st = (hipStream_t)s;
+    if (dd == MI_F32) launch_convert_from<F32>(dst, src, ds, n, st);
+    else if (dd == MI_F16) launch_convert_from<F16>(dst, src, ds, n, st);
+    else launch_convert_from<BF16>(dst, src, ds, n, st);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+MI_API int32_t mi_make_causal_mask(uint8_t *m, int64_t len, mi_stream s) {
+    if (len < 0) return mi_set_error(MI_EINVAL, "mi_make_causal_mask: negative length");
+    if (len == 0) return MI_OK;
+    if (!m) return mi_set_error(MI_EINVAL, "mi_make_causal_mask: null pointer");
+    hipLaunchKernelGGL(causal_mask_kernel, dim3(grid_for(len * len)), dim3(256), 0, (hipStream_t)s, m, len);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}

@@ -1,0 +1,14 @@
+"""Python mirror of NNlib.jl's attention-path operators on MI355X (gfx950).
+
+Host-side stand-in for the Julia module: same operator names and semantics, column-major
+Julia-shaped arrays, all computation behind the C ABI of ``libmi355attn.so``.
+"""
+from . import _lib
+from ._lib import ArgumentError, DimensionMismatch, MIError
+from .array import BatchedTranspose, CausalMask, DeviceArray, batched_adjoint, batched_transpose
+from .ops import (batched_mul, batched_mul_, dot_product_attention, dot_product_attention_scores,
+                  last_attention_kernel, make_causal_mask, softmax, softmax_)
+
+__all__ = ["ArgumentError", "DimensionMismatch", "MIError", "DeviceArray", "BatchedTranspose", "CausalMask",
+           "batched_adjoint", "batched_transpose", "batched_mul", "batched_mul_", "dot_product_attention",
+           "dot_product_attention_scores", "last_attention_kernel", "make_causal_mask", "softmax", "softmax_"]

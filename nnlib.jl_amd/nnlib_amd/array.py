@@ -1,0 +1,179 @@
+"""Julia-shaped device arrays for the Python mirror of the NNlib attention API.
+
+A ``DeviceArray`` has a Julia ``size`` tuple and column-major memory, exactly as the arrays the
+reference operates on; element ``(i1, i2, ...)`` is at ``i1 + i2*size[0] + ...``.  PyTorch is used
+only as the owner of the device allocation (and for host<->device copies).
+"""
+import numpy as np
+import torch
+
+from . import _lib
+
+_TORCH = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "bool": torch.uint8}
+_CODE = {"f32": _lib.MI_F32, "f16": _lib.MI_F16, "bf16": _lib.MI_BF16}
+_NP2NAME = {np.dtype(np.float32): "f32", np.dtype(np.float16): "f16", np.dtype(np.bool_): "bool",
+            np.dtype(np.uint8): "bool"}
+
+
+def _require_gpu():
+    if not torch.cuda.is_available():
+        raise RuntimeError("nnlib_amd needs a GPU (torch.cuda.is_available() is False); there is no CPU path")
+
+
+class DeviceArray:
+    """Column-major array in device memory.
+
+    ``dims`` is the Julia size; ``strides`` are element strides (Julia ``strides``), which lets
+    ``batched_transpose`` and friends be lazy views like the reference's wrappers
+    (src/batched/batchedadjtrans.jl:23-92)."""
+
+    def __init__(self, storage, dims, dtype, strides=None, offset=0):
+        self.storage = storage          # 1-D torch tensor that owns the memory
+        self.dims = tuple(int(d) for d in dims)
+        self.dtype = dtype              # "f32" | "f16" | "bf16" | "bool"
+        if strides is None:
+            strides, acc = [], 1
+            for d in self.dims:
+                strides.append(acc)
+                acc *= d
+        self.strides = tuple(int(s) for s in strides)
+        self.offset = int(offset)       # in elements
+
+    # ---- construction --------------------------------------------------------------------
+    @classmethod
+    def empty(cls, dims, dtype="f32"):
+        _require_gpu()
+        n = int(np.prod(dims, dtype=np.int64)) if len(dims) else 1
+        return cls(torch.empty(max(n, 1), dtype=_TORCH[dtype], device="cuda"), dims, dtype)
+
+    @classmethod
+    def zeros(cls, dims, dtype="f32"):
+        a = cls.empty(dims, dtype)
+        a.storage.zero_()
+        return a
+
+    @classmethod
+    def from_numpy(cls, a, dtype=None):
+        """``a`` is indexed like the Julia array (any memory order). ``dtype`` may narrow it
+        ("bf16" rounds to nearest even from the array's float values)."""
+        _require_gpu()
+        a = np.asarray(a)
+        if dtype is None:
+            if a.dtype not in _NP2NAME:
+                a = a.astype(np.float32)
+            dtype = _NP2NAME[a.dtype]
+        if dtype == "bool":
+            flat = np.ascontiguousarray(a.astype(np.uint8).ravel(order="F"))
+            t = torch.from_numpy(flat).cuda()
+        else:
+            src = a.astype(np.float32) if a.dtype not in (np.float32, np.float16) else a
+            flat = np.ascontiguousarray(src.ravel(order="F"))
+            t = torch.from_numpy(flat).cuda().to(_TORCH[dtype])
+        if t.numel() == 0:
+            t = torch.empty(1, dtype=_TORCH[dtype], device="cuda")
+        return cls(t, a.shape, dtype)
+
+    @classmethod
+    def from_torch(cls, t, dims, dtype):
+        """Wrap an existing 1-D (or contiguous) device tensor whose memory already is column-major ``dims``."""
+        return cls(t.reshape(-1), dims, dtype)
+
+    # ---- views ---------------------------------------------------------------------------
+    @property
+    def ndim(self):
+        return len(self.dims)
+
+    def size(self, d=None):
+        return self.dims if d is None else (self.dims[d - 1] if d <= len(self.dims) else 1)
+
+    @property
+    def length(self):
+        return int(np.prod(self.dims, dtype=np.int64)) if self.dims else 1
+
+    def is_contiguous(self):
+        acc = 1
+        for d, s in zip(self.dims, self.strides):
+            if d != 1 and s != acc:
+                return False
+            acc *= d
+        return True
+
+    def reshape(self, *dims):
+        if len(dims) == 1 and isinstance(dims[0], (tuple, list)):
+            dims = tuple(dims[0])
+        if -1 in dims:
+            known = int(np.prod([d for d in dims if d != -1], dtype=np.int64))
+            dims = tuple(self.length // max(known, 1) if d == -1 else d for d in dims)
+        assert self.is_contiguous(), "reshape needs a contiguous array"
+        assert int(np.prod(dims, dtype=np.int64)) == self.length, "reshape must keep the element count"
+        return DeviceArray(self.storage, dims, self.dtype, None, self.offset)
+
+    @property
+    def itemsize(self):
+        return self.storage.element_size()
+
+    @property
+    def ptr(self):
+        return self.storage.data_ptr() + self.offset * self.itemsize
+
+    @property
+    def code(self):
+        return _CODE[self.dtype]
+
+    # ---- host copies ---------------------------------------------------------------------
+    def to_numpy(self):
+        """Julia-shaped numpy array (Fortran order). bf16 comes back as float32, bool as bool."""
+        assert self.is_contiguous(), "materialise a lazy transpose before copying to the host"
+        flat = self.storage[self.offset:self.offset + self.length]
+        if self.dtype == "bf16":
+            flat = flat.float()
+        h = flat.cpu().numpy()
+        if self.dtype == "bool":
+            h = h.astype(bool)
+        return h.reshape(self.dims, order="F")
+
+    def __repr__(self):
+        return f"DeviceArray{{{self.dtype}}}{self.dims}"
+
+
+class BatchedTranspose(DeviceArray):
+    """Lazy per-slice transpose of a 3-D array (src/batched/batchedadjtrans.jl:23-52)."""
+
+    def __init__(self, parent):
+        assert parent.ndim == 3, "batched_transpose expects a 3-D array"
+        d, s = parent.dims, parent.strides
+        super().__init__(parent.storage, (d[1], d[0], d[2]), parent.dtype, (s[1], s[0], s[2]), parent.offset)
+        self.parent = parent
+
+
+def batched_transpose(A):
+    """batched_transpose(A) (src/batched/batchedadjtrans.jl:37-38); transposing twice unwraps."""
+    return A.parent if isinstance(A, BatchedTranspose) else BatchedTranspose(A)
+
+
+def batched_adjoint(A):
+    """batched_adjoint(A): all element types here are real, so it equals batched_transpose
+    (src/batched/batchedadjtrans.jl:50-51)."""
+    return batched_transpose(A)
+
+
+class CausalMask:
+    """What ``make_causal_mask`` returns for device arrays: the (len, len) pattern
+    ``m[i, j] = i <= j`` (src/attention.jl:145) kept symbolic so that the attention kernel can
+    apply it from indices instead of reading len*len bytes.  ``materialize()`` gives the dense
+    Bool array the reference would have produced."""
+
+    def __init__(self, length):
+        self.length = int(length)
+        self.dims = (self.length, self.length)
+
+    def size(self, d=None):
+        return self.dims if d is None else (self.dims[d - 1] if d <= 2 else 1)
+
+    def materialize(self):
+        out = DeviceArray.empty(self.dims, "bool")
+        _lib.check(_lib.load().mi_make_causal_mask(out.ptr, self.length, None))
+        return out
+
+    def to_numpy(self):
+        return self.materialize().to_numpy()

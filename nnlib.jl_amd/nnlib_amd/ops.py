@@ -1,0 +1,303 @@
+"""Python mirror of the reference's operator interface for the attention path.
+
+Same names, argument meaning and error behaviour as NNlib.jl (citations are paths in the
+NNlib.jl source tree).  Every function marshals arguments and calls the C ABI
+(``include/mi355attn.h``); all arithmetic happens in the HIP kernels.
+"""
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+from ._lib import ArgumentError, DimensionMismatch
+from .array import BatchedTranspose, CausalMask, DeviceArray
+
+__all__ = ["dot_product_attention", "dot_product_attention_scores", "make_causal_mask", "softmax", "softmax_",
+           "batched_mul", "batched_mul_", "last_attention_kernel"]
+
+_last_kernel = None
+_workspace = None
+
+
+def identity(x):
+    return x
+
+
+def last_attention_kernel():
+    """Name of the kernel family the most recent attention call dispatched to."""
+    return _lib.KERNEL_NAMES.get(_last_kernel)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _get_workspace(nbytes):
+    global _workspace
+    if nbytes == 0:
+        return None, 0
+    if _workspace is None or _workspace.numel() < nbytes:
+        _workspace = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    return _workspace, _workspace.numel()
+
+
+def _broadcast_strides(x, target, what):
+    """Element strides of ``x`` against the 4-D score tensor ``target`` = (kv, q, H, B); 0 where
+    ``x`` has extent 1.  Julia broadcasting raises DimensionMismatch otherwise."""
+    dims = tuple(x.dims) + (1,) * (4 - len(x.dims))
+    strides = tuple(x.strides) + (0,) * (4 - len(x.strides))
+    if len(dims) > 4 and any(d != 1 for d in dims[4:]):
+        raise DimensionMismatch(f"{what} of size {x.dims} is not broadcastable to {target}")
+    out = []
+    for d, s, t in zip(dims[:4], strides[:4], target):
+        if d == 1:
+            out.append(0)
+        elif d == t:
+            out.append(s)
+        else:
+            raise DimensionMismatch(f"arrays could not be broadcast to a common size: {what} has size {x.dims}, "
+                                    f"attention scores have size {target}")
+    return out
+
+
+def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_weights, weights_dtype, flags):
+    """One mi_attention_fwd call on flattened (F, L, B) operands."""
+    global _last_kernel
+    lib = _lib.load()
+    d = _lib.mi_attn_desc()
+    d.struct_size = ctypes.sizeof(_lib.mi_attn_desc)
+    d.dtype = q.code
+    d.flags = flags
+    d.E, d.Ev, d.Lq, d.Lkv, d.H, d.B = E, Ev, Lq, Lkv, H, B
+    d.q, d.k = q.ptr, k.ptr
+    d.v = v.ptr if v is not None else None
+    target = (Lkv, Lq, H, B)
+    keep = [q, k, v]
+    if bias is not None:
+        if bias.dtype != q.dtype:
+            raise ArgumentError(f"bias must have the element type of q ({q.dtype}), got {bias.dtype}")
+        st = _broadcast_strides(bias, target, "bias")
+        d.bias = bias.ptr
+        d.bias_strides = (ctypes.c_int64 * 4)(*st)
+    d.causal = 0
+    if isinstance(mask, CausalMask):
+        if mask.length != Lkv or mask.length != Lq:
+            raise DimensionMismatch(f"arrays could not be broadcast to a common size: mask has size {mask.dims}, "
+                                    f"attention scores have size {target}")
+        d.causal = 1
+    elif mask is not None:
+        if mask.dtype != "bool":
+            raise ArgumentError("mask must be a Bool array")
+        st = _broadcast_strides(mask, target, "mask")
+        d.mask = mask.ptr
+        d.mask_strides = (ctypes.c_int64 * 4)(*st)
+    out = DeviceArray.empty((Ev, Lq, B), q.dtype) if want_out else None
+    wdt = weights_dtype or q.dtype
+    alpha = DeviceArray.empty((Lkv, Lq, H, B), wdt) if want_weights else None
+    d.out = out.ptr if out is not None else None
+    d.weights = alpha.ptr if alpha is not None else None
+    d.weights_dtype = alpha.code if alpha is not None else q.code
+    kernel, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
+    _lib.check(lib.mi_attention_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))
+    wbuf, wsize = _get_workspace(ws.value)
+    if wbuf is not None:
+        d.workspace, d.workspace_bytes = wbuf.data_ptr(), wsize
+    _lib.check(lib.mi_attention_fwd(ctypes.byref(d), _stream()))
+    _last_kernel = kernel.value
+    del keep
+    return out, alpha
+
+
+def _contig(x, name):
+    if not isinstance(x, DeviceArray):
+        raise ArgumentError(f"{name} must be a DeviceArray")
+    if not x.is_contiguous():
+        raise ArgumentError(f"{name} must be a dense column-major array")
+    return x
+
+
+def dot_product_attention(q, k, v, bias=None, *, fdrop=identity, mask=None, nheads=1, return_weights=True,
+                          weights_dtype=None, _flags=0):
+    """dot_product_attention(query, key, value, [bias]; [fdrop, mask, nheads])  (src/attention.jl:40-84).
+
+    q (qk_dim, q_len, batch...), k (qk_dim, kv_len, batch...), v (v_dim, kv_len, batch...).
+    Returns ``(x, alpha)``: x (v_dim, q_len, batch...), alpha (kv_len, q_len, nheads, batch...).
+
+    Beyond the reference: ``return_weights=False`` skips materialising alpha (``None`` is returned
+    in its place) and ``weights_dtype="f32"`` asks for Float32 weights from 16-bit inputs."""
+    q, k, v = _contig(q, "q"), _contig(k, "k"), _contig(v, "v")
+    if not (q.ndim == k.ndim == v.ndim) or q.ndim < 2:
+        raise ArgumentError("query, key and value must have the same number of dimensions (at least 2)")
+    if not (q.dtype == k.dtype == v.dtype) or q.dtype == "bool":
+        raise ArgumentError("query, key and value must share a floating-point element type")
+    bq, bk, bv = q.dims[2:], k.dims[2:], v.dims[2:]
+    if not (bq == bk == bv):                                     # src/attention.jl:42, :63
+        raise ArgumentError("Batch dimensions have to be the same.")
+    B = int(np.prod(bq, dtype=np.int64)) if bq else 1
+    E, Lq, Lkv, Ev = q.dims[0], q.dims[1], k.dims[1], v.dims[0]
+    if E % nheads or k.dims[0] % nheads or Ev % nheads:          # src/attention.jl:55
+        raise ArgumentError("First dimension in query, key and value must be divisible by `nheads`.\n"
+                            f"Instead:\n- size(q): {q.dims}\n- size(k): {k.dims}\n- size(v): {v.dims}\n- nheads: {nheads}")
+    if E != k.dims[0]:                                           # src/attention.jl:69
+        raise ArgumentError("First dimension in query and key has to be the same. Instead:\n"
+                            f"- size(q): {q.dims}\n- size(k): {k.dims}")
+    if Lkv != v.dims[1]:                                         # src/attention.jl:74
+        raise ArgumentError("Second dimension in key and value has to be the same. Instead:\n"
+                            f"- size(k): {k.dims}\n- size(v): {v.dims}")
+    if fdrop is identity:
+        x, alpha = _attention_call(q, k, v, bias, mask, nheads, B, E, Ev, Lq, Lkv, True, return_weights,
+                                   weights_dtype, _flags)
+    else:
+        # alpha handed back is post-fdrop (src/attention.jl:126); the value product then runs as a
+        # batched GEMM on the caller-visible weights, as src/attention.jl:96-98 does.
+        _, alpha = _attention_call(q, k, None, bias, mask, nheads, B, E, Ev, Lq, Lkv, False, True, weights_dtype,
+                                   _flags)
+        alpha = fdrop(alpha)
+        x = _weights_times_values(alpha, v, nheads, B, Ev, Lq, Lkv)
+    x = x.reshape((Ev, Lq) + tuple(bq))
+    if alpha is not None:
+        alpha = alpha.reshape((Lkv, Lq, nheads) + tuple(bq))
+    return x, alpha
+
+
+def _weights_times_values(alpha, v, H, B, Ev, Lq, Lkv):
+    """x[d,h,i,b] = sum_j alpha[j,i,h,b] v[d,h,j,b] as strided batched GEMMs over heads, one per batch
+    (no permuted copies: a head of v is a (Dv, Lkv) matrix with column stride Ev)."""
+    if alpha.dtype != v.dtype:
+        raise ArgumentError("fdrop must keep the element type of the attention weights")
+    lib = _lib.load()
+    Dv = Ev // H
+    out = DeviceArray.empty((Ev, Lq, B), v.dtype)
+    es = v.itemsize
+    for b in range(B):
+        _lib.check(lib.mi_batched_gemm(v.code, b"N", b"N", Dv, Lq, Lkv, 1.0,
+                                       v.ptr + es * b * Ev * Lkv, Ev, Dv,
+                                       alpha.ptr + es * b * Lkv * Lq * H, Lkv, Lkv * Lq, 0.0,
+                                       out.ptr + es * b * Ev * Lq, Ev, Dv, H, _stream()), DimensionMismatch)
+    return out
+
+
+def dot_product_attention_scores(q, k, bias=None, *, fdrop=identity, mask=None, weights_dtype=None, _flags=0):
+    """dot_product_attention_scores(query, key, [bias]; [fdrop, mask])  (src/attention.jl:112-127).
+    Inputs are 4-D (num_features / nheads, nheads, sequence_length, batch_size)."""
+    q, k = _contig(q, "q"), _contig(k, "k")
+    if q.ndim != 4 or k.ndim != 4:
+        raise ArgumentError("dot_product_attention_scores expects 4-D (D, nheads, L, batch) arrays")
+    if q.dtype != k.dtype:
+        raise ArgumentError("query and key must share an element type")
+    D, H, Lq, B = q.dims
+    if k.dims[0] != D or k.dims[1] != H or k.dims[3] != B:
+        raise DimensionMismatch(f"query {q.dims} and key {k.dims} disagree in feature, head or batch size")
+    Lkv = k.dims[2]
+    _, alpha = _attention_call(q, k, None, bias, mask, H, B, D * H, D * H, Lq, Lkv, False, True, weights_dtype, _flags)
+    return fdrop(alpha)
+
+
+def make_causal_mask(x, *, dims=2):
+    """make_causal_mask(x; dims=2)  (src/attention.jl:149-153): square mask of side size(x, dims) with
+    m[i, j] = i <= j.  Returned lazily (see CausalMask); ``.materialize()`` gives the dense Bool array."""
+    return CausalMask(x.size(dims))
+
+
+# ---- softmax -------------------------------------------------------------------------------------
+
+def softmax(x, *, dims=1):
+    """softmax(x; dims=1)  (src/softmax.jl:56)."""
+    if not isinstance(x, DeviceArray):
+        # src/softmax.jl:215-218
+        raise ArgumentError("`softmax(x)` called with a number, but it expects an array.")
+    out = DeviceArray.empty(x.dims, x.dtype)
+    return softmax_(out, x, dims=dims)
+
+
+def softmax_(out, x=None, *, dims=1):
+    """softmax!(out, x; dims=1) and softmax!(x; dims=1)  (src/softmax.jl:64-66)."""
+    if x is None:
+        x = out
+    if dims != 1:
+        raise NotImplementedError("only dims=1 (the attention path) is built; other dims are out of scope")
+    x, out = _contig(x, "x"), _contig(out, "out")
+    if out.dims != x.dims:
+        raise DimensionMismatch(f"output size {out.dims} differs from input size {x.dims}")
+    if x.dtype == "bool" or out.dtype != x.dtype:
+        raise ArgumentError("softmax needs floating-point input and output of one element type")
+    rows = x.dims[0] if x.dims else 1
+    cols = x.length // rows if rows else 0
+    _lib.check(_lib.load().mi_softmax_dim1(x.code, x.ptr, out.ptr, rows, cols, _stream()))
+    return out
+
+
+# ---- batched_mul ---------------------------------------------------------------------------------
+
+def _blas_layout(X, name):
+    """('N' | 'T', leading dimension, batch stride) from strides, the decision table of
+    _batched_try_gemm! (src/batched/batchedmul.jl:272-294); layouts BLAS cannot address raise as
+    ext/NNlibAMDGPUExt/batched_mul.jl:1-9 does."""
+    s1, s2, s3 = X.strides
+    if s2 == 1 and X.dims[0] > 1:
+        flag, ld = b"T", s1
+    elif s1 == 1:
+        flag, ld = b"N", s2
+    elif s2 == 1:
+        flag, ld = b"T", s1
+    else:
+        raise ArgumentError(f"Unsupported array layout for batched mul.\n- Size: {X.dims}\n- Strides: {X.strides}")
+    rows = X.dims[0] if flag == b"N" else X.dims[1]
+    return flag, max(ld, rows, 1), s3
+
+
+def batched_mul_(C, A, B, alpha=1.0, beta=0.0):
+    """batched_mul!(C, A, B, alpha=1, beta=0)  (src/batched/batchedmul.jl:238-254)."""
+    if not (C.ndim == A.ndim == B.ndim) or C.ndim < 3:
+        raise DimensionMismatch("batched_mul! needs arrays of equal dimensionality (at least 3)")
+    if C.ndim > 3:
+        bs = C.dims[2:]
+        if A.dims[2:] != bs:
+            raise DimensionMismatch("batch size of A must match C")      # :246
+        if B.dims[2:] != bs:
+            raise DimensionMismatch("batch size of B must match C")      # :247
+        C3 = C.reshape(C.dims[0], C.dims[1], -1)
+        batched_mul_(C3, A.reshape(A.dims[0], A.dims[1], -1), B.reshape(B.dims[0], B.dims[1], -1), alpha, beta)
+        return C
+    if not (A.dtype == B.dtype == C.dtype) or A.dtype == "bool":
+        raise ArgumentError("batched_mul! needs one floating-point element type for A, B and C")
+    nb = C.dims[2]
+    if A.dims[2] not in (nb, 1):
+        raise DimensionMismatch("batch size mismatch: A != C")            # src/gemm.jl:99
+    if B.dims[2] not in (nb, 1):
+        raise DimensionMismatch("batch size mismatch: B != C")            # src/gemm.jl:100
+    m, ka = A.dims[0], A.dims[1]
+    kb, n = B.dims[0], B.dims[1]
+    if ka != kb or m != C.dims[0] or n != C.dims[1]:                      # src/gemm.jl:106-108
+        raise DimensionMismatch(f"A1 has size ({m},{ka}), B1 has size ({kb},{n}), C1 has size {C.dims[:2]}")
+    tA, lda, sA = _blas_layout(A, "A")
+    tB, ldb, sB = _blas_layout(B, "B")
+    if C.strides[0] != 1:
+        raise ArgumentError(f"Unsupported array layout for batched mul.\n- Size: {C.dims}\n- Strides: {C.strides}")
+    sA = 0 if A.dims[2] == 1 else sA                                     # src/gemm.jl:117-118
+    sB = 0 if B.dims[2] == 1 else sB
+    _lib.check(_lib.load().mi_batched_gemm(C.code, tA, tB, m, n, ka, float(alpha), A.ptr, lda, sA, B.ptr, ldb, sB,
+                                           float(beta), C.ptr, max(C.strides[1], m, 1), C.strides[2], nb, _stream()),
+               DimensionMismatch)
+    return C
+
+
+def batched_mul(A, B):
+    """batched_mul(A, B)  (src/batched/batchedmul.jl:47-60): C[:,:,k...] = A[:,:,k...] * B[:,:,k...];
+    a 3-D operand with batch extent 1 is shared by every batch."""
+    if not isinstance(A, DeviceArray) or not isinstance(B, DeviceArray):
+        raise ArgumentError("batched_mul expects DeviceArrays")
+    if A.ndim != B.ndim or A.ndim < 3:
+        raise DimensionMismatch("batched_mul needs two arrays of equal dimensionality (at least 3)")
+    if A.ndim > 3:
+        bs = A.dims[2:]
+        assert bs == B.dims[2:], "batch size has to be the same for the two arrays."   # :49
+        z = batched_mul(A.reshape(A.dims[0], A.dims[1], -1), B.reshape(B.dims[0], B.dims[1], -1))
+        return z.reshape((z.dims[0], z.dims[1]) + tuple(bs))
+    if not (A.dims[2] == B.dims[2] or A.dims[2] == 1 or B.dims[2] == 1):
+        raise DimensionMismatch("batch size mismatch: A != B")                          # :57-58
+    if A.dtype != B.dtype:
+        raise ArgumentError("batched_mul needs one element type for A and B")
+    C = DeviceArray.empty((A.dims[0], B.dims[1], max(A.dims[2], B.dims[2])), A.dtype)
+    return batched_mul_(C, A, B)

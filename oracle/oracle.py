@@ -1,0 +1,196 @@
+"""ctypes front end of the C oracle (``nnlib_oracle.c``) plus an independent numpy statement.
+
+TEST INFRASTRUCTURE ONLY.  Nothing under the product package imports this module; it is used
+by ``tests/``, by the smoke check and by the benchmark's CPU-baseline leg.
+
+Arrays follow the Julia convention of the reference: an array of Julia size ``(E, L, B)`` is a
+numpy array of shape ``(E, L, B)`` in Fortran (column-major) memory order.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+def build(force=False):
+    """Compile the C oracle next to its source (gcc, a second or two)."""
+    so = os.path.join(_HERE, "libnnlib_oracle.so")
+    if force and os.path.exists(so):
+        os.remove(so)
+    subprocess.run(["make", "-s", "-C", _HERE], check=True)
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        so = os.path.join(_HERE, "libnnlib_oracle.so")
+        if not os.path.exists(so):
+            build()
+        L = ctypes.CDLL(so)
+        i64, f32, f64, vp, ci = ctypes.c_int64, ctypes.c_float, ctypes.c_double, ctypes.c_void_p, ctypes.c_int
+        L.orc_batched_gemm_f32.argtypes = [ci, ci, i64, i64, i64, f32, vp, i64, i64, i64, vp, i64, i64, i64,
+                                           f32, vp, i64, i64, i64, ci]
+        L.orc_batched_gemm_f32.restype = None
+        L.orc_batched_gemm_f64.argtypes = [ci, ci, i64, i64, i64, f64, vp, i64, i64, vp, i64, i64, f64, vp,
+                                           i64, i64, i64]
+        L.orc_batched_gemm_f64.restype = None
+        L.orc_softmax_dim1_f32.argtypes = [vp, vp, i64, i64]
+        L.orc_softmax_dim1_f32.restype = None
+        L.orc_softmax_dim1_f64.argtypes = [vp, vp, i64, i64]
+        L.orc_softmax_dim1_f64.restype = None
+        L.orc_make_causal_mask.argtypes = [vp, i64]
+        L.orc_make_causal_mask.restype = None
+        L.orc_nnlib_attention_f32.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, ci]
+        L.orc_nnlib_attention_f32.restype = None
+        L.orc_attention_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp]
+        L.orc_attention_f64.restype = None
+        _LIB = L
+    return _LIB
+
+
+def _f(a, dt):
+    return np.asfortranarray(np.asarray(a, dtype=dt))
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def broadcast_strides(shape, target_ndim=4):
+    """Element strides (column-major) of an array broadcast against a ``target_ndim``-D tensor.
+
+    Dimensions of extent 1 (or missing trailing dimensions) get stride 0, which is how
+    Julia broadcasting treats them (reference src/attention.jl:131,137)."""
+    shape = tuple(shape) + (1,) * (target_ndim - len(shape))
+    out, acc = [], 1
+    for n in shape:
+        out.append(0 if n == 1 else acc)
+        acc *= n
+    return (ctypes.c_int64 * target_ndim)(*out)
+
+
+def _flatten3(x):
+    """(F, L, batch...) -> (F, L, prod(batch)) as the N-D method does (src/attention.jl:43)."""
+    x = np.asarray(x)
+    return x.reshape(x.shape[0], x.shape[1], -1, order="F")
+
+
+def make_causal_mask(length):
+    m = np.zeros((length, length), dtype=np.uint8, order="F")
+    lib().orc_make_causal_mask(_ptr(m), length)
+    return m.astype(bool)
+
+
+def softmax_dim1(x, dtype=np.float32):
+    x = _f(x, dtype)
+    rows = x.shape[0] if x.ndim else 1
+    cols = x.size // max(rows, 1)
+    y = np.empty_like(x, order="F")
+    fn = lib().orc_softmax_dim1_f32 if dtype == np.float32 else lib().orc_softmax_dim1_f64
+    fn(_ptr(x), _ptr(y), rows, cols)
+    return y
+
+
+def batched_gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, C=None, dtype=np.float32, nthreads=1):
+    """3-D column-major batched GEMM; a batch extent of 1 on A or B broadcasts."""
+    A, B = _f(A, dtype), _f(B, dtype)
+    m, ka = (A.shape[1], A.shape[0]) if transA else (A.shape[0], A.shape[1])
+    kb, n = (B.shape[1], B.shape[0]) if transB else (B.shape[0], B.shape[1])
+    assert ka == kb
+    batch = max(A.shape[2], B.shape[2])
+    if C is None:
+        C = np.zeros((m, n, batch), dtype=dtype, order="F")
+    else:
+        C = _f(C, dtype).copy(order="F")
+    sA = 0 if A.shape[2] == 1 else A.shape[0] * A.shape[1]
+    sB = 0 if B.shape[2] == 1 else B.shape[0] * B.shape[1]
+    if dtype == np.float32:
+        lib().orc_batched_gemm_f32(int(transA), int(transB), m, n, ka, alpha, _ptr(A), A.shape[0], sA, A.size,
+                                   _ptr(B), B.shape[0], sB, B.size, beta, _ptr(C), m, m * n, batch, nthreads)
+    else:
+        lib().orc_batched_gemm_f64(int(transA), int(transB), m, n, ka, alpha, _ptr(A), A.shape[0], sA,
+                                   _ptr(B), B.shape[0], sB, beta, _ptr(C), m, m * n, batch)
+    return C
+
+
+def _attention(q, k, v, bias, mask, nheads, dtype, want_out, nthreads):
+    bshape = tuple(np.shape(q)[2:])
+    q3, k3 = _f(_flatten3(q), dtype), _f(_flatten3(k), dtype)
+    v3 = _f(_flatten3(v), dtype) if v is not None else None
+    E, Lq, B = q3.shape
+    Lkv = k3.shape[1]
+    Ev = v3.shape[0] if v3 is not None else E
+    H = nheads
+    bs = ms = None
+    if bias is not None:
+        bias = _f(bias, dtype)
+        bs = broadcast_strides(bias.shape)
+    if mask is not None:
+        mask = np.asfortranarray(np.asarray(mask).astype(np.uint8))
+        ms = broadcast_strides(mask.shape)
+    alpha = np.empty((Lkv, Lq, H, B), dtype=dtype, order="F")
+    out = np.empty((Ev, Lq, B), dtype=dtype, order="F") if want_out else None
+    if dtype == np.float32:
+        lib().orc_nnlib_attention_f32(_ptr(q3), _ptr(k3), _ptr(v3), _ptr(bias), bs, _ptr(mask), ms,
+                                      E, Ev, Lq, Lkv, H, B, _ptr(out), _ptr(alpha), nthreads)
+    else:
+        lib().orc_attention_f64(_ptr(q3), _ptr(k3), _ptr(v3), _ptr(bias), bs, _ptr(mask), ms,
+                                E, Ev, Lq, Lkv, H, B, _ptr(out), _ptr(alpha))
+    alpha = alpha.reshape((Lkv, Lq, H) + bshape, order="F")
+    if want_out:
+        out = out.reshape((Ev, Lq) + bshape, order="F")
+    return out, alpha
+
+
+def nnlib_attention_f32(q, k, v, bias=None, mask=None, nheads=1, nthreads=1):
+    """The reference's op sequence in Float32 (src/attention.jl:52-127). Returns (x, alpha)."""
+    return _attention(q, k, v, bias, mask, nheads, np.float32, True, nthreads)
+
+
+def attention_f64(q, k, v, bias=None, mask=None, nheads=1):
+    """Defining formula in double precision. Returns (x, alpha)."""
+    return _attention(q, k, v, bias, mask, nheads, np.float64, True, 1)
+
+
+def scores4_f64(q4, k4, bias=None, mask=None):
+    """dot_product_attention_scores on 4-D (D, H, L, B) inputs (src/attention.jl:112-127)."""
+    q4, k4 = np.asarray(q4), np.asarray(k4)
+    D, H, Lq, B = q4.shape
+    q3 = q4.reshape(D * H, Lq, B, order="F")
+    k3 = k4.reshape(D * H, k4.shape[2], B, order="F")
+    return _attention(q3, k3, None, bias, mask, H, np.float64, False, 1)[1]
+
+
+# ---------------------------------------------------------------------------------------------
+# Independent numpy statement (no C involved): used to cross-check the C oracle itself.
+# ---------------------------------------------------------------------------------------------
+
+def numpy_attention(q, k, v, bias=None, mask=None, nheads=1):
+    """x[d,h,i,b] = sum_j softmax_j(sum_d k[d,h,j,b] q[d,h,i,b]/sqrt(D) + bias, masked) v[d,h,j,b]
+    evaluated with einsum in float64 on Julia-shaped arrays."""
+    bshape = tuple(np.shape(q)[2:])
+    q3, k3, v3 = (_flatten3(np.asarray(a, dtype=np.float64)) for a in (q, k, v))
+    E, Lq, B = q3.shape
+    Lkv, Ev, H = k3.shape[1], v3.shape[0], nheads
+    D, Dv = E // H, Ev // H
+    q4 = q3.reshape(D, H, Lq, B, order="F")
+    k4 = k3.reshape(D, H, Lkv, B, order="F")
+    v4 = v3.reshape(Dv, H, Lkv, B, order="F")
+    logits = np.einsum("dhjb,dhib->jihb", k4, q4 / np.sqrt(np.float64(D)))
+    if bias is not None:
+        b = np.asarray(bias, dtype=np.float64)
+        logits = logits + b.reshape(b.shape + (1,) * (4 - b.ndim))
+    if mask is not None:
+        m = np.asarray(mask, dtype=bool)
+        logits = np.where(m.reshape(m.shape + (1,) * (4 - m.ndim)), logits, -np.inf)
+    with np.errstate(invalid="ignore", over="ignore"):
+        mx = logits.max(axis=0, keepdims=True)
+        e = np.where(np.isposinf(mx), np.where(np.isposinf(logits), 1.0, 0.0), np.exp(logits - mx))
+        alpha = e / e.sum(axis=0, keepdims=True)
+    x = np.einsum("jihb,dhjb->dhib", alpha, v4).reshape(Ev, Lq, B, order="F")
+    return x.reshape((Ev, Lq) + bshape, order="F"), alpha.reshape((Lkv, Lq, H) + bshape, order="F")

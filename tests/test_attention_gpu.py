@@ -1,0 +1,227 @@
+"""GPU parity of dot_product_attention / dot_product_attention_scores against the CPU oracle.
+
+Patterned on the reference's own tests (test/attention.jl, test/ext_amdgpu/attention.jl).
+Tolerances: Float32 max error <= 1e-4 of output scale; Float16/BFloat16 <= 1e-2 against the
+Float32 CPU result on the same (already rounded) inputs; weight columns sum to 1 within 1e-5
+(checked on Float32 weights).
+"""
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+
+from conftest import rel_err, round_to
+
+pytestmark = pytest.mark.gpu
+TOL = {"f32": 1e-4, "f16": 1e-2, "bf16": 1e-2}
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _run(nn, q, k, v, dtype, bias=None, mask=None, nheads=1, causal=False, **kw):
+    dq, dk, dv = (nn.DeviceArray.from_numpy(a, dtype) for a in (q, k, v))
+    db = nn.DeviceArray.from_numpy(bias, dtype) if bias is not None else None
+    if causal:
+        dm = nn.make_causal_mask(dq, dims=2)
+    else:
+        dm = nn.DeviceArray.from_numpy(mask) if mask is not None else None
+    y, a = nn.dot_product_attention(dq, dk, dv, db, mask=dm, nheads=nheads, **kw)
+    return y.to_numpy(), (a.to_numpy() if a is not None else None)
+
+
+def _check(nn, oracle, rng, dtype, E, Lq, Lkv, B, H, *, Ev=None, causal=False, bias_shape=None, mask_shape=None,
+           scale=1.0, expect=None, weights=True, batch_shape=None, flags=0):
+    Ev = Ev or E
+    bs = batch_shape if batch_shape is not None else (B,)
+    q = round_to(rng.standard_normal((E, Lq) + bs) * scale, dtype)
+    k = round_to(rng.standard_normal((E, Lkv) + bs) * scale, dtype)
+    v = round_to(rng.standard_normal((Ev, Lkv) + bs), dtype)
+    bias = round_to(0.5 * rng.standard_normal(bias_shape), dtype) if bias_shape else None
+    mask = None
+    if mask_shape:
+        mask = rng.random(mask_shape) < 0.9
+        mask[0, ...] = True          # no fully masked column
+    omask = mask
+    if causal:
+        omask = oracle.make_causal_mask(Lq)
+    y, a = _run(nn, q, k, v, dtype, bias, mask, H, causal, return_weights=weights,
+                weights_dtype="f32" if weights else None, _flags=flags)
+    if expect:
+        assert nn.last_attention_kernel() == expect, nn.last_attention_kernel()
+    yr, ar = oracle.nnlib_attention_f32(q, k, v, bias, omask, H, nthreads=8)
+    assert y.shape == yr.shape
+    yerr = rel_err(y, yr)
+    assert yerr <= TOL[dtype], (yerr, nn.last_attention_kernel())
+    if weights:
+        assert a.shape == ar.shape
+        werr = float(np.abs(a - ar).max())
+        assert werr <= TOL[dtype], werr
+        colsum_err = float(np.abs(a.sum(axis=0) - 1).max())
+        assert colsum_err <= 1e-5, colsum_err
+        if omask is not None:
+            keep = np.broadcast_to(np.asarray(omask).reshape(omask.shape + (1,) * (a.ndim - omask.ndim)), a.shape)
+            n_leaked = int(np.count_nonzero(a[~keep]))
+            assert n_leaked == 0, n_leaked
+    return y, a
+
+
+def test_specific_results(nn):
+    """Golden vectors of test/attention.jl:25-34."""
+    g = json.load(open(os.path.join(GOLD, "attention_specific_results.json")))
+    q = (np.arange(1, 13, dtype=np.float32) / 12).reshape(4, 3, 1, order="F")
+    y, a = _run(nn, q, q, q, "f32", nheads=2)
+    assert np.abs(y - np.array(g["ytrue"]).reshape(4, 3, 1, order="F")).max() < 1e-5
+    assert np.abs(a - np.array(g["alphatrue"]).reshape(3, 3, 2, 1, order="F")).max() < 1e-5
+
+
+@pytest.mark.parametrize("batch_shape", [(), (1,), (2,), (2, 1, 3)])
+@pytest.mark.parametrize("nheads", [1, 3, 5])
+def test_different_batchsizes(nn, oracle, batch_shape, nheads):
+    """Shape grid of test/attention.jl:1-15 and test/ext_amdgpu/attention.jl:1-23."""
+    rng = np.random.default_rng(0)
+    n, lenq, lenkv = 15, 3, 4
+    q = rng.random((n, lenq) + batch_shape, dtype=np.float32)
+    k = rng.random((n, lenkv) + batch_shape, dtype=np.float32)
+    v = rng.random((n, lenkv) + batch_shape, dtype=np.float32)
+    y, a = _run(nn, q, k, v, "f32", nheads=nheads)
+    assert y.shape == (n, lenq) + batch_shape
+    assert a.shape == (lenkv, lenq, nheads) + batch_shape
+    assert np.allclose(a.sum(axis=0), 1, atol=1e-6)
+    yr, ar = oracle.nnlib_attention_f32(q, k, v, nheads=nheads)
+    assert np.abs(y - yr).max() < 1e-5 and np.abs(a - ar).max() < 1e-5
+
+
+def test_scores_equal_attention_weights(nn):
+    """test/attention.jl:17-23."""
+    q = (np.arange(1, 25, dtype=np.float32) / 24).reshape(4, 2, 3, 1, order="F")
+    dq = nn.DeviceArray.from_numpy(q)
+    a = nn.dot_product_attention_scores(dq, dq).to_numpy()
+    q2 = nn.DeviceArray.from_numpy(q.reshape(8, 3, 1, order="F"))
+    _, a2 = nn.dot_product_attention(q2, q2, q2, nheads=2)
+    assert np.allclose(a, a2.to_numpy(), atol=1e-6)
+
+
+def test_mask_zero_pattern(nn):
+    """test/attention.jl:36-52: weights are positive exactly where the mask keeps."""
+    rng = np.random.default_rng(1)
+    q = rng.random((4, 2, 3, 1), dtype=np.float32)
+    k = rng.random((4, 2, 5, 1), dtype=np.float32)
+    mask = rng.random((5, 3)) < 0.5
+    mask[0, :] = True
+    a = nn.dot_product_attention_scores(nn.DeviceArray.from_numpy(q), nn.DeviceArray.from_numpy(k),
+                                        mask=nn.DeviceArray.from_numpy(mask)).to_numpy()
+    assert np.all((a[:, :, 0, 0] > 0) == mask) and np.all((a[:, :, 1, 0] > 0) == mask)
+    x = nn.DeviceArray.from_numpy(rng.random((4, 2, 3, 1), dtype=np.float32))
+    cm = nn.make_causal_mask(x, dims=3)
+    a = nn.dot_product_attention_scores(x, x, mask=cm).to_numpy()
+    dense = cm.to_numpy()
+    assert dense.dtype == bool and np.array_equal(dense, np.triu(np.ones((3, 3), bool)))
+    assert np.all((a[:, :, 0, 0] > 0) == dense) and np.all((a[:, :, 1, 0] > 0) == dense)
+
+
+def test_bias_shapes(nn, oracle):
+    """test/attention.jl:61-68."""
+    rng = np.random.default_rng(2)
+    q = rng.random((4, 5, 1), dtype=np.float32)
+    k = rng.random((4, 3, 1), dtype=np.float32)
+    bias = rng.standard_normal((3, 5)).astype(np.float32)
+    y, a = _run(nn, q, k, k, "f32", bias=bias, nheads=2)
+    assert a.shape == (3, 5, 2, 1) and y.shape == (4, 5, 1)
+    yr, ar = oracle.nnlib_attention_f32(q, k, k, bias, None, 2)
+    assert np.abs(y - yr).max() < 1e-5 and np.abs(a - ar).max() < 1e-5
+
+
+def test_dropout_path(nn):
+    """test/attention.jl:54-59: a non-identity fdrop runs scores -> fdrop -> batched_mul, and the
+    returned weights are the dropped ones."""
+    rng = np.random.default_rng(3)
+    x = nn.DeviceArray.from_numpy(rng.random((10, 10, 10), dtype=np.float32))
+
+    def fdrop(alpha, p=0.5):
+        h = alpha.to_numpy()
+        keep = np.random.default_rng(4).random(h.shape) > p
+        return nn.DeviceArray.from_numpy((keep * h / (1 - p)).astype(np.float32))
+
+    y, a = nn.dot_product_attention(x, x, x, nheads=2, fdrop=fdrop)
+    a = a.to_numpy()
+    assert 0.4 < np.mean(a > 0) < 0.6
+    v4 = x.to_numpy().reshape(5, 2, 10, 10, order="F")
+    ref = np.einsum("jihb,dhjb->dhib", a, v4).reshape(10, 10, 10, order="F")
+    assert np.abs(y.to_numpy() - ref).max() < 1e-5
+
+
+def test_errors(nn):
+    """ArgumentError conditions of src/attention.jl:42,55-78."""
+    z = lambda *d: nn.DeviceArray.zeros(d)
+    with pytest.raises(nn.ArgumentError, match="divisible"):
+        nn.dot_product_attention(z(6, 3, 1), z(6, 4, 1), z(6, 4, 1), nheads=4)
+    with pytest.raises(nn.ArgumentError, match="Batch dimensions"):
+        nn.dot_product_attention(z(6, 3, 2), z(6, 4, 1), z(6, 4, 1))
+    with pytest.raises(nn.ArgumentError, match="query and key"):
+        nn.dot_product_attention(z(6, 3, 1), z(4, 4, 1), z(6, 4, 1))
+    with pytest.raises(nn.ArgumentError, match="key and value"):
+        nn.dot_product_attention(z(6, 3, 1), z(6, 4, 1), z(6, 5, 1))
+    with pytest.raises(nn.DimensionMismatch):
+        nn.dot_product_attention(z(6, 3, 1), z(6, 4, 1), z(6, 4, 1), z(5, 3))
+
+
+# ---- MFMA flash kernels against the oracle ---------------------------------------------------------
+
+FLASH16_CASES = [
+    # dtype, E, Lq, Lkv, B, H, kwargs
+    ("bf16", 256, 128, 128, 2, 2, {}),
+    ("bf16", 256, 200, 333, 1, 2, {}),                       # ragged tails in both lengths
+    ("bf16", 256, 256, 256, 2, 2, dict(causal=True)),
+    ("bf16", 256, 130, 130, 1, 2, dict(causal=True)),
+    ("f16", 128, 96, 160, 2, 2, {}),
+    ("f16", 128, 192, 192, 1, 2, dict(causal=True)),
+    ("f16", 128, 64, 320, 2, 2, dict(bias_shape=(320, 64, 2, 2), mask_shape=(320, 64))),
+    ("f16", 128, 70, 131, 2, 2, dict(bias_shape=(131, 70), mask_shape=(131, 70, 1, 2))),   # unaligned strides
+    ("bf16", 128, 64, 256, 1, 1, dict(bias_shape=(256, 1, 1, 1))),
+    ("bf16", 256, 128, 128, 1, 2, dict(causal=True, mask_shape=(128, 128))),
+    ("f16", 64, 33, 65, 3, 1, {}),
+]
+
+
+@pytest.mark.parametrize("case", FLASH16_CASES, ids=lambda c: f"{c[0]}-E{c[1]}-Lq{c[2]}-Lkv{c[3]}-B{c[4]}-H{c[5]}-" + "-".join(c[6]))
+@pytest.mark.parametrize("weights", [False, True], ids=["noweights", "weights"])
+def test_flash16_parity(nn, oracle, case, weights):
+    dtype, E, Lq, Lkv, B, H, kw = case
+    rng = np.random.default_rng(hash((E, Lq, Lkv, B, H)) % 2**32)
+    _check(nn, oracle, rng, dtype, E, Lq, Lkv, B, H, expect="flash16", weights=weights, **kw)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_generic_kernel_parity(nn, oracle, dtype):
+    """The generic kernel on a shape the MFMA kernels do not take (head dims 24 / 40)."""
+    rng = np.random.default_rng(7)
+    _check(nn, oracle, rng, dtype, 48, 37, 75, 2, 2, Ev=80, bias_shape=(75, 37, 2, 1), mask_shape=(75, 37),
+           expect="generic")
+
+
+def test_flash16_matches_generic_on_device(nn):
+    """Both kernels on identical device buffers (bf16, causal)."""
+    rng = np.random.default_rng(8)
+    q, k, v = (nn.DeviceArray.from_numpy(rng.standard_normal((256, 192, 2)).astype(np.float32), "bf16") for _ in range(3))
+    cm = nn.make_causal_mask(q)
+    y1, a1 = nn.dot_product_attention(q, k, v, mask=cm, nheads=2, weights_dtype="f32")
+    assert nn.last_attention_kernel() == "flash16"
+    y2, a2 = nn.dot_product_attention(q, k, v, mask=cm, nheads=2, weights_dtype="f32", _flags=1)
+    assert nn.last_attention_kernel() == "generic"
+    assert rel_err(y1.to_numpy(), y2.to_numpy()) < 1e-2
+    assert np.abs(a1.to_numpy() - a2.to_numpy()).max() < 1e-2
+
+
+def test_fully_masked_column_is_nan(nn):
+    """src/softmax.jl:73-75 gives exp(-Inf - -Inf) = NaN for an all-dropped column (by code reading;
+    no reference test pins it).  Both kernel families must agree with that."""
+    rng = np.random.default_rng(9)
+    for dtype, E, H, flags in (("f32", 16, 2, 0), ("bf16", 128, 1, 0)):
+        q = rng.standard_normal((E, 40, 1)).astype(np.float32)
+        k = rng.standard_normal((E, 70, 1)).astype(np.float32)
+        mask = np.ones((70, 40), bool)
+        mask[:, 5] = False
+        y, a = _run(nn, q, k, k, dtype, mask=mask, nheads=H, weights_dtype="f32")
+        assert np.isnan(y[:, 5, 0]).all() and np.isnan(a[:, 5]).all()
+        assert np.isfinite(np.delete(y, 5, axis=1)).all()
