@@ -1,0 +1,246 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5] [--no-cpu]
+
+A "step" is one dot_product_attention call on synthetic inputs that are already resident in HBM.
+The default workload is C3 (bf16 causal prefill, head dim 128, L = 4096), the configuration the
+prefill target is quoted on; the decode workload C5 is measured in the same run and reported under
+"decode" in the same JSON line.  Timing is by HIP events on the stream the kernels are launched on.
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "nnlib.jl_amd"))
+
+PEAK = {"bf16": 2516.0, "f16": 2516.0, "f32": 157.3}   # dense MFMA TFLOP/s
+HBM_PEAK = 8000.0                                       # GB/s
+
+# name -> description of BASELINE.json's configs
+WORKLOADS = {
+    "c1": dict(name="C1 self-attention f32 (512,128,4) H=8, weights returned", dtype="f32", E=512, Lq=128, Lkv=128,
+               B=4, H=8, causal=False, weights=True, scale=1.0, seed=0x5EED0000),
+    "c2": dict(name="C2 causal self-attention f32 (1024,1024,8) H=16, weights returned", dtype="f32", E=1024,
+               Lq=1024, Lkv=1024, B=8, H=16, causal=True, weights=True, scale=0.125, seed=0x5EED0001),
+    "c3": dict(name="C3 causal prefill bf16 (4096,4096,2) H=32 D=128, weights not materialised", dtype="bf16",
+               E=4096, Lq=4096, Lkv=4096, B=2, H=32, causal=True, weights=False, scale=1.0, seed=0x5EED0002),
+    "c4": dict(name="C4 cross-attention f16 q(1024,256,4) kv(1024,8192,4) H=16 + bias (8192,256,16,4) + mask (8192,256)",
+               dtype="f16", E=1024, Lq=256, Lkv=8192, B=4, H=16, causal=False, weights=False, scale=1.0,
+               bias=True, mask=True, seed=0x5EED0003),
+    "c5": dict(name="C5 decode bf16 q(4096,1,16) kv(4096,32768,16) H=32 D=128", dtype="bf16", E=4096, Lq=1,
+               Lkv=32768, B=16, H=32, causal=False, weights=False, scale=1.0, seed=0x5EED0004),
+}
+
+
+def algorithmic_work(w):
+    """(FLOPs, compulsory HBM bytes) of one call: 4*Lq*Lkv*D*H*B FLOP (QK^T and PV; causal counts the
+    unmasked triangle only), every input read once and every output written once."""
+    E, Lq, Lkv, B, H = w["E"], w["Lq"], w["Lkv"], w["B"], w["H"]
+    D = E // H
+    es = 4 if w["dtype"] == "f32" else 2
+    pairs = Lq * (Lq + 1) // 2 if w["causal"] else Lq * Lkv
+    flops = 4 * D * H * B * pairs
+    nbytes = es * (E * Lq * B + 2 * E * Lkv * B + E * Lq * B)
+    if w["weights"]:
+        nbytes += es * Lkv * Lq * H * B
+    if w.get("bias"):
+        nbytes += es * Lkv * Lq * H * B
+    if w.get("mask"):
+        nbytes += Lkv * Lq
+    if w["causal"] and w["weights"]:
+        nbytes += Lq * Lkv   # the dense Bool mask the reference would read
+    return flops, nbytes
+
+
+class Runner:
+    """Owns the device buffers of one workload and launches it through the C ABI."""
+
+    def __init__(self, key):
+        import torch
+        import nnlib_amd
+        from nnlib_amd import _lib
+        self.torch, self.nn, self._lib = torch, nnlib_amd, _lib
+        self.lib = _lib.load()
+        _lib.check(self.lib.mi_init(0))
+        w = self.w = WORKLOADS[key]
+        dt = w["dtype"]
+        E, Lq, Lkv, B, H = w["E"], w["Lq"], w["Lkv"], w["B"], w["H"]
+        DA = nnlib_amd.DeviceArray
+        self.q, self.k, self.v = DA.empty((E, Lq, B), dt), DA.empty((E, Lkv, B), dt), DA.empty((E, Lkv, B), dt)
+        for sid, a in enumerate((self.q, self.k, self.v)):
+            sc = w["scale"] if sid < 2 else 1.0
+            _lib.check(self.lib.mi_randn_fill(a.ptr, a.code, a.length, w["seed"], sid, sc, None))
+        self.bias = self.mask = None
+        if w.get("bias"):
+            self.bias = DA.empty((Lkv, Lq, H, B), dt)
+            _lib.check(self.lib.mi_randn_fill(self.bias.ptr, self.bias.code, self.bias.length, w["seed"], 3, 0.5, None))
+        if w.get("mask"):
+            self.mask = DA.empty((Lkv, Lq), "bool")
+            _lib.check(self.lib.mi_bernoulli_fill(self.mask.ptr, self.mask.length, w["seed"], 4, 0.9, None))
+        self.out = DA.empty((E, Lq, B), dt)
+        self.alpha = DA.empty((Lkv, Lq, H, B), dt) if w["weights"] else None
+        d = self.desc = _lib.mi_attn_desc()
+        d.struct_size = ctypes.sizeof(_lib.mi_attn_desc)
+        d.dtype = self.q.code
+        d.weights_dtype = self.q.code
+        d.causal = int(w["causal"])
+        d.E, d.Ev, d.Lq, d.Lkv, d.H, d.B = E, E, Lq, Lkv, H, B
+        d.q, d.k, d.v, d.out = self.q.ptr, self.k.ptr, self.v.ptr, self.out.ptr
+        d.weights = self.alpha.ptr if self.alpha is not None else None
+        if self.bias is not None:
+            d.bias = self.bias.ptr
+            d.bias_strides = (ctypes.c_int64 * 4)(1, Lkv, Lkv * Lq, Lkv * Lq * H)
+        if self.mask is not None:
+            d.mask = self.mask.ptr
+            d.mask_strides = (ctypes.c_int64 * 4)(1, Lkv, 0, 0)
+        kern, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
+        _lib.check(self.lib.mi_attention_plan(ctypes.byref(d), ctypes.byref(kern), ctypes.byref(ws)))
+        self.kernel = _lib.KERNEL_NAMES[kern.value]
+        self.ws = torch.empty(max(ws.value, 1), dtype=torch.uint8, device="cuda")
+        d.workspace, d.workspace_bytes = self.ws.data_ptr(), ws.value
+
+    def step(self):
+        self._lib.check(self.lib.mi_attention_fwd(ctypes.byref(self.desc), None))
+
+    def time(self, steps, warmup):
+        """Average ms per call over `steps` back-to-back launches, HIP events on the launch stream."""
+        lib, _lib = self.lib, self._lib
+        e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+        _lib.check(lib.mi_event_create(ctypes.byref(e0)))
+        _lib.check(lib.mi_event_create(ctypes.byref(e1)))
+        for _ in range(warmup):
+            self.step()
+        _lib.check(lib.mi_device_sync())
+        t0 = time.perf_counter()
+        _lib.check(lib.mi_event_record(e0, None))
+        for _ in range(steps):
+            self.step()
+        _lib.check(lib.mi_event_record(e1, None))
+        _lib.check(lib.mi_event_sync(e1))
+        _lib.check(lib.mi_device_sync())
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        ms = ctypes.c_float(0)
+        _lib.check(lib.mi_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+        lib.mi_event_destroy(e0)
+        lib.mi_event_destroy(e1)
+        return ms.value / steps, wall_ms
+
+
+def cpu_baseline(key, budget_s=20.0):
+    """The CPU oracle (NNlib's op sequence restated in C, Float32, NNlib's thread policy) timed on a
+    bounded sample of the same workload: a subset of heads of one batch element, scaled to the job."""
+    import numpy as np
+    from oracle import oracle as O
+    w = WORKLOADS[key]
+    E, Lq, Lkv, B, H = w["E"], w["Lq"], w["Lkv"], w["B"], w["H"]
+    D = E // H
+    cores = os.cpu_count() or 1
+    flops_full = 4 * D * Lq * Lkv            # per (head, batch), unmasked (the reference computes every score)
+    # aim for about budget_s seconds assuming ~3 GFLOP/s/core effective on the whole unfused chain
+    est_rate = 3e9 * cores
+    nh = int(max(1, min(H, budget_s * est_rate / flops_full)))
+    rng = np.random.default_rng(w["seed"] & 0xFFFF)
+    q = np.asfortranarray((rng.standard_normal((nh * D, Lq, 1)) * w["scale"]).astype(np.float32))
+    k = np.asfortranarray((rng.standard_normal((nh * D, Lkv, 1)) * w["scale"]).astype(np.float32))
+    v = np.asfortranarray(rng.standard_normal((nh * D, Lkv, 1)).astype(np.float32))
+    bias = (0.5 * rng.standard_normal((Lkv, Lq, nh, 1))).astype(np.float32) if w.get("bias") else None
+    mask = None
+    if w.get("mask"):
+        mask = rng.random((Lkv, Lq)) < 0.9
+    if w["causal"]:
+        mask = O.make_causal_mask(Lq)
+    O.lib()
+    t0 = time.perf_counter()
+    O.nnlib_attention_f32(q, k, v, bias, mask, nh, nthreads=cores)
+    dt = time.perf_counter() - t0
+    flops, nbytes = algorithmic_work(w)
+    frac = nh / (H * B)
+    full_s = dt / frac
+    return dict(seconds_sample=dt, seconds_full_job=full_s, heads_in_sample=nh, cores=cores,
+                sample=f"{nh} of {H * B} (head, batch) slices of the same workload, Float32, "
+                       f"{cores} threads over batch slices (NNlib policy), scaled by {1 / frac:.0f}x",
+                tflops=flops / full_s / 1e12, gbps=nbytes / full_s / 1e9)
+
+
+def measure(key, steps, warmup, with_cpu):
+    w = WORKLOADS[key]
+    r = Runner(key)
+    ms, wall_ms = r.time(steps, warmup)
+    flops, nbytes = algorithmic_work(w)
+    tflops = flops / (ms * 1e-3) / 1e12
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    hbm_bound = key in ("c4", "c5")
+    if hbm_bound:
+        roof = dict(bound="hbm", achieved=gbps, peak=HBM_PEAK, unit="GB/s", frac=gbps / HBM_PEAK, traffic=None)
+    else:
+        pk = PEAK[w["dtype"]]
+        roof = dict(bound="mfma", achieved=tflops, peak=pk, unit="TFLOP/s", frac=tflops / pk, traffic=None)
+    res = dict(workload=w["name"], kernel=r.kernel, ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, gbps=gbps,
+               flops_per_step=flops, bytes_per_step=nbytes, roofline=roof)
+    if with_cpu:
+        c = cpu_baseline(key)
+        if hbm_bound:
+            res["cpu_baseline"] = dict(value=c["gbps"], unit="GB/s", cores=c["cores"], kind="port", sample=c["sample"],
+                                       seconds_sample=c["seconds_sample"])
+        else:
+            res["cpu_baseline"] = dict(value=c["tflops"], unit="TFLOP/s", cores=c["cores"], kind="port",
+                                       sample=c["sample"], seconds_sample=c["seconds_sample"])
+    del r
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (heads and batches shard without communication; "
+                 "see DESIGN.md). Run with --gpus 1.")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the attention path has no CPU fallback")
+
+    main_res = measure(args.workload, args.steps, args.warmup, not args.no_cpu)
+    w = WORKLOADS[args.workload]
+    prefill = args.workload not in ("c4", "c5")
+    line = {
+        "metric": "attention TFLOP/s (prefill)" if prefill else "attention GB/s (HBM-bound)",
+        "value": main_res["tflops"] if prefill else main_res["gbps"],
+        "unit": "TFLOP/s" if prefill else "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": main_res["workload"], "kernel": main_res["kernel"], "E": w["E"], "Lq": w["Lq"],
+                   "Lkv": w["Lkv"], "B": w["B"], "nheads": w["H"], "causal": w["causal"]},
+        "roofline": main_res["roofline"],
+        "flops_per_step": main_res["flops_per_step"], "bytes_per_step": main_res["bytes_per_step"],
+    }
+    if "cpu_baseline" in main_res:
+        line["cpu_baseline"] = main_res["cpu_baseline"]
+    if args.workload == "c3" and not args.no_decode:
+        dsteps = max(5, min(args.steps, 20))
+        dec = measure("c5", dsteps, min(args.warmup, 3), not args.no_cpu)
+        line["decode"] = {"metric": "attention GB/s (decode)", "value": dec["gbps"], "unit": "GB/s",
+                          "ms_per_step": dec["ms_per_step"], "steps": dsteps, "dtype": "bf16",
+                          "config": {"workload": dec["workload"], "kernel": dec["kernel"]},
+                          "roofline": dec["roofline"]}
+        if "cpu_baseline" in dec:
+            line["decode"]["cpu_baseline"] = dec["cpu_baseline"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
