@@ -1,8 +1,199 @@
-// split-kv decode path (placeholder until the kernel lands).
+// Split-kv attention for a single query per (head, batch) ("decode" shape, Lq = 1), bf16 / f16.
+//
+// The work is a stream over K and V: every byte is read once and used once, so the kernel is
+// organised around HBM, not around the matrix cores.  A kv row (all heads) is E contiguous elements;
+// a wavefront owns a 512-element segment of the row (4 heads at D = 128, 8 heads at D = 64), each
+// lane 8 consecutive features (one 16-byte load), and walks a contiguous range of kv rows.  The
+// dot product over a head is finished with a butterfly over the D/8 lanes that share the head.
+// Each (segment, kv-split, batch) wavefront keeps an online-softmax state (m, l, o[8]) and writes it
+// to a workspace; a second small kernel merges the splits.
+//
+// Same arithmetic as the reference chain (src/attention.jl:112-127, fdrop = identity, no bias/mask):
+//   s_j = sum_d k[d,j] * q[d] / sqrt(D),  a = softmax_j(s),  x[d] = sum_j a_j v[d,j].
 #include "common.h"
 #include "attention_params.h"
-bool attention_decode_supports(const AttnParams &) { return false; }
-size_t attention_decode_workspace(const AttnParams &) { return 0; }
-int32_t launch_attention_decode(const AttnParams &, hipStream_t) {
-    return mi_set_error(MI_EINVAL, "decode kernel not built");
+
+namespace {
+
+constexpr int ROWS = 8;        // kv rows in flight per lane and tensor
+constexpr int SEG = 512;       // features per wavefront
+
+struct DecodeArgs {
+    AttnParams p;
+    float c;           // log2(e) / sqrt(D)
+    int32_t nsplit;
+    int32_t rows_per_split;
+    int32_t nseg;      // ceil(E / 512)
+};
+
+__device__ inline void unpack8(const u32x4_t &v, float *out, BF16) {
+    const bf16x8_t h = __builtin_bit_cast(bf16x8_t, v);
+#pragma unroll
+    for (int e = 0; e < 8; e++) out[e] = (float)h[e];
+}
+__device__ inline void unpack8(const u32x4_t &v, float *out, F16) {
+    const f16x8_t h = __builtin_bit_cast(f16x8_t, v);
+#pragma unroll
+    for (int e = 0; e < 8; e++) out[e] = (float)h[e];
+}
+
+// workspace layout: [B][nsplit][E] floats of o, then [B][nsplit][H] of m, then [B][nsplit][H] of l
+template <typename T, int D>
+__global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
+    const AttnParams &p = a.p;
+    typedef typename T::type t;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int seg = blockIdx.x * 4 + wave;
+    const int split = blockIdx.y;
+    const int64_t b = blockIdx.z;
+    const int64_t f = (int64_t)seg * SEG + lane * 8;   // first feature of this lane
+    const bool lane_ok = f < p.E;                      // E is a multiple of 8 (D is 64 or 128)
+    if (seg >= a.nseg) return;
+
+    const t *kb = (const t *)p.k + p.E * p.Lkv * b + (lane_ok ? f : 0);
+    const t *vb = (const t *)p.v + p.E * p.Lkv * b + (lane_ok ? f : 0);
+    float qf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (lane_ok) unpack8(*(const u32x4_t *)((const t *)p.q + p.E * b + f), qf, T());
+
+    const int64_t j_begin = (int64_t)split * a.rows_per_split;
+    int64_t j_end = j_begin + a.rows_per_split;
+    if (j_end > p.Lkv) j_end = p.Lkv;
+
+    float m = MI_NEG_INF, l = 0.0f;
+    float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const u32x4_t zero = {0, 0, 0, 0};
+
+    for (int64_t j = j_begin; j < j_end; j += ROWS) {
+        u32x4_t kr[ROWS], vr[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            const bool ok = lane_ok && j + r < j_end;
+            kr[r] = ok ? *(const u32x4_t *)(kb + p.E * (j + r)) : zero;
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            const bool ok = lane_ok && j + r < j_end;
+            vr[r] = ok ? *(const u32x4_t *)(vb + p.E * (j + r)) : zero;
+        }
+        float s[ROWS];
+        float mx = MI_NEG_INF;
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            float kf[8];
+            unpack8(kr[r], kf, T());
+            float d = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) d = fmaf(kf[e], qf[e], d);
+#pragma unroll
+            for (int off = 1; off < D / 8; off <<= 1) d += __shfl_xor(d, off, 64);
+            s[r] = j + r < j_end ? d : MI_NEG_INF;
+            mx = fmaxf(mx, s[r]);
+        }
+        const float mnew = fmaxf(m, mx);      // finite: at least one row of the chunk is valid
+        const float resc = mi_exp2((m - mnew) * a.c);
+        m = mnew;
+        l *= resc;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] *= resc;
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            const float pr = mi_exp2((s[r] - mnew) * a.c);
+            l += pr;
+            float vf[8];
+            unpack8(vr[r], vf, T());
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = fmaf(pr, vf[e], o[e]);
+        }
+    }
+    if (!lane_ok) return;
+    float *ws = (float *)p.workspace;
+    const int64_t slot = b * a.nsplit + split;
+    float *wo = ws + slot * p.E + f;
+    *(floatx4_t *)wo = (floatx4_t){o[0], o[1], o[2], o[3]};
+    *(floatx4_t *)(wo + 4) = (floatx4_t){o[4], o[5], o[6], o[7]};
+    if ((lane & (D / 8 - 1)) == 0) {
+        const int64_t h = f / D;
+        float *wm = ws + (int64_t)p.B * a.nsplit * p.E;
+        float *wl = wm + (int64_t)p.B * a.nsplit * p.H;
+        wm[slot * p.H + h] = m;
+        wl[slot * p.H + h] = l;
+    }
+}
+
+// one thread per output feature: merge the splits with the usual log-sum-exp rule
+template <typename T>
+__global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
+    const AttnParams &p = a.p;
+    const int64_t b = blockIdx.y;
+    const int64_t f = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (f >= p.E) return;
+    const int64_t h = f / p.D;
+    const float *ws = (const float *)p.workspace;
+    const float *wm = ws + (int64_t)p.B * a.nsplit * p.E;
+    const float *wl = wm + (int64_t)p.B * a.nsplit * p.H;
+    float m = MI_NEG_INF;
+    for (int s = 0; s < a.nsplit; s++) m = fmaxf(m, wm[(b * a.nsplit + s) * p.H + h]);
+    float l = 0.0f, o = 0.0f;
+    for (int s = 0; s < a.nsplit; s++) {
+        const int64_t slot = b * a.nsplit + s;
+        const float w = mi_exp2((wm[slot * p.H + h] - m) * a.c);
+        l = fmaf(wl[slot * p.H + h], w, l);
+        o = fmaf(ws[slot * p.E + f], w, o);
+    }
+    ((typename T::type *)p.out)[p.E * b + f] = T::from_f32(o / l);
+}
+
+int pick_nsplit(const AttnParams &p) {
+    // enough wavefronts to cover the chip several times over, at least 256 rows per split
+    const int64_t nseg = (p.E + SEG - 1) / SEG;
+    int64_t want = 8192 / (nseg * p.B > 0 ? nseg * p.B : 1);
+    int64_t maxs = (p.Lkv + 255) / 256;
+    if (want > maxs) want = maxs;
+    if (want < 1) want = 1;
+    if (want > 1024) want = 1024;
+    return (int)want;
+}
+
+}  // namespace
+
+bool attention_decode_supports(const AttnParams &p) {
+    if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
+    if (p.Lq != 1 || p.weights || p.bias || p.mask || !p.out) return false;
+    if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
+    if (p.Lkv < 512) return false;   // short contexts: the tiled kernel is fine
+    if (p.B > 65535) return false;
+    auto al = [](const void *x) { return (((uintptr_t)x) & 15) == 0; };
+    return al(p.q) && al(p.k) && al(p.v);
+}
+
+size_t attention_decode_workspace(const AttnParams &p) {
+    const size_t ns = (size_t)pick_nsplit(p);
+    return sizeof(float) * ns * (size_t)p.B * (size_t)(p.E + 2 * p.H);
+}
+
+int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
+    DecodeArgs a;
+    a.p = p;
+    a.c = MI_LOG2E / sqrtf((float)p.D);
+    a.nsplit = pick_nsplit(p);
+    a.rows_per_split = (int32_t)((p.Lkv + a.nsplit - 1) / a.nsplit);
+    a.nsplit = (int32_t)((p.Lkv + a.rows_per_split - 1) / a.rows_per_split);  // no empty split
+    a.nseg = (int32_t)((p.E + SEG - 1) / SEG);
+    if ((((uintptr_t)p.workspace) & 15) != 0)
+        return mi_set_error(MI_EWORKSPACE, "decode workspace must be 16-byte aligned");
+    dim3 grid((unsigned)((a.nseg + 3) / 4), (unsigned)a.nsplit, (unsigned)p.B);
+    dim3 mgrid((unsigned)((p.E + 255) / 256), (unsigned)p.B);
+    if (p.dtype == MI_BF16) {
+        if (p.D == 128) hipLaunchKernelGGL((decode_split_kernel<BF16, 128>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((decode_split_kernel<BF16, 64>), grid, dim3(256), 0, st, a);
+        MI_LAUNCH_CHECK();
+        hipLaunchKernelGGL(decode_merge_kernel<BF16>, mgrid, dim3(256), 0, st, a);
+    } else {
+        if (p.D == 128) hipLaunchKernelGGL((decode_split_kernel<F16, 128>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((decode_split_kernel<F16, 64>), grid, dim3(256), 0, st, a);
+        MI_LAUNCH_CHECK();
+        hipLaunchKernelGGL(decode_merge_kernel<F16>, mgrid, dim3(256), 0, st, a);
+    }
+    MI_LAUNCH_CHECK();
+    return MI_OK;
 }

@@ -1,8 +1,252 @@
-// fp32 MFMA flash forward (placeholder until the kernel lands: reports "not supported" so that
-// the dispatcher falls back to the generic kernel).
-#include "common.h"
-#include "attention_params.h"
-bool attention_flash32_supports(const AttnParams &) { return false; }
-int32_t launch_attention_flash32(const AttnParams &, hipStream_t) {
-    return mi_set_error(MI_EINVAL, "fp32 flash kernel not built");
+// Flash-style attention forward for Float32 inputs on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
+//
+// Same decomposition as the 16-bit kernel: S^T = K Q^T with keys as MFMA rows and queries as
+// columns, online softmax per lane-owned query column, O^T += V^T P^T.  With one fp32 per register
+// no transposition is needed anywhere: the A operand of the second product is a plain 4-byte LDS
+// read of V[key][feature = lane], and the B operand is the softmax accumulator register itself.
+// Products and sums are true fp32 (no down-conversion), which keeps the 1e-4 parity bound.
+//
+// The contraction index of QK^T is permuted so that a lane fetches K with 16-byte LDS reads:
+// k-step 4c+j of half-wave hh multiplies feature d = 8c + 4hh + j (Q is loaded with the same map).
+#include "flash_common.h"
+
+namespace {
+
+typedef F32 T;
+constexpr int BN = FLASH_BN;
+
+template <int D, int QB>
+struct Frag32 {
+    float q[QB][D / 2];
+    floatx16_t o[QB][D / 32];
+    float m[QB], l[QB];
+};
+
+template <int D>
+struct Cfg {
+    static constexpr int KS = D + 4;   // K row stride (floats): rows 4 banks apart, conflict-free b128 reads
+    static constexpr int VS = D + 8;   // V row stride (floats): rows 4 apart land 32 banks apart
+    static constexpr int CHUNKS = BN * D / 4 / 256;  // 16-byte chunks per thread, tile and tensor
+    static constexpr size_t SMEM = sizeof(float) * 2 * BN * (KS + VS);
+};
+
+__device__ inline floatx4_t ldg16f(const float *p, bool ok) {
+    floatx4_t z = {0.f, 0.f, 0.f, 0.f};
+    return ok ? *(const floatx4_t *)p : z;
+}
+
+template <int D, int QB, bool CAUSAL, bool EXTRAS, int PHASE>
+__device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *Ks, float *Vs, int64_t b, int64_t h,
+                                   int64_t iw, int n_tiles) {
+    constexpr int KS = Cfg<D>::KS, VS = Cfg<D>::VS, CHUNKS = Cfg<D>::CHUNKS;
+    const AttnParams &p = a.p;
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hh = lane >> 5;
+    constexpr bool NEED_V = PHASE != PHASE_STATS;
+    const bool do_pv = NEED_V && p.out != nullptr;
+
+    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + D * h;
+    const float *vbase = NEED_V && p.v ? (const float *)p.v + p.Ev * (p.Lkv * b) + D * h : nullptr;
+
+    floatx4_t kreg[CHUNKS], vreg[CHUNKS];
+    auto load_tile = [&](int jt) {
+        const int64_t j0 = (int64_t)jt * BN;
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            const bool ok = j0 + row < p.Lkv;
+            kreg[u] = ldg16f(kbase + p.E * (j0 + row) + col, ok);
+            if (NEED_V) vreg[u] = ldg16f(vbase + p.Ev * (j0 + row) + col, ok && do_pv);
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            *(floatx4_t *)(Ks + (buf * BN + row) * KS + col) = kreg[u];
+            if (NEED_V) *(floatx4_t *)(Vs + (buf * BN + row) * VS + col) = vreg[u];
+        }
+    };
+
+    if (n_tiles <= 0) return;
+    load_tile(0);
+    __syncthreads();
+    store_tile(0);
+    __syncthreads();
+
+    for (int jt = 0; jt < n_tiles; jt++) {
+        const int buf = jt & 1;
+        const int64_t j0 = (int64_t)jt * BN;
+        if (jt + 1 < n_tiles) load_tile(jt + 1);
+
+        const bool active = !CAUSAL || j0 <= iw + 32 * QB - 1;
+        if (active) {
+            floatx16_t s[QB][2];
+#pragma unroll
+            for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) s[qb][kb] = (floatx16_t){0};
+            const float *kt = Ks + (buf * BN + r) * KS + 4 * hh;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int c = 0; c < D / 8; c++) {
+                    const floatx4_t k4 = *(const floatx4_t *)(kt + kb * 32 * KS + 8 * c);
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int qb = 0; qb < QB; qb++)
+                            s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(k4[j], f.q[qb][4 * c + j], s[qb][kb], 0, 0, 0);
+                }
+
+            flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0);
+
+            if (do_pv) {
+                // k-step v of key block kb multiplies key 32*kb + 8*(v/4) + 4*hh + v%4: exactly the key
+                // whose weight sits in accumulator register v of this lane
+                const float *vt = Vs + (buf * BN + 4 * hh) * VS + r;
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const float *src = vt + (32 * kb + 8 * (v / 4) + (v % 4)) * VS;
+#pragma unroll
+                        for (int dvb = 0; dvb < D / 32; dvb++) {
+                            const float va = src[32 * dvb];
+#pragma unroll
+                            for (int qb = 0; qb < QB; qb++)
+                                f.o[qb][dvb] = __builtin_amdgcn_mfma_f32_32x32x2f32(va, s[qb][kb][v], f.o[qb][dvb], 0, 0, 0);
+                        }
+                    }
+            }
+        }
+        if (jt + 1 < n_tiles) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+}
+
+template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS>
+__global__ __launch_bounds__(256, 1) void flash32_kernel(FlashArgs a) {
+    constexpr int KS = Cfg<D>::KS, VS = Cfg<D>::VS;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char flash_smem[];
+    float *Ks = (float *)flash_smem;     // [2][BN][KS]
+    float *Vs = Ks + 2 * BN * KS;        // [2][BN][VS]
+    (void)VS;
+    constexpr int BM = 128 * QB;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t id = blockIdx.x;
+    const int64_t hb = id % HB;
+    const int64_t qt = a.n_qtiles - 1 - id / HB;   // heaviest (latest) query tiles first
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t i0 = qt * BM, iw = i0 + (int64_t)wave * 32 * QB;
+
+    Frag32<D, QB> f;
+    const float *qbase = (const float *)p.q + p.E * (p.Lq * b) + D * h;
+    const float sq = sqrtf((float)D);
+#pragma unroll
+    for (int qb = 0; qb < QB; qb++) {
+        const int64_t qi = iw + 32 * qb + r;
+#pragma unroll
+        for (int c = 0; c < D / 8; c++) {
+            const floatx4_t q4 = ldg16f(qbase + p.E * qi + 8 * c + 4 * hh, qi < p.Lq);
+            // the reference divides q by sqrt(D) before the product (src/attention.jl:118)
+#pragma unroll
+            for (int j = 0; j < 4; j++) f.q[qb][4 * c + j] = q4[j] / sq;
+        }
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++) f.o[qb][dvb] = (floatx16_t){0};
+        f.m[qb] = MI_NEG_INF;
+        f.l[qb] = 0.0f;
+    }
+
+    int64_t kv_end = p.Lkv;
+    if (CAUSAL && i0 + BM < kv_end) kv_end = i0 + BM;
+    const int n_tiles = (int)((kv_end + BN - 1) / BN);
+
+    if (!WEIGHTS) {
+        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_ONLINE>(a, f, Ks, Vs, b, h, iw, n_tiles);
+    } else {
+        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_STATS>(a, f, Ks, Vs, b, h, iw, n_tiles);
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) {
+            const float l = f.l[qb] + mi_swap32(f.l[qb]);
+            f.l[qb] = 1.0f / l;
+        }
+        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_FINAL>(a, f, Ks, Vs, b, h, iw, n_tiles);
+        if (CAUSAL && p.weights) flash_zero_skipped_weights<QB, float>(a, b, h, iw, n_tiles);
+    }
+
+    if (p.out) {
+        float *obase = (float *)p.out + p.Ev * (p.Lq * b) + D * h;
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) {
+            const int64_t qi = iw + 32 * qb + r;
+            float inv = 1.0f;
+            if (!WEIGHTS) {
+                const float l = f.l[qb] + mi_swap32(f.l[qb]);
+                inv = 1.0f / l;
+            }
+            if (qi < p.Lq) {
+#pragma unroll
+                for (int dvb = 0; dvb < D / 32; dvb++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        floatx4_t o4;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o4[e] = f.o[qb][dvb][4 * g + e] * inv;
+                        *(floatx4_t *)(obase + p.Ev * qi + 32 * dvb + 8 * g + 4 * hh) = o4;
+                    }
+            }
+        }
+    }
+}
+
+template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS>
+int32_t launch_one(const FlashArgs &a, hipStream_t st) {
+    const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B;
+    constexpr size_t smem = Cfg<D>::SMEM;
+    auto kern = flash32_kernel<D, QB, CAUSAL, EXTRAS, WEIGHTS>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(256), smem, st, a);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+template <int D, int QB>
+int32_t launch_d(const FlashArgs &a, hipStream_t st) {
+    const bool extras = a.p.bias || a.p.mask, w = a.p.weights != nullptr;
+    if (a.p.causal) {
+        if (extras) return w ? launch_one<D, QB, true, true, true>(a, st) : launch_one<D, QB, true, true, false>(a, st);
+        return w ? launch_one<D, QB, true, false, true>(a, st) : launch_one<D, QB, true, false, false>(a, st);
+    }
+    if (extras) return w ? launch_one<D, QB, false, true, true>(a, st) : launch_one<D, QB, false, true, false>(a, st);
+    return w ? launch_one<D, QB, false, false, true>(a, st) : launch_one<D, QB, false, false, false>(a, st);
+}
+
+}  // namespace
+
+bool attention_flash32_supports(const AttnParams &p) {
+    if (p.dtype != MI_F32) return false;
+    if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
+    auto al = [](const void *x) { return (((uintptr_t)x) & 15) == 0; };
+    if (!al(p.q) || !al(p.k) || (p.out && (!al(p.v) || !al(p.out)))) return false;
+    const int64_t tiles = (p.Lq + 127) / 128;
+    return tiles * p.H * p.B <= 2147483647LL;
+}
+
+int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
+    FlashArgs a;
+    a.p = p;
+    a.c = MI_LOG2E;  // q is pre-divided by sqrt(D); only the change of base remains
+    a.n_qtiles = (int32_t)((p.Lq + 127) / 128);
+    flash_fill_vec_flags(a);
+    return p.D == 64 ? launch_d<64, 1>(a, st) : launch_d<128, 1>(a, st);
 }

@@ -49,6 +49,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
 // ---- element traits ----------------------------------------------------------------
 struct F32 {
     typedef float type;
+    typedef floatx4_t vec4;
     static constexpr int id = MI_F32;
     __device__ static inline float to_f32(float x) { return x; }
     __device__ static inline float from_f32(float x) { return x; }

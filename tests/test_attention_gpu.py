@@ -225,3 +225,43 @@ def test_fully_masked_column_is_nan(nn):
         y, a = _run(nn, q, k, k, dtype, mask=mask, nheads=H, weights_dtype="f32")
         assert np.isnan(y[:, 5, 0]).all() and np.isnan(a[:, 5]).all()
         assert np.isfinite(np.delete(y, 5, axis=1)).all()
+
+
+FLASH32_CASES = [
+    ("f32", 128, 128, 128, 2, 2, {}),
+    ("f32", 128, 200, 333, 1, 2, {}),
+    ("f32", 256, 130, 130, 1, 2, dict(causal=True)),
+    ("f32", 128, 256, 256, 2, 2, dict(causal=True, scale=0.125)),
+    ("f32", 128, 64, 320, 2, 2, dict(bias_shape=(320, 64, 2, 2), mask_shape=(320, 64))),
+    ("f32", 128, 70, 131, 2, 2, dict(bias_shape=(131, 70), mask_shape=(131, 70, 1, 2))),
+    ("f32", 256, 96, 96, 1, 2, dict(causal=True, mask_shape=(96, 96))),
+    ("f32", 64, 33, 65, 3, 1, {}),
+]
+
+
+@pytest.mark.parametrize("case", FLASH32_CASES, ids=lambda c: f"{c[0]}-E{c[1]}-Lq{c[2]}-Lkv{c[3]}-B{c[4]}-H{c[5]}-" + "-".join(c[6]))
+@pytest.mark.parametrize("weights", [False, True], ids=["noweights", "weights"])
+def test_flash32_parity(nn, oracle, case, weights):
+    dtype, E, Lq, Lkv, B, H, kw = case
+    rng = np.random.default_rng(hash((E, Lq, Lkv, B, H, 32)) % 2**32)
+    _check(nn, oracle, rng, dtype, E, Lq, Lkv, B, H, expect="flash32", weights=weights, **kw)
+
+
+@pytest.mark.parametrize("dtype,E,H,Lkv,B", [("bf16", 512, 4, 1500, 2), ("bf16", 256, 2, 4096, 3), ("f16", 512, 8, 777, 1),
+                                             ("f16", 1024, 8, 2048, 2), ("bf16", 128, 1, 513, 1)])
+def test_decode_parity(nn, oracle, dtype, E, H, Lkv, B):
+    """Split-kv path for a single query per (head, batch)."""
+    rng = np.random.default_rng(E + Lkv)
+    _check(nn, oracle, rng, dtype, E, 1, Lkv, B, H, expect="decode", weights=False)
+
+
+def test_decode_matches_flash16_on_device(nn):
+    rng = np.random.default_rng(11)
+    q = nn.DeviceArray.from_numpy(rng.standard_normal((512, 1, 2)).astype(np.float32), "bf16")
+    k = nn.DeviceArray.from_numpy(rng.standard_normal((512, 3000, 2)).astype(np.float32), "bf16")
+    v = nn.DeviceArray.from_numpy(rng.standard_normal((512, 3000, 2)).astype(np.float32), "bf16")
+    y1, _ = nn.dot_product_attention(q, k, v, nheads=4, return_weights=False)
+    assert nn.last_attention_kernel() == "decode"
+    y2, _ = nn.dot_product_attention(q, k, v, nheads=4, return_weights=True)   # weights force the tiled kernel
+    assert nn.last_attention_kernel() == "flash16"
+    assert rel_err(y1.to_numpy(), y2.to_numpy()) < 1e-2
