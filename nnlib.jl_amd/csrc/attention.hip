@@ -6,6 +6,10 @@ int32_t launch_flash16_bf16_d64(const AttnParams &, hipStream_t);
 int32_t launch_flash16_bf16_d128(const AttnParams &, hipStream_t);
 int32_t launch_flash16_f16_d64(const AttnParams &, hipStream_t);
 int32_t launch_flash16_f16_d128(const AttnParams &, hipStream_t);
+int32_t launch_flash16_fast_bf16(const AttnParams &, hipStream_t);
+int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t);
+bool flash16_fast_supports_bf16(const AttnParams &);
+bool flash16_fast_supports_f16(const AttnParams &);
 
 static inline bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
 
@@ -20,6 +24,8 @@ bool attention_flash16_supports(const AttnParams &p) {
 }
 
 int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
+    if (p.dtype == MI_BF16 && flash16_fast_supports_bf16(p)) return launch_flash16_fast_bf16(p, st);
+    if (p.dtype == MI_F16 && flash16_fast_supports_f16(p)) return launch_flash16_fast_f16(p, st);
     if (p.dtype == MI_BF16) return p.D == 64 ? launch_flash16_bf16_d64(p, st) : launch_flash16_bf16_d128(p, st);
     return p.D == 64 ? launch_flash16_f16_d64(p, st) : launch_flash16_f16_d128(p, st);
 }
