@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libmi355attn.so"))
+# MI355ATTN_LIB overrides the in-tree build (e.g. to load a library built with other flags)
+LIB_PATH = os.environ.get("MI355ATTN_LIB") or os.path.normpath(os.path.join(_HERE, "..", "lib", "libmi355attn.so"))
 
 MI_OK, MI_EINVAL, MI_EDTYPE, MI_ESHAPE, MI_EHIP, MI_ENOMEM, MI_EWORKSPACE = range(7)
 MI_F32, MI_F16, MI_BF16 = 0, 1, 2
