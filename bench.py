@@ -199,8 +199,8 @@ def measure(key, steps, warmup, with_cpu):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
@@ -231,8 +231,8 @@ def main():
     if "cpu_baseline" in main_res:
         line["cpu_baseline"] = main_res["cpu_baseline"]
     if args.workload == "c3" and not args.no_decode:
-        dsteps = max(5, min(args.steps, 20))
-        dec = measure("c5", dsteps, min(args.warmup, 3), not args.no_cpu)
+        dsteps = max(5, min(args.steps, 50))
+        dec = measure("c5", dsteps, min(args.warmup, 10), not args.no_cpu)
         line["decode"] = {"metric": "attention GB/s (decode)", "value": dec["gbps"], "unit": "GB/s",
                           "ms_per_step": dec["ms_per_step"], "steps": dsteps, "dtype": "bf16",
                           "config": {"workload": dec["workload"], "kernel": dec["kernel"]},
