@@ -133,39 +133,47 @@ class Runner:
         return ms.value / steps, wall_ms
 
 
-def cpu_baseline(key, budget_s=20.0):
+def cpu_baseline(key, budget_s=15.0):
     """The CPU oracle (NNlib's op sequence restated in C, Float32, NNlib's thread policy) timed on a
-    bounded sample of the same workload: a subset of heads of one batch element, scaled to the job."""
+    bounded sample of the same workload: whole (head, batch) slices of it, as many as fit in about
+    `budget_s` seconds (sized from a one-slice-per-thread trial run), scaled to the whole job."""
     import numpy as np
     from oracle import oracle as O
     w = WORKLOADS[key]
     E, Lq, Lkv, B, H = w["E"], w["Lq"], w["Lkv"], w["B"], w["H"]
     D = E // H
-    cores = os.cpu_count() or 1
-    flops_full = 4 * D * Lq * Lkv            # per (head, batch), unmasked (the reference computes every score)
-    # aim for about budget_s seconds assuming ~3 GFLOP/s/core effective on the whole unfused chain
-    est_rate = 3e9 * cores
-    nh = int(max(1, min(H, budget_s * est_rate / flops_full)))
+    cores = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
     rng = np.random.default_rng(w["seed"] & 0xFFFF)
-    q = np.asfortranarray((rng.standard_normal((nh * D, Lq, 1)) * w["scale"]).astype(np.float32))
-    k = np.asfortranarray((rng.standard_normal((nh * D, Lkv, 1)) * w["scale"]).astype(np.float32))
-    v = np.asfortranarray(rng.standard_normal((nh * D, Lkv, 1)).astype(np.float32))
-    bias = (0.5 * rng.standard_normal((Lkv, Lq, nh, 1))).astype(np.float32) if w.get("bias") else None
+    f32 = np.float32
     mask = None
     if w.get("mask"):
         mask = rng.random((Lkv, Lq)) < 0.9
     if w["causal"]:
         mask = O.make_causal_mask(Lq)
     O.lib()
-    t0 = time.perf_counter()
-    O.nnlib_attention_f32(q, k, v, bias, mask, nh, nthreads=cores)
-    dt = time.perf_counter() - t0
+
+    def run(nh, nb):
+        q = np.asfortranarray(rng.standard_normal((nh * D, Lq, nb), dtype=f32) * f32(w["scale"]))
+        k = np.asfortranarray(rng.standard_normal((nh * D, Lkv, nb), dtype=f32) * f32(w["scale"]))
+        v = np.asfortranarray(rng.standard_normal((nh * D, Lkv, nb), dtype=f32))
+        bias = f32(0.5) * rng.standard_normal((Lkv, Lq, nh, nb), dtype=f32) if w.get("bias") else None
+        t0 = time.perf_counter()
+        O.nnlib_attention_f32(q, k, v, bias, mask, nh, nthreads=cores)
+        return time.perf_counter() - t0
+
+    trial_h = min(H, cores)
+    t_trial = run(trial_h, 1)
+    slices = H * B
+    want = int(max(trial_h, min(slices, trial_h * budget_s / max(t_trial, 1e-6))))
+    nh = min(H, want)
+    nb = max(1, min(B, want // nh))
+    dt = run(nh, nb) if nh * nb > trial_h else t_trial
+    n = nh * nb if nh * nb > trial_h else trial_h
     flops, nbytes = algorithmic_work(w)
-    frac = nh / (H * B)
-    full_s = dt / frac
-    return dict(seconds_sample=dt, seconds_full_job=full_s, heads_in_sample=nh, cores=cores,
-                sample=f"{nh} of {H * B} (head, batch) slices of the same workload, Float32, "
-                       f"{cores} threads over batch slices (NNlib policy), scaled by {1 / frac:.0f}x",
+    full_s = dt * slices / n
+    return dict(seconds_sample=dt, seconds_full_job=full_s, cores=cores,
+                sample=f"{n} of {slices} (head, batch) slices of the same workload ({dt:.1f} s), Float32, "
+                       f"{cores} threads over batch slices (NNlib's policy), scaled by {slices / n:.3g}x",
                 tflops=flops / full_s / 1e12, gbps=nbytes / full_s / 1e9)
 
 
