@@ -204,12 +204,30 @@ def measure(key, steps, warmup, with_cpu):
     return res
 
 
+def copy_calibration(steps):
+    """A plain copy kernel of known size (1 GiB read, 1 GiB written per launch): the reference point
+    that the FETCH_SIZE / WRITE_SIZE counters are scaled by when HBM traffic is read with rocprofv3."""
+    import torch
+    import nnlib_amd
+    from nnlib_amd import _lib
+    lib = _lib.load()
+    _lib.check(lib.mi_init(0))
+    n = 1 << 28
+    src = nnlib_amd.DeviceArray.zeros((n,), "f32")
+    dst = nnlib_amd.DeviceArray.empty((n,), "f32")
+    for _ in range(steps):
+        _lib.check(lib.mi_convert(dst.ptr, _lib.MI_F32, src.ptr, _lib.MI_F32, n, None))
+    _lib.check(lib.mi_device_sync())
+    print(json.dumps({"workload": "copy", "kernel": "convert_kernel<F32, F32>", "bytes_read": 4 * n,
+                      "bytes_written": 4 * n, "launches": steps}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
     args = ap.parse_args()
@@ -220,6 +238,8 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the attention path has no CPU fallback")
 
+    if args.workload == "copy":
+        return copy_calibration(min(args.steps, 10))
     main_res = measure(args.workload, args.steps, args.warmup, not args.no_cpu)
     w = WORKLOADS[args.workload]
     prefill = args.workload not in ("c4", "c5")
