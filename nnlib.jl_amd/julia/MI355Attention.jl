@@ -1,0 +1,283 @@
+# MI355Attention.jl -- Julia host side of the MI355X attention library.
+#
+# Thin marshalling layer over the C ABI of libmi355attn.so (include/mi355attn.h).  It owns a
+# column-major device array type and defines, for that type, the operators NNlib.jl exports for
+# the attention path, with NNlib's signatures, return values and exception types:
+#
+#   dot_product_attention(q, k, v, [bias]; fdrop, mask, nheads)   NNlib src/attention.jl:40-84
+#   dot_product_attention_scores(q, k, [bias]; fdrop, mask)        NNlib src/attention.jl:112-127
+#   make_causal_mask(x; dims)                                      NNlib src/attention.jl:149-153
+#   softmax(x; dims=1), softmax!(out, x; dims=1)                   NNlib src/softmax.jl:56-66
+#   batched_mul(A, B), batched_mul!(C, A, B, alpha, beta)          NNlib src/batched/batchedmul.jl:47-60,238-254
+#   batched_transpose, batched_adjoint                             NNlib src/batched/batchedadjtrans.jl:37-52
+#
+# All arithmetic happens in the library.  This file has not been executed in the build environment
+# (no Julia toolchain there); the Python mirror in nnlib_amd/ exercises the same entry points.
+module MI355Attention
+
+export DeviceArray, CausalMask, dot_product_attention, dot_product_attention_scores, make_causal_mask,
+       softmax, softmax!, batched_mul, batched_mul!, batched_transpose, batched_adjoint
+
+const libmi = get(ENV, "MI355ATTN_LIB", joinpath(@__DIR__, "..", "lib", "libmi355attn.so"))
+
+# ---- status codes and element types (include/mi355attn.h) ----------------------------------------
+const MI_OK, MI_EINVAL, MI_EDTYPE, MI_ESHAPE, MI_EHIP, MI_ENOMEM, MI_EWORKSPACE = Int32.(0:6)
+const MI_F32, MI_F16, MI_BF16 = Int32(0), Int32(1), Int32(2)
+
+primitive type BFloat16 <: AbstractFloat 16 end     # storage only; use BFloat16s.jl for arithmetic
+const MIFloat = Union{Float32, Float16, BFloat16}
+dtype_code(::Type{Float32}) = MI_F32
+dtype_code(::Type{Float16}) = MI_F16
+dtype_code(::Type{BFloat16}) = MI_BF16
+
+last_error() = unsafe_string(ccall((:mi_last_error_string, libmi), Cstring, ()))
+
+# Status -> the exception NNlib raises for the same condition (src/attention.jl:42,55-78 throw
+# ArgumentError; src/batched/batchedmul.jl:57-58 and src/gemm.jl:106-108 throw DimensionMismatch).
+function check(rc::Int32; shape_error = ArgumentError)
+    rc == MI_OK && return nothing
+    msg = last_error()
+    rc == MI_ESHAPE && throw(shape_error(msg))
+    (rc == MI_EINVAL || rc == MI_EDTYPE) && throw(ArgumentError(msg))
+    rc == MI_ENOMEM && throw(OutOfMemoryError())
+    error("mi355attn status $rc: $msg")
+end
+
+__init__() = check(ccall((:mi_init, libmi), Int32, (Int32,), Int32(0)))
+
+# ---- device arrays ---------------------------------------------------------------------------------
+# Column-major, like Array.  `strides` lets batched_transpose be a lazy view, as NNlib's
+# BatchedTranspose is (src/batched/batchedadjtrans.jl:23-27).
+mutable struct DeviceArray{T, N} <: AbstractArray{T, N}
+    ptr::Ptr{Cvoid}
+    dims::NTuple{N, Int}
+    strides::NTuple{N, Int}
+    owner::Any                      # `nothing` if this object owns ptr, else the parent array
+    function DeviceArray{T, N}(ptr, dims, strides, owner) where {T, N}
+        a = new{T, N}(ptr, dims, strides, owner)
+        owner === nothing && finalizer(free!, a)
+        a
+    end
+end
+
+dense_strides(dims) = ntuple(i -> prod(dims[1:i-1]; init = 1), length(dims))
+
+function DeviceArray{T}(::UndefInitializer, dims::Vararg{Int, N}) where {T, N}
+    p = Ref{Ptr{Cvoid}}(C_NULL)
+    check(ccall((:mi_malloc, libmi), Int32, (Ptr{Ptr{Cvoid}}, Csize_t), p, max(prod(dims), 1) * sizeof(T)))
+    DeviceArray{T, N}(p[], dims, dense_strides(dims), nothing)
+end
+DeviceArray{T}(u::UndefInitializer, dims::Tuple) where {T} = DeviceArray{T}(u, dims...)
+
+function free!(a::DeviceArray)
+    # mi_free is hipFree: it may block until the device is idle, which is acceptable at GC time
+    a.ptr == C_NULL || ccall((:mi_free, libmi), Int32, (Ptr{Cvoid},), a.ptr)
+    a.ptr = C_NULL
+    nothing
+end
+
+function DeviceArray(h::Array{T, N}) where {T <: Union{MIFloat, Bool}, N}
+    d = DeviceArray{T}(undef, size(h)...)
+    check(ccall((:mi_memcpy_h2d, libmi), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), d.ptr, h, sizeof(h), C_NULL))
+    d
+end
+
+function Base.Array(d::DeviceArray{T, N}) where {T, N}
+    is_dense(d) || throw(ArgumentError("materialise a lazy transpose before copying to the host"))
+    h = Array{T, N}(undef, d.dims)
+    check(ccall((:mi_memcpy_d2h, libmi), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), h, d.ptr, sizeof(h), C_NULL))
+    h
+end
+
+Base.size(a::DeviceArray) = a.dims
+Base.strides(a::DeviceArray) = a.strides
+Base.elsize(::Type{<:DeviceArray{T}}) where {T} = sizeof(T)
+Base.unsafe_convert(::Type{Ptr{T}}, a::DeviceArray{T}) where {T} = convert(Ptr{T}, a.ptr)
+Base.similar(a::DeviceArray, ::Type{T}, dims::Dims) where {T} = DeviceArray{T}(undef, dims...)
+Base.getindex(::DeviceArray, I...) = error("scalar indexing of a DeviceArray is not supported; copy with Array(x)")
+is_dense(a::DeviceArray) = a.strides == dense_strides(a.dims)
+
+function Base.reshape(a::DeviceArray{T}, dims::Dims{N}) where {T, N}
+    is_dense(a) || throw(ArgumentError("reshape needs a dense array"))
+    prod(dims) == length(a) || throw(DimensionMismatch("new dimensions $dims must be consistent with array size $(length(a))"))
+    DeviceArray{T, N}(a.ptr, dims, dense_strides(dims), a)
+end
+
+batched_transpose(a::DeviceArray{T, 3}) where {T} =
+    DeviceArray{T, 3}(a.ptr, (a.dims[2], a.dims[1], a.dims[3]), (a.strides[2], a.strides[1], a.strides[3]), a)
+batched_adjoint(a::DeviceArray{<:Real, 3}) = batched_transpose(a)
+
+# ---- masks -----------------------------------------------------------------------------------------
+# make_causal_mask on a device array returns this lazy stand-in for triu(trues(len, len)); the kernel
+# applies m[i, j] = i <= j (src/attention.jl:145) from indices.  collect(m) gives the dense Bool matrix.
+struct CausalMask <: AbstractMatrix{Bool}
+    len::Int
+end
+Base.size(m::CausalMask) = (m.len, m.len)
+Base.getindex(m::CausalMask, i::Int, j::Int) = i <= j
+make_causal_mask(x::DeviceArray; dims::Int = 2) = CausalMask(size(x, dims))
+
+# ---- attention -------------------------------------------------------------------------------------
+# Mirror of `mi_attn_desc` (include/mi355attn.h); field order and sizes must match the header.
+struct AttnDesc
+    struct_size::Int32; dtype::Int32; weights_dtype::Int32; causal::Int32; flags::UInt32; reserved::Int32
+    E::Int64; Ev::Int64; Lq::Int64; Lkv::Int64; H::Int64; B::Int64
+    q::Ptr{Cvoid}; k::Ptr{Cvoid}; v::Ptr{Cvoid}; out::Ptr{Cvoid}; weights::Ptr{Cvoid}
+    bias::Ptr{Cvoid}; bias_strides::NTuple{4, Int64}
+    mask::Ptr{Cvoid}; mask_strides::NTuple{4, Int64}
+    workspace::Ptr{Cvoid}; workspace_bytes::Csize_t
+end
+
+# element strides of x against the (kv, q, head, batch) score tensor; 0 where x has extent 1
+function broadcast_strides(x::DeviceArray, target::NTuple{4, Int}, what)
+    ntuple(4) do i
+        d = i <= ndims(x) ? size(x, i) : 1
+        d == 1 ? Int64(0) : d == target[i] ? Int64(strides(x)[i]) :
+            throw(DimensionMismatch("arrays could not be broadcast to a common size: $what has size $(size(x)), attention scores have size $target"))
+    end
+end
+
+function attention_call(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v, bias, mask, H::Int; want_out::Bool,
+                        want_weights::Bool) where {T <: MIFloat}
+    E, Lq, B = size(q); Lkv = size(k, 2); Ev = v === nothing ? E : size(v, 1)
+    target = (Lkv, Lq, H, B)
+    out = want_out ? DeviceArray{T}(undef, Ev, Lq, B) : nothing
+    alpha = want_weights ? DeviceArray{T}(undef, Lkv, Lq, H, B) : nothing
+    causal, mptr, mstr = Int32(0), C_NULL, ntuple(_ -> Int64(0), 4)
+    if mask isa CausalMask
+        (mask.len == Lkv == Lq) || throw(DimensionMismatch("arrays could not be broadcast to a common size: mask has size $(size(mask)), attention scores have size $target"))
+        causal = Int32(1)
+    elseif mask !== nothing
+        mask isa DeviceArray{Bool} || throw(ArgumentError("mask must be a Bool DeviceArray or a CausalMask"))
+        mptr, mstr = mask.ptr, broadcast_strides(mask, target, "mask")
+    end
+    bptr, bstr = C_NULL, ntuple(_ -> Int64(0), 4)
+    if bias !== nothing
+        bias isa DeviceArray{T} || throw(ArgumentError("bias must be a DeviceArray with the element type of q"))
+        bptr, bstr = bias.ptr, broadcast_strides(bias, target, "bias")
+    end
+    mk(ws, wsbytes) = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0),
+                               E, Ev, Lq, Lkv, H, B, q.ptr, k.ptr, v === nothing ? C_NULL : v.ptr,
+                               out === nothing ? C_NULL : out.ptr, alpha === nothing ? C_NULL : alpha.ptr,
+                               bptr, bstr, mptr, mstr, ws, wsbytes)
+    need = Ref{Csize_t}(0)
+    check(ccall((:mi_attention_workspace_size, libmi), Int32, (Ref{AttnDesc}, Ptr{Csize_t}), mk(C_NULL, 0), need))
+    ws = need[] > 0 ? DeviceArray{UInt8}(undef, Int(need[])) : nothing
+    GC.@preserve q k v bias mask out alpha ws begin
+        check(ccall((:mi_attention_fwd, libmi), Int32, (Ref{AttnDesc}, Ptr{Cvoid}),
+                    mk(ws === nothing ? C_NULL : ws.ptr, need[]), C_NULL))
+    end
+    out, alpha
+end
+
+function dot_product_attention(q::DeviceArray{T, N}, k::DeviceArray{T, N}, v::DeviceArray{T, N}, args...; kws...) where {T, N}
+    batch_size = size(q)[3:end]
+    batch_size == size(k)[3:end] == size(v)[3:end] || throw(ArgumentError("Batch dimensions have to be the same."))
+    q, k, v = map(x -> reshape(x, (size(x, 1), size(x, 2), prod(size(x)[3:end]; init = 1))), (q, k, v))
+    x, α = dot_product_attention(q, k, v, args...; kws...)
+    x = reshape(x, (size(x, 1), size(x, 2), batch_size...))
+    α === nothing || (α = reshape(α, (size(α)[1:3]..., batch_size...)))
+    return x, α
+end
+
+# `return_weights = false` is this library's one addition: it skips materialising α and returns
+# `nothing` in its place (the reference always returns α).
+function dot_product_attention(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::DeviceArray{T, 3}, bias = nothing;
+                               fdrop = identity, mask = nothing, nheads = 1, return_weights = true) where {T <: MIFloat}
+    all(size.((q, k, v), 1) .% nheads .== 0) || throw(ArgumentError("First dimension in query, key and value must be divisible by `nheads`.\nInstead:\n- size(q): $(size(q))\n- size(k): $(size(k))\n- size(v): $(size(v))\n- nheads: $nheads"))
+    size(q, 3) == size(k, 3) == size(v, 3) || throw(ArgumentError("Batch dimensions have to be the same. Instead:\n- size(q): $(size(q))\n- size(k): $(size(k))\n- size(v): $(size(v))"))
+    size(q, 1) == size(k, 1) || throw(ArgumentError("First dimension in query and key has to be the same. Instead:\n- size(q): $(size(q))\n- size(k): $(size(k))"))
+    size(k, 2) == size(v, 2) || throw(ArgumentError("Second dimension in key and value has to be the same. Instead:\n- size(k): $(size(k))\n- size(v): $(size(v))"))
+    if fdrop === identity
+        return attention_call(q, k, v, bias, mask, nheads; want_out = true, want_weights = return_weights)
+    end
+    # any other fdrop acts on the weights the caller sees (src/attention.jl:126): scores -> fdrop -> PV
+    _, α = attention_call(q, k, nothing, bias, mask, nheads; want_out = false, want_weights = true)
+    α = fdrop(α)
+    return weights_times_values(α, v, nheads), α
+end
+
+function dot_product_attention_scores(q::DeviceArray{T, 4}, k::DeviceArray{T, 4}, bias = nothing;
+                                      fdrop = identity, mask = nothing) where {T <: MIFloat}
+    D, H, Lq, B = size(q)
+    (size(k, 1), size(k, 2), size(k, 4)) == (D, H, B) || throw(DimensionMismatch("query $(size(q)) and key $(size(k)) disagree in feature, head or batch size"))
+    _, α = attention_call(reshape(q, (D * H, Lq, B)), reshape(k, (D * H, size(k, 3), B)), nothing, bias, mask, H;
+                          want_out = false, want_weights = true)
+    return fdrop(α)
+end
+
+# x[d,h,i,b] = sum_j α[j,i,h,b] v[d,h,j,b]: one strided batched GEMM over heads per batch element
+function weights_times_values(α::DeviceArray{T, 4}, v::DeviceArray{T, 3}, H::Int) where {T}
+    Ev, Lkv, B = size(v); Lq = size(α, 2); Dv = Ev ÷ H
+    out = DeviceArray{T}(undef, Ev, Lq, B)
+    for b in 0:B-1
+        gemm!('N', 'N', Dv, Lq, Lkv, 1f0, v.ptr + sizeof(T) * b * Ev * Lkv, Ev, Dv,
+              α.ptr + sizeof(T) * b * Lkv * Lq * H, Lkv, Lkv * Lq, 0f0, out.ptr + sizeof(T) * b * Ev * Lq, Ev, Dv, H, T)
+    end
+    out
+end
+
+# ---- softmax ---------------------------------------------------------------------------------------
+softmax(x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = softmax!(similar(x, T, size(x)), x; dims)
+softmax!(x::DeviceArray; dims = 1) = softmax!(x, x; dims)
+function softmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloat}
+    dims == 1 || error("only dims = 1 is built; use NNlib's generic method for other dims")
+    size(out) == size(x) || throw(DimensionMismatch("output size $(size(out)) differs from input size $(size(x))"))
+    rows = size(x, 1); cols = rows == 0 ? 0 : length(x) ÷ rows
+    GC.@preserve out x check(ccall((:mi_softmax_dim1, libmi), Int32, (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Ptr{Cvoid}),
+                                   dtype_code(T), x.ptr, out.ptr, rows, cols, C_NULL))
+    out
+end
+
+# ---- batched_mul -----------------------------------------------------------------------------------
+function gemm!(tA, tB, m, n, k, α, A, lda, sA, B, ldb, sB, β, C, ldc, sC, batch, ::Type{T}) where {T}
+    check(ccall((:mi_batched_gemm, libmi), Int32,
+                (Int32, Cchar, Cchar, Int64, Int64, Int64, Float32, Ptr{Cvoid}, Int64, Int64, Ptr{Cvoid}, Int64, Int64,
+                 Float32, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
+                dtype_code(T), tA, tB, m, n, k, α, A, lda, sA, B, ldb, sB, β, C, ldc, sC, batch, C_NULL);
+          shape_error = DimensionMismatch)
+end
+
+# ('N' | 'T', leading dimension) from strides: the table of _batched_try_gemm!, src/batched/batchedmul.jl:272-294
+function blas_layout(X::DeviceArray{T, 3}) where {T}
+    s1, s2, _ = strides(X)
+    if s2 == 1 && size(X, 1) > 1
+        'T', max(s1, size(X, 2), 1)
+    elseif s1 == 1
+        'N', max(s2, size(X, 1), 1)
+    elseif s2 == 1
+        'T', max(s1, size(X, 2), 1)
+    else
+        throw(ArgumentError("Unsupported array layout for batched mul.\n- Size: $(size(X))\n- Strides: $(strides(X))"))
+    end
+end
+
+function batched_mul!(C::DeviceArray{T, 3}, A::DeviceArray{T, 3}, B::DeviceArray{T, 3}, α::Number = one(Float32),
+                      β::Number = zero(Float32)) where {T <: MIFloat}
+    size(A, 3) == size(C, 3) || size(A, 3) == 1 || throw(DimensionMismatch("batch size mismatch: A != C"))
+    size(B, 3) == size(C, 3) || size(B, 3) == 1 || throw(DimensionMismatch("batch size mismatch: B != C"))
+    m, ka = size(A, 1), size(A, 2); kb, n = size(B, 1), size(B, 2)
+    (ka == kb && m == size(C, 1) && n == size(C, 2)) ||
+        throw(DimensionMismatch("A1 has size ($m,$ka), B1 has size ($kb,$n), C1 has size $(size(C)[1:2])"))
+    (tA, lda), (tB, ldb) = blas_layout(A), blas_layout(B)
+    strides(C)[1] == 1 || throw(ArgumentError("Unsupported array layout for batched mul.\n- Size: $(size(C))\n- Strides: $(strides(C))"))
+    sA = size(A, 3) == 1 ? 0 : strides(A)[3]          # src/gemm.jl:117-118
+    sB = size(B, 3) == 1 ? 0 : strides(B)[3]
+    GC.@preserve A B C gemm!(tA, tB, m, n, ka, Float32(α), A.ptr, lda, sA, B.ptr, ldb, sB, Float32(β), C.ptr,
+                              max(strides(C)[2], m, 1), strides(C)[3], size(C, 3), T)
+    C
+end
+
+function batched_mul(A::DeviceArray{T, 3}, B::DeviceArray{T, 3}) where {T <: MIFloat}
+    size(A, 3) == size(B, 3) || size(A, 3) == 1 || size(B, 3) == 1 || throw(DimensionMismatch("batch size mismatch: A != B"))
+    batched_mul!(DeviceArray{T}(undef, size(A, 1), size(B, 2), max(size(A, 3), size(B, 3))), A, B)
+end
+
+function batched_mul(x::DeviceArray{T, N}, y::DeviceArray{T, N}) where {T <: MIFloat, N}
+    batch_size = size(x)[3:end]
+    @assert batch_size == size(y)[3:end] "batch size has to be the same for the two arrays."
+    z = batched_mul(reshape(x, (size(x, 1), size(x, 2), prod(batch_size))), reshape(y, (size(y, 1), size(y, 2), prod(batch_size))))
+    reshape(z, (size(z, 1), size(z, 2), batch_size...))
+end
+
+end # module
