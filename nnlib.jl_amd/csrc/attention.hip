@@ -11,7 +11,47 @@ int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t);
 bool flash16_fast_supports_bf16(const AttnParams &);
 bool flash16_fast_supports_f16(const AttnParams &);
 
+#include "flash_common.h"
+
 static inline bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
+
+// ---- merge of split-kv partials -------------------------------------------------------------------
+// out[e, q, b] = sum_s o_s * 2^(m_s - m) / sum_s l_s * 2^(m_s - m), m = max_s m_s.  A row whose every
+// piece was fully masked has m = -Inf and comes out NaN, as the unsplit kernel (and the reference) gives.
+template <typename T>
+__global__ __launch_bounds__(256) void flash_merge_kernel(const float *ws, typename T::type *out, int nsplit, int64_t B,
+                                                           int64_t Lq, int64_t Ev, int64_t H) {
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t qi = blockIdx.y, b = blockIdx.z;
+    if (e >= Ev) return;
+    const int64_t h = e / (Ev / H);
+    const float *wml = ws + (int64_t)nsplit * B * Lq * Ev;
+    float m = MI_NEG_INF;
+    for (int s = 0; s < nsplit; s++) m = fmaxf(m, wml[((((int64_t)s * B + b) * H + h) * Lq + qi) * 2]);
+    float o = 0.0f, l = 0.0f;
+    for (int s = 0; s < nsplit; s++) {
+        const float *ml = wml + ((((int64_t)s * B + b) * H + h) * Lq + qi) * 2;
+        const float w = mi_exp2(ml[0] - m);
+        l = fmaf(ml[1], w, l);
+        o = fmaf(ws[(((int64_t)s * B + b) * Lq + qi) * Ev + e], w, o);
+    }
+    out[Ev * (Lq * b + qi) + e] = T::from_f32(o / l);
+}
+
+int32_t launch_flash_merge(const AttnParams &p, int nsplit, hipStream_t st) {
+    if (p.Lq > 65535 || p.B > 65535) return mi_set_error(MI_ESHAPE, "split-kv merge supports at most 65535 queries and batches");
+    dim3 grid((unsigned)((p.Ev + 255) / 256), (unsigned)p.Lq, (unsigned)p.B);
+    const float *ws = (const float *)p.workspace;
+    if (p.dtype == MI_BF16)
+        hipLaunchKernelGGL(flash_merge_kernel<BF16>, grid, dim3(256), 0, st, ws, (__bf16 *)p.out, nsplit, p.B, p.Lq, p.Ev, p.H);
+    else
+        hipLaunchKernelGGL(flash_merge_kernel<F16>, grid, dim3(256), 0, st, ws, (_Float16 *)p.out, nsplit, p.B, p.Lq, p.Ev, p.H);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+// true when the call takes the software-pipelined head-dim-128 kernel (which never splits)
+static bool takes_fast_path(const AttnParams &p);
 
 bool attention_flash16_supports(const AttnParams &p) {
     if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
@@ -21,6 +61,10 @@ bool attention_flash16_supports(const AttnParams &p) {
     const int64_t tiles = (p.Lq + 127) / 128;
     if (tiles * p.H * p.B > 2147483647LL) return false;
     return true;
+}
+
+static bool takes_fast_path(const AttnParams &p) {
+    return (p.dtype == MI_BF16 && flash16_fast_supports_bf16(p)) || (p.dtype == MI_F16 && flash16_fast_supports_f16(p));
 }
 
 int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
@@ -85,7 +129,10 @@ static int32_t choose(const mi_attn_desc *d, const AttnParams &p, size_t *ws) {
         *ws = attention_decode_workspace(p);
         return MI_ATTN_KERNEL_DECODE;
     }
-    if (attention_flash16_supports(p)) return MI_ATTN_KERNEL_FLASH16;
+    if (attention_flash16_supports(p)) {
+        if (!takes_fast_path(p)) *ws = flash_split_workspace(p, flash_pick_nsplit(p, 128));
+        return MI_ATTN_KERNEL_FLASH16;
+    }
     if (attention_flash32_supports(p)) return MI_ATTN_KERNEL_FLASH32;
     return MI_ATTN_KERNEL_GENERIC;
 }

@@ -245,6 +245,8 @@ bool attention_flash32_supports(const AttnParams &p) {
 int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     FlashArgs a;
     a.p = p;
+    a.nsplit = 1;
+    a.tiles_per_split = 0;
     a.c = MI_LOG2E;  // q is pre-divided by sqrt(D); only the change of base remains
     a.n_qtiles = (int32_t)((p.Lq + 127) / 128);
     flash_fill_vec_flags(a);

@@ -17,7 +17,28 @@ struct FlashArgs {
     int32_t bias_vec;  // bias rows may be read 4 keys at a time
     int32_t mask_vec;
     int32_t w_vec;     // weight rows may be written 4 keys at a time
+    int32_t nsplit;    // key range is cut into this many pieces, one workgroup each (1 = no split)
+    int32_t tiles_per_split;
 };
+
+// Split-kv bookkeeping shared by the planner (workspace size) and the launchers.
+// Partials live in the caller's workspace: o as [split][B][Lq][Ev] floats, then (m, l) as
+// [split][B][H][Lq][2] floats, m in log2 units.
+inline int flash_pick_nsplit(const AttnParams &p, int bm) {
+    if (p.weights || !p.out) return 1;                      // weights need the global maximum up front
+    const int64_t wgs = ((p.Lq + bm - 1) / bm) * p.H * p.B;
+    if (wgs >= 512 || p.Lkv < 2048) return 1;
+    int64_t n = (1024 + wgs - 1) / wgs;
+    const int64_t max_by_len = p.Lkv / 512;                 // at least 512 keys per piece
+    if (n > max_by_len) n = max_by_len;
+    if (n > 64) n = 64;
+    return n < 1 ? 1 : (int)n;
+}
+inline size_t flash_split_workspace(const AttnParams &p, int nsplit) {
+    if (nsplit <= 1) return 0;
+    return sizeof(float) * (size_t)nsplit * (size_t)p.B * (size_t)p.Lq * (size_t)(p.Ev + 2 * p.H);
+}
+int32_t launch_flash_merge(const AttnParams &p, int nsplit, hipStream_t st);
 
 enum { PHASE_ONLINE = 0, PHASE_STATS = 1, PHASE_FINAL = 2 };
 

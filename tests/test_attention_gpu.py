@@ -265,3 +265,36 @@ def test_decode_matches_flash16_on_device(nn):
     y2, _ = nn.dot_product_attention(q, k, v, nheads=4, return_weights=True)   # weights force the tiled kernel
     assert nn.last_attention_kernel() == "flash16"
     assert rel_err(y1.to_numpy(), y2.to_numpy()) < 1e-2
+
+
+SPLIT_CASES = [
+    ("f16", 128, 100, 3000, 1, 2, dict(bias_shape=(3000, 100, 2, 1), mask_shape=(3000, 100))),
+    ("f16", 128, 256, 4096, 2, 2, dict(bias_shape=(4096, 256, 2, 2))),
+    ("bf16", 128, 2048, 2048, 1, 2, dict(causal=True)),            # head dim 64: general kernel, causal pieces
+    ("bf16", 64, 70, 2500, 3, 1, {}),
+    ("f16", 256, 130, 2100, 1, 2, dict(mask_shape=(2100, 130))),    # head dim 128 with a mask
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_CASES, ids=lambda c: f"{c[0]}-E{c[1]}-Lq{c[2]}-Lkv{c[3]}-B{c[4]}-H{c[5]}-" + "-".join(c[6]))
+def test_split_kv_parity(nn, oracle, case):
+    """Few (query tile, head, batch) workgroups and a long key range: the key range is cut into pieces,
+    one workgroup each, and a second kernel merges the partial (m, l, o)."""
+    dtype, E, Lq, Lkv, B, H, kw = case
+    rng = np.random.default_rng(hash((E, Lq, Lkv, B, H, 7)) % 2**32)
+    import ctypes
+    _check(nn, oracle, rng, dtype, E, Lq, Lkv, B, H, expect="flash16", weights=False, **kw)
+    from nnlib_amd import ops
+    assert ops._workspace is not None and ops._workspace.numel() > 0      # the split path was taken
+
+
+def test_split_kv_fully_masked_query(nn):
+    rng = np.random.default_rng(12)
+    q = rng.standard_normal((128, 40, 1)).astype(np.float32)
+    k = rng.standard_normal((128, 2600, 1)).astype(np.float32)
+    mask = np.ones((2600, 40), bool)
+    mask[:, 7] = False
+    mask[:2000, 9] = False             # whole pieces masked, but not the query
+    y, _ = _run(nn, q, k, k, "f16", mask=mask, nheads=2, return_weights=False)
+    assert np.isnan(y[:, 7, 0]).all()
+    assert np.isfinite(np.delete(y, 7, axis=1)).all()
