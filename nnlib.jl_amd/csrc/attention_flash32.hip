@@ -100,7 +100,7 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
                             s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(k4[j], f.q[qb][4 * c + j], s[qb][kb], 0, 0, 0);
                 }
 
-            flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0);
+            flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0);
 
             if (do_pv) {
                 // k-step v of key block kb multiplies key 32*kb + 8*(v/4) + 4*hh + v%4: exactly the key

@@ -44,6 +44,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2_t;
 typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
 
 // ---- element traits ----------------------------------------------------------------

@@ -19,6 +19,8 @@ struct FlashArgs {
     int32_t w_vec;     // weight rows may be written 4 keys at a time
     int32_t nsplit;    // key range is cut into this many pieces, one workgroup each (1 = no split)
     int32_t tiles_per_split;
+    int32_t bias_lds;  // 16-bit kernels: bias / mask tiles may be staged through LDS with 16-byte DMA pieces
+    int32_t mask_lds;
 };
 
 // Split-kv bookkeeping shared by the planner (workspace size) and the launchers.
@@ -41,6 +43,9 @@ inline size_t flash_split_workspace(const AttnParams &p, int nsplit) {
 int32_t launch_flash_merge(const AttnParams &p, int nsplit, hipStream_t st);
 
 enum { PHASE_ONLINE = 0, PHASE_STATS = 1, PHASE_FINAL = 2 };
+// how a kernel variant reads bias / mask: not at all, straight from global memory with arbitrary
+// strides, or from tiles staged through LDS (FlashStaged; every array present must qualify)
+enum { EXTRAS_NONE = 0, EXTRAS_DIRECT = 1, EXTRAS_STAGED = 2 };
 
 inline void flash_fill_vec_flags(FlashArgs &a) {
     const AttnParams &p = a.p;
@@ -51,17 +56,128 @@ inline void flash_fill_vec_flags(FlashArgs &a) {
     a.mask_vec = p.mask && p.mask_strides[0] == 1 && mult4(p.mask_strides[1]) && mult4(p.mask_strides[2]) &&
                  mult4(p.mask_strides[3]) && mult4(p.Lkv) && (((uintptr_t)p.mask) & 3) == 0;
     a.w_vec = p.weights && mult4(p.Lkv) && (((uintptr_t)p.weights) & 15) == 0;
+    // LDS staging moves 16-byte pieces addressed with 32-bit byte offsets from the (head, batch) slice:
+    // rows must start 16-byte aligned and the slice (plus one query tile of slack) must stay below 2 GiB.
+    auto fits = [&](const int64_t *st, size_t elem) {
+        const int64_t reach = ((p.Lq + 256) * st[1] + p.Lkv + FLASH_BN) * (int64_t)elem;
+        const int64_t per16 = 16 / (int64_t)elem;
+        return st[0] == 1 && st[1] % per16 == 0 && st[2] % per16 == 0 && st[3] % per16 == 0 && reach < (int64_t)0x7fffffff;
+    };
+    a.bias_lds = p.bias && es == 2 && fits(p.bias_strides, es) && (((uintptr_t)p.bias) & 15) == 0;
+    a.mask_lds = p.mask && es == 2 && fits(p.mask_strides, 1) && (((uintptr_t)p.mask) & 15) == 0;
 }
+
+// Encoding of s_waitcnt for "at most N vector memory operations outstanding" (vmcnt[3:0] | expcnt[6:4] |
+// lgkmcnt[11:8] | vmcnt[15:14]); the other counters are left unconstrained.
+#define FLASH_WAIT_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (((N) >> 4) << 14) | (7 << 4) | (15 << 8))
+
+// One 1 KiB piece global -> LDS (64 lanes x 16 bytes, lane l lands at lds_addr + 16*l; lanes whose
+// offset is outside the buffer write zeros).  Issued as inline assembly so that the compiler does not
+// serialise later LDS reads behind it; completion is tracked by hand with FLASH_WAIT_VMCNT (vector
+// memory loads complete in order).
+__device__ inline void flash_dma_1k(const i32x4_t &rsrc, unsigned lds_addr, int voffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voffset), "s"(rsrc)
+                 : "memory", "m0");
+}
+
+__device__ inline i32x4_t flash_make_rsrc(const void *base, uint32_t bytes) {
+    const uint64_t addr = (uint64_t)base;
+    i32x4_t rs;
+    rs[0] = __builtin_amdgcn_readfirstlane((int)(addr & 0xffffffffu));
+    rs[1] = __builtin_amdgcn_readfirstlane((int)((addr >> 32) & 0xffffu));  // stride 0: raw buffer
+    rs[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+    rs[3] = 0x00020000;
+    return rs;
+}
+
+// Bias / mask tiles of one wavefront staged through LDS (16-bit kernels).  A wavefront owns 32*QB query
+// rows; per kv tile it needs, for each of them, 64 bias elements (128 bytes) and 64 mask bytes.  Reading
+// those straight from global memory in the accumulator layout makes every load instruction touch 32
+// different cache lines for 16 (bias) or 8 (mask) bytes each; instead the wavefront copies the
+// [rows][64] tile with full-width DMA pieces into a private LDS region, one tile ahead, and reads it
+// back in the accumulator layout.  16-byte chunks are XOR-swizzled per row so that those reads spread
+// over all banks.  The regions are private to the wavefront: no barrier is involved, only vmcnt.
+typedef __attribute__((address_space(3))) const unsigned char flash_lds_cu8;
+template <int QB>
+struct FlashStaged {
+    static constexpr int BIAS_STAGE = 32 * QB * 128, MASK_STAGE = 32 * QB * 64;  // bytes per stage
+    static constexpr int BYTES_PER_WAVE = 2 * (BIAS_STAGE + MASK_STAGE);
+    bool bias = false, mask = false;
+    i32x4_t brs, mrs;
+    unsigned blds, mlds;                 // LDS byte addresses of the two-stage regions
+    int bvoff[4 * QB], mvoff[2 * QB];    // per-lane global byte offsets of the DMA pieces (tile term excluded)
+
+    __device__ static int bias_swz(int row) { return (row >> 1) & 7; }
+    __device__ static int mask_swz(int row) { return (row >> 2) & 3; }
+
+    __device__ void init(const FlashArgs &a, unsigned lds_wave_base, int lane, int64_t iw, int64_t h, int64_t b) {
+        const AttnParams &p = a.p;
+        bias = a.bias_lds;
+        mask = a.mask_lds;
+        blds = __builtin_amdgcn_readfirstlane(lds_wave_base);  // wave-uniform: goes into M0
+        mlds = blds + 2 * BIAS_STAGE;
+        {   // set up unconditionally so that the resource words stay in scalar registers
+            const int64_t s1 = p.bias_strides[1];
+            const char *base = (const char *)p.bias + 2 * (h * p.bias_strides[2] + b * p.bias_strides[3]);
+            brs = flash_make_rsrc(base, (uint32_t)(2 * ((p.Lq - 1) * s1 + p.Lkv)));
+#pragma unroll
+            for (int i = 0; i < 4 * QB; i++) {
+                const int row = 8 * i + (lane >> 3);
+                bvoff[i] = (int)(2 * (iw + row) * s1) + (((lane & 7) ^ bias_swz(row)) << 4);
+            }
+        }
+        {
+            const int64_t s1 = p.mask_strides[1];
+            const char *base = (const char *)p.mask + h * p.mask_strides[2] + b * p.mask_strides[3];
+            mrs = flash_make_rsrc(base, (uint32_t)((p.Lq - 1) * s1 + p.Lkv));
+#pragma unroll
+            for (int i = 0; i < 2 * QB; i++) {
+                const int row = 16 * i + (lane >> 2);
+                mvoff[i] = (int)((iw + row) * s1) + (((lane & 3) ^ mask_swz(row)) << 4);
+            }
+        }
+    }
+    // start the copy of the tile whose first key is j0 into `stage`
+    __device__ void issue(int stage, int64_t j0) const {
+        if (bias) {
+#pragma unroll
+            for (int i = 0; i < 4 * QB; i++) flash_dma_1k(brs, blds + stage * BIAS_STAGE + i * 1024, bvoff[i] + (int)(2 * j0));
+        }
+        if (mask) {
+#pragma unroll
+            for (int i = 0; i < 2 * QB; i++) flash_dma_1k(mrs, mlds + stage * MASK_STAGE + i * 1024, mvoff[i] + (int)j0);
+        }
+    }
+    // all copies issued so far have landed
+    __device__ void wait() const {
+        if (bias || mask) {
+            FLASH_WAIT_VMCNT(0);
+            asm volatile("" ::: "memory");
+        }
+    }
+    // 4 consecutive bias elements (8 bytes) / mask bytes of wavefront row `row`, keys 8*c8 + 4*hh .. +3 of the tile
+    template <typename V4>
+    __device__ V4 bias4(int stage, int row, int c8, int hh) const {
+        const unsigned addr = blds + stage * BIAS_STAGE + row * 128 + ((c8 ^ bias_swz(row)) << 4) + 8 * hh;
+        return *(__attribute__((address_space(3))) const V4 *)(uintptr_t)addr;
+    }
+    __device__ uint32_t mask4(int stage, int row, int c8, int hh) const {
+        const unsigned addr = mlds + stage * MASK_STAGE + row * 64 + (((c8 >> 1) ^ mask_swz(row)) << 4) + 8 * (c8 & 1) + 4 * hh;
+        return *(__attribute__((address_space(3))) const uint32_t *)(uintptr_t)addr;
+    }
+};
 
 // On entry s[qb][kb] holds raw dot products k.q of tile rows [j0, j0+64) for the wavefront's query
 // blocks; on exit it holds exp2(x - m) (ONLINE / STATS) or the final normalised weights (FINAL),
 // with m, l (and, ONLINE only, the output accumulators o) updated.
 //   T      element traits of the bias array
 //   NDV    number of 32-row blocks of the output accumulator
-template <typename T, int QB, int NDV, bool CAUSAL, bool EXTRAS, int PHASE, typename TW>
+template <typename T, int QB, int NDV, bool CAUSAL, int EXTRAS, int PHASE, typename TW>
 __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB][2], floatx16_t (&o)[QB][NDV],
                                           float (&fm)[QB], float (&fl)[QB], int64_t b, int64_t h, int64_t iw,
-                                          int64_t j0) {
+                                          int64_t j0, const FlashStaged<QB> &sg = FlashStaged<QB>(), int stage = 0) {
     const AttnParams &p = a.p;
     typedef typename T::type elem_t;
     constexpr int BN = FLASH_BN;
@@ -85,30 +201,43 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                     bool keep[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) keep[e] = kv + e < p.Lkv && (!CAUSAL || kv + e <= qi);
-                    if (bias && qok) {
-                        if (a.bias_vec) {
-                            if (kv < p.Lkv) {
-                                typename T::vec4 t4 = *(const typename T::vec4 *)(bias + boff + kv);
+                    if (EXTRAS == EXTRAS_STAGED) {
+                        if (sg.bias) {
+                            typename T::vec4 t4 = sg.template bias4<typename T::vec4>(stage, 32 * qb + r, 4 * kb + g, hh);
 #pragma unroll
-                                for (int e = 0; e < 4; e++) bv[e] = T::to_f32(t4[e]);
-                            }
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                if (kv + e < p.Lkv) bv[e] = T::to_f32(bias[boff + (kv + e) * p.bias_strides[0]]);
+                            for (int e = 0; e < 4; e++) bv[e] = T::to_f32(t4[e]);
                         }
-                    }
-                    if (p.mask && qok) {
-                        if (a.mask_vec) {
-                            if (kv < p.Lkv) {
-                                uint32_t m4 = *(const uint32_t *)(p.mask + moff + kv);
+                        if (sg.mask) {
+                            const uint32_t m4 = sg.mask4(stage, 32 * qb + r, 4 * kb + g, hh);
 #pragma unroll
-                                for (int e = 0; e < 4; e++) keep[e] = keep[e] && ((m4 >> (8 * e)) & 0xFF);
+                            for (int e = 0; e < 4; e++) keep[e] = keep[e] && ((m4 >> (8 * e)) & 0xFF);
+                        }
+                    } else {
+                        if (bias && qok) {
+                            if (a.bias_vec) {
+                                if (kv < p.Lkv) {
+                                    typename T::vec4 t4 = *(const typename T::vec4 *)(bias + boff + kv);
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) bv[e] = T::to_f32(t4[e]);
+                                }
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    if (kv + e < p.Lkv) bv[e] = T::to_f32(bias[boff + (kv + e) * p.bias_strides[0]]);
                             }
-                        } else {
+                        }
+                        if (p.mask && qok) {
+                            if (a.mask_vec) {
+                                if (kv < p.Lkv) {
+                                    uint32_t m4 = *(const uint32_t *)(p.mask + moff + kv);
 #pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                if (kv + e < p.Lkv) keep[e] = keep[e] && p.mask[moff + (kv + e) * p.mask_strides[0]];
+                                    for (int e = 0; e < 4; e++) keep[e] = keep[e] && ((m4 >> (8 * e)) & 0xFF);
+                                }
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    if (kv + e < p.Lkv) keep[e] = keep[e] && p.mask[moff + (kv + e) * p.mask_strides[0]];
+                            }
                         }
                     }
 #pragma unroll

@@ -181,6 +181,10 @@ FLASH16_CASES = [
     ("bf16", 128, 64, 256, 1, 1, dict(bias_shape=(256, 1, 1, 1))),
     ("bf16", 256, 128, 128, 1, 2, dict(causal=True, mask_shape=(128, 128))),
     ("f16", 64, 33, 65, 3, 1, {}),
+    # 16-byte aligned bias / mask rows: tiles staged through LDS; ragged tails in both lengths
+    ("f16", 128, 70, 336, 2, 2, dict(bias_shape=(336, 70, 2, 2), mask_shape=(336, 70, 1, 2))),
+    ("bf16", 256, 150, 400, 1, 2, dict(bias_shape=(400, 150, 1, 1), mask_shape=(400, 1, 2, 1))),
+    ("bf16", 128, 192, 192, 2, 2, dict(causal=True, bias_shape=(192, 192, 2, 1))),
 ]
 
 
