@@ -248,6 +248,7 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     a.nsplit = 1;
     a.tiles_per_split = 0;
     a.c = MI_LOG2E;  // q is pre-divided by sqrt(D); only the change of base remains
+    a.cn = 1.0f;
     a.n_qtiles = (int32_t)((p.Lq + 127) / 128);
     flash_fill_vec_flags(a);
     return p.D == 64 ? launch_d<64, 1>(a, st) : launch_d<128, 1>(a, st);

@@ -12,7 +12,8 @@ constexpr int FLASH_BN = 64;  // keys per tile
 
 struct FlashArgs {
     AttnParams p;
-    float c;           // log2(e) / sqrt(D)
+    float c;           // log2(e) * cn
+    float cn;          // factor that turns an accumulator into the reference's logit: 1/sqrt(D), or 1 when q is pre-scaled
     int32_t n_qtiles;
     int32_t bias_vec;  // bias rows may be read 4 keys at a time
     int32_t mask_vec;
@@ -187,8 +188,38 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
     for (int qb = 0; qb < QB; qb++) {
         const int64_t qi = iw + 32 * qb + r;
         const bool qok = qi < p.Lq;
-        // ---- scale, bias, mask: x = log2(e) * (reference logit) --------------------------------
-        if (EXTRAS) {
+        // ---- scale, bias, mask.  With bias / mask the accumulators end up holding the reference's
+        // logits (natural units); without, they keep the raw dot products and the positive factor c
+        // is folded into the exponent below (max commutes with a positive scale).
+        if (EXTRAS == EXTRAS_STAGED) {
+            const int row = 32 * qb + r;
+            if (sg.bias) {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const typename T::vec4 t4 = sg.template bias4<typename T::vec4>(stage, row, 4 * kb + g, hh);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) s[qb][kb][4 * g + e] = fmaf(s[qb][kb][4 * g + e], a.cn, T::to_f32(t4[e]));
+                    }
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) s[qb][kb][v] *= a.cn;
+            }
+            if (sg.mask) {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const uint32_t m4 = sg.mask4(stage, row, 4 * kb + g, hh);
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            s[qb][kb][4 * g + e] = (m4 & (0xFFu << (8 * e))) ? s[qb][kb][4 * g + e] : MI_NEG_INF;
+                    }
+            }
+        } else if (EXTRAS == EXTRAS_DIRECT) {
             const elem_t *bias = (const elem_t *)p.bias;
             const int64_t boff = qi * p.bias_strides[1] + h * p.bias_strides[2] + b * p.bias_strides[3];
             const int64_t moff = qi * p.mask_strides[1] + h * p.mask_strides[2] + b * p.mask_strides[3];
@@ -201,66 +232,56 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                     bool keep[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) keep[e] = kv + e < p.Lkv && (!CAUSAL || kv + e <= qi);
-                    if (EXTRAS == EXTRAS_STAGED) {
-                        if (sg.bias) {
-                            typename T::vec4 t4 = sg.template bias4<typename T::vec4>(stage, 32 * qb + r, 4 * kb + g, hh);
+                    if (bias && qok) {
+                        if (a.bias_vec) {
+                            if (kv < p.Lkv) {
+                                typename T::vec4 t4 = *(const typename T::vec4 *)(bias + boff + kv);
 #pragma unroll
-                            for (int e = 0; e < 4; e++) bv[e] = T::to_f32(t4[e]);
-                        }
-                        if (sg.mask) {
-                            const uint32_t m4 = sg.mask4(stage, 32 * qb + r, 4 * kb + g, hh);
-#pragma unroll
-                            for (int e = 0; e < 4; e++) keep[e] = keep[e] && ((m4 >> (8 * e)) & 0xFF);
-                        }
-                    } else {
-                        if (bias && qok) {
-                            if (a.bias_vec) {
-                                if (kv < p.Lkv) {
-                                    typename T::vec4 t4 = *(const typename T::vec4 *)(bias + boff + kv);
-#pragma unroll
-                                    for (int e = 0; e < 4; e++) bv[e] = T::to_f32(t4[e]);
-                                }
-                            } else {
-#pragma unroll
-                                for (int e = 0; e < 4; e++)
-                                    if (kv + e < p.Lkv) bv[e] = T::to_f32(bias[boff + (kv + e) * p.bias_strides[0]]);
+                                for (int e = 0; e < 4; e++) bv[e] = T::to_f32(t4[e]);
                             }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (kv + e < p.Lkv) bv[e] = T::to_f32(bias[boff + (kv + e) * p.bias_strides[0]]);
                         }
-                        if (p.mask && qok) {
-                            if (a.mask_vec) {
-                                if (kv < p.Lkv) {
-                                    uint32_t m4 = *(const uint32_t *)(p.mask + moff + kv);
+                    }
+                    if (p.mask && qok) {
+                        if (a.mask_vec) {
+                            if (kv < p.Lkv) {
+                                uint32_t m4 = *(const uint32_t *)(p.mask + moff + kv);
 #pragma unroll
-                                    for (int e = 0; e < 4; e++) keep[e] = keep[e] && ((m4 >> (8 * e)) & 0xFF);
-                                }
-                            } else {
-#pragma unroll
-                                for (int e = 0; e < 4; e++)
-                                    if (kv + e < p.Lkv) keep[e] = keep[e] && p.mask[moff + (kv + e) * p.mask_strides[0]];
+                                for (int e = 0; e < 4; e++) keep[e] = keep[e] && ((m4 >> (8 * e)) & 0xFF);
                             }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (kv + e < p.Lkv) keep[e] = keep[e] && p.mask[moff + (kv + e) * p.mask_strides[0]];
                         }
                     }
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        float x = fmaf(s[qb][kb][4 * g + e], a.c, bv[e] * MI_LOG2E);
+                        float x = fmaf(s[qb][kb][4 * g + e], a.cn, bv[e]);
                         s[qb][kb][4 * g + e] = keep[e] ? x : MI_NEG_INF;
                     }
                 }
-        } else if (edge) {
+        }
+        if (EXTRAS != EXTRAS_DIRECT && edge) {
+            // keys past the end of the sequence or, causal, after the query: tile-local limit per lane
+            int64_t lim64 = p.Lkv - j0;
+            if (CAUSAL && qi - j0 + 1 < lim64) lim64 = qi - j0 + 1;
+            const int lim = lim64 > BN ? BN : (lim64 < 0 ? 0 : (int)lim64);
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
-                    const int64_t kv = j0 + 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4);
-                    const bool keep = kv < p.Lkv && (!CAUSAL || kv <= qi);
-                    s[qb][kb][v] = keep ? s[qb][kb][v] : MI_NEG_INF;
+                    const int kvl = 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4);
+                    s[qb][kb][v] = kvl < lim ? s[qb][kb][v] : MI_NEG_INF;
                 }
         }
-        // Without EXTRAS the accumulators still hold raw dot products; the positive factor c is
-        // folded into the exponent below (max commutes with a positive scale).
-        const float cs = EXTRAS ? 1.0f : a.c;
+        const float cs = EXTRAS ? MI_LOG2E : a.c;
 
         float pmul = 1.0f, msafe;
+        bool pinf;  // the running maximum is +Inf: weights become the normalised indicator of the +Inf entries
         if (PHASE != PHASE_FINAL) {
             float mx = MI_NEG_INF;
 #pragma unroll
@@ -273,6 +294,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             msafe = mnew == MI_NEG_INF ? 0.0f : mnew;
             float resc = mi_exp2((mold - msafe) * cs);
             if (EXTRAS && mold == mnew) resc = 1.0f;  // also covers +Inf == +Inf
+            pinf = mnew == MI_POS_INF;
             fm[qb] = mnew;
             fl[qb] *= resc;
             if (PHASE == PHASE_ONLINE) {
@@ -283,7 +305,19 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             }
         } else {
             msafe = fm[qb] == MI_NEG_INF ? 0.0f : fm[qb];
+            pinf = fm[qb] == MI_POS_INF;
             pmul = fl[qb];  // holds 1 / (row sum) in the final phase
+        }
+        // src/softmax.jl:74-75.  Only bias or an upstream overflow can produce +Inf logits, so the
+        // per-element work sits behind a wavefront-uniform test.
+        if (EXTRAS && __builtin_expect(__builtin_amdgcn_ballot_w64(pinf) != 0, 0)) {
+            if (pinf) {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) s[qb][kb][v] = s[qb][kb][v] == MI_POS_INF ? 0.0f : MI_NEG_INF;
+                msafe = 0.0f;
+            }
         }
         const float moff2 = -msafe * cs;
         float lsum = 0.0f;
@@ -293,7 +327,6 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             for (int v = 0; v < 16; v++) {
                 float x = s[qb][kb][v];
                 float e = mi_exp2(fmaf(x, cs, moff2));
-                if (EXTRAS) e = (x == MI_POS_INF) ? 1.0f : e;  // src/softmax.jl:74-75
                 if (PHASE == PHASE_FINAL) e *= pmul;
                 lsum += e;
                 s[qb][kb][v] = e;
