@@ -302,3 +302,31 @@ def test_split_kv_fully_masked_query(nn):
     y, _ = _run(nn, q, k, k, "f16", mask=mask, nheads=2, return_weights=False)
     assert np.isnan(y[:, 7, 0]).all()
     assert np.isfinite(np.delete(y, 7, axis=1)).all()
+
+
+@pytest.mark.parametrize("dtype,E,Lkv,expect", [("f32", 128, 136, "flash32"), ("f16", 128, 144, "flash16"),
+                                                ("bf16", 128, 131, "flash16"), ("f16", 48, 75, "generic")],
+                         ids=["flash32", "flash16-staged", "flash16-direct", "generic"])
+@pytest.mark.parametrize("weights", [False, True], ids=["noweights", "weights"])
+def test_plus_inf_logits(nn, oracle, dtype, E, Lkv, expect, weights):
+    """src/softmax.jl:69-75: a column whose maximum is +Inf becomes the normalised indicator of its +Inf
+    entries.  +Inf enters through the bias; one query has it in two tiles, one in a later tile only."""
+    rng = np.random.default_rng(31)
+    Lq, B, H = 40, 2, 2
+    q = round_to(rng.standard_normal((E, Lq, B)), dtype)
+    k = round_to(rng.standard_normal((E, Lkv, B)), dtype)
+    v = round_to(rng.standard_normal((E, Lkv, B)), dtype)
+    bias = round_to(0.5 * rng.standard_normal((Lkv, Lq, H, B)), dtype)
+    bias[3, 5] = np.inf
+    bias[Lkv - 2, 5] = np.inf
+    bias[70, 9] = np.inf
+    bias[0, 11, 1, 0] = np.inf
+    y, a = _run(nn, q, k, v, dtype, bias, None, H, return_weights=weights, weights_dtype="f32")
+    assert nn.last_attention_kernel() == expect
+    yr, ar = oracle.nnlib_attention_f32(q, k, v, bias, None, H)
+    assert np.isfinite(yr).all()
+    tol = 1e-4 if dtype == "f32" else 1e-2
+    assert rel_err(y, yr) < tol
+    if weights:
+        assert np.allclose(a, ar, atol=tol)
+        assert a[3, 5, 0, 0] == 0.5 and a[Lkv - 2, 5, 1, 1] == 0.5 and a[70, 9, 0, 1] == 1.0 and a[1, 5, 0, 0] == 0.0
