@@ -21,26 +21,37 @@ static inline bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0;
 template <typename T>
 __global__ __launch_bounds__(256) void flash_merge_kernel(const float *ws, typename T::type *out, int nsplit, int64_t B,
                                                            int64_t Lq, int64_t Ev, int64_t H) {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    // one thread per 4 consecutive output features (same head: head dims are multiples of 4)
+    const int64_t e = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     const int64_t qi = blockIdx.y, b = blockIdx.z;
     if (e >= Ev) return;
     const int64_t h = e / (Ev / H);
-    const float *wml = ws + (int64_t)nsplit * B * Lq * Ev;
+    const float *wml = ws + (int64_t)nsplit * B * Lq * Ev + ((b * H + h) * Lq + qi) * 2;
+    const int64_t ml_step = B * H * Lq * 2, o_step = B * Lq * Ev;
+    const float *wo = ws + (b * Lq + qi) * Ev + e;
     float m = MI_NEG_INF;
-    for (int s = 0; s < nsplit; s++) m = fmaxf(m, wml[((((int64_t)s * B + b) * H + h) * Lq + qi) * 2]);
-    float o = 0.0f, l = 0.0f;
+    for (int s = 0; s < nsplit; s++) m = fmaxf(m, wml[s * ml_step]);
+    floatx4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
+    float l = 0.0f;
+#pragma unroll 4
     for (int s = 0; s < nsplit; s++) {
-        const float *ml = wml + ((((int64_t)s * B + b) * H + h) * Lq + qi) * 2;
+        const floatx2_t ml = *(const floatx2_t *)(wml + s * ml_step);
+        const floatx4_t o4 = *(const floatx4_t *)(wo + s * o_step);
         const float w = mi_exp2(ml[0] - m);
         l = fmaf(ml[1], w, l);
-        o = fmaf(ws[(((int64_t)s * B + b) * Lq + qi) * Ev + e], w, o);
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = fmaf(o4[i], w, o[i]);
     }
-    out[Ev * (Lq * b + qi) + e] = T::from_f32(o / l);
+    const float inv = 1.0f / l;
+    typename T::vec4 r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r[i] = T::from_f32(o[i] * inv);
+    *(typename T::vec4 *)(out + Ev * (Lq * b + qi) + e) = r;
 }
 
 int32_t launch_flash_merge(const AttnParams &p, int nsplit, hipStream_t st) {
     if (p.Lq > 65535 || p.B > 65535) return mi_set_error(MI_ESHAPE, "split-kv merge supports at most 65535 queries and batches");
-    dim3 grid((unsigned)((p.Ev + 255) / 256), (unsigned)p.Lq, (unsigned)p.B);
+    dim3 grid((unsigned)((p.Ev / 4 + 255) / 256), (unsigned)p.Lq, (unsigned)p.B);
     const float *ws = (const float *)p.workspace;
     if (p.dtype == MI_BF16)
         hipLaunchKernelGGL(flash_merge_kernel<BF16>, grid, dim3(256), 0, st, ws, (__bf16 *)p.out, nsplit, p.B, p.Lq, p.Ev, p.H);
