@@ -127,7 +127,8 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
 }
 
 template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS>
-__global__ __launch_bounds__(256, 1) void flash32_kernel(FlashArgs a) {
+// Head dim 64 without bias / mask fits two workgroups per CU (256 registers, 70 KiB of LDS each).
+__global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_kernel(FlashArgs a) {
     constexpr int KS = Cfg<D>::KS, VS = Cfg<D>::VS;
     const AttnParams &p = a.p;
     extern __shared__ __attribute__((aligned(16))) unsigned char flash_smem[];
