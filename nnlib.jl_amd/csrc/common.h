@@ -65,6 +65,14 @@ struct F16 {
     __device__ static inline floatx16_t mfma32(vec8 a, vec8 b, floatx16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
+    // D = A*B + C with D in other registers than C (the builtin always ties D to C, which costs a
+    // 16-register copy when C stays live).  The compiler does not know this is an MFMA: the caller
+    // keeps VALU reads of the result at least one later MFMA away.
+    __device__ static inline floatx16_t mfma32_keep_c(vec8 a, vec8 b, const floatx16_t &c) {
+        floatx16_t d;
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+        return d;
+    }
 };
 struct BF16 {
     typedef __bf16 type;
@@ -75,6 +83,11 @@ struct BF16 {
     __device__ static inline __bf16 from_f32(float x) { return (__bf16)x; }
     __device__ static inline floatx16_t mfma32(vec8 a, vec8 b, floatx16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    __device__ static inline floatx16_t mfma32_keep_c(vec8 a, vec8 b, const floatx16_t &c) {
+        floatx16_t d;
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(a), "v"(b), "v"(c));
+        return d;
     }
 };
 
@@ -88,6 +101,14 @@ __device__ static inline float mi_swap32(float x) {
 }
 
 __device__ static inline float mi_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// max(a, b, c) as one instruction with no quieting of the inputs (fmaxf on MFMA results costs an extra
+// v_max x, x per operand); a NaN operand is ignored like fmaxf does.
+__device__ static inline float mi_max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 
 // wavefront (64 lanes) reductions
 __device__ static inline float mi_wave_max(float v) {
