@@ -156,6 +156,26 @@ int32_t mi_make_causal_mask(uint8_t *m, int64_t len, mi_stream stream);
 int32_t mi_softmax_dim1(int32_t dtype, const void *x, void *y, int64_t rows, int64_t cols,
                         mi_stream stream);
 
+/* ---- softmax family over any run of adjacent dimensions --------------------------- */
+/* The array is viewed as (inner, len, outer): element (i, j, o) at i + inner*(j + len*o), and the
+ * reduction runs over j.  `dims = d` of an N-d column-major array gives inner = prod(size[1:d-1]),
+ * len = size[d], outer = prod(size[d+1:N]); `dims = :` gives (1, length, 1); a tuple of adjacent
+ * dims multiplies their extents into len.  y may alias x.  Arithmetic in fp32. */
+enum { MI_SOFTMAX = 0, MI_LOGSOFTMAX = 1 };
+/* op = MI_SOFTMAX: softmax(x; dims) (src/softmax.jl:56-79).  op = MI_LOGSOFTMAX: logsoftmax(x; dims)
+ * (src/softmax.jl:133-147), including its +Inf rule: a column whose maximum is +Inf gives 0 at the
+ * +Inf entries and -Inf elsewhere before the log-sum is subtracted. */
+int32_t mi_softmax(int32_t op, int32_t dtype, const void *x, void *y, int64_t inner, int64_t len,
+                   int64_t outer, mi_stream stream);
+/* logsumexp(x; dims) (src/softmax.jl:200-203): y (inner, outer) = max + log(sum(exp(x - max))). */
+int32_t mi_logsumexp(int32_t dtype, const void *x, void *y, int64_t inner, int64_t len,
+                     int64_t outer, mi_stream stream);
+/* Gradients given the forward RESULT y and the cotangent dy; dx may alias dy.
+ * op = MI_SOFTMAX:    dx = dy*y - y*sum(dy*y)   (_∇softmax!, src/softmax.jl:107-110)
+ * op = MI_LOGSOFTMAX: dx = dy - sum(dy)*exp(y)  (_∇logsoftmax!, src/softmax.jl:175-177) */
+int32_t mi_softmax_bwd(int32_t op, int32_t dtype, const void *dy, const void *y, void *dx,
+                       int64_t inner, int64_t len, int64_t outer, mi_stream stream);
+
 /* ---- batched GEMM ---------------------------------------------------------------- */
 /* C[:,:,b] = alpha * op(A[:,:,b]) * op(B[:,:,b]) + beta * C[:,:,b],  b in [0, batch).
  * The signature follows the backend hook NNlib._batched_gemm!(transA, transB, alpha,

@@ -7,7 +7,9 @@
 #   dot_product_attention(q, k, v, [bias]; fdrop, mask, nheads)   NNlib src/attention.jl:40-84
 #   dot_product_attention_scores(q, k, [bias]; fdrop, mask)        NNlib src/attention.jl:112-127
 #   make_causal_mask(x; dims)                                      NNlib src/attention.jl:149-153
-#   softmax(x; dims=1), softmax!(out, x; dims=1)                   NNlib src/softmax.jl:56-66
+#   softmax(x; dims), softmax!(out, x; dims)                       NNlib src/softmax.jl:56-66
+#   logsoftmax, logsoftmax!, logsumexp                             NNlib src/softmax.jl:133-147,200-203
+#   ∇softmax, ∇softmax!, ∇logsoftmax, ∇logsoftmax!                 NNlib src/softmax.jl:87-110,155-177
 #   batched_mul(A, B), batched_mul!(C, A, B, alpha, beta)          NNlib src/batched/batchedmul.jl:47-60,238-254
 #   batched_transpose, batched_adjoint                             NNlib src/batched/batchedadjtrans.jl:37-52
 #
@@ -16,7 +18,8 @@
 module MI355Attention
 
 export DeviceArray, CausalMask, dot_product_attention, dot_product_attention_scores, make_causal_mask,
-       softmax, softmax!, batched_mul, batched_mul!, batched_transpose, batched_adjoint
+       softmax, softmax!, logsoftmax, logsoftmax!, logsumexp, ∇softmax, ∇softmax!, ∇logsoftmax, ∇logsoftmax!,
+       batched_mul, batched_mul!, batched_transpose, batched_adjoint
 
 const libmi = get(ENV, "MI355ATTN_LIB", joinpath(@__DIR__, "..", "lib", "libmi355attn.so"))
 
@@ -217,17 +220,62 @@ function weights_times_values(α::DeviceArray{T, 4}, v::DeviceArray{T, 3}, H::In
     out
 end
 
-# ---- softmax ---------------------------------------------------------------------------------------
-softmax(x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = softmax!(similar(x, T, size(x)), x; dims)
-softmax!(x::DeviceArray; dims = 1) = softmax!(x, x; dims)
-function softmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloat}
-    dims == 1 || error("only dims = 1 is built; use NNlib's generic method for other dims")
+# ---- softmax family (NNlib src/softmax.jl) ---------------------------------------------------------
+const MI_SOFTMAX, MI_LOGSOFTMAX = Int32(0), Int32(1)
+
+# (inner, len, outer) of a reduction over `dims` (an integer, a tuple of adjacent dimensions, or :)
+function reduction_geometry(sz::Dims, dims)
+    dims isa Colon && return (1, prod(sz), 1)
+    ds = sort!(unique!(collect(Int, dims)))
+    (isempty(ds) || first(ds) < 1) && throw(ArgumentError("dims must be positive dimension numbers, got $dims"))
+    ds == collect(first(ds):last(ds)) ||
+        throw(ArgumentError("dims = $dims: only runs of adjacent dimensions are supported on device arrays"))
+    ext(d) = d <= length(sz) ? sz[d] : 1
+    n = max(length(sz), last(ds))
+    (prod(ext, 1:first(ds)-1; init = 1), prod(ext, ds; init = 1), prod(ext, last(ds)+1:n; init = 1))
+end
+
+function softmax_like!(op::Int32, out::DeviceArray{T}, x::DeviceArray{T}, dims) where {T <: MIFloat}
     size(out) == size(x) || throw(DimensionMismatch("output size $(size(out)) differs from input size $(size(x))"))
-    rows = size(x, 1); cols = rows == 0 ? 0 : length(x) ÷ rows
-    GC.@preserve out x check(ccall((:mi_softmax_dim1, libmi), Int32, (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Ptr{Cvoid}),
-                                   dtype_code(T), x.ptr, out.ptr, rows, cols, C_NULL))
+    inner, len, outer = reduction_geometry(size(x), dims)
+    GC.@preserve out x check(ccall((:mi_softmax, libmi), Int32,
+                                   (Int32, Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
+                                   op, dtype_code(T), x.ptr, out.ptr, inner, len, outer, C_NULL))
     out
 end
+
+softmax(x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = softmax!(similar(x, T, size(x)), x; dims)
+softmax!(x::DeviceArray; dims = 1) = softmax!(x, x; dims)
+softmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = softmax_like!(MI_SOFTMAX, out, x, dims)
+
+logsoftmax(x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = logsoftmax!(similar(x, T, size(x)), x; dims)
+logsoftmax!(x::DeviceArray; dims = 1) = logsoftmax!(x, x; dims)
+logsoftmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = softmax_like!(MI_LOGSOFTMAX, out, x, dims)
+
+# logsumexp(x; dims = :) returns a scalar for dims = : (one device-to-host copy), else an array that
+# keeps the reduced dimensions with extent 1, as NNlib's does (src/softmax.jl:200-203).
+function logsumexp(x::DeviceArray{T, N}; dims = :) where {T <: MIFloat, N}
+    inner, len, outer = reduction_geometry(size(x), dims)
+    kept = dims isa Colon ? () : ntuple(d -> d in dims ? 1 : size(x, d), N)
+    out = similar(x, T, kept)
+    GC.@preserve out x check(ccall((:mi_logsumexp, libmi), Int32,
+                                   (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
+                                   dtype_code(T), x.ptr, out.ptr, inner, len, outer, C_NULL))
+    dims isa Colon ? Array(out)[] : out
+end
+
+function softmax_grad!(op::Int32, dx::DeviceArray{T}, dy::DeviceArray{T}, y::DeviceArray{T}, dims) where {T <: MIFloat}
+    size(dx) == size(dy) == size(y) || throw(DimensionMismatch("dx, dy and y must have one size"))
+    inner, len, outer = reduction_geometry(size(y), dims)
+    GC.@preserve dx dy y check(ccall((:mi_softmax_bwd, libmi), Int32,
+                                     (Int32, Int32, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
+                                     op, dtype_code(T), dy.ptr, y.ptr, dx.ptr, inner, len, outer, C_NULL))
+    dx
+end
+∇softmax!(dx::DeviceArray, dy::DeviceArray, y::DeviceArray; dims = 1) = softmax_grad!(MI_SOFTMAX, dx, dy, y, dims)
+∇softmax(dy::DeviceArray{T}, y::DeviceArray{T}; dims = 1) where {T} = ∇softmax!(similar(y, T, size(y)), dy, y; dims)
+∇logsoftmax!(dx::DeviceArray, dy::DeviceArray, y::DeviceArray; dims = 1) = softmax_grad!(MI_LOGSOFTMAX, dx, dy, y, dims)
+∇logsoftmax(dy::DeviceArray{T}, y::DeviceArray{T}; dims = 1) where {T} = ∇logsoftmax!(similar(y, T, size(y)), dy, y; dims)
 
 # ---- batched_mul -----------------------------------------------------------------------------------
 function gemm!(tA, tB, m, n, k, α, A, lda, sA, B, ldb, sB, β, C, ldc, sC, batch, ::Type{T}) where {T}

@@ -14,6 +14,7 @@ MI_F32, MI_F16, MI_BF16 = 0, 1, 2
 KERNEL_GENERIC, KERNEL_FLASH16, KERNEL_FLASH32, KERNEL_DECODE = 0, 1, 2, 3
 KERNEL_NAMES = {0: "generic", 1: "flash16", 2: "flash32", 3: "decode"}
 MI_ATTN_FORCE_GENERIC = 1
+MI_SOFTMAX, MI_LOGSOFTMAX = 0, 1
 
 c_i32, c_i64, c_u64, c_f32 = ctypes.c_int32, ctypes.c_int64, ctypes.c_uint64, ctypes.c_float
 c_vp, c_sz = ctypes.c_void_p, ctypes.c_size_t
@@ -58,6 +59,9 @@ SIGNATURES = {
     "mi_attention_fwd": (c_i32, [ctypes.POINTER(mi_attn_desc), c_vp]),
     "mi_make_causal_mask": (c_i32, [c_vp, c_i64, c_vp]),
     "mi_softmax_dim1": (c_i32, [c_i32, c_vp, c_vp, c_i64, c_i64, c_vp]),
+    "mi_softmax": (c_i32, [c_i32, c_i32, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
+    "mi_logsumexp": (c_i32, [c_i32, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
+    "mi_softmax_bwd": (c_i32, [c_i32, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "mi_batched_gemm": (c_i32, [c_i32, ctypes.c_char, ctypes.c_char, c_i64, c_i64, c_i64, c_f32, c_vp, c_i64, c_i64,
                                 c_vp, c_i64, c_i64, c_f32, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "mi_randn_fill": (c_i32, [c_vp, c_i32, c_i64, c_u64, c_u64, c_f32, c_vp]),

@@ -14,7 +14,8 @@ from ._lib import ArgumentError, DimensionMismatch
 from .array import BatchedTranspose, CausalMask, DeviceArray
 
 __all__ = ["dot_product_attention", "dot_product_attention_scores", "make_causal_mask", "softmax", "softmax_",
-           "batched_mul", "batched_mul_", "last_attention_kernel"]
+           "logsoftmax", "logsoftmax_", "logsumexp", "grad_softmax", "grad_softmax_", "grad_logsoftmax",
+           "grad_logsoftmax_", "batched_mul", "batched_mul_", "last_attention_kernel"]
 
 _last_kernel = None
 _workspace = None
@@ -200,32 +201,117 @@ def make_causal_mask(x, *, dims=2):
     return CausalMask(x.size(dims))
 
 
-# ---- softmax -------------------------------------------------------------------------------------
+# ---- softmax family --------------------------------------------------------------------------------
 
-def softmax(x, *, dims=1):
-    """softmax(x; dims=1)  (src/softmax.jl:56)."""
-    if not isinstance(x, DeviceArray):
-        # src/softmax.jl:215-218
-        raise ArgumentError("`softmax(x)` called with a number, but it expects an array.")
-    out = DeviceArray.empty(x.dims, x.dtype)
-    return softmax_(out, x, dims=dims)
+def _reduction_geometry(dims_of_x, dims):
+    """(inner, len, outer, kept) for a reduction over ``dims`` of a column-major array: ``dims`` is a
+    1-based dimension, a tuple of adjacent dimensions, or ``None`` for Julia's ``:``.  ``kept`` is the
+    size of the reduced result (extent 1 along ``dims``, as Julia's ``sum(x; dims)`` keeps them)."""
+    size = tuple(dims_of_x)
+    if dims is None:
+        n = int(np.prod(size, dtype=np.int64)) if size else 1
+        return 1, n, 1, ()
+    ds = sorted({int(d) for d in (dims if isinstance(dims, (tuple, list)) else (dims,))})
+    if not ds or ds[0] < 1:
+        raise ArgumentError(f"dims must be positive dimension numbers, got {dims}")
+    ds = [d for d in ds if d <= len(size)]       # trailing singleton dimensions reduce to themselves
+    if not ds:
+        return int(np.prod(size, dtype=np.int64)) if size else 1, 1, 1, size
+    if ds != list(range(ds[0], ds[-1] + 1)):
+        raise ArgumentError(f"dims = {dims}: only runs of adjacent dimensions are supported on device arrays")
+    lo, hi = ds[0] - 1, ds[-1]
+    prod = lambda t: int(np.prod(t, dtype=np.int64)) if t else 1
+    kept = size[:lo] + (1,) * (hi - lo) + size[hi:]
+    return prod(size[:lo]), prod(size[lo:hi]), prod(size[hi:]), kept
 
 
-def softmax_(out, x=None, *, dims=1):
-    """softmax!(out, x; dims=1) and softmax!(x; dims=1)  (src/softmax.jl:64-66)."""
-    if x is None:
-        x = out
-    if dims != 1:
-        raise NotImplementedError("only dims=1 (the attention path) is built; other dims are out of scope")
+def _number_error(name):
+    # src/softmax.jl:213-218
+    return ArgumentError(f"`{name}(x)` called with a number, but it expects an array. Usually this is because a layer "
+                         f"like `Dense(3,4,softmax)` is broadcasting it like an activation function; `{name}` needs to "
+                         "be outside the layer.")
+
+
+def _softmax_like(name, op, out, x, dims):
+    if not isinstance(x, DeviceArray) or not isinstance(out, DeviceArray):
+        raise _number_error(name)
     x, out = _contig(x, "x"), _contig(out, "out")
     if out.dims != x.dims:
         raise DimensionMismatch(f"output size {out.dims} differs from input size {x.dims}")
     if x.dtype == "bool" or out.dtype != x.dtype:
-        raise ArgumentError("softmax needs floating-point input and output of one element type")
-    rows = x.dims[0] if x.dims else 1
-    cols = x.length // rows if rows else 0
-    _lib.check(_lib.load().mi_softmax_dim1(x.code, x.ptr, out.ptr, rows, cols, _stream()))
+        raise ArgumentError(f"{name} needs floating-point input and output of one element type")
+    inner, n, outer, _ = _reduction_geometry(x.dims, dims)
+    _lib.check(_lib.load().mi_softmax(op, x.code, x.ptr, out.ptr, inner, n, outer, _stream()))
     return out
+
+
+def softmax(x, *, dims=1):
+    """softmax(x; dims=1)  (src/softmax.jl:56).  ``dims=None`` is Julia's ``dims=:``."""
+    if not isinstance(x, DeviceArray):
+        raise _number_error("softmax")
+    return softmax_(DeviceArray.empty(x.dims, x.dtype), x, dims=dims)
+
+
+def softmax_(out, x=None, *, dims=1):
+    """softmax!(out, x; dims=1) and softmax!(x; dims=1)  (src/softmax.jl:64-66)."""
+    return _softmax_like("softmax!", _lib.MI_SOFTMAX, out, out if x is None else x, dims)
+
+
+def logsoftmax(x, *, dims=1):
+    """logsoftmax(x; dims=1)  (src/softmax.jl:133)."""
+    if not isinstance(x, DeviceArray):
+        raise _number_error("logsoftmax")
+    return logsoftmax_(DeviceArray.empty(x.dims, x.dtype), x, dims=dims)
+
+
+def logsoftmax_(out, x=None, *, dims=1):
+    """logsoftmax!(out, x; dims=1) and logsoftmax!(x; dims=1)  (src/softmax.jl:141-143)."""
+    return _softmax_like("logsoftmax!", _lib.MI_LOGSOFTMAX, out, out if x is None else x, dims)
+
+
+def logsumexp(x, *, dims=None):
+    """logsumexp(x; dims=:)  (src/softmax.jl:200-203).  With ``dims=None`` the result is a 0-d
+    DeviceArray holding the scalar; otherwise the reduced dimensions are kept with extent 1."""
+    if not isinstance(x, DeviceArray):
+        raise _number_error("logsumexp")
+    x = _contig(x, "x")
+    if x.dtype == "bool":
+        raise ArgumentError("logsumexp needs a floating-point array")
+    inner, n, outer, kept = _reduction_geometry(x.dims, dims)
+    out = DeviceArray.empty(kept, x.dtype)
+    _lib.check(_lib.load().mi_logsumexp(x.code, x.ptr, out.ptr, inner, n, outer, _stream()))
+    return out
+
+
+def _softmax_grad(name, op, dx, dy, y, dims):
+    dy, y, dx = _contig(dy, "dy"), _contig(y, "y"), _contig(dx, "dx")
+    if not (dy.dims == y.dims == dx.dims):
+        raise DimensionMismatch(f"{name}: dx {dx.dims}, dy {dy.dims} and y {y.dims} must have one size")
+    if y.dtype == "bool" or not (dy.dtype == y.dtype == dx.dtype):
+        raise ArgumentError(f"{name} needs one floating-point element type for dx, dy and y")
+    inner, n, outer, _ = _reduction_geometry(y.dims, dims)
+    _lib.check(_lib.load().mi_softmax_bwd(op, y.code, dy.ptr, y.ptr, dx.ptr, inner, n, outer, _stream()))
+    return dx
+
+
+def grad_softmax(dy, y, *, dims=1):
+    """∇softmax(dy, y; dims=1)  (src/softmax.jl:87-98): gradient of softmax given its RESULT y."""
+    return _softmax_grad("∇softmax", _lib.MI_SOFTMAX, DeviceArray.empty(y.dims, y.dtype), dy, y, dims)
+
+
+def grad_softmax_(dx, dy, y, *, dims=1):
+    """∇softmax!(dx, dy, y; dims=1)  (src/softmax.jl:105-110)."""
+    return _softmax_grad("∇softmax!", _lib.MI_SOFTMAX, dx, dy, y, dims)
+
+
+def grad_logsoftmax(dy, y, *, dims=1):
+    """∇logsoftmax(dy, y; dims=1)  (src/softmax.jl:155-166)."""
+    return _softmax_grad("∇logsoftmax", _lib.MI_LOGSOFTMAX, DeviceArray.empty(y.dims, y.dtype), dy, y, dims)
+
+
+def grad_logsoftmax_(dx, dy, y, *, dims=1):
+    """∇logsoftmax!(dx, dy, y; dims=1)  (src/softmax.jl:173-177)."""
+    return _softmax_grad("∇logsoftmax!", _lib.MI_LOGSOFTMAX, dx, dy, y, dims)
 
 
 # ---- batched_mul ---------------------------------------------------------------------------------

@@ -49,6 +49,12 @@ def lib():
         L.orc_nnlib_attention_f32.restype = None
         L.orc_attention_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp]
         L.orc_attention_f64.restype = None
+        for suf in ("f32", "f64"):
+            getattr(L, "orc_softmax_nd_" + suf).argtypes = [ci, vp, vp, i64, i64, i64]
+            getattr(L, "orc_logsumexp_" + suf).argtypes = [vp, vp, i64, i64, i64]
+            getattr(L, "orc_softmax_bwd_" + suf).argtypes = [ci, vp, vp, vp, i64, i64, i64]
+            for n in ("orc_softmax_nd_", "orc_logsumexp_", "orc_softmax_bwd_"):
+                getattr(L, n + suf).restype = None
         _LIB = L
     return _LIB
 
@@ -94,6 +100,61 @@ def softmax_dim1(x, dtype=np.float32):
     fn = lib().orc_softmax_dim1_f32 if dtype == np.float32 else lib().orc_softmax_dim1_f64
     fn(_ptr(x), _ptr(y), rows, cols)
     return y
+
+
+def reduction_geometry(shape, dims):
+    """(inner, len, outer, kept shape) of a reduction over ``dims`` (1-based dimension, tuple of adjacent
+    dimensions, or None for Julia's ``:``) of a column-major array."""
+    shape = tuple(shape)
+    if dims is None:
+        return 1, int(np.prod(shape, dtype=np.int64)), 1, ()
+    ds = sorted(set(dims if isinstance(dims, (tuple, list)) else (dims,)))
+    assert ds == list(range(ds[0], ds[-1] + 1))
+    nd = len(shape)
+    padded = shape + (1,) * max(0, ds[-1] - nd)       # dimensions past ndims have extent 1 in Julia
+    lo, hi = ds[0] - 1, ds[-1]
+    prod = lambda t: int(np.prod(t, dtype=np.int64)) if t else 1
+    kept = (padded[:lo] + (1,) * (hi - lo) + padded[hi:])[:nd]
+    return prod(padded[:lo]), prod(padded[lo:hi]), prod(padded[hi:]), kept
+
+
+def _suffix(dtype):
+    return "f32" if dtype == np.float32 else "f64"
+
+
+def softmax(x, dims=1, dtype=np.float64, log=False):
+    """softmax / logsoftmax over ``dims`` (src/softmax.jl:69-79, 137-147)."""
+    x = _f(x, dtype)
+    inner, n, outer, _ = reduction_geometry(x.shape, dims)
+    y = np.empty_like(x, order="F")
+    getattr(lib(), "orc_softmax_nd_" + _suffix(dtype))(int(log), _ptr(x), _ptr(y), inner, n, outer)
+    return y
+
+
+def logsoftmax(x, dims=1, dtype=np.float64):
+    return softmax(x, dims, dtype, log=True)
+
+
+def logsumexp(x, dims=None, dtype=np.float64):
+    """logsumexp(x; dims) (src/softmax.jl:200-203); reduced dimensions are kept with extent 1."""
+    x = _f(x, dtype)
+    inner, n, outer, kept = reduction_geometry(x.shape, dims)
+    y = np.empty(kept, dtype=dtype, order="F")
+    getattr(lib(), "orc_logsumexp_" + _suffix(dtype))(_ptr(x), _ptr(y), inner, n, outer)
+    return y
+
+
+def grad_softmax(dy, y, dims=1, dtype=np.float64, log=False):
+    """∇softmax / ∇logsoftmax given the forward result y (src/softmax.jl:107-110, 175-177)."""
+    dy, y = _f(dy, dtype), _f(y, dtype)
+    inner, n, outer, _ = reduction_geometry(y.shape, dims)
+    dx = np.empty_like(y, order="F")
+    getattr(lib(), "orc_softmax_bwd_" + _suffix(dtype))(int(log), _ptr(dy), _ptr(y), _ptr(dx), inner, n, outer)
+    return dx
+
+
+def grad_logsoftmax(dy, y, dims=1, dtype=np.float64):
+    return grad_softmax(dy, y, dims, dtype, log=True)
 
 
 def batched_gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, C=None, dtype=np.float32, nthreads=1):

@@ -19,6 +19,10 @@ def softmax_gold():
     return json.load(open(os.path.join(GOLD, "softmax_reference_values.json")))
 
 
+def softmax_family_gold():
+    return json.load(open(os.path.join(GOLD, "softmax_family_reference_values.json")))
+
+
 def attention_gold():
     g = json.load(open(os.path.join(GOLD, "attention_specific_results.json")))
     q = (np.arange(1, 13, dtype=np.float64) / 12).reshape(4, 3, 1, order="F")

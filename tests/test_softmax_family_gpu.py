@@ -1,0 +1,105 @@
+"""GPU parity of softmax over any dims, logsoftmax, logsumexp and the two gradients, through the C ABI,
+against the reference's own values (test/softmax.jl) and the CPU oracle."""
+import numpy as np
+import pytest
+
+import reference_cases as R
+from conftest import round_to
+
+pytestmark = pytest.mark.gpu
+G = R.softmax_family_gold()
+TOL = {"f32": 2e-6, "f16": 2e-3, "bf16": 2e-2}
+
+
+def _dev(nn, x, dtype="f32"):
+    return nn.DeviceArray.from_numpy(np.asarray(x, dtype=np.float32), dtype)
+
+
+def test_reference_values(nn):
+    d = G["doctest_matrix_dims2"]
+    assert np.allclose(nn.softmax(_dev(nn, R.rows(d["x_rows"])), dims=2).to_numpy(), R.rows(d["y_rows"]), atol=1e-6)
+    t = G["inf_table_other_dims"]
+    x = _dev(nn, R.rows(t["x_rows"]))
+    assert np.allclose(nn.softmax(x, dims=2).to_numpy(), R.rows(t["dims2"]), atol=1e-6)
+    assert np.allclose(nn.softmax(x, dims=None).to_numpy(), R.rows(t["dims_all"]))
+    assert np.allclose(nn.softmax(x, dims=(1, 2)).to_numpy(), R.rows(t["dims_1_2"]))
+    d = G["logsoftmax_vector"]
+    assert np.allclose(nn.logsoftmax(_dev(nn, d["x"])).to_numpy(), d["y"])
+    d = G["logsoftmax_matrix"]
+    x = _dev(nn, R.rows(d["x_rows"]))
+    assert np.allclose(nn.logsoftmax(x).to_numpy(), R.rows(d["y_rows"]))
+    ones = _dev(nn, np.ones((2, 3)))
+    assert np.allclose(nn.grad_logsoftmax(ones, nn.logsoftmax(x)).to_numpy(), R.rows(G["grad_logsoftmax_ones"]["dx_rows"]))
+    assert np.allclose(nn.grad_softmax(ones, nn.softmax(x)).to_numpy(), 0)
+    t = G["pytorch_logsoftmax_table"]
+    x = _dev(nn, R.rows(t["x_rows"]))
+    ones = _dev(nn, np.ones((3, 6)))
+    assert np.allclose(nn.grad_logsoftmax(ones, nn.logsoftmax(x)).to_numpy(), R.rows(t["dx_rows"]), rtol=1e-4, atol=1e-6)
+    assert np.allclose(nn.grad_softmax(ones, nn.softmax(x)).to_numpy(), 0, atol=1e-6)
+    for rows in ([[1, 2], [3, "Inf"]], [[1, "-Inf"], [3, "Inf"]], [[1, "Inf"], [3, "Inf"]]):   # test/softmax.jl:72-74
+        x = _dev(nn, R.rows(rows))
+        assert np.allclose(np.exp(nn.logsoftmax(x).to_numpy()), nn.softmax(x).to_numpy())
+    x = _dev(nn, R.rows([[1, 2], [3, "NaN"]]))
+    y = nn.logsoftmax(x).to_numpy()
+    assert np.isnan(y[:, 1]).all() and np.isfinite(y[:, 0]).all()
+
+
+SHAPES = [((2, 2, 2, 2, 2), d) for d in (1, 2, 3, 4, 5)] + [
+    ((5, 7), 2), ((3, 4), None), ((33, 65, 3), 2), ((64, 100, 5), 2), ((130, 17, 2), (2, 3)), ((7, 3000, 2), 2),
+    ((1, 5000, 3), 2), ((300, 70, 2), 2), ((5000,), 1), ((70000,), None), ((4, 9, 6), (1, 2)), ((128, 40), 1),
+    ((9, 5), 3)]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape,dims", SHAPES)
+def test_forward_against_oracle(nn, oracle, dtype, shape, dims):
+    """Every dims of test/softmax.jl:8-14's 2^5 array, plus shapes on both sides of each kernel
+    boundary (inner below / above 64, columns that fit registers or are re-read)."""
+    rng = np.random.default_rng(abs(hash((shape, str(dims)))) % 2**31)
+    x = round_to(rng.standard_normal(shape) * 2, dtype)
+    dx = _dev(nn, x, dtype)
+    tol = TOL[dtype]
+    sm = nn.softmax(dx, dims=dims).to_numpy()
+    assert np.abs(sm - oracle.softmax(x, dims)).max() <= tol
+    ls_ref = oracle.logsoftmax(x, dims)
+    ls = nn.logsoftmax(dx, dims=dims).to_numpy()
+    assert np.abs(ls - ls_ref).max() <= tol * max(1.0, np.abs(ls_ref).max())
+    lse_ref = oracle.logsumexp(x, dims)
+    lse = nn.logsumexp(dx, dims=dims)
+    assert lse.dims == lse_ref.shape
+    assert np.abs(lse.to_numpy() - lse_ref).max() <= tol * max(1.0, np.abs(lse_ref).max())
+    # in place (softmax!(x), logsoftmax!(x)): test/softmax.jl:8-14
+    d2 = _dev(nn, x, dtype)
+    nn.logsoftmax_(d2, dims=dims)
+    assert np.array_equal(d2.to_numpy(), ls)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("shape,dims", SHAPES)
+def test_gradients_against_oracle(nn, oracle, dtype, shape, dims):
+    rng = np.random.default_rng(abs(hash((shape, str(dims), 1))) % 2**31)
+    x = rng.standard_normal(shape) * 2
+    dy = round_to(rng.standard_normal(shape), dtype)
+    tol = TOL[dtype] * 4
+    for log in (False, True):
+        y = round_to(oracle.softmax(x, dims, log=log), dtype)
+        ref = oracle.grad_softmax(dy, y, dims, log=log)
+        fn = nn.grad_logsoftmax if log else nn.grad_softmax
+        got = fn(_dev(nn, dy, dtype), _dev(nn, y, dtype), dims=dims).to_numpy()
+        assert np.abs(got - ref).max() <= tol * max(1.0, np.abs(ref).max()), (log, np.abs(got - ref).max())
+    # ∇softmax!(dx, dy, y) writing over dy
+    y = round_to(oracle.softmax(x, dims), dtype)
+    ddy = _dev(nn, dy, dtype)
+    nn.grad_softmax_(ddy, ddy, _dev(nn, y, dtype), dims=dims)
+    assert np.abs(ddy.to_numpy() - oracle.grad_softmax(dy, y, dims)).max() <= tol
+
+
+def test_errors(nn):
+    with pytest.raises(nn.ArgumentError, match="expects an array"):
+        nn.logsoftmax(1.0)
+    with pytest.raises(nn.ArgumentError, match="expects an array"):
+        nn.logsumexp(1.0)
+    with pytest.raises(nn.ArgumentError, match="adjacent"):
+        nn.softmax(nn.DeviceArray.zeros((2, 3, 4)), dims=(1, 3))
+    with pytest.raises(nn.DimensionMismatch):
+        nn.grad_softmax_(nn.DeviceArray.zeros((3, 2)), nn.DeviceArray.zeros((2, 3)), nn.DeviceArray.zeros((2, 3)))
