@@ -145,6 +145,40 @@ int32_t mi_attention_plan(const mi_attn_desc *desc, int32_t *kernel, size_t *wor
 int32_t mi_attention_workspace_size(const mi_attn_desc *desc, size_t *bytes);
 int32_t mi_attention_fwd(const mi_attn_desc *desc, mi_stream stream);
 
+/*
+ * Gradient of one dot_product_attention call (fdrop = identity).  The reference has no hand-written
+ * rule: reverse-mode AD walks src/attention.jl:86-127 backwards through the rrule of batched_mul
+ * (src/batched/batchedmul.jl:96-110) and _∇softmax! (src/softmax.jl:107-110); this entry point is
+ * that chain fused, never materialising the (Lkv, Lq, H, B) tensors.  Its results are checked the
+ * way the reference checks its gradients (test/attention.jl:70-76: against finite differences).
+ *
+ *   fwd      : the forward call (dtype, sizes, q, k, v, bias, mask, causal, flags).  fwd.out may
+ *              hold the forward RESULT x; the MFMA kernels need it and the call falls back to the
+ *              generic kernels without it.  fwd.weights and fwd.workspace are ignored.
+ *   dout     : (Ev, Lq, B) cotangent of x, `dtype`.
+ *   dweights : NULL, or (Lkv, Lq, H, B) cotangent of the returned weights, `dtype`.
+ *   dq, dk, dv : gradients with the shapes of q, k, v, `dtype`; any may be NULL (not computed).
+ *   dbias    : NULL, or FLOAT32 array addressed with fwd.bias_strides; the gradient is ADDED into
+ *              it (dims with stride 0 receive the sum over that dim), so the caller zero-fills it.
+ *   workspace: at least mi_attention_bwd_plan()'s size, 16-byte aligned.
+ * A query whose keys are all dropped has NaN weights in the forward pass and NaN gradients here.
+ */
+typedef struct mi_attn_bwd_desc {
+    int32_t struct_size; /* = sizeof(mi_attn_bwd_desc) */
+    int32_t reserved;
+    mi_attn_desc fwd;
+    const void *dout;
+    const void *dweights;
+    void *dq;
+    void *dk;
+    void *dv;
+    float *dbias;
+    void *workspace;
+    size_t workspace_bytes;
+} mi_attn_bwd_desc;
+int32_t mi_attention_bwd_plan(const mi_attn_bwd_desc *desc, int32_t *kernel, size_t *workspace_bytes);
+int32_t mi_attention_bwd(const mi_attn_bwd_desc *desc, mi_stream stream);
+
 /* make_causal_mask (src/attention.jl:149-153): m (len, len) uint8, m[i,j] = (i <= j). */
 int32_t mi_make_causal_mask(uint8_t *m, int64_t len, mi_stream stream);
 

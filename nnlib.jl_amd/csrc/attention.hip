@@ -88,7 +88,7 @@ int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
 // Validation.  The first four conditions are the reference's ArgumentErrors
 // (src/attention.jl:55-78); with (E, L, B) sizes passed as scalars, "batch dimensions equal",
 // "qk feature dims equal" and "kv lengths equal" hold by construction, which leaves divisibility.
-static int32_t validate(const mi_attn_desc *d, AttnParams *out) {
+int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_backward) {
     if (!d) return mi_set_error(MI_EINVAL, "mi_attention: desc is NULL");
     if (d->struct_size != (int32_t)sizeof(mi_attn_desc))
         return mi_set_error(MI_EINVAL, "mi_attention: desc.struct_size is %d, library expects %zu", d->struct_size,
@@ -105,13 +105,14 @@ static int32_t validate(const mi_attn_desc *d, AttnParams *out) {
     if (d->causal && d->Lq != d->Lkv)
         return mi_set_error(MI_ESHAPE, "mi_attention: a causal (len, len) mask needs Lq == Lkv (got %lld, %lld)",
                             (long long)d->Lq, (long long)d->Lkv);
-    if (!d->out && !d->weights) return mi_set_error(MI_EINVAL, "mi_attention: both out and weights are NULL");
+    if (!for_backward && !d->out && !d->weights) return mi_set_error(MI_EINVAL, "mi_attention: both out and weights are NULL");
     if (d->weights && d->weights_dtype != d->dtype && d->weights_dtype != MI_F32)
         return mi_set_error(MI_EDTYPE, "mi_attention: weights_dtype must equal dtype or be MI_F32");
     const bool empty = d->Lq == 0 || d->B == 0 || (d->E == 0 && d->Ev == 0);
     if (!empty) {
         if (d->Lkv > 0 && d->E > 0 && (!d->q || !d->k)) return mi_set_error(MI_EINVAL, "mi_attention: q or k is NULL");
-        if (d->out && d->Lkv > 0 && d->Ev > 0 && !d->v) return mi_set_error(MI_EINVAL, "mi_attention: v is NULL but out is not");
+        if ((d->out || for_backward) && d->Lkv > 0 && d->Ev > 0 && !d->v)
+            return mi_set_error(MI_EINVAL, "mi_attention: v is NULL but out is not");
     }
     for (int i = 0; i < 4; i++) {
         if (d->bias && d->bias_strides[i] < 0) return mi_set_error(MI_ESHAPE, "mi_attention: negative bias stride");
@@ -150,7 +151,7 @@ static int32_t choose(const mi_attn_desc *d, const AttnParams &p, size_t *ws) {
 
 MI_API int32_t mi_attention_plan(const mi_attn_desc *d, int32_t *kernel, size_t *workspace_bytes) {
     AttnParams p;
-    int32_t rc = validate(d, &p);
+    int32_t rc = attention_validate(d, &p);
     if (rc != MI_OK) return rc;
     size_t ws = 0;
     int32_t k = choose(d, p, &ws);
@@ -166,7 +167,7 @@ MI_API int32_t mi_attention_workspace_size(const mi_attn_desc *d, size_t *bytes)
 
 MI_API int32_t mi_attention_fwd(const mi_attn_desc *d, mi_stream s) {
     AttnParams p;
-    int32_t rc = validate(d, &p);
+    int32_t rc = attention_validate(d, &p);
     if (rc != MI_OK) return rc;
     hipStream_t st = (hipStream_t)s;
     if (p.Lq == 0 || p.B == 0) return MI_OK;  // empty outputs

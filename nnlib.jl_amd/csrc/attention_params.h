@@ -13,6 +13,23 @@ struct AttnParams {
     int32_t dtype, weights_dtype, causal;
 };
 
+// One backward call: the forward call it differentiates plus cotangents and gradient buffers.
+struct AttnBwdParams {
+    AttnParams p;
+    const void *dout, *dweights;
+    void *dq, *dk, *dv;
+    float *dbias;      // addressed with p.bias_strides
+    float *stats;      // workspace: per (query, head, batch) softmax statistics
+    void *workspace;
+};
+
+int32_t launch_attention_bwd_generic(const AttnBwdParams &bp, hipStream_t st);
+int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp, hipStream_t st);
+bool attention_bwd_flash16_supports(const AttnBwdParams &bp);
+size_t attention_bwd_flash16_workspace(const AttnParams &p);
+size_t attention_bwd_generic_workspace(const AttnParams &p);
+int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_backward = false);
+
 int32_t launch_attention_generic(const AttnParams &p, hipStream_t st);
 int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st);
 int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st);

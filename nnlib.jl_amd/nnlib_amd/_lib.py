@@ -32,6 +32,14 @@ class mi_attn_desc(ctypes.Structure):
     ]
 
 
+class mi_attn_bwd_desc(ctypes.Structure):
+    _fields_ = [
+        ("struct_size", c_i32), ("reserved", c_i32), ("fwd", mi_attn_desc),
+        ("dout", c_vp), ("dweights", c_vp), ("dq", c_vp), ("dk", c_vp), ("dv", c_vp), ("dbias", c_vp),
+        ("workspace", c_vp), ("workspace_bytes", c_sz),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/mi355attn.h declares
 SIGNATURES = {
     "mi_version": (c_i32, []),
@@ -57,6 +65,8 @@ SIGNATURES = {
     "mi_attention_plan": (c_i32, [ctypes.POINTER(mi_attn_desc), ctypes.POINTER(c_i32), ctypes.POINTER(c_sz)]),
     "mi_attention_workspace_size": (c_i32, [ctypes.POINTER(mi_attn_desc), ctypes.POINTER(c_sz)]),
     "mi_attention_fwd": (c_i32, [ctypes.POINTER(mi_attn_desc), c_vp]),
+    "mi_attention_bwd_plan": (c_i32, [ctypes.POINTER(mi_attn_bwd_desc), ctypes.POINTER(c_i32), ctypes.POINTER(c_sz)]),
+    "mi_attention_bwd": (c_i32, [ctypes.POINTER(mi_attn_bwd_desc), c_vp]),
     "mi_make_causal_mask": (c_i32, [c_vp, c_i64, c_vp]),
     "mi_softmax_dim1": (c_i32, [c_i32, c_vp, c_vp, c_i64, c_i64, c_vp]),
     "mi_softmax": (c_i32, [c_i32, c_i32, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),

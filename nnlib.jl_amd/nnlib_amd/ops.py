@@ -15,7 +15,8 @@ from .array import BatchedTranspose, CausalMask, DeviceArray
 
 __all__ = ["dot_product_attention", "dot_product_attention_scores", "make_causal_mask", "softmax", "softmax_",
            "logsoftmax", "logsoftmax_", "logsumexp", "grad_softmax", "grad_softmax_", "grad_logsoftmax",
-           "grad_logsoftmax_", "batched_mul", "batched_mul_", "last_attention_kernel"]
+           "grad_logsoftmax_", "batched_mul", "batched_mul_", "batched_mul_pullback", "last_attention_kernel",
+           "dot_product_attention_grad", "last_attention_bwd_kernel"]
 
 _last_kernel = None
 _workspace = None
@@ -62,19 +63,15 @@ def _broadcast_strides(x, target, what):
     return out
 
 
-def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_weights, weights_dtype, flags):
-    """One mi_attention_fwd call on flattened (F, L, B) operands."""
-    global _last_kernel
-    lib = _lib.load()
-    d = _lib.mi_attn_desc()
+def _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags):
+    """Forward-call part of a descriptor: element type, sizes, inputs, bias / mask strides."""
     d.struct_size = ctypes.sizeof(_lib.mi_attn_desc)
-    d.dtype = q.code
+    d.dtype = d.weights_dtype = q.code
     d.flags = flags
     d.E, d.Ev, d.Lq, d.Lkv, d.H, d.B = E, Ev, Lq, Lkv, H, B
     d.q, d.k = q.ptr, k.ptr
     d.v = v.ptr if v is not None else None
     target = (Lkv, Lq, H, B)
-    keep = [q, k, v]
     if bias is not None:
         if bias.dtype != q.dtype:
             raise ArgumentError(f"bias must have the element type of q ({q.dtype}), got {bias.dtype}")
@@ -93,6 +90,14 @@ def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_we
         st = _broadcast_strides(mask, target, "mask")
         d.mask = mask.ptr
         d.mask_strides = (ctypes.c_int64 * 4)(*st)
+
+
+def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_weights, weights_dtype, flags):
+    """One mi_attention_fwd call on flattened (F, L, B) operands."""
+    global _last_kernel
+    lib = _lib.load()
+    d = _lib.mi_attn_desc()
+    _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags)
     out = DeviceArray.empty((Ev, Lq, B), q.dtype) if want_out else None
     wdt = weights_dtype or q.dtype
     alpha = DeviceArray.empty((Lkv, Lq, H, B), wdt) if want_weights else None
@@ -106,7 +111,6 @@ def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_we
         d.workspace, d.workspace_bytes = wbuf.data_ptr(), wsize
     _lib.check(lib.mi_attention_fwd(ctypes.byref(d), _stream()))
     _last_kernel = kernel.value
-    del keep
     return out, alpha
 
 
@@ -118,15 +122,8 @@ def _contig(x, name):
     return x
 
 
-def dot_product_attention(q, k, v, bias=None, *, fdrop=identity, mask=None, nheads=1, return_weights=True,
-                          weights_dtype=None, _flags=0):
-    """dot_product_attention(query, key, value, [bias]; [fdrop, mask, nheads])  (src/attention.jl:40-84).
-
-    q (qk_dim, q_len, batch...), k (qk_dim, kv_len, batch...), v (v_dim, kv_len, batch...).
-    Returns ``(x, alpha)``: x (v_dim, q_len, batch...), alpha (kv_len, q_len, nheads, batch...).
-
-    Beyond the reference: ``return_weights=False`` skips materialising alpha (``None`` is returned
-    in its place) and ``weights_dtype="f32"`` asks for Float32 weights from 16-bit inputs."""
+def _check_qkv(q, k, v, nheads):
+    """The argument checks of src/attention.jl:40-78; returns (B, E, Ev, Lq, Lkv, batch dims)."""
     q, k, v = _contig(q, "q"), _contig(k, "k"), _contig(v, "v")
     if not (q.ndim == k.ndim == v.ndim) or q.ndim < 2:
         raise ArgumentError("query, key and value must have the same number of dimensions (at least 2)")
@@ -146,6 +143,19 @@ def dot_product_attention(q, k, v, bias=None, *, fdrop=identity, mask=None, nhea
     if Lkv != v.dims[1]:                                         # src/attention.jl:74
         raise ArgumentError("Second dimension in key and value has to be the same. Instead:\n"
                             f"- size(k): {k.dims}\n- size(v): {v.dims}")
+    return B, E, Ev, Lq, Lkv, tuple(bq)
+
+
+def dot_product_attention(q, k, v, bias=None, *, fdrop=identity, mask=None, nheads=1, return_weights=True,
+                          weights_dtype=None, _flags=0):
+    """dot_product_attention(query, key, value, [bias]; [fdrop, mask, nheads])  (src/attention.jl:40-84).
+
+    q (qk_dim, q_len, batch...), k (qk_dim, kv_len, batch...), v (v_dim, kv_len, batch...).
+    Returns ``(x, alpha)``: x (v_dim, q_len, batch...), alpha (kv_len, q_len, nheads, batch...).
+
+    Beyond the reference: ``return_weights=False`` skips materialising alpha (``None`` is returned
+    in its place) and ``weights_dtype="f32"`` asks for Float32 weights from 16-bit inputs."""
+    B, E, Ev, Lq, Lkv, bq = _check_qkv(q, k, v, nheads)
     if fdrop is identity:
         x, alpha = _attention_call(q, k, v, bias, mask, nheads, B, E, Ev, Lq, Lkv, True, return_weights,
                                    weights_dtype, _flags)
@@ -160,6 +170,57 @@ def dot_product_attention(q, k, v, bias=None, *, fdrop=identity, mask=None, nhea
     if alpha is not None:
         alpha = alpha.reshape((Lkv, Lq, nheads) + tuple(bq))
     return x, alpha
+
+
+_last_bwd_kernel = None
+
+
+def last_attention_bwd_kernel():
+    """Name of the kernel family the most recent attention gradient call dispatched to."""
+    return _lib.KERNEL_NAMES.get(_last_bwd_kernel)
+
+
+def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, mask=None, nheads=1, _flags=0):
+    """Pullback of ``dot_product_attention(q, k, v, bias; mask, nheads)`` with ``fdrop = identity``:
+    given the cotangent ``dy`` of the output (and optionally ``dalpha`` of the returned weights) it
+    returns ``(dq, dk, dv, dbias)``; ``dbias`` is ``None`` without a bias and has the bias's size
+    otherwise (Float32).  The reference gets the same values from AD through src/attention.jl:86-127
+    (rrule of batched_mul, src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110).
+    ``y`` is the forward result; passing it lets the MFMA kernels run."""
+    global _last_bwd_kernel
+    B, E, Ev, Lq, Lkv, bq = _check_qkv(q, k, v, nheads)
+    dy = _contig(dy, "dy")
+    if dy.dims != (Ev, Lq) + bq or dy.dtype != q.dtype:
+        raise DimensionMismatch(f"dy must have the size and element type of the output {(Ev, Lq) + bq}, got {dy.dims}")
+    lib = _lib.load()
+    d = _lib.mi_attn_bwd_desc()
+    d.struct_size = ctypes.sizeof(_lib.mi_attn_bwd_desc)
+    _fill_desc(d.fwd, q, k, v, bias, mask, nheads, B, E, Ev, Lq, Lkv, _flags)
+    if y is not None:
+        y = _contig(y, "y")
+        if y.dims != dy.dims or y.dtype != q.dtype:
+            raise DimensionMismatch("y must have the size and element type of dy")
+        d.fwd.out = y.ptr
+    d.dout = dy.ptr
+    if dalpha is not None:
+        dalpha = _contig(dalpha, "dalpha")
+        if dalpha.dims != (Lkv, Lq, nheads) + bq or dalpha.dtype != q.dtype:
+            raise DimensionMismatch(f"dalpha must have size {(Lkv, Lq, nheads) + bq} and the element type of q")
+        d.dweights = dalpha.ptr
+    dq, dk, dv = DeviceArray.empty(q.dims, q.dtype), DeviceArray.empty(k.dims, q.dtype), DeviceArray.empty(v.dims, q.dtype)
+    d.dq, d.dk, d.dv = dq.ptr, dk.ptr, dv.ptr
+    dbias = None
+    if bias is not None:
+        dbias = DeviceArray.zeros(bias.dims, "f32")
+        d.dbias = dbias.ptr
+    kernel, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
+    _lib.check(lib.mi_attention_bwd_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))
+    wbuf, wsize = _get_workspace(ws.value)
+    if wbuf is not None:
+        d.workspace, d.workspace_bytes = wbuf.data_ptr(), wsize
+    _lib.check(lib.mi_attention_bwd(ctypes.byref(d), _stream()))
+    _last_bwd_kernel = kernel.value
+    return dq, dk, dv, dbias
 
 
 def _weights_times_values(alpha, v, H, B, Ev, Lq, Lkv):
@@ -387,3 +448,39 @@ def batched_mul(A, B):
         raise ArgumentError("batched_mul needs one element type for A and B")
     C = DeviceArray.empty((A.dims[0], B.dims[1], max(A.dims[2], B.dims[2])), A.dtype)
     return batched_mul_(C, A, B)
+
+
+def batched_mul_pullback(A, B, dC):
+    """The pullback of ``batched_mul(A, B)`` (rrule at src/batched/batchedmul.jl:96-110):
+    ``dA = dC * B'`` and ``dB = A' * dC`` per slice; an operand whose batch extent is 1 was shared by
+    every slice, so its gradient is the sum over slices."""
+    from .array import batched_adjoint
+    if A.ndim != 3 or B.ndim != 3 or dC.ndim != 3:
+        raise DimensionMismatch("batched_mul_pullback expects 3-D arrays")
+    nb = dC.dims[2]
+
+    def summed(X, make):
+        if X.dims[2] != 1 or nb == 1:
+            return make(None)
+        # sum over slices: accumulate slice by slice into one (m, n, 1) result with beta = 1
+        out = DeviceArray.zeros(X.dims, X.dtype)
+        for b in range(nb):
+            make((out, b))
+        return out
+
+    def slice3(X, b):
+        return DeviceArray(X.storage, X.dims[:2] + (1,), X.dtype, X.strides, X.offset + (b * X.strides[2] if X.dims[2] > 1 else 0))
+
+    def dA_of(acc):
+        if acc is None:
+            return batched_mul(dC, batched_adjoint(B))
+        out, b = acc
+        return batched_mul_(out, slice3(dC, b), batched_adjoint(slice3(B, b)), 1.0, 1.0)
+
+    def dB_of(acc):
+        if acc is None:
+            return batched_mul(batched_adjoint(A), dC)
+        out, b = acc
+        return batched_mul_(out, batched_adjoint(slice3(A, b)), slice3(dC, b), 1.0, 1.0)
+
+    return summed(A, dA_of), summed(B, dB_of)

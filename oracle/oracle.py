@@ -49,6 +49,8 @@ def lib():
         L.orc_nnlib_attention_f32.restype = None
         L.orc_attention_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp]
         L.orc_attention_f64.restype = None
+        L.orc_attention_bwd_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp, vp]
+        L.orc_attention_bwd_f64.restype = None
         for suf in ("f32", "f64"):
             getattr(L, "orc_softmax_nd_" + suf).argtypes = [ci, vp, vp, i64, i64, i64]
             getattr(L, "orc_logsumexp_" + suf).argtypes = [vp, vp, i64, i64, i64]
@@ -225,6 +227,57 @@ def scores4_f64(q4, k4, bias=None, mask=None):
     q3 = q4.reshape(D * H, Lq, B, order="F")
     k3 = k4.reshape(D * H, k4.shape[2], B, order="F")
     return _attention(q3, k3, None, bias, mask, H, np.float64, False, 1)[1]
+
+
+def attention_bwd_f64(q, k, v, dout, bias=None, mask=None, nheads=1, dweights=None):
+    """Gradient of dot_product_attention with respect to q, k, v and bias, given the cotangent ``dout``
+    of the output (and optionally ``dweights`` of the returned weights): the reverse of the op chain of
+    src/attention.jl:86-127.  Returns (dq, dk, dv, dbias); dbias has the shape of ``bias`` (None without)."""
+    f8 = np.float64
+    bshape = tuple(np.shape(q)[2:])
+    q3, k3, v3, do3 = (_f(_flatten3(a), f8) for a in (q, k, v, dout))
+    E, Lq, B = q3.shape
+    Lkv, Ev, H = k3.shape[1], v3.shape[0], nheads
+    _, alpha = _attention(q, k, v, bias, mask, nheads, f8, True, 1)
+    alpha = _f(alpha.reshape(Lkv, Lq, H, B, order="F"), f8)
+    dq, dk, dv = (np.empty(a.shape, dtype=f8, order="F") for a in (q3, k3, v3))
+    dw = None if dweights is None else _f(np.asarray(dweights).reshape(Lkv, Lq, H, B, order="F"), f8)
+    db = bs = None
+    if bias is not None:
+        db = np.zeros(np.shape(bias), dtype=f8, order="F")
+        bs = broadcast_strides(db.shape)
+    lib().orc_attention_bwd_f64(_ptr(q3), _ptr(k3), _ptr(v3), _ptr(alpha), _ptr(do3), _ptr(dw), bs,
+                                E, Ev, Lq, Lkv, H, B, _ptr(dq), _ptr(dk), _ptr(dv), _ptr(db))
+    return (dq.reshape(np.shape(q), order="F"), dk.reshape(np.shape(k), order="F"),
+            dv.reshape(np.shape(v), order="F"), db)
+
+
+def numpy_attention_bwd(q, k, v, dout, bias=None, mask=None, nheads=1, dweights=None):
+    """Independent einsum statement of the same gradient (no C involved)."""
+    f8 = np.float64
+    q3, k3, v3, do3 = (_flatten3(np.asarray(a, dtype=f8)) for a in (q, k, v, dout))
+    E, Lq, B = q3.shape
+    Lkv, Ev, H = k3.shape[1], v3.shape[0], nheads
+    D, Dv = E // H, Ev // H
+    _, alpha = numpy_attention(q, k, v, bias, mask, nheads)
+    alpha = alpha.reshape(Lkv, Lq, H, B, order="F")
+    q4, k4 = q3.reshape(D, H, Lq, B, order="F"), k3.reshape(D, H, Lkv, B, order="F")
+    v4, do4 = v3.reshape(Dv, H, Lkv, B, order="F"), do3.reshape(Dv, H, Lq, B, order="F")
+    da = np.einsum("dhjb,dhib->jihb", v4, do4)
+    if dweights is not None:
+        da = da + np.asarray(dweights, dtype=f8).reshape(Lkv, Lq, H, B, order="F")
+    dv4 = np.einsum("jihb,dhib->dhjb", alpha, do4)
+    dl = alpha * (da - (alpha * da).sum(axis=0, keepdims=True))
+    c = 1.0 / np.sqrt(f8(D))
+    dq4 = c * np.einsum("jihb,dhjb->dhib", dl, k4)
+    dk4 = c * np.einsum("jihb,dhib->dhjb", dl, q4)
+    db = None
+    if bias is not None:
+        bshape = tuple(np.shape(bias)) + (1,) * (4 - np.ndim(bias))
+        axes = tuple(a for a in range(4) if bshape[a] == 1)
+        db = dl.sum(axis=axes, keepdims=True).reshape(np.shape(bias), order="F")
+    return (dq4.reshape(np.shape(q), order="F"), dk4.reshape(np.shape(k), order="F"),
+            dv4.reshape(np.shape(v), order="F"), db)
 
 
 # ---------------------------------------------------------------------------------------------
