@@ -1,9 +1,34 @@
-// MFMA backward for bf16/f16 inputs (placeholder selection logic until the kernels land).
+// MFMA attention backward for bf16/f16 inputs: eligibility, workspace size and dispatch to the
+// per-(dtype, head dim) instantiations of attention_backward_flash16.inc.
 #include "common.h"
 #include "attention_params.h"
 
-bool attention_bwd_flash16_supports(const AttnBwdParams &) { return false; }
-size_t attention_bwd_flash16_workspace(const AttnParams &) { return 0; }
-int32_t launch_attention_bwd_flash16(const AttnBwdParams &, hipStream_t) {
-    return mi_set_error(MI_EINVAL, "MFMA attention backward is not available for this call");
+int32_t launch_bwd_flash16_bf16_d64(const AttnBwdParams &, hipStream_t);
+int32_t launch_bwd_flash16_bf16_d128(const AttnBwdParams &, hipStream_t);
+int32_t launch_bwd_flash16_f16_d64(const AttnBwdParams &, hipStream_t);
+int32_t launch_bwd_flash16_f16_d128(const AttnBwdParams &, hipStream_t);
+
+static inline bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
+
+bool attention_bwd_flash16_supports(const AttnBwdParams &bp) {
+    const AttnParams &p = bp.p;
+    if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
+    if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
+    // the kernels need the forward result (for delta), take no weight cotangent and give no bias gradient
+    if (!p.out || bp.dweights || bp.dbias) return false;
+    if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.out) || !aligned16(bp.dout)) return false;
+    if ((bp.dq && !aligned16(bp.dq)) || (bp.dk && !aligned16(bp.dk)) || (bp.dv && !aligned16(bp.dv))) return false;
+    const int64_t tiles = (p.Lq + 127) / 128 > (p.Lkv + 127) / 128 ? (p.Lq + 127) / 128 : (p.Lkv + 127) / 128;
+    return tiles * p.H * p.B <= 2147483647LL;
+}
+
+// three float planes [B*H][Lq rounded up to 128]: row maximum (log2 units), 1 / row sum, delta
+size_t attention_bwd_flash16_workspace(const AttnParams &p) {
+    return sizeof(float) * 3 * (size_t)(p.B * p.H) * (size_t)((p.Lq + 127) / 128 * 128);
+}
+
+int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp, hipStream_t st) {
+    const AttnParams &p = bp.p;
+    if (p.dtype == MI_BF16) return p.D == 64 ? launch_bwd_flash16_bf16_d64(bp, st) : launch_bwd_flash16_bf16_d128(bp, st);
+    return p.D == 64 ? launch_bwd_flash16_f16_d64(bp, st) : launch_bwd_flash16_f16_d128(bp, st);
 }
