@@ -137,6 +137,15 @@ typedef struct mi_attn_desc {
     int64_t mask_strides[4];
     void *workspace;
     size_t workspace_bytes;
+    /* fdrop = dropout(., p) fused into the kernel (src/dropout.jl:38-53 applied at
+     * src/attention.jl:126): each weight is zeroed with probability dropout_p, else multiplied by
+     * 1/(1 - dropout_p), after the softmax and before the value product; returned weights are
+     * post-dropout, as the reference returns them.  The keep decision of weight (kv, q, h, b) is
+     * that of mi_dropout() at linear index kv + Lkv*(q + Lq*(h + H*b)) with the same seed, so the
+     * fused and the unfused route give the same result.  0 = no dropout. */
+    float dropout_p;
+    uint32_t reserved2;
+    uint64_t dropout_seed;
 } mi_attn_desc;
 
 /* Validates shapes the way src/attention.jl:55-78 does (MI_ESHAPE on failure) and
@@ -181,6 +190,13 @@ int32_t mi_attention_bwd(const mi_attn_bwd_desc *desc, mi_stream stream);
 
 /* make_causal_mask (src/attention.jl:149-153): m (len, len) uint8, m[i,j] = (i <= j). */
 int32_t mi_make_causal_mask(uint8_t *m, int64_t len, mi_stream stream);
+
+/* ---- dropout --------------------------------------------------------------------- */
+/* y[i] = keep_i ? x[i] / (1 - p) : 0 with keep_i ~ Bernoulli(1 - p) from the counter-based generator
+ * keyed by (seed, i): dropout(x, p; dims = :) of src/dropout.jl:38-53 with a reproducible stream in
+ * place of Julia's RNG.  y may alias x.  0 <= p <= 1 (p = 1 zeroes everything). */
+int32_t mi_dropout(int32_t dtype, const void *x, void *y, int64_t n, float p, uint64_t seed,
+                   mi_stream stream);
 
 /* ---- softmax over the first dimension -------------------------------------------- */
 /* y[:, c] = softmax(x[:, c]) for a (rows, cols) column-major matrix; y may alias x

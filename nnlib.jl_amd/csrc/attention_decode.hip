@@ -158,7 +158,7 @@ int pick_nsplit(const AttnParams &p) {
 
 bool attention_decode_supports(const AttnParams &p) {
     if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
-    if (p.Lq != 1 || p.weights || p.bias || p.mask || !p.out) return false;
+    if (p.Lq != 1 || p.weights || p.bias || p.mask || !p.out || p.drop_thresh) return false;
     if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
     if (p.Lkv < 512) return false;   // short contexts: the tiled kernel is fine
     if (p.B > 65535) return false;

@@ -69,6 +69,8 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(AttnParams p) {
         float a = 0.0f;
         if (j < p.Lkv) {
             a = generic_term(score(j), m) / l;
+            if (p.drop_thresh)   // fdrop = dropout: src/attention.jl:126, src/dropout.jl:38-53
+                a = mi_dropout_keep(p.drop_key, (uint64_t)(j + p.Lkv * (i + p.Lq * (h + p.H * b))), p.drop_thresh) ? a * p.drop_scale : 0.0f;
             if (w) w[j] = (TW)a;
         }
         if (v) {

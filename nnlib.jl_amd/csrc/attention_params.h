@@ -11,6 +11,11 @@ struct AttnParams {
     int64_t bias_strides[4], mask_strides[4];
     int64_t E, Ev, Lq, Lkv, H, B, D, Dv;
     int32_t dtype, weights_dtype, causal;
+    // fused dropout of the weights: element (kv, q, h, b) is kept when mi_dropout_keep(drop_key,
+    // kv + Lkv*(q + Lq*(h + H*b)), drop_thresh); kept weights are multiplied by drop_scale.  thresh 0 = off
+    uint64_t drop_key;
+    uint32_t drop_thresh;
+    float drop_scale;
 };
 
 // One backward call: the forward call it differentiates plus cotangents and gradient buffers.

@@ -110,6 +110,31 @@ __device__ static inline float mi_max3(float a, float b, float c) {
     return r;
 }
 
+// ---- counter-based random bits ------------------------------------------------------------------
+// bits(seed, stream, i) = mix64(mix64(seed ^ stream * C) + i * G); one 64-bit word per element index.
+__host__ __device__ static inline uint64_t mi_mix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+__host__ __device__ static inline uint64_t mi_stream_key(uint64_t seed, uint64_t stream_id) {
+    return mi_mix64(seed ^ (stream_id * 0xD1342543DE82EF95ull));
+}
+__host__ __device__ static inline uint64_t mi_counter_bits(uint64_t key, uint64_t i) {
+    return mi_mix64(key + i * 0x9E3779B97F4A7C15ull);
+}
+// Dropout keep decision for element i: a 24-bit uniform u = bits[63:40] / 2^24 is kept when u >= p,
+// i.e. when its integer value reaches thresh = ceil(p * 2^24).
+#define MI_DROPOUT_STREAM 0x64726F70ull   // stream id reserved for dropout masks
+static inline uint32_t mi_dropout_threshold(float p) {
+    const double t = ceil((double)p * 16777216.0);
+    return t <= 0.0 ? 0u : (t >= 16777216.0 ? 16777216u : (uint32_t)t);
+}
+__device__ static inline bool mi_dropout_keep(uint64_t key, uint64_t i, uint32_t thresh) {
+    return (uint32_t)(mi_counter_bits(key, i) >> 40) >= thresh;
+}
+
 // wavefront (64 lanes) reductions
 __device__ static inline float mi_wave_max(float v) {
 #pragma unroll

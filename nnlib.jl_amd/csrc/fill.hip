@@ -1,15 +1,8 @@
 // Reproducible input generators, dtype conversion and make_causal_mask.
 #include "common.h"
 
-__device__ static inline uint64_t mix64(uint64_t z) {
-    z += 0x9E3779B97F4A7C15ull;
-    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
-    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-    return z ^ (z >> 31);
-}
-
 __device__ static inline uint64_t counter_bits(uint64_t seed, uint64_t stream_id, uint64_t i) {
-    return mix64(mix64(seed ^ (stream_id * 0xD1342543DE82EF95ull)) + i * 0x9E3779B97F4A7C15ull);
+    return mi_counter_bits(mi_stream_key(seed, stream_id), i);
 }
 
 template <typename T>
@@ -34,6 +27,15 @@ __global__ void bernoulli_kernel(uint8_t *p, int64_t n, uint64_t seed, uint64_t 
         float u = (float)((r >> 40) & 0xFFFFFF) * (1.0f / 16777216.0f);
         p[i] = (uint8_t)(u < keep);
     }
+}
+
+// dropout(x, p; dims = :)  (src/dropout.jl:38-53)
+template <typename T>
+__global__ void dropout_kernel(const typename T::type *x, typename T::type *y, int64_t n, uint64_t key, uint32_t thresh,
+                               float scale) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) y[i] = T::from_f32(mi_dropout_keep(key, (uint64_t)i, thresh) ? T::to_f32(x[i]) * scale : 0.0f);
 }
 
 template <typename TD, typename TS>
@@ -81,6 +83,24 @@ MI_API int32_t mi_bernoulli_fill(uint8_t *mask, int64_t n, uint64_t seed, uint64
     if (!mask) return mi_set_error(MI_EINVAL, "mi_bernoulli_fill: null pointer");
     hipLaunchKernelGGL(bernoulli_kernel, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)s, mask, n, seed, stream_id,
                        keep_prob);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+MI_API int32_t mi_dropout(int32_t dtype, const void *x, void *y, int64_t n, float p, uint64_t seed, mi_stream s) {
+    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_dropout: unknown dtype %d", dtype);
+    if (n < 0) return mi_set_error(MI_EINVAL, "mi_dropout: negative length");
+    if (!(p >= 0.0f && p <= 1.0f)) return mi_set_error(MI_EINVAL, "dropout expects a probability 0 <= p <= 1");   // src/dropout.jl:43
+    if (n == 0) return MI_OK;
+    if (!x || !y) return mi_set_error(MI_EINVAL, "mi_dropout: null pointer");
+    const uint64_t key = mi_stream_key(seed, MI_DROPOUT_STREAM);
+    const uint32_t thresh = mi_dropout_threshold(p);
+    const float scale = p < 1.0f ? 1.0f / (1.0f - p) : 0.0f;
+    dim3 g(grid_for(n)), b(256);
+    hipStream_t st = (hipStream_t)s;
+    if (dtype == MI_F32) hipLaunchKernelGGL(dropout_kernel<F32>, g, b, 0, st, (const float *)x, (float *)y, n, key, thresh, scale);
+    else if (dtype == MI_F16) hipLaunchKernelGGL(dropout_kernel<F16>, g, b, 0, st, (const _Float16 *)x, (_Float16 *)y, n, key, thresh, scale);
+    else hipLaunchKernelGGL(dropout_kernel<BF16>, g, b, 0, st, (const __bf16 *)x, (__bf16 *)y, n, key, thresh, scale);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }

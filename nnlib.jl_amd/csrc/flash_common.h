@@ -337,6 +337,19 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             }
         if (PHASE != PHASE_FINAL) fl[qb] += lsum;
 
+        // fdrop = dropout (src/attention.jl:126): after the softmax, so the row sum above is untouched;
+        // before the value product and before the weights are written, which are post-dropout.
+        if (PHASE != PHASE_STATS && p.drop_thresh != 0) {
+            const uint64_t row0 = (uint64_t)(p.Lkv * (qi + p.Lq * (h + p.H * b)) + j0 + 4 * hh);
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const bool keep = mi_dropout_keep(p.drop_key, row0 + (uint64_t)(32 * kb + 8 * (v / 4) + (v % 4)), p.drop_thresh);
+                    s[qb][kb][v] = keep ? s[qb][kb][v] * p.drop_scale : 0.0f;
+                }
+        }
+
         if (PHASE == PHASE_FINAL && p.weights && qok) {
             TW *w = (TW *)p.weights + p.Lkv * (qi + p.Lq * (h + p.H * b));
 #pragma unroll

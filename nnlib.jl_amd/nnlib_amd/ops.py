@@ -16,7 +16,7 @@ from .array import BatchedTranspose, CausalMask, DeviceArray
 __all__ = ["dot_product_attention", "dot_product_attention_scores", "make_causal_mask", "softmax", "softmax_",
            "logsoftmax", "logsoftmax_", "logsumexp", "grad_softmax", "grad_softmax_", "grad_logsoftmax",
            "grad_logsoftmax_", "batched_mul", "batched_mul_", "batched_mul_pullback", "last_attention_kernel",
-           "dot_product_attention_grad", "last_attention_bwd_kernel"]
+           "dot_product_attention_grad", "last_attention_bwd_kernel", "Dropout", "dropout"]
 
 _last_kernel = None
 _workspace = None
@@ -24,6 +24,33 @@ _workspace = None
 
 def identity(x):
     return x
+
+
+class Dropout:
+    """``fdrop = Dropout(p, seed)``: the reference's ``x -> dropout(x, p)`` (src/dropout.jl:38-53) with a
+    reproducible counter-based stream.  ``dot_product_attention`` recognises it and applies the dropout
+    inside the attention kernel; called on an array it runs the standalone kernel, with the same keep
+    decisions for the same seed."""
+
+    def __init__(self, p, seed=0):
+        if not 0 <= p <= 1:
+            raise ArgumentError("dropout expects a probability 0 <= p <= 1")      # src/dropout.jl:43
+        self.p, self.seed = float(p), int(seed)
+
+    def __call__(self, x):
+        return dropout(x, self.p, seed=self.seed)
+
+
+def dropout(x, p, *, seed=0, dims=None):
+    """dropout(A, p; dims = :)  (src/dropout.jl:38-53): zero with probability p, else scale by 1/(1-p)."""
+    if dims is not None:
+        raise NotImplementedError("dropout along dims (one decision per slice) is not built")
+    x = _contig(x, "x")
+    if x.dtype == "bool":
+        raise ArgumentError("dropout needs a floating-point array")
+    out = DeviceArray.empty(x.dims, x.dtype)
+    _lib.check(_lib.load().mi_dropout(x.code, x.ptr, out.ptr, x.length, float(p), int(seed), _stream()))
+    return out
 
 
 def last_attention_kernel():
@@ -63,9 +90,11 @@ def _broadcast_strides(x, target, what):
     return out
 
 
-def _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags):
+def _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags, fdrop=None):
     """Forward-call part of a descriptor: element type, sizes, inputs, bias / mask strides."""
     d.struct_size = ctypes.sizeof(_lib.mi_attn_desc)
+    if fdrop is not None:
+        d.dropout_p, d.dropout_seed = fdrop.p, fdrop.seed
     d.dtype = d.weights_dtype = q.code
     d.flags = flags
     d.E, d.Ev, d.Lq, d.Lkv, d.H, d.B = E, Ev, Lq, Lkv, H, B
@@ -92,12 +121,13 @@ def _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags):
         d.mask_strides = (ctypes.c_int64 * 4)(*st)
 
 
-def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_weights, weights_dtype, flags):
+def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_weights, weights_dtype, flags,
+                    fdrop=None):
     """One mi_attention_fwd call on flattened (F, L, B) operands."""
     global _last_kernel
     lib = _lib.load()
     d = _lib.mi_attn_desc()
-    _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags)
+    _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags, fdrop)
     out = DeviceArray.empty((Ev, Lq, B), q.dtype) if want_out else None
     wdt = weights_dtype or q.dtype
     alpha = DeviceArray.empty((Lkv, Lq, H, B), wdt) if want_weights else None
@@ -156,9 +186,9 @@ def dot_product_attention(q, k, v, bias=None, *, fdrop=identity, mask=None, nhea
     Beyond the reference: ``return_weights=False`` skips materialising alpha (``None`` is returned
     in its place) and ``weights_dtype="f32"`` asks for Float32 weights from 16-bit inputs."""
     B, E, Ev, Lq, Lkv, bq = _check_qkv(q, k, v, nheads)
-    if fdrop is identity:
+    if fdrop is identity or isinstance(fdrop, Dropout):
         x, alpha = _attention_call(q, k, v, bias, mask, nheads, B, E, Ev, Lq, Lkv, True, return_weights,
-                                   weights_dtype, _flags)
+                                   weights_dtype, _flags, fdrop if isinstance(fdrop, Dropout) else None)
     else:
         # alpha handed back is post-fdrop (src/attention.jl:126); the value product then runs as a
         # batched GEMM on the caller-visible weights, as src/attention.jl:96-98 does.
@@ -252,8 +282,10 @@ def dot_product_attention_scores(q, k, bias=None, *, fdrop=identity, mask=None, 
     if k.dims[0] != D or k.dims[1] != H or k.dims[3] != B:
         raise DimensionMismatch(f"query {q.dims} and key {k.dims} disagree in feature, head or batch size")
     Lkv = k.dims[2]
-    _, alpha = _attention_call(q, k, None, bias, mask, H, B, D * H, D * H, Lq, Lkv, False, True, weights_dtype, _flags)
-    return fdrop(alpha)
+    fused = fdrop if isinstance(fdrop, Dropout) else None
+    _, alpha = _attention_call(q, k, None, bias, mask, H, B, D * H, D * H, Lq, Lkv, False, True, weights_dtype, _flags,
+                               fused)
+    return alpha if fused is not None else fdrop(alpha)
 
 
 def make_causal_mask(x, *, dims=2):

@@ -104,6 +104,31 @@ def softmax_dim1(x, dtype=np.float32):
     return y
 
 
+_M64 = np.uint64(0xFFFFFFFFFFFFFFFF)
+
+
+def _mix64(z):
+    """splitmix64 finaliser on uint64 arrays (wraps modulo 2^64)."""
+    with np.errstate(over="ignore"):
+        z = z + np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+def dropout_keep_mask(shape, p, seed):
+    """Keep decisions (column-major linear index order) of the library's dropout stream: the published
+    definition restated in numpy: bits(i) = mix64(mix64(seed ^ stream*C) + i*G), u = bits >> 40 (24 bits),
+    keep = u >= ceil(p * 2^24).  The product's kernels must reproduce exactly this mask."""
+    n = int(np.prod(shape, dtype=np.int64))
+    with np.errstate(over="ignore"):
+        key = _mix64(np.array([seed], dtype=np.uint64) ^ (np.uint64(0x64726F70) * np.uint64(0xD1342543DE82EF95)))
+        bits = _mix64(key + np.arange(n, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15))
+    thresh = min(max(int(np.ceil(np.float32(p).astype(np.float64) * 16777216.0)), 0), 16777216)
+    keep = (bits >> np.uint64(40)).astype(np.int64) >= thresh
+    return keep.reshape(shape, order="F")
+
+
 def reduction_geometry(shape, dims):
     """(inner, len, outer, kept shape) of a reduction over ``dims`` (1-based dimension, tuple of adjacent
     dimensions, or None for Julia's ``:``) of a column-major array."""

@@ -1,0 +1,88 @@
+"""Dropout of the attention weights (fdrop = dropout(., p), src/attention.jl:126 with src/dropout.jl:38-53):
+the standalone kernel and the copy fused into the attention kernels, against the CPU oracle combined
+with a numpy restatement of the library's published keep-decision stream."""
+import numpy as np
+import pytest
+
+from conftest import rel_err, round_to
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("p", [0.0, 0.3, 0.5, 1.0])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_standalone_dropout_matches_the_published_stream(nn, oracle, p, dtype):
+    rng = np.random.default_rng(0)
+    x = round_to(rng.standard_normal((37, 11, 3)) + 3.0, dtype)          # no zeros in x
+    y = nn.dropout(nn.DeviceArray.from_numpy(x, dtype), p, seed=42).to_numpy()
+    keep = oracle.dropout_keep_mask(x.shape, p, 42)
+    assert np.array_equal(y != 0, keep)
+    scale = 0.0 if p == 1.0 else 1.0 / (1.0 - np.float32(p))
+    assert np.allclose(y, np.where(keep, x * scale, 0), rtol=1e-2 if dtype == "bf16" else 1e-6)
+    # another seed gives another mask; the kept fraction is 1 - p (docstring example of src/dropout.jl:16-18)
+    big = nn.dropout(nn.DeviceArray.from_numpy(np.ones((10000, 5), dtype=np.float32)), p, seed=7).to_numpy()
+    assert abs(big.mean() - (0.0 if p == 1.0 else 1.0)) < 0.03
+
+
+def test_reference_statistical_test(nn):
+    """test/attention.jl:54-59 and test/ext_amdgpu/attention.jl:36-42: about half the weights survive p = 0.5."""
+    rng = np.random.default_rng(1)
+    q = nn.DeviceArray.from_numpy(rng.random((10, 10, 10)).astype(np.float32))
+    for fdrop in (nn.Dropout(0.5, seed=3), lambda a: nn.dropout(a, 0.5, seed=3)):
+        y, alpha = nn.dot_product_attention(q, q, q, nheads=2, fdrop=fdrop)
+        assert 0.6 > (alpha.to_numpy() > 0).mean() > 0.4
+
+
+CASES = [
+    # dtype, E, Lq, Lkv, B, H, causal, weights, expected kernel
+    ("f32", 30, 7, 9, 2, 3, False, True, "generic"),
+    ("f32", 128, 96, 160, 2, 2, False, True, "flash32"),
+    ("f32", 128, 100, 100, 1, 2, True, False, "flash32"),
+    ("bf16", 128, 70, 200, 2, 2, False, False, "flash16"),
+    ("bf16", 256, 130, 130, 2, 2, True, True, "flash16"),
+    ("f16", 128, 64, 4096, 1, 2, False, False, "flash16"),      # few query tiles, long keys: split-kv + merge
+    ("bf16", 256, 300, 300, 1, 2, True, False, "flash16"),      # head dim 128: would take the fast kernel without dropout
+]
+
+
+@pytest.mark.parametrize("dtype,E,Lq,Lkv,B,H,causal,weights,expect", CASES)
+def test_fused_dropout_against_oracle(nn, oracle, dtype, E, Lq, Lkv, B, H, causal, weights, expect):
+    rng = np.random.default_rng(E + Lq + Lkv)
+    p, seed = 0.25, 2024
+    q = round_to(rng.standard_normal((E, Lq, B)) * 0.5, dtype)
+    k = round_to(rng.standard_normal((E, Lkv, B)) * 0.5, dtype)
+    v = round_to(rng.standard_normal((E, Lkv, B)), dtype)
+    D = nn.DeviceArray.from_numpy
+    dq_, dk_, dv_ = D(q, dtype), D(k, dtype), D(v, dtype)
+    mask = nn.make_causal_mask(dq_) if causal else None
+    y, a = nn.dot_product_attention(dq_, dk_, dv_, mask=mask, nheads=H, fdrop=nn.Dropout(p, seed), return_weights=weights,
+                                    weights_dtype="f32")
+    assert nn.last_attention_kernel() == expect
+    _, a_ref = oracle.attention_f64(q, k, v, None, oracle.make_causal_mask(Lq) if causal else None, H)
+    keep = oracle.dropout_keep_mask(a_ref.shape, p, seed)
+    a_ref = np.where(keep, a_ref / (1.0 - np.float32(p)), 0.0)            # alpha = fdrop(softmax(...))
+    Dh = E // H
+    y_ref = np.einsum("jihb,dhjb->dhib", a_ref, v.reshape(Dh, H, Lkv, B, order="F")).reshape(E, Lq, B, order="F")
+    assert rel_err(y.to_numpy(), y_ref) <= (1e-4 if dtype == "f32" else 1e-2)
+    if weights:
+        an = a.to_numpy()
+        assert np.array_equal(an != 0, a_ref != 0)                        # returned weights are post-dropout
+        assert np.abs(an - a_ref).max() <= (1e-5 if dtype == "f32" else 1e-2)
+    # the unfused route (scores -> standalone dropout -> batched product) takes the same decisions
+    y2, a2 = nn.dot_product_attention(dq_, dk_, dv_, mask=mask, nheads=H, fdrop=lambda w: nn.dropout(w, p, seed=seed))
+    assert rel_err(y2.to_numpy(), y_ref) <= (1e-4 if dtype == "f32" else 2e-2)
+    assert np.array_equal(a2.to_numpy() != 0, a_ref != 0)
+
+
+def test_scores_with_fused_dropout_and_edge_probabilities(nn):
+    rng = np.random.default_rng(5)
+    q = nn.DeviceArray.from_numpy(rng.random((4, 2, 3, 1)).astype(np.float32))
+    a0 = nn.dot_product_attention_scores(q, q).to_numpy()
+    assert np.array_equal(nn.dot_product_attention_scores(q, q, fdrop=nn.Dropout(0.0)).to_numpy(), a0)
+    assert np.all(nn.dot_product_attention_scores(q, q, fdrop=nn.Dropout(1.0)).to_numpy() == 0)
+    a = nn.dot_product_attention_scores(q, q, fdrop=nn.Dropout(0.5, seed=1)).to_numpy()
+    assert np.all((a == 0) | np.isclose(a, 2 * a0))
+    with pytest.raises(nn.ArgumentError, match="probability"):
+        nn.Dropout(1.5)
+    with pytest.raises(nn.ArgumentError, match="probability"):
+        nn.dropout(q, -0.1)
