@@ -240,6 +240,13 @@ int32_t mi_batched_gemm(int32_t dtype, char transA, char transB, int64_t m, int6
                         int64_t ldb, int64_t strideB, float beta, void *C, int64_t ldc,
                         int64_t strideC, int64_t batch, mi_stream stream);
 
+/* ---- materialising lazy views ------------------------------------------------------ */
+/* dst (contiguous column-major d0 x d1 x d2) = src read with element strides (s0, s1, s2): the copy(X)
+ * the reference makes of a PermutedDimsArray / transposed view before a BLAS call cannot address it
+ * (_copy_if_faster, src/batched/batchedmul.jl:76-83).  elem_bytes is 1, 2 or 4. */
+int32_t mi_strided_copy(void *dst, const void *src, int32_t elem_bytes, int64_t d0, int64_t d1, int64_t d2,
+                        int64_t s0, int64_t s1, int64_t s2, mi_stream stream);
+
 /* ---- reproducible inputs --------------------------------------------------------- */
 /* ptr[i] = dtype(scale * z_i), z_i ~ N(0,1) from a counter-based generator keyed by
  * (seed, stream_id, i); the same call always produces the same bits.  No counterpart

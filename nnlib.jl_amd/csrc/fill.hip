@@ -1,5 +1,6 @@
 // Reproducible input generators, dtype conversion and make_causal_mask.
 #include "common.h"
+#include <type_traits>
 
 __device__ static inline uint64_t counter_bits(uint64_t seed, uint64_t stream_id, uint64_t i) {
     return mi_counter_bits(mi_stream_key(seed, stream_id), i);
@@ -43,6 +44,22 @@ __global__ void convert_kernel(typename TD::type *d, const typename TS::type *s,
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) d[i] = TD::from_f32(TS::to_f32(s[i]));
+}
+
+// dst (contiguous, column-major d0 x d1 x d2) = src addressed with element strides (s0, s1, s2):
+// materialises a lazy PermutedDimsArray / transpose view (what the reference's copy(X) does in
+// _copy_if_faster, src/batched/batchedmul.jl:76-83)
+template <int BYTES>
+__global__ void strided_copy_kernel(void *dst, const void *src, int64_t d0, int64_t d1, int64_t d2, int64_t s0, int64_t s1,
+                                    int64_t s2) {
+    typedef typename std::conditional<BYTES == 4, uint32_t, typename std::conditional<BYTES == 2, uint16_t, uint8_t>::type>::type word;
+    const int64_t n = d0 * d1 * d2;
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; idx < n; idx += stride) {
+        const int64_t i0 = idx % d0, i1 = (idx / d0) % d1, i2 = idx / (d0 * d1);
+        ((word *)dst)[idx] = ((const word *)src)[i0 * s0 + i1 * s1 + i2 * s2];
+    }
 }
 
 // m[i + j*len] = (i <= j): reference src/attention.jl:145,149-153
@@ -123,6 +140,22 @@ MI_API int32_t mi_convert(void *dst, int32_t dd, const void *src, int32_t ds, in
     if (dd == MI_F32) launch_convert_from<F32>(dst, src, ds, n, st);
     else if (dd == MI_F16) launch_convert_from<F16>(dst, src, ds, n, st);
     else launch_convert_from<BF16>(dst, src, ds, n, st);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+MI_API int32_t mi_strided_copy(void *dst, const void *src, int32_t elem_bytes, int64_t d0, int64_t d1, int64_t d2, int64_t s0,
+                               int64_t s1, int64_t s2, mi_stream s) {
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) return mi_set_error(MI_EINVAL, "mi_strided_copy: element size must be 1, 2 or 4 bytes");
+    if (d0 < 0 || d1 < 0 || d2 < 0 || s0 < 0 || s1 < 0 || s2 < 0) return mi_set_error(MI_EINVAL, "mi_strided_copy: negative size or stride");
+    const int64_t n = d0 * d1 * d2;
+    if (n == 0) return MI_OK;
+    if (!dst || !src) return mi_set_error(MI_EINVAL, "mi_strided_copy: null pointer");
+    dim3 g(grid_for(n)), b(256);
+    hipStream_t st = (hipStream_t)s;
+    if (elem_bytes == 4) hipLaunchKernelGGL(strided_copy_kernel<4>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
+    else if (elem_bytes == 2) hipLaunchKernelGGL(strided_copy_kernel<2>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
+    else hipLaunchKernelGGL(strided_copy_kernel<1>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }

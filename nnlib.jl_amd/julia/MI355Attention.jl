@@ -12,6 +12,9 @@
 #   ∇softmax, ∇softmax!, ∇logsoftmax, ∇logsoftmax!                 NNlib src/softmax.jl:87-110,155-177
 #   batched_mul(A, B), batched_mul!(C, A, B, alpha, beta)          NNlib src/batched/batchedmul.jl:47-60,238-254
 #   batched_transpose, batched_adjoint                             NNlib src/batched/batchedadjtrans.jl:37-52
+#   batched_vec, matrix x 3-array forms of batched_mul             NNlib src/batched/batchedmul.jl:140-218
+#   Dropout(p, seed) as fdrop, dropout(x, p)                       NNlib src/dropout.jl:38-53
+#   ∇dot_product_attention, batched_mul_pullback                   what AD derives from src/attention.jl:86-127
 #
 # All arithmetic happens in the library.  This file has not been executed in the build environment
 # (no Julia toolchain there); the Python mirror in nnlib_amd/ exercises the same entry points.
@@ -19,7 +22,8 @@ module MI355Attention
 
 export DeviceArray, CausalMask, dot_product_attention, dot_product_attention_scores, make_causal_mask,
        softmax, softmax!, logsoftmax, logsoftmax!, logsumexp, ∇softmax, ∇softmax!, ∇logsoftmax, ∇logsoftmax!,
-       batched_mul, batched_mul!, batched_transpose, batched_adjoint
+       batched_mul, batched_mul!, batched_vec, batched_transpose, batched_adjoint, batched_mul_pullback,
+       Dropout, dropout, ∇dot_product_attention
 
 const libmi = get(ENV, "MI355ATTN_LIB", joinpath(@__DIR__, "..", "lib", "libmi355attn.so"))
 
@@ -129,6 +133,36 @@ struct AttnDesc
     bias::Ptr{Cvoid}; bias_strides::NTuple{4, Int64}
     mask::Ptr{Cvoid}; mask_strides::NTuple{4, Int64}
     workspace::Ptr{Cvoid}; workspace_bytes::Csize_t
+    dropout_p::Float32; reserved2::UInt32; dropout_seed::UInt64
+end
+
+# Mirror of `mi_attn_bwd_desc`.
+struct AttnBwdDesc
+    struct_size::Int32; reserved::Int32
+    fwd::AttnDesc
+    dout::Ptr{Cvoid}; dweights::Ptr{Cvoid}; dq::Ptr{Cvoid}; dk::Ptr{Cvoid}; dv::Ptr{Cvoid}; dbias::Ptr{Cvoid}
+    workspace::Ptr{Cvoid}; workspace_bytes::Csize_t
+end
+
+# fdrop = Dropout(p, seed): NNlib's `x -> dropout(x, p)` (src/dropout.jl:38-53) with a reproducible
+# counter-based stream.  dot_product_attention applies it inside the attention kernel; called on an
+# array it runs the standalone kernel, with the same keep decisions for the same seed.
+struct Dropout
+    p::Float32
+    seed::UInt64
+    function Dropout(p::Real, seed::Integer = 0)
+        0 <= p <= 1 || throw(ArgumentError("dropout expects a probability 0 <= p <= 1"))
+        new(Float32(p), UInt64(seed))
+    end
+end
+(d::Dropout)(x::DeviceArray) = dropout(x, d.p; seed = d.seed)
+function dropout(x::DeviceArray{T}, p::Real; seed::Integer = 0) where {T <: MIFloat}
+    0 <= p <= 1 || throw(ArgumentError("dropout expects a probability 0 <= p <= 1"))
+    is_dense(x) || throw(ArgumentError("dropout needs a dense array"))
+    y = similar(x, T, size(x))
+    GC.@preserve x y check(ccall((:mi_dropout, libmi), Int32, (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Float32, UInt64, Ptr{Cvoid}),
+                                 dtype_code(T), x.ptr, y.ptr, length(x), Float32(p), UInt64(seed), C_NULL))
+    y
 end
 
 # element strides of x against the (kv, q, head, batch) score tensor; 0 where x has extent 1
@@ -140,12 +174,9 @@ function broadcast_strides(x::DeviceArray, target::NTuple{4, Int}, what)
     end
 end
 
-function attention_call(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v, bias, mask, H::Int; want_out::Bool,
-                        want_weights::Bool) where {T <: MIFloat}
-    E, Lq, B = size(q); Lkv = size(k, 2); Ev = v === nothing ? E : size(v, 1)
-    target = (Lkv, Lq, H, B)
-    out = want_out ? DeviceArray{T}(undef, Ev, Lq, B) : nothing
-    alpha = want_weights ? DeviceArray{T}(undef, Lkv, Lq, H, B) : nothing
+# (causal flag, mask pointer + strides, bias pointer + strides) of a call
+function mask_and_bias(::Type{T}, bias, mask, target::NTuple{4, Int}) where {T}
+    Lkv, Lq = target[1], target[2]
     causal, mptr, mstr = Int32(0), C_NULL, ntuple(_ -> Int64(0), 4)
     if mask isa CausalMask
         (mask.len == Lkv == Lq) || throw(DimensionMismatch("arrays could not be broadcast to a common size: mask has size $(size(mask)), attention scores have size $target"))
@@ -159,10 +190,20 @@ function attention_call(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v, bias, mas
         bias isa DeviceArray{T} || throw(ArgumentError("bias must be a DeviceArray with the element type of q"))
         bptr, bstr = bias.ptr, broadcast_strides(bias, target, "bias")
     end
+    causal, mptr, mstr, bptr, bstr
+end
+
+function attention_call(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v, bias, mask, H::Int; want_out::Bool,
+                        want_weights::Bool, fdrop::Union{Nothing, Dropout} = nothing) where {T <: MIFloat}
+    E, Lq, B = size(q); Lkv = size(k, 2); Ev = v === nothing ? E : size(v, 1)
+    causal, mptr, mstr, bptr, bstr = mask_and_bias(T, bias, mask, (Lkv, Lq, H, B))
+    out = want_out ? DeviceArray{T}(undef, Ev, Lq, B) : nothing
+    alpha = want_weights ? DeviceArray{T}(undef, Lkv, Lq, H, B) : nothing
+    p, seed = fdrop === nothing ? (0f0, UInt64(0)) : (fdrop.p, fdrop.seed)
     mk(ws, wsbytes) = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0),
                                E, Ev, Lq, Lkv, H, B, q.ptr, k.ptr, v === nothing ? C_NULL : v.ptr,
                                out === nothing ? C_NULL : out.ptr, alpha === nothing ? C_NULL : alpha.ptr,
-                               bptr, bstr, mptr, mstr, ws, wsbytes)
+                               bptr, bstr, mptr, mstr, ws, wsbytes, p, UInt32(0), seed)
     need = Ref{Csize_t}(0)
     check(ccall((:mi_attention_workspace_size, libmi), Int32, (Ref{AttnDesc}, Ptr{Csize_t}), mk(C_NULL, 0), need))
     ws = need[] > 0 ? DeviceArray{UInt8}(undef, Int(need[])) : nothing
@@ -191,8 +232,9 @@ function dot_product_attention(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::De
     size(q, 3) == size(k, 3) == size(v, 3) || throw(ArgumentError("Batch dimensions have to be the same. Instead:\n- size(q): $(size(q))\n- size(k): $(size(k))\n- size(v): $(size(v))"))
     size(q, 1) == size(k, 1) || throw(ArgumentError("First dimension in query and key has to be the same. Instead:\n- size(q): $(size(q))\n- size(k): $(size(k))"))
     size(k, 2) == size(v, 2) || throw(ArgumentError("Second dimension in key and value has to be the same. Instead:\n- size(k): $(size(k))\n- size(v): $(size(v))"))
-    if fdrop === identity
-        return attention_call(q, k, v, bias, mask, nheads; want_out = true, want_weights = return_weights)
+    if fdrop === identity || fdrop isa Dropout
+        return attention_call(q, k, v, bias, mask, nheads; want_out = true, want_weights = return_weights,
+                              fdrop = fdrop isa Dropout ? fdrop : nothing)
     end
     # any other fdrop acts on the weights the caller sees (src/attention.jl:126): scores -> fdrop -> PV
     _, α = attention_call(q, k, nothing, bias, mask, nheads; want_out = false, want_weights = true)
@@ -205,8 +247,35 @@ function dot_product_attention_scores(q::DeviceArray{T, 4}, k::DeviceArray{T, 4}
     D, H, Lq, B = size(q)
     (size(k, 1), size(k, 2), size(k, 4)) == (D, H, B) || throw(DimensionMismatch("query $(size(q)) and key $(size(k)) disagree in feature, head or batch size"))
     _, α = attention_call(reshape(q, (D * H, Lq, B)), reshape(k, (D * H, size(k, 3), B)), nothing, bias, mask, H;
-                          want_out = false, want_weights = true)
-    return fdrop(α)
+                          want_out = false, want_weights = true, fdrop = fdrop isa Dropout ? fdrop : nothing)
+    return fdrop isa Dropout ? α : fdrop(α)
+end
+
+# Pullback of dot_product_attention(q, k, v, bias; mask, nheads) with fdrop = identity: returns
+# (dq, dk, dv, dbias) for the cotangent dy of the output (and optionally dα of the returned weights).
+# NNlib gets these from AD through src/attention.jl:86-127 (rrule of batched_mul,
+# src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110).  `y` is the forward result;
+# passing it lets the MFMA kernels run.  A ChainRulesCore.rrule for DeviceArray arguments is three lines
+# on top of this function: call the forward, close over (q, k, v, bias, y), return this pullback.
+function ∇dot_product_attention(dy::DeviceArray{T, 3}, q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::DeviceArray{T, 3},
+                                bias = nothing; y = nothing, dα = nothing, mask = nothing, nheads = 1) where {T <: MIFloat}
+    E, Lq, B = size(q); Lkv = size(k, 2); Ev = size(v, 1)
+    size(dy) == (Ev, Lq, B) || throw(DimensionMismatch("dy must have the size of the output $((Ev, Lq, B)), got $(size(dy))"))
+    causal, mptr, mstr, bptr, bstr = mask_and_bias(T, bias, mask, (Lkv, Lq, nheads, B))
+    dq, dk, dv = similar(q, T, size(q)), similar(k, T, size(k)), similar(v, T, size(v))
+    dbias = bias === nothing ? nothing : DeviceArray{Float32}(undef, size(bias)...)
+    dbias === nothing || check(ccall((:mi_fill_zero, libmi), Int32, (Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), dbias.ptr, sizeof(Float32) * length(dbias), C_NULL))
+    fwd = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0), E, Ev, Lq, Lkv, nheads, B,
+                   q.ptr, k.ptr, v.ptr, y === nothing ? C_NULL : y.ptr, C_NULL, bptr, bstr, mptr, mstr, C_NULL, 0, 0f0, UInt32(0), UInt64(0))
+    mk(ws, wsbytes) = AttnBwdDesc(Int32(sizeof(AttnBwdDesc)), Int32(0), fwd, dy.ptr, dα === nothing ? C_NULL : dα.ptr, dq.ptr, dk.ptr,
+                                  dv.ptr, dbias === nothing ? C_NULL : dbias.ptr, ws, wsbytes)
+    need = Ref{Csize_t}(0)
+    check(ccall((:mi_attention_bwd_plan, libmi), Int32, (Ref{AttnBwdDesc}, Ptr{Int32}, Ptr{Csize_t}), mk(C_NULL, 0), C_NULL, need))
+    ws = need[] > 0 ? DeviceArray{UInt8}(undef, Int(need[])) : nothing
+    GC.@preserve dy q k v bias mask y dα dq dk dv dbias ws begin
+        check(ccall((:mi_attention_bwd, libmi), Int32, (Ref{AttnBwdDesc}, Ptr{Cvoid}), mk(ws === nothing ? C_NULL : ws.ptr, need[]), C_NULL))
+    end
+    dq, dk, dv, dbias
 end
 
 # x[d,h,i,b] = sum_j α[j,i,h,b] v[d,h,j,b]: one strided batched GEMM over heads per batch element
@@ -307,6 +376,11 @@ function batched_mul!(C::DeviceArray{T, 3}, A::DeviceArray{T, 3}, B::DeviceArray
     m, ka = size(A, 1), size(A, 2); kb, n = size(B, 1), size(B, 2)
     (ka == kb && m == size(C, 1) && n == size(C, 2)) ||
         throw(DimensionMismatch("A1 has size ($m,$ka), B1 has size ($kb,$n), C1 has size $(size(C)[1:2])"))
+    if strides(C)[1] != 1 && strides(C)[2] == 1 && size(C, 1) > 1
+        # C is a lazily permuted array: C' = B' * A' (src/batched/batchedmul.jl:268-270)
+        batched_mul!(batched_transpose(C), batched_transpose(B), batched_transpose(A), α, β)
+        return C
+    end
     (tA, lda), (tB, ldb) = blas_layout(A), blas_layout(B)
     strides(C)[1] == 1 || throw(ArgumentError("Unsupported array layout for batched mul.\n- Size: $(size(C))\n- Strides: $(strides(C))"))
     sA = size(A, 3) == 1 ? 0 : strides(A)[3]          # src/gemm.jl:117-118
@@ -316,9 +390,66 @@ function batched_mul!(C::DeviceArray{T, 3}, A::DeviceArray{T, 3}, B::DeviceArray
     C
 end
 
+# lazy PermutedDimsArray(A, perm) and matrix transpose: same memory, permuted size and strides
+permuted(a::DeviceArray{T, N}, perm::NTuple{N, Int}) where {T, N} =
+    DeviceArray{T, N}(a.ptr, ntuple(i -> a.dims[perm[i]], N), ntuple(i -> a.strides[perm[i]], N), a)
+Base.transpose(a::DeviceArray{T, 2}) where {T} = permuted(a, (2, 1))
+Base.adjoint(a::DeviceArray{T, 2}) where {T <: Real} = permuted(a, (2, 1))
+with_batch(a::DeviceArray{T, 2}) where {T} = DeviceArray{T, 3}(a.ptr, (a.dims..., 1), (a.strides..., length(a)), a)
+
+# dense copy of a lazy view of up to 3 dimensions (copy(X) in _copy_if_faster, src/batched/batchedmul.jl:76-83)
+function Base.copy(a::DeviceArray{T, N}) where {T, N}
+    N <= 3 || throw(ArgumentError("copy of a strided DeviceArray is built for up to 3 dimensions"))
+    out = DeviceArray{T}(undef, size(a)...)
+    d = (size(a)..., ntuple(_ -> 1, 3 - N)...); s = (strides(a)..., ntuple(_ -> 0, 3 - N)...)
+    GC.@preserve a out check(ccall((:mi_strided_copy, libmi), Int32,
+                                   (Ptr{Cvoid}, Ptr{Cvoid}, Int32, Int64, Int64, Int64, Int64, Int64, Int64, Ptr{Cvoid}),
+                                   out.ptr, a.ptr, sizeof(T), d[1], d[2], d[3], s[1], s[2], s[3], C_NULL))
+    out
+end
+
+# layouts the GEMM kernel cannot address are materialised first (the reference copies the stride(X,3) == 1
+# case and hands the rest to batched_mul_generic!; the results are the same)
+function copy_if_faster(X::DeviceArray{T, 3}) where {T}
+    s1, s2, s3 = strides(X)
+    ((s3 == 1 && s1 != 1 && size(X, 3) > 1) || (s1 != 1 && s2 != 1 && size(X, 1) > 1 && size(X, 2) > 1)) ? copy(X) : X
+end
+
 function batched_mul(A::DeviceArray{T, 3}, B::DeviceArray{T, 3}) where {T <: MIFloat}
     size(A, 3) == size(B, 3) || size(A, 3) == 1 || size(B, 3) == 1 || throw(DimensionMismatch("batch size mismatch: A != B"))
-    batched_mul!(DeviceArray{T}(undef, size(A, 1), size(B, 2), max(size(A, 3), size(B, 3))), A, B)
+    batched_mul!(DeviceArray{T}(undef, size(A, 1), size(B, 2), max(size(A, 3), size(B, 3))), copy_if_faster(A), copy_if_faster(B))
+end
+# a matrix (plain or lazily transposed) on either side is shared by every batch (src/batched/batchedmul.jl:140-164)
+batched_mul(A::DeviceArray{T, 3}, B::DeviceArray{T, 2}) where {T <: MIFloat} = batched_mul(A, with_batch(B))
+batched_mul(A::DeviceArray{T, 2}, B::DeviceArray{T, 3}) where {T <: MIFloat} = batched_mul(with_batch(A), B)
+
+# batched_vec (src/batched/batchedmul.jl:166-218)
+function batched_vec(A::DeviceArray{T}, B::DeviceArray{T}) where {T <: MIFloat}
+    ndims(A) == ndims(B) + 1 || throw(DimensionMismatch("batched_vec requires ndims(A) == ndims(B) + 1, got ndims(A)=$(ndims(A)) and ndims(B)=$(ndims(B))"))
+    size(A)[3:end] == size(B)[2:end] || throw(DimensionMismatch("batch dimensions must match: size(A)[3:end]=$(size(A)[3:end]) != size(B)[2:end]=$(size(B)[2:end])"))
+    Bd = is_dense(B) ? B : copy(B)
+    C = batched_mul(A, reshape(Bd, (size(B, 1), 1, size(B)[2:end]...)))
+    reshape(C, (size(C, 1), size(C)[3:end]...))
+end
+batched_vec(A::DeviceArray{T, 3}, b::DeviceArray{T, 1}) where {T <: MIFloat} =
+    reshape(batched_mul(A, reshape(b, (length(b), 1, 1))), (size(A, 1), size(A, 3)))
+
+# pullback of batched_mul (rrule at src/batched/batchedmul.jl:96-110); an operand with batch extent 1 was
+# shared by every slice, so its gradient accumulates over slices (beta = 1)
+function batched_mul_pullback(A::DeviceArray{T, 3}, B::DeviceArray{T, 3}, Δ::DeviceArray{T, 3}) where {T <: MIFloat}
+    nb = size(Δ, 3)
+    slice(X, b) = DeviceArray{T, 3}(X.ptr + sizeof(T) * (size(X, 3) > 1 ? b * strides(X)[3] : 0), (size(X, 1), size(X, 2), 1), strides(X), X)
+    function grad(X, f)
+        (size(X, 3) != 1 || nb == 1) && return f(Δ, A, B, nothing)
+        out = DeviceArray{T}(undef, size(X)...)
+        for b in 0:nb-1
+            f(slice(Δ, b), slice(A, b), slice(B, b), (out, b == 0 ? 0f0 : 1f0))
+        end
+        out
+    end
+    dA = grad(A, (Δ, A, B, acc) -> acc === nothing ? batched_mul(Δ, batched_adjoint(B)) : batched_mul!(acc[1], Δ, batched_adjoint(B), 1f0, acc[2]))
+    dB = grad(B, (Δ, A, B, acc) -> acc === nothing ? batched_mul(batched_adjoint(A), Δ) : batched_mul!(acc[1], batched_adjoint(A), Δ, 1f0, acc[2]))
+    dA, dB
 end
 
 function batched_mul(x::DeviceArray{T, N}, y::DeviceArray{T, N}) where {T <: MIFloat, N}

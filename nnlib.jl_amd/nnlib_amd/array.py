@@ -108,6 +108,29 @@ class DeviceArray:
         assert int(np.prod(dims, dtype=np.int64)) == self.length, "reshape must keep the element count"
         return DeviceArray(self.storage, dims, self.dtype, None, self.offset)
 
+    def permuted(self, *perm):
+        """Lazy ``PermutedDimsArray(A, perm)`` (1-based ``perm`` as in Julia): same memory, permuted
+        size and strides."""
+        if len(perm) == 1 and isinstance(perm[0], (tuple, list)):
+            perm = tuple(perm[0])
+        assert sorted(perm) == list(range(1, self.ndim + 1)), "perm must be a permutation of 1:ndims"
+        return DeviceArray(self.storage, [self.dims[p - 1] for p in perm], self.dtype,
+                           [self.strides[p - 1] for p in perm], self.offset)
+
+    def with_trailing(self, n):
+        """Same memory viewed with ``n`` extra trailing dimensions of extent 1 (``reshape(A, size(A)..., 1)``
+        for views whose strides must be kept)."""
+        return DeviceArray(self.storage, self.dims + (1,) * n, self.dtype, self.strides + (self.length,) * n, self.offset)
+
+    def copy(self):
+        """Dense column-major copy (``copy(X)`` / ``permutedims``): materialises a lazy view of up to 3 dims."""
+        assert self.ndim <= 3, "copy of a strided view is built for up to 3 dimensions"
+        d = self.dims + (1,) * (3 - self.ndim)
+        s = self.strides + (0,) * (3 - self.ndim)
+        out = DeviceArray.empty(self.dims, self.dtype)
+        _lib.check(_lib.load().mi_strided_copy(out.ptr, self.ptr, self.itemsize, d[0], d[1], d[2], s[0], s[1], s[2], None))
+        return out
+
     @property
     def itemsize(self):
         return self.storage.element_size()
@@ -123,7 +146,8 @@ class DeviceArray:
     # ---- host copies ---------------------------------------------------------------------
     def to_numpy(self):
         """Julia-shaped numpy array (Fortran order). bf16 comes back as float32, bool as bool."""
-        assert self.is_contiguous(), "materialise a lazy transpose before copying to the host"
+        if not self.is_contiguous():
+            return self.copy().to_numpy()
         flat = self.storage[self.offset:self.offset + self.length]
         if self.dtype == "bf16":
             flat = flat.float()
@@ -149,6 +173,15 @@ class BatchedTranspose(DeviceArray):
 def batched_transpose(A):
     """batched_transpose(A) (src/batched/batchedadjtrans.jl:37-38); transposing twice unwraps."""
     return A.parent if isinstance(A, BatchedTranspose) else BatchedTranspose(A)
+
+
+def transpose(M):
+    """Lazy transpose of a matrix (Julia's ``transpose(M)`` / ``M'`` for the real element types here)."""
+    assert M.ndim == 2, "transpose expects a matrix"
+    return M.permuted(2, 1)
+
+
+adjoint = transpose
 
 
 def batched_adjoint(A):

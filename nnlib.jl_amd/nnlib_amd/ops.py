@@ -11,12 +11,12 @@ import torch
 
 from . import _lib
 from ._lib import ArgumentError, DimensionMismatch
-from .array import BatchedTranspose, CausalMask, DeviceArray
+from .array import BatchedTranspose, CausalMask, DeviceArray, batched_transpose
 
 __all__ = ["dot_product_attention", "dot_product_attention_scores", "make_causal_mask", "softmax", "softmax_",
            "logsoftmax", "logsoftmax_", "logsumexp", "grad_softmax", "grad_softmax_", "grad_logsoftmax",
            "grad_logsoftmax_", "batched_mul", "batched_mul_", "batched_mul_pullback", "last_attention_kernel",
-           "dot_product_attention_grad", "last_attention_bwd_kernel", "Dropout", "dropout"]
+           "dot_product_attention_grad", "last_attention_bwd_kernel", "Dropout", "dropout", "batched_vec"]
 
 _last_kernel = None
 _workspace = None
@@ -450,6 +450,11 @@ def batched_mul_(C, A, B, alpha=1.0, beta=0.0):
     kb, n = B.dims[0], B.dims[1]
     if ka != kb or m != C.dims[0] or n != C.dims[1]:                      # src/gemm.jl:106-108
         raise DimensionMismatch(f"A1 has size ({m},{ka}), B1 has size ({kb},{n}), C1 has size {C.dims[:2]}")
+    if C.strides[0] != 1 and C.strides[1] == 1 and C.dims[0] > 1:
+        # C is a lazily transposed / permuted array: compute C' = B' * A' into its parent layout
+        # (_batched_try_gemm!, src/batched/batchedmul.jl:268-270: "transposing C = A * B into C' = B' * A'")
+        batched_mul_(batched_transpose(C), batched_transpose(B), batched_transpose(A), alpha, beta)
+        return C
     tA, lda, sA = _blas_layout(A, "A")
     tB, ldb, sB = _blas_layout(B, "B")
     if C.strides[0] != 1:
@@ -462,11 +467,26 @@ def batched_mul_(C, A, B, alpha=1.0, beta=0.0):
     return C
 
 
+def _copy_if_faster(X):
+    """_copy_if_faster (src/batched/batchedmul.jl:76-83) widened to every layout the GEMM kernel cannot
+    address (neither of the first two strides is 1): such views are materialised; the reference would
+    hand them to batched_mul_generic!, with the same result."""
+    s1, s2, s3 = X.strides
+    if (s3 == 1 and s1 != 1 and X.dims[2] > 1) or (s1 != 1 and s2 != 1 and X.dims[0] > 1 and X.dims[1] > 1):
+        return X.copy()
+    return X
+
+
 def batched_mul(A, B):
-    """batched_mul(A, B)  (src/batched/batchedmul.jl:47-60): C[:,:,k...] = A[:,:,k...] * B[:,:,k...];
-    a 3-D operand with batch extent 1 is shared by every batch."""
+    """batched_mul(A, B)  (src/batched/batchedmul.jl:47-60, 140-164): C[:,:,k...] = A[:,:,k...] * B[:,:,k...];
+    a 3-D operand with batch extent 1 is shared by every batch, and so is a plain (or lazily
+    transposed) matrix on either side.  Lazy views (batched_transpose, permuted) are accepted."""
     if not isinstance(A, DeviceArray) or not isinstance(B, DeviceArray):
         raise ArgumentError("batched_mul expects DeviceArrays")
+    if A.ndim == 3 and B.ndim == 2:            # _semi_batched_mul, src/batched/batchedmul.jl:143-150
+        return batched_mul(A, B.with_trailing(1))
+    if A.ndim == 2 and B.ndim == 3:            # src/batched/batchedmul.jl:152-164
+        return batched_mul(A.with_trailing(1), B)
     if A.ndim != B.ndim or A.ndim < 3:
         raise DimensionMismatch("batched_mul needs two arrays of equal dimensionality (at least 3)")
     if A.ndim > 3:
@@ -479,7 +499,24 @@ def batched_mul(A, B):
     if A.dtype != B.dtype:
         raise ArgumentError("batched_mul needs one element type for A and B")
     C = DeviceArray.empty((A.dims[0], B.dims[1], max(A.dims[2], B.dims[2])), A.dtype)
-    return batched_mul_(C, A, B)
+    return batched_mul_(C, _copy_if_faster(A), _copy_if_faster(B))
+
+
+def batched_vec(A, B):
+    """batched_vec(A, B)  (src/batched/batchedmul.jl:166-218): C[:,k...] = A[:,:,k...] * B[:,k...]; a vector
+    ``B`` is shared by every batch."""
+    if not isinstance(A, DeviceArray) or not isinstance(B, DeviceArray):
+        raise ArgumentError("batched_vec expects DeviceArrays")
+    if A.ndim == 3 and B.ndim == 1:                                                    # :217-218
+        return batched_mul(A, B.reshape(B.dims[0], 1, 1)).reshape(A.dims[0], A.dims[2])
+    if A.ndim != B.ndim + 1:                                                           # :198-199
+        raise DimensionMismatch(f"batched_vec requires ndims(A) == ndims(B) + 1, got ndims(A)={A.ndim} and ndims(B)={B.ndim}")
+    if A.dims[2:] != B.dims[1:]:                                                       # :200-201
+        raise DimensionMismatch(f"batch dimensions must match: size(A)[3:end]={A.dims[2:]} != size(B)[2:end]={B.dims[1:]}")
+    if not B.is_contiguous():
+        B = B.copy()                                                                   # :213-215: a transposed B is copied
+    C = batched_mul(A, B.reshape((B.dims[0], 1) + B.dims[1:]))
+    return C.reshape((C.dims[0],) + C.dims[2:])
 
 
 def batched_mul_pullback(A, B, dC):

@@ -94,3 +94,92 @@ def test_errors(nn):
         nn.batched_mul(z(2, 3, 2), z(4, 2, 2))
     with pytest.raises(nn.DimensionMismatch):
         nn.batched_mul_(z(2, 2, 3), z(2, 2, 2), z(2, 2, 2))
+
+
+# ---- the wider batched_mul surface (src/batched/batchedmul.jl:140-218) --------------------------------
+
+def _slices(A, B):
+    nb = max(A.shape[2], B.shape[2])
+    return np.stack([A[:, :, k if A.shape[2] > 1 else 0] @ B[:, :, k if B.shape[2] > 1 else 0] for k in range(nb)], axis=2)
+
+
+@pytest.mark.parametrize("perm", [(1, 3, 2), (2, 1, 3), (3, 2, 1)])
+@pytest.mark.parametrize("adj", [False, True])
+def test_permuted_dims_inputs(nn, perm, adj):
+    """test/batchedmul.jl:80-88: lazy PermutedDimsArray operands equal their materialised permutedims;
+    perm (3,2,1) has stride 1 along the batch and is copied first (_copy_if_faster)."""
+    rng = np.random.default_rng(sum(perm))
+    A = rng.standard_normal((4, 4, 4)).astype(np.float32)
+    B = rng.standard_normal((4, 4, 4)).astype(np.float32)
+    ax = tuple(p - 1 for p in perm)
+    dA, dB = nn.DeviceArray.from_numpy(A), nn.DeviceArray.from_numpy(B)
+    fun = nn.batched_adjoint if adj else (lambda x: x)
+    Ah = A.transpose(1, 0, 2) if adj else A
+    got = nn.batched_mul(fun(dA), dB.permuted(perm)).to_numpy()
+    assert np.abs(got - _slices(Ah, B.transpose(ax))).max() < 1e-5
+    got = nn.batched_mul(fun(dA.permuted(perm)), dB).to_numpy()
+    Ap = A.transpose(ax)
+    assert np.abs(got - _slices(Ap.transpose(1, 0, 2) if adj else Ap, B)).max() < 1e-5
+    assert np.array_equal(dA.permuted(perm).copy().to_numpy(), Ap)          # permutedims
+
+
+def test_permuted_dims_output_and_five_argument_form(nn):
+    """test/batchedmul.jl:90-101: C = PermutedDimsArray(zeros(5,2,4), (3,1,2)) is written through its
+    transpose; 10*C1 and C1 + 100 with the alpha / beta arguments."""
+    rng = np.random.default_rng(2)
+    A = rng.standard_normal((4, 3, 2)).astype(np.float32)
+    Bp = rng.standard_normal((5, 3, 2)).astype(np.float32)
+    dA, dB = nn.DeviceArray.from_numpy(A), nn.batched_adjoint(nn.DeviceArray.from_numpy(Bp))
+    C1 = nn.batched_mul(dA, dB).to_numpy()
+    assert np.abs(C1 - _slices(A, Bp.transpose(1, 0, 2))).max() < 1e-5
+    parent = nn.DeviceArray.zeros((5, 2, 4))
+    C2 = parent.permuted(3, 1, 2)
+    assert C2.dims == (4, 5, 2)
+    nn.batched_mul_(C2, dA, dB)
+    assert np.abs(C2.to_numpy() - C1).max() < 1e-5
+    nn.batched_mul_(C2, dA, dB, 10)
+    assert np.abs(C2.to_numpy() - 10 * C1).max() < 1e-4
+    parent.storage.fill_(10.0)
+    nn.batched_mul_(C2, dA, dB, 1, 10)
+    assert np.abs(C2.to_numpy() - (C1 + 100)).max() < 1e-4
+
+
+def test_matrix_operands_and_batched_vec(nn):
+    """test/batchedmul.jl:225-236: a matrix (plain or lazily transposed) on either side is shared by every
+    batch; batched_vec treats the matrix as a batch of vectors."""
+    rng = np.random.default_rng(3)
+    A = rng.standard_normal((3, 3, 3)).astype(np.float32)
+    M = rng.standard_normal((3, 3)).astype(np.float32)
+    V = rng.standard_normal(3).astype(np.float32)
+    dA, dM, dV = (nn.DeviceArray.from_numpy(x) for x in (A, M, V))
+    cat = lambda f: np.stack([f(k) for k in range(3)], axis=2)
+    assert np.abs(nn.batched_mul(dA, dM).to_numpy() - cat(lambda k: A[:, :, k] @ M)).max() < 1e-5
+    assert np.abs(nn.batched_mul(dA, nn.transpose(dM)).to_numpy() - cat(lambda k: A[:, :, k] @ M.T)).max() < 1e-5
+    assert np.abs(nn.batched_mul(dM, dA).to_numpy() - cat(lambda k: M @ A[:, :, k])).max() < 1e-5
+    assert np.abs(nn.batched_mul(nn.adjoint(dM), dA).to_numpy() - cat(lambda k: M.T @ A[:, :, k])).max() < 1e-5
+    hcat = lambda f: np.stack([f(k) for k in range(3)], axis=1)
+    assert np.abs(nn.batched_vec(dA, dM).to_numpy() - hcat(lambda k: A[:, :, k] @ M[:, k])).max() < 1e-5
+    assert np.abs(nn.batched_vec(dA, nn.transpose(dM)).to_numpy() - hcat(lambda k: A[:, :, k] @ M.T[:, k])).max() < 1e-5
+    assert np.abs(nn.batched_vec(dA, dV).to_numpy() - hcat(lambda k: A[:, :, k] @ V)).max() < 1e-5
+
+
+def test_batched_vec_nd(nn):
+    """test/batchedmul.jl:337-365 and the size doctests of src/batched/batchedmul.jl:182-196."""
+    rng = np.random.default_rng(4)
+    A4, B3 = rng.standard_normal((4, 5, 3, 2)).astype(np.float32), rng.standard_normal((5, 3, 2)).astype(np.float32)
+    C = nn.batched_vec(nn.DeviceArray.from_numpy(A4), nn.DeviceArray.from_numpy(B3))
+    assert C.dims == (4, 3, 2)
+    assert np.abs(C.to_numpy() - np.einsum("mkij,kij->mij", A4, B3)).max() < 1e-5
+    A5, B4 = rng.standard_normal((3, 4, 2, 3, 2)).astype(np.float32), rng.standard_normal((4, 2, 3, 2)).astype(np.float32)
+    C5 = nn.batched_vec(nn.DeviceArray.from_numpy(A5), nn.DeviceArray.from_numpy(B4))
+    assert C5.dims == (3, 2, 3, 2)
+    assert np.abs(C5.to_numpy() - np.einsum("mkabc,kabc->mabc", A5, B4)).max() < 1e-5
+    Z = nn.DeviceArray.zeros
+    assert nn.batched_vec(Z((16, 8, 32)), Z((8, 32))).dims == (16, 32)
+    assert nn.batched_vec(Z((16, 8, 32)), Z((8,))).dims == (16, 32)
+    assert nn.batched_mul(Z((16, 8, 32)), Z((8, 4))).dims == (16, 4, 32)
+    assert nn.batched_mul(Z((16, 8)), Z((8, 4, 32))).dims == (16, 4, 32)
+    with pytest.raises(nn.DimensionMismatch):
+        nn.batched_vec(Z((3, 4, 2)), Z((4, 3)))
+    with pytest.raises(nn.DimensionMismatch):
+        nn.batched_vec(Z((3, 4, 2, 3)), Z((4, 2, 2)))
