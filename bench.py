@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|bwd|logsoftmax|softmax_dims2] [--no-cpu]
 
 A "step" is one dot_product_attention call on synthetic inputs that are already resident in HBM.
 The default workload is C3 (bf16 causal prefill, head dim 128, L = 4096), the configuration the
@@ -228,6 +228,115 @@ def measure(key, steps, warmup, with_cpu):
     return res
 
 
+# ---- the rows built after the five configurations: gradient and softmax family ------------------------
+
+EXTRA = {
+    "bwd": "gradient of C3: causal bf16 (4096,4096,2) H=32 D=128, dq + dk + dv from dy and the forward result",
+    "logsoftmax": "logsoftmax(x; dims=1), x (4096, 65536) f32 (1 GiB in, 1 GiB out)",
+    "softmax_dims2": "softmax(x; dims=2), x (256, 4096, 128) bf16 (256 MiB in, 256 MiB out), reduction over the strided dim",
+}
+
+
+def _event_time(lib, _lib, fn, steps, warmup):
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    _lib.check(lib.mi_event_create(ctypes.byref(e0)))
+    _lib.check(lib.mi_event_create(ctypes.byref(e1)))
+    for _ in range(warmup):
+        fn()
+    _lib.check(lib.mi_device_sync())
+    _lib.check(lib.mi_event_record(e0, None))
+    for _ in range(steps):
+        fn()
+    _lib.check(lib.mi_event_record(e1, None))
+    _lib.check(lib.mi_event_sync(e1))
+    ms = ctypes.c_float(0)
+    _lib.check(lib.mi_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    lib.mi_event_destroy(e0)
+    lib.mi_event_destroy(e1)
+    return ms.value / steps
+
+
+def measure_extra(key, steps, warmup, with_cpu):
+    """One JSON line for a workload outside BASELINE.json's five configurations (same fields)."""
+    import numpy as np
+    import nnlib_amd as nn
+    from nnlib_amd import _lib
+    lib = _lib.load()
+    _lib.check(lib.mi_init(0))
+    DA = nn.DeviceArray
+    cores = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
+    if key == "bwd":
+        w = WORKLOADS["c3"]
+        E, L, B, H = w["E"], w["Lq"], w["B"], w["H"]
+        D = E // H
+        arrs = [DA.empty((E, L, B), "bf16") for _ in range(4)]
+        for sid, a in enumerate(arrs):
+            _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, w["seed"], sid, 1.0, None))
+        q, k, v, dy = arrs
+        y, _ = nn.dot_product_attention(q, k, v, mask=nn.make_causal_mask(q), nheads=H, return_weights=False)
+        d = _lib.mi_attn_bwd_desc()
+        d.struct_size = ctypes.sizeof(_lib.mi_attn_bwd_desc)
+        nn.ops._fill_desc(d.fwd, q, k, v, None, nn.make_causal_mask(q), H, B, E, E, L, L, 0)
+        d.fwd.out, d.dout = y.ptr, dy.ptr
+        grads = [DA.empty((E, L, B), "bf16") for _ in range(3)]
+        d.dq, d.dk, d.dv = (g.ptr for g in grads)
+        kern, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
+        _lib.check(lib.mi_attention_bwd_plan(ctypes.byref(d), ctypes.byref(kern), ctypes.byref(ws)))
+        wsbuf = DA.empty((ws.value // 4 + 4,), "f32")
+        d.workspace, d.workspace_bytes = wsbuf.ptr, ws.value
+        ms = _event_time(lib, _lib, lambda: _lib.check(lib.mi_attention_bwd(ctypes.byref(d), None)), steps, warmup)
+        # five products (S, dP, dV, dK, dQ) of 2*D FLOP per unmasked (query, key) pair
+        flops = 10 * D * H * B * (L * (L + 1) // 2)
+        val = flops / (ms * 1e-3) / 1e12
+        line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype="bf16",
+                    roofline=dict(bound="mfma", achieved=val, peak=PEAK["bf16"], unit="TFLOP/s", frac=val / PEAK["bf16"], traffic=None),
+                    config=dict(workload=EXTRA[key], kernel=_lib.KERNEL_NAMES[kern.value]), flops_per_step=flops)
+        if with_cpu:
+            from oracle import oracle as O
+            rng = np.random.default_rng(0)
+            a1 = [np.asfortranarray(rng.standard_normal((D, L, 1))) for _ in range(4)]
+            t0 = time.perf_counter()
+            O.attention_bwd_f64(a1[0], a1[1], a1[2], a1[3], None, O.make_causal_mask(L), 1)
+            dt = time.perf_counter() - t0
+            line["cpu_baseline"] = dict(value=flops / (dt * H * B) / 1e12, unit="TFLOP/s", cores=1, kind="port",
+                                        sample=f"1 of {H * B} (head, batch) slices, forward + gradient oracle in Float64 on one thread "
+                                               f"({dt:.1f} s), scaled by {H * B}x")
+    else:
+        if key == "logsoftmax":
+            dims, dt_name, shape, op = 1, "f32", (4096, 65536), _lib.MI_LOGSOFTMAX
+        else:
+            dims, dt_name, shape, op = 2, "bf16", (256, 4096, 128), _lib.MI_SOFTMAX
+        nsets = 2 if key == "logsoftmax" else 4          # rotate past the 256 MiB last-level cache
+        xs = [DA.empty(shape, dt_name) for _ in range(nsets)]
+        ys = [DA.empty(shape, dt_name) for _ in range(nsets)]
+        for x in xs:
+            _lib.check(lib.mi_randn_fill(x.ptr, x.code, x.length, 7, 0, 1.0, None))
+        inner, n, outer, _ = nn.ops._reduction_geometry(shape, dims)
+        state = {"i": 0}
+
+        def fn():
+            i = state["i"] = (state["i"] + 1) % nsets
+            _lib.check(lib.mi_softmax(op, xs[i].code, xs[i].ptr, ys[i].ptr, inner, n, outer, None))
+        ms = _event_time(lib, _lib, fn, steps, warmup)
+        nbytes = 2 * xs[0].length * xs[0].itemsize       # one read, one write
+        val = nbytes / (ms * 1e-3) / 1e9
+        line = dict(metric=f"{key} GB/s", value=val, unit="GB/s", dtype=dt_name,
+                    roofline=dict(bound="hbm", achieved=val, peak=HBM_PEAK, unit="GB/s", frac=val / HBM_PEAK, traffic=None),
+                    config=dict(workload=EXTRA[key], kernel="softmax_nd_kernel"), bytes_per_step=nbytes)
+        if with_cpu:
+            from oracle import oracle as O
+            small = (shape[0], shape[1] // 16) + shape[2:]
+            xh = np.asfortranarray(np.random.default_rng(0).standard_normal(small).astype(np.float32))
+            t0 = time.perf_counter()
+            O.softmax(xh, dims, np.float32, log=(key == "logsoftmax"))
+            dt = time.perf_counter() - t0
+            line["cpu_baseline"] = dict(value=nbytes / 16 / dt / 1e9, unit="GB/s", cores=1, kind="port",
+                                        sample=f"1/16 of the array, Float32 oracle on one thread as the reference's passes are ({dt:.2f} s)")
+    line.update(n_gpus=1, steps=steps, warmup=warmup, ms_per_step=ms, higher_is_better=True, scaling="weak", vs_baseline=None,
+                data="synthetic")
+    print(json.dumps(line))
+
+
 def copy_calibration(steps):
     """A plain copy kernel of known size (1 GiB read, 1 GiB written per launch): the reference point
     that the FETCH_SIZE / WRITE_SIZE counters are scaled by when HBM traffic is read with rocprofv3."""
@@ -251,7 +360,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["copy"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + sorted(EXTRA) + ["copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
     args = ap.parse_args()
@@ -264,6 +373,8 @@ def main():
 
     if args.workload == "copy":
         return copy_calibration(min(args.steps, 10))
+    if args.workload in EXTRA:
+        return measure_extra(args.workload, min(args.steps, 50), min(args.warmup, 10), not args.no_cpu)
     main_res = measure(args.workload, args.steps, args.warmup, not args.no_cpu)
     w = WORKLOADS[args.workload]
     prefill = args.workload not in ("c4", "c5")

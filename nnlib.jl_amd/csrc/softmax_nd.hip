@@ -43,10 +43,13 @@ __device__ inline float reduce_slices(float v, int ti_log2, float *red) {
     return r;
 }
 
+// e^x through the hardware 2^x (the reference's own exp is @fastmath, src/softmax.jl:72)
+__device__ inline float fast_exp(float x) { return mi_exp2(x * MI_LOG2E); }
+
 // the reference's elementwise rules given the column maximum m
 __device__ inline float softmax_term(float x, float m) {   // src/softmax.jl:72-75
     if (m == MI_POS_INF) return x == MI_POS_INF ? 1.0f : 0.0f;
-    return expf(x - m);
+    return fast_exp(x - m);
 }
 __device__ inline float logsoftmax_shift(float x, float m) {   // src/softmax.jl:140-144
     if (m == MI_POS_INF) return x == MI_POS_INF ? 0.0f : MI_NEG_INF;
@@ -95,12 +98,12 @@ __global__ __launch_bounds__(256) void softmax_nd_kernel(const typename T::type 
                 for (int c = 0; c < CACHE; c++) {
                     const int64_t j = js + (int64_t)tj * c;
                     if (ok && j < g.len)
-                        yc[g.inner * j] = T::from_f32(OP == OP_GRAD_SOFTMAX ? v2[c] * (v[c] - s) : v[c] - s * expf(v2[c]));
+                        yc[g.inner * j] = T::from_f32(OP == OP_GRAD_SOFTMAX ? v2[c] * (v[c] - s) : v[c] - s * fast_exp(v2[c]));
                 }
             } else if (ok) {
                 for (int64_t j = js; j < g.len; j += tj) {
                     const float dy = T::to_f32(xc[g.inner * j]), yy = T::to_f32(x2c[g.inner * j]);
-                    yc[g.inner * j] = T::from_f32(OP == OP_GRAD_SOFTMAX ? yy * (dy - s) : dy - s * expf(yy));
+                    yc[g.inner * j] = T::from_f32(OP == OP_GRAD_SOFTMAX ? yy * (dy - s) : dy - s * fast_exp(yy));
                 }
             }
             continue;
@@ -125,8 +128,8 @@ __global__ __launch_bounds__(256) void softmax_nd_kernel(const typename T::type 
         float s = 0.0f;
         auto term = [&](float xv) {
             if (OP == OP_SOFTMAX) return softmax_term(xv, m);
-            if (OP == OP_LOGSOFTMAX) return expf(logsoftmax_shift(xv, m));
-            return expf(xv - m);   // logsumexp: no special cases (src/softmax.jl:202)
+            if (OP == OP_LOGSOFTMAX) return fast_exp(logsoftmax_shift(xv, m));
+            return fast_exp(xv - m);   // logsumexp: no special cases (src/softmax.jl:202)
         };
         if (cached) {
 #pragma unroll
@@ -159,6 +162,176 @@ __global__ __launch_bounds__(256) void softmax_nd_kernel(const typename T::type 
     }
 }
 
+// ---- reductions over a strided dimension with wide rows ----------------------------------------------
+// inner is a multiple of VEC (16 bytes of elements) and every row starts 16-byte aligned: a thread owns
+// VEC consecutive `inner` positions and walks j in steps of TJ; TI threads side by side cover TI*VEC
+// positions, so a wavefront reads 64/TI rows of TI*16 contiguous bytes per load.  One pass finds the
+// maximum and the sum together (running maximum, sum rescaled when it grows), a second pass writes:
+// two reads and one write per element.
+template <typename T, int VEC>
+struct VecIO {
+    typedef typename T::type t;
+    __device__ static void unpack(const u32x4_t &raw, float (&v)[VEC]) {
+        if constexpr (VEC == 4) {
+            const floatx4_t f = __builtin_bit_cast(floatx4_t, raw);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = f[e];
+        } else {
+            const typename T::vec8 h = __builtin_bit_cast(typename T::vec8, raw);
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = T::to_f32(h[e]);
+        }
+    }
+    __device__ static void store(t *p, const float (&v)[VEC]) {
+        if constexpr (VEC == 4) {
+            floatx4_t f;
+#pragma unroll
+            for (int e = 0; e < 4; e++) f[e] = v[e];
+            *(floatx4_t *)p = f;
+        } else {
+            typename T::vec8 h;
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = T::from_f32(v[e]);
+            *(u32x4_t *)p = __builtin_bit_cast(u32x4_t, h);
+        }
+    }
+};
+
+// running (maximum, sum of exponentials against it); the special cases keep the reference's results:
+// nothing but -Inf so far contributes no terms, a +Inf maximum counts the +Inf entries (src/softmax.jl:72-75)
+__device__ inline void online_add(float x, float &m, float &s) {
+    if (x > m) {
+        s = (m == MI_NEG_INF) ? 0.0f : s * fast_exp(m - x);
+        m = x;
+    }
+    if (m != MI_NEG_INF) s += softmax_term(x, m);
+}
+__device__ inline void online_merge(float m2, float s2, float &m, float &s) {
+    if (m2 > m) {
+        s = (m == MI_NEG_INF) ? s2 : s2 + s * fast_exp(m - m2);
+        m = m2;
+    } else if (m2 != MI_NEG_INF) {
+        s += (m2 == m) ? s2 : s2 * fast_exp(m2 - m);
+    }
+}
+
+template <typename T, int OP, int VEC>
+__global__ __launch_bounds__(256) void softmax_nd_vec_kernel(const typename T::type *x, const typename T::type *x2,
+                                                              typename T::type *y, Geometry g) {
+    typedef typename T::type t;
+    typedef VecIO<T, VEC> IO;
+    constexpr int U = 4;   // rows in flight per thread: all loads of a group are issued before any arithmetic
+    constexpr bool GRAD = OP >= OP_GRAD_SOFTMAX;
+    __shared__ float red_m[256 * VEC], red_s[256 * VEC];
+    const int ti = 1 << g.ti_log2, tj = 256 >> g.ti_log2;
+    const int il = threadIdx.x & (ti - 1), js = threadIdx.x >> g.ti_log2;
+    const int64_t n_tiles = g.n_itiles * g.outer;
+    const int64_t step = g.inner * tj;   // elements between consecutive rows of one thread
+    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const int64_t o = tile / g.n_itiles, i = ((tile % g.n_itiles) * ti + il) * VEC;
+        const bool ok = i < g.inner;
+        const int64_t base = i + g.inner * g.len * o + g.inner * js;
+        const int64_t nrows = ok && js < g.len ? (g.len - js + tj - 1) / tj : 0;   // rows js, js+tj, ... of this thread
+        float m[VEC], s[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            m[e] = MI_NEG_INF;
+            s[e] = 0.0f;
+        }
+        for (int64_t r0 = 0; r0 < nrows; r0 += U) {
+            u32x4_t raw[U], raw2[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int64_t at = base + step * (r0 + u < nrows ? r0 + u : nrows - 1);   // the tail repeats the last row (ignored below)
+                raw[u] = *(const u32x4_t *)(x + at);
+                if (OP == OP_GRAD_SOFTMAX) raw2[u] = *(const u32x4_t *)(x2 + at);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (r0 + u >= nrows) break;
+                float v[VEC], v2[VEC];
+                IO::unpack(raw[u], v);
+                if constexpr (GRAD) {
+                    if (OP == OP_GRAD_SOFTMAX) IO::unpack(raw2[u], v2);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) s[e] += OP == OP_GRAD_SOFTMAX ? v[e] * v2[e] : v[e];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) online_add(v[e], m[e], s[e]);
+                }
+            }
+        }
+        // combine the TJ slices of each position through LDS
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            red_m[(js * ti + il) * VEC + e] = m[e];
+            red_s[(js * ti + il) * VEC + e] = s[e];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            float mm = MI_NEG_INF, ss = 0.0f;
+            for (int q = 0; q < tj; q++) {
+                const float m2 = red_m[(q * ti + il) * VEC + e], s2 = red_s[(q * ti + il) * VEC + e];
+                if constexpr (GRAD) ss += s2;
+                else online_merge(m2, s2, mm, ss);
+            }
+            m[e] = mm;
+            s[e] = ss;
+        }
+        if (!ok) continue;
+        if constexpr (OP == OP_LOGSUMEXP) {
+            if (js == 0) {
+                float r[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; e++)   // the reference's x - max is Inf - Inf for an infinite maximum
+                    r[e] = (m[e] == MI_POS_INF || m[e] == MI_NEG_INF) ? __builtin_nanf("") : m[e] + logf(s[e]);
+                IO::store(y + i + g.inner * o, r);
+            }
+            continue;
+        }
+        // per-position constants of the second pass; `plain`: finite maxima, so no special cases
+        float c0[VEC], c1[VEC];
+        bool plain = true;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            plain = plain && m[e] > MI_NEG_INF && m[e] < MI_POS_INF;
+            if (OP == OP_SOFTMAX) {
+                c0[e] = -m[e] * MI_LOG2E;
+                c1[e] = 1.0f / s[e];
+            } else if (OP == OP_LOGSOFTMAX) {
+                c0[e] = logf(s[e]);
+                c1[e] = -m[e] - c0[e];
+            }
+        }
+        for (int64_t r0 = 0; r0 < nrows; r0 += U) {
+            u32x4_t raw[U], raw2[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int64_t at = base + step * (r0 + u < nrows ? r0 + u : nrows - 1);
+                raw[u] = *(const u32x4_t *)(x + at);
+                if (GRAD) raw2[u] = *(const u32x4_t *)(x2 + at);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (r0 + u >= nrows) break;
+                float v[VEC], v2[VEC], r[VEC];
+                IO::unpack(raw[u], v);
+                if (GRAD) IO::unpack(raw2[u], v2);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    if (OP == OP_SOFTMAX) r[e] = plain ? mi_exp2(fmaf(v[e], MI_LOG2E, c0[e])) * c1[e] : softmax_term(v[e], m[e]) / s[e];
+                    else if (OP == OP_LOGSOFTMAX) r[e] = plain ? v[e] + c1[e] : logsoftmax_shift(v[e], m[e]) - c0[e];
+                    else if (OP == OP_GRAD_SOFTMAX) r[e] = v2[e] * (v[e] - s[e]);
+                    else r[e] = v[e] - s[e] * fast_exp(v2[e]);
+                }
+                IO::store(y + base + step * (r0 + u), r);
+            }
+        }
+    }
+}
+
 template <typename T, int OP>
 void launch_nd(const void *x, const void *x2, void *y, int64_t inner, int64_t len, int64_t outer, hipStream_t st) {
     typedef typename T::type t;
@@ -166,6 +339,22 @@ void launch_nd(const void *x, const void *x2, void *y, int64_t inner, int64_t le
     g.inner = inner;
     g.len = len;
     g.outer = outer;
+    constexpr int VEC = 16 / (int)sizeof(t);
+    const auto al = [](const void *p) { return (((uintptr_t)p) & 15) == 0; };
+    if (inner % VEC == 0 && inner >= 4 * VEC && len > 64 && al(x) && al(y) && (!x2 || al(x2))) {
+        // wide rows and columns too long for the register cache of the scalar kernel
+        const int64_t chunks = inner / VEC;
+        g.ti_log2 = 0;
+        while ((1 << g.ti_log2) < 64 && ((int64_t)1 << g.ti_log2) < chunks) g.ti_log2++;
+        // enough workgroups to fill the chip, but rows of at least 64 contiguous bytes per wavefront load
+        while (g.ti_log2 > 2 && ((chunks + (1 << g.ti_log2) - 1) >> g.ti_log2) * outer < 2048) g.ti_log2--;
+        g.n_itiles = (chunks + (1 << g.ti_log2) - 1) >> g.ti_log2;
+        int64_t blocks = g.n_itiles * outer;
+        if (blocks > 262144) blocks = 262144;
+        hipLaunchKernelGGL((softmax_nd_vec_kernel<T, OP, VEC>), dim3((unsigned)blocks), dim3(256), 0, st, (const t *)x,
+                           (const t *)x2, (t *)y, g);
+        return;
+    }
     g.ti_log2 = 0;
     while ((1 << g.ti_log2) < 64 && ((int64_t)1 << g.ti_log2) < inner) g.ti_log2++;
     g.n_itiles = (inner + (1 << g.ti_log2) - 1) >> g.ti_log2;

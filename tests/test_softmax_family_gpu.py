@@ -47,7 +47,7 @@ def test_reference_values(nn):
 SHAPES = [((2, 2, 2, 2, 2), d) for d in (1, 2, 3, 4, 5)] + [
     ((5, 7), 2), ((3, 4), None), ((33, 65, 3), 2), ((64, 100, 5), 2), ((130, 17, 2), (2, 3)), ((7, 3000, 2), 2),
     ((1, 5000, 3), 2), ((300, 70, 2), 2), ((5000,), 1), ((70000,), None), ((4, 9, 6), (1, 2)), ((128, 40), 1),
-    ((9, 5), 3)]
+    ((9, 5), 3), ((256, 1000, 3), 2), ((96, 129, 2), 2), ((32, 70, 2, 2), (2, 3)), ((1024, 65), 2)]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
@@ -103,3 +103,33 @@ def test_errors(nn):
         nn.softmax(nn.DeviceArray.zeros((2, 3, 4)), dims=(1, 3))
     with pytest.raises(nn.DimensionMismatch):
         nn.grad_softmax_(nn.DeviceArray.zeros((3, 2)), nn.DeviceArray.zeros((2, 3)), nn.DeviceArray.zeros((2, 3)))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_special_values_on_the_wide_row_kernel(nn, oracle, dtype):
+    """The one-pass maximum-and-sum of the strided kernel keeps the +-Inf / NaN rules of
+    src/softmax.jl:72-75, 140-144 wherever the special entry sits in the column."""
+    rng = np.random.default_rng(11)
+    x = round_to(rng.standard_normal((64, 200, 2)), dtype)
+    x[0, :, 0] = -np.inf                      # all -Inf: NaN
+    x[1, 5, 0] = np.inf                       # one +Inf
+    x[2, [3, 150], 0] = np.inf                # two +Inf: 0.5 each
+    x[3, 0, 0] = -np.inf                      # -Inf first, finite later
+    x[4, 199, 0] = -np.inf
+    x[5, 77, 0] = np.nan                      # NaN poisons its column only
+    x[6, :100, 1] = -np.inf                   # a long run of -Inf before the first finite entry
+    x[7, 0, 1] = np.inf
+    x[7, 1:, 1] = -np.inf
+    d = _dev(nn, x, dtype)
+    tol = TOL[dtype]
+    with np.errstate(invalid="ignore"):
+        for fn, ref in ((nn.softmax, oracle.softmax(x, 2)), (nn.logsoftmax, oracle.logsoftmax(x, 2))):
+            got = fn(d, dims=2).to_numpy()
+            assert np.array_equal(np.isnan(got), np.isnan(ref))
+            assert np.array_equal(np.isinf(got), np.isinf(ref))
+            fin = np.isfinite(ref)
+            assert np.abs(got[fin] - ref[fin]).max() <= tol * max(1.0, np.abs(ref[fin]).max())
+        got, ref = nn.logsumexp(d, dims=2).to_numpy(), oracle.logsumexp(x, 2)
+        assert np.array_equal(np.isnan(got), np.isnan(ref)) and np.array_equal(np.isinf(got), np.isinf(ref))
+        fin = np.isfinite(ref)
+        assert np.abs(got[fin] - ref[fin]).max() <= tol * 10
