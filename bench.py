@@ -273,11 +273,12 @@ def measure_extra(key, steps, warmup, with_cpu):
         for sid, a in enumerate(arrs):
             _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, w["seed"], sid, 1.0, None))
         q, k, v, dy = arrs
-        y, _ = nn.dot_product_attention(q, k, v, mask=nn.make_causal_mask(q), nheads=H, return_weights=False)
+        y, _ = nn.dot_product_attention(q, k, v, mask=nn.make_causal_mask(q), nheads=H, return_weights=False,
+                                        save_for_backward=True)   # as an AD rule would: the pullback reuses the row statistics
         d = _lib.mi_attn_bwd_desc()
         d.struct_size = ctypes.sizeof(_lib.mi_attn_bwd_desc)
         nn.ops._fill_desc(d.fwd, q, k, v, None, nn.make_causal_mask(q), H, B, E, E, L, L, 0)
-        d.fwd.out, d.dout = y.ptr, dy.ptr
+        d.fwd.out, d.dout, d.fwd.stats = y.ptr, dy.ptr, y.saved_stats.ptr
         grads = [DA.empty((E, L, B), "bf16") for _ in range(3)]
         d.dq, d.dk, d.dv = (g.ptr for g in grads)
         kern, ws = ctypes.c_int32(0), ctypes.c_size_t(0)

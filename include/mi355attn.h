@@ -146,6 +146,14 @@ typedef struct mi_attn_desc {
     float dropout_p;
     uint32_t reserved2;
     uint64_t dropout_seed;
+    /* Optional: softmax row statistics saved for mi_attention_bwd (what an AD rule keeps between the
+     * forward and the backward call).  NULL, or a buffer of mi_attention_stats_size() bytes, 16-byte
+     * aligned.  Written only by calls that mi_attention_plan() reports as MI_ATTN_KERNEL_FLASH16 (such
+     * calls then do not split the key range); other kernels leave it untouched.  Contents are private
+     * to the library.  In mi_attn_bwd_desc.fwd: pass the buffer a FLASH16 forward call of the same
+     * arguments filled (the backward call also writes into it), or NULL to have the statistics
+     * recomputed. */
+    float *stats;
 } mi_attn_desc;
 
 /* Validates shapes the way src/attention.jl:55-78 does (MI_ESHAPE on failure) and
@@ -153,6 +161,7 @@ typedef struct mi_attn_desc {
 int32_t mi_attention_plan(const mi_attn_desc *desc, int32_t *kernel, size_t *workspace_bytes);
 int32_t mi_attention_workspace_size(const mi_attn_desc *desc, size_t *bytes);
 int32_t mi_attention_fwd(const mi_attn_desc *desc, mi_stream stream);
+int32_t mi_attention_stats_size(const mi_attn_desc *desc, size_t *bytes);
 
 /*
  * Gradient of one dot_product_attention call (fdrop = identity).  The reference has no hand-written

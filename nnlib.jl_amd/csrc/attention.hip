@@ -121,6 +121,8 @@ int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_back
     AttnParams p;
     p.q = d->q; p.k = d->k; p.v = d->v; p.out = d->out; p.weights = d->weights;
     p.bias = d->bias; p.mask = d->mask; p.workspace = d->workspace;
+    p.stats = d->stats;
+    if (d->stats && (((uintptr_t)d->stats) & 15) != 0) return mi_set_error(MI_EINVAL, "mi_attention: stats must be 16-byte aligned");
     for (int i = 0; i < 4; i++) {
         p.bias_strides[i] = d->bias ? d->bias_strides[i] : 0;
         p.mask_strides[i] = d->mask ? d->mask_strides[i] : 0;
@@ -164,6 +166,15 @@ MI_API int32_t mi_attention_plan(const mi_attn_desc *d, int32_t *kernel, size_t 
     int32_t k = choose(d, p, &ws);
     if (kernel) *kernel = k;
     if (workspace_bytes) *workspace_bytes = ws;
+    return MI_OK;
+}
+
+MI_API int32_t mi_attention_stats_size(const mi_attn_desc *d, size_t *bytes) {
+    if (!bytes) return mi_set_error(MI_EINVAL, "mi_attention_stats_size: bytes is NULL");
+    AttnParams p;
+    int32_t rc = attention_validate(d, &p, true);
+    if (rc != MI_OK) return rc;
+    *bytes = attention_stats_bytes(p);
     return MI_OK;
 }
 

@@ -22,15 +22,20 @@ static int32_t validate_bwd(const mi_attn_bwd_desc *d, AttnBwdParams *out) {
     bp.dv = d->dv;
     bp.dbias = d->dbias;
     bp.workspace = d->workspace;
-    bp.stats = (float *)d->workspace;
+    bp.have_stats = d->fwd.stats != nullptr;
+    bp.stats = bp.have_stats ? d->fwd.stats : (float *)d->workspace;
     *out = bp;
     return MI_OK;
 }
 
 static int32_t choose_bwd(const mi_attn_bwd_desc *d, const AttnBwdParams &bp, size_t *ws) {
     if (!(d->fwd.flags & MI_ATTN_FORCE_GENERIC) && attention_bwd_flash16_supports(bp)) {
-        *ws = attention_bwd_flash16_workspace(bp.p);
+        *ws = bp.have_stats ? 0 : attention_bwd_flash16_workspace(bp.p);
         return MI_ATTN_KERNEL_FLASH16;
+    }
+    if (bp.have_stats) {   // the generic kernels keep their own statistics, in their own layout
+        *ws = attention_bwd_generic_workspace(bp.p);
+        return MI_ATTN_KERNEL_GENERIC;
     }
     *ws = attention_bwd_generic_workspace(bp.p);
     return MI_ATTN_KERNEL_GENERIC;
@@ -68,5 +73,7 @@ MI_API int32_t mi_attention_bwd(const mi_attn_bwd_desc *d, mi_stream s) {
                             d->workspace ? d->workspace_bytes : (size_t)0);
     if ((((uintptr_t)d->workspace) & 15) != 0) return mi_set_error(MI_EWORKSPACE, "mi_attention_bwd: workspace must be 16-byte aligned");
     if (kernel == MI_ATTN_KERNEL_FLASH16) return launch_attention_bwd_flash16(bp, st);
+    bp.stats = (float *)d->workspace;
+    bp.have_stats = 0;
     return launch_attention_bwd_generic(bp, st);
 }

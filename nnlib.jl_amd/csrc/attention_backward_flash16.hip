@@ -23,9 +23,7 @@ bool attention_bwd_flash16_supports(const AttnBwdParams &bp) {
 }
 
 // three float planes [B*H][Lq rounded up to 128]: row maximum (log2 units), 1 / row sum, delta
-size_t attention_bwd_flash16_workspace(const AttnParams &p) {
-    return sizeof(float) * 3 * (size_t)(p.B * p.H) * (size_t)((p.Lq + 127) / 128 * 128);
-}
+size_t attention_bwd_flash16_workspace(const AttnParams &p) { return attention_stats_bytes(p); }
 
 int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp, hipStream_t st) {
     const AttnParams &p = bp.p;

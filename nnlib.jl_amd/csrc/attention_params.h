@@ -8,6 +8,7 @@ struct AttnParams {
     const void *bias;
     const uint8_t *mask;
     void *workspace;
+    float *stats;      // optional: row statistics for the backward call, three planes [B*H][Lq rounded up to 128]
     int64_t bias_strides[4], mask_strides[4];
     int64_t E, Ev, Lq, Lkv, H, B, D, Dv;
     int32_t dtype, weights_dtype, causal;
@@ -24,9 +25,16 @@ struct AttnBwdParams {
     const void *dout, *dweights;
     void *dq, *dk, *dv;
     float *dbias;      // addressed with p.bias_strides
-    float *stats;      // workspace: per (query, head, batch) softmax statistics
+    float *stats;      // per (query, head, batch) softmax statistics: the workspace, or the buffer a forward call saved
+    int32_t have_stats; // the forward call already filled the first two planes of `stats`
     void *workspace;
 };
+
+// size of the statistics planes shared by the forward kernels that save them and the backward kernels
+__host__ __device__ static inline int64_t attention_stats_lq_pad(int64_t Lq) { return (Lq + 127) / 128 * 128; }
+static inline size_t attention_stats_bytes(const AttnParams &p) {
+    return sizeof(float) * 3 * (size_t)(p.B * p.H) * (size_t)attention_stats_lq_pad(p.Lq);
+}
 
 int32_t launch_attention_bwd_generic(const AttnBwdParams &bp, hipStream_t st);
 int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp, hipStream_t st);

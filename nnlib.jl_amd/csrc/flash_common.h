@@ -24,11 +24,22 @@ struct FlashArgs {
     int32_t mask_lds;
 };
 
+// Row statistics saved for the backward call: planes (maximum in log2 units, 1 / row sum, delta) of
+// [B*H][Lq rounded up to 128] floats; the forward kernels fill the first two.  Rows past Lq inside the
+// padding get zeros, which make their weights vanish in the backward kernels.
+__device__ inline void flash_save_stats(const AttnParams &p, int64_t b, int64_t h, int64_t qi, float m2, float linv) {
+    const int64_t pad = attention_stats_lq_pad(p.Lq);
+    if (qi >= pad) return;
+    const int64_t at = (b * p.H + h) * pad + qi;
+    p.stats[at] = qi < p.Lq ? m2 : 0.0f;
+    p.stats[p.B * p.H * pad + at] = qi < p.Lq ? linv : 0.0f;
+}
+
 // Split-kv bookkeeping shared by the planner (workspace size) and the launchers.
 // Partials live in the caller's workspace: o as [split][B][Lq][Ev] floats, then (m, l) as
 // [split][B][H][Lq][2] floats, m in log2 units.
 inline int flash_pick_nsplit(const AttnParams &p, int bm) {
-    if (p.weights || !p.out) return 1;                      // weights need the global maximum up front
+    if (p.weights || !p.out || p.stats) return 1;           // weights need the global maximum up front; saved statistics are per whole row
     const int64_t wgs = ((p.Lq + bm - 1) / bm) * p.H * p.B;
     if (wgs >= 512 || p.Lkv < 2048) return 1;
     // aim at one resident round: two workgroups per CU on 256 CUs (measured best on the f16 cross-attention case)

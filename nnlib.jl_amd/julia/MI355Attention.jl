@@ -134,6 +134,7 @@ struct AttnDesc
     mask::Ptr{Cvoid}; mask_strides::NTuple{4, Int64}
     workspace::Ptr{Cvoid}; workspace_bytes::Csize_t
     dropout_p::Float32; reserved2::UInt32; dropout_seed::UInt64
+    stats::Ptr{Cvoid}
 end
 
 # Mirror of `mi_attn_bwd_desc`.
@@ -193,8 +194,10 @@ function mask_and_bias(::Type{T}, bias, mask, target::NTuple{4, Int}) where {T}
     causal, mptr, mstr, bptr, bstr
 end
 
+# `stats`: nothing, or a Float32 DeviceArray of mi_attention_stats_size bytes that receives the softmax
+# row statistics for ∇dot_product_attention (written by the 16-bit MFMA kernels only)
 function attention_call(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v, bias, mask, H::Int; want_out::Bool,
-                        want_weights::Bool, fdrop::Union{Nothing, Dropout} = nothing) where {T <: MIFloat}
+                        want_weights::Bool, fdrop::Union{Nothing, Dropout} = nothing, stats = nothing) where {T <: MIFloat}
     E, Lq, B = size(q); Lkv = size(k, 2); Ev = v === nothing ? E : size(v, 1)
     causal, mptr, mstr, bptr, bstr = mask_and_bias(T, bias, mask, (Lkv, Lq, H, B))
     out = want_out ? DeviceArray{T}(undef, Ev, Lq, B) : nothing
@@ -203,11 +206,11 @@ function attention_call(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v, bias, mas
     mk(ws, wsbytes) = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0),
                                E, Ev, Lq, Lkv, H, B, q.ptr, k.ptr, v === nothing ? C_NULL : v.ptr,
                                out === nothing ? C_NULL : out.ptr, alpha === nothing ? C_NULL : alpha.ptr,
-                               bptr, bstr, mptr, mstr, ws, wsbytes, p, UInt32(0), seed)
+                               bptr, bstr, mptr, mstr, ws, wsbytes, p, UInt32(0), seed, stats === nothing ? C_NULL : stats.ptr)
     need = Ref{Csize_t}(0)
     check(ccall((:mi_attention_workspace_size, libmi), Int32, (Ref{AttnDesc}, Ptr{Csize_t}), mk(C_NULL, 0), need))
     ws = need[] > 0 ? DeviceArray{UInt8}(undef, Int(need[])) : nothing
-    GC.@preserve q k v bias mask out alpha ws begin
+    GC.@preserve q k v bias mask out alpha ws stats begin
         check(ccall((:mi_attention_fwd, libmi), Int32, (Ref{AttnDesc}, Ptr{Cvoid}),
                     mk(ws === nothing ? C_NULL : ws.ptr, need[]), C_NULL))
     end
@@ -224,17 +227,23 @@ function dot_product_attention(q::DeviceArray{T, N}, k::DeviceArray{T, N}, v::De
     return x, α
 end
 
+# attention_stats(q, nheads): buffer for the `stats` keyword of dot_product_attention (forward, written)
+# and ∇dot_product_attention (backward, read): saves the gradient its own pass over the keys
+function attention_stats(q::DeviceArray{T, 3}, nheads::Int) where {T}
+    DeviceArray{Float32}(undef, 3 * size(q, 3) * nheads * (cld(size(q, 2), 128) * 128))
+end
+
 # `return_weights = false` is this library's one addition: it skips materialising α and returns
 # `nothing` in its place (the reference always returns α).
 function dot_product_attention(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::DeviceArray{T, 3}, bias = nothing;
-                               fdrop = identity, mask = nothing, nheads = 1, return_weights = true) where {T <: MIFloat}
+                               fdrop = identity, mask = nothing, nheads = 1, return_weights = true, stats = nothing) where {T <: MIFloat}
     all(size.((q, k, v), 1) .% nheads .== 0) || throw(ArgumentError("First dimension in query, key and value must be divisible by `nheads`.\nInstead:\n- size(q): $(size(q))\n- size(k): $(size(k))\n- size(v): $(size(v))\n- nheads: $nheads"))
     size(q, 3) == size(k, 3) == size(v, 3) || throw(ArgumentError("Batch dimensions have to be the same. Instead:\n- size(q): $(size(q))\n- size(k): $(size(k))\n- size(v): $(size(v))"))
     size(q, 1) == size(k, 1) || throw(ArgumentError("First dimension in query and key has to be the same. Instead:\n- size(q): $(size(q))\n- size(k): $(size(k))"))
     size(k, 2) == size(v, 2) || throw(ArgumentError("Second dimension in key and value has to be the same. Instead:\n- size(k): $(size(k))\n- size(v): $(size(v))"))
     if fdrop === identity || fdrop isa Dropout
         return attention_call(q, k, v, bias, mask, nheads; want_out = true, want_weights = return_weights,
-                              fdrop = fdrop isa Dropout ? fdrop : nothing)
+                              fdrop = fdrop isa Dropout ? fdrop : nothing, stats)
     end
     # any other fdrop acts on the weights the caller sees (src/attention.jl:126): scores -> fdrop -> PV
     _, α = attention_call(q, k, nothing, bias, mask, nheads; want_out = false, want_weights = true)
@@ -258,7 +267,7 @@ end
 # passing it lets the MFMA kernels run.  A ChainRulesCore.rrule for DeviceArray arguments is three lines
 # on top of this function: call the forward, close over (q, k, v, bias, y), return this pullback.
 function ∇dot_product_attention(dy::DeviceArray{T, 3}, q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::DeviceArray{T, 3},
-                                bias = nothing; y = nothing, dα = nothing, mask = nothing, nheads = 1) where {T <: MIFloat}
+                                bias = nothing; y = nothing, dα = nothing, mask = nothing, nheads = 1, stats = nothing) where {T <: MIFloat}
     E, Lq, B = size(q); Lkv = size(k, 2); Ev = size(v, 1)
     size(dy) == (Ev, Lq, B) || throw(DimensionMismatch("dy must have the size of the output $((Ev, Lq, B)), got $(size(dy))"))
     causal, mptr, mstr, bptr, bstr = mask_and_bias(T, bias, mask, (Lkv, Lq, nheads, B))
@@ -266,13 +275,13 @@ function ∇dot_product_attention(dy::DeviceArray{T, 3}, q::DeviceArray{T, 3}, k
     dbias = bias === nothing ? nothing : DeviceArray{Float32}(undef, size(bias)...)
     dbias === nothing || check(ccall((:mi_fill_zero, libmi), Int32, (Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), dbias.ptr, sizeof(Float32) * length(dbias), C_NULL))
     fwd = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0), E, Ev, Lq, Lkv, nheads, B,
-                   q.ptr, k.ptr, v.ptr, y === nothing ? C_NULL : y.ptr, C_NULL, bptr, bstr, mptr, mstr, C_NULL, 0, 0f0, UInt32(0), UInt64(0))
+                   q.ptr, k.ptr, v.ptr, y === nothing ? C_NULL : y.ptr, C_NULL, bptr, bstr, mptr, mstr, C_NULL, 0, 0f0, UInt32(0), UInt64(0), stats === nothing ? C_NULL : stats.ptr)
     mk(ws, wsbytes) = AttnBwdDesc(Int32(sizeof(AttnBwdDesc)), Int32(0), fwd, dy.ptr, dα === nothing ? C_NULL : dα.ptr, dq.ptr, dk.ptr,
                                   dv.ptr, dbias === nothing ? C_NULL : dbias.ptr, ws, wsbytes)
     need = Ref{Csize_t}(0)
     check(ccall((:mi_attention_bwd_plan, libmi), Int32, (Ref{AttnBwdDesc}, Ptr{Int32}, Ptr{Csize_t}), mk(C_NULL, 0), C_NULL, need))
     ws = need[] > 0 ? DeviceArray{UInt8}(undef, Int(need[])) : nothing
-    GC.@preserve dy q k v bias mask y dα dq dk dv dbias ws begin
+    GC.@preserve dy q k v bias mask y dα dq dk dv dbias ws stats begin
         check(ccall((:mi_attention_bwd, libmi), Int32, (Ref{AttnBwdDesc}, Ptr{Cvoid}), mk(ws === nothing ? C_NULL : ws.ptr, need[]), C_NULL))
     end
     dq, dk, dv, dbias

@@ -30,6 +30,7 @@ class mi_attn_desc(ctypes.Structure):
         ("mask", c_vp), ("mask_strides", c_i64 * 4),
         ("workspace", c_vp), ("workspace_bytes", c_sz),
         ("dropout_p", c_f32), ("reserved2", ctypes.c_uint32), ("dropout_seed", c_u64),
+        ("stats", c_vp),
     ]
 
 
@@ -66,6 +67,7 @@ SIGNATURES = {
     "mi_attention_plan": (c_i32, [ctypes.POINTER(mi_attn_desc), ctypes.POINTER(c_i32), ctypes.POINTER(c_sz)]),
     "mi_attention_workspace_size": (c_i32, [ctypes.POINTER(mi_attn_desc), ctypes.POINTER(c_sz)]),
     "mi_attention_fwd": (c_i32, [ctypes.POINTER(mi_attn_desc), c_vp]),
+    "mi_attention_stats_size": (c_i32, [ctypes.POINTER(mi_attn_desc), ctypes.POINTER(c_sz)]),
     "mi_attention_bwd_plan": (c_i32, [ctypes.POINTER(mi_attn_bwd_desc), ctypes.POINTER(c_i32), ctypes.POINTER(c_sz)]),
     "mi_attention_bwd": (c_i32, [ctypes.POINTER(mi_attn_bwd_desc), c_vp]),
     "mi_make_causal_mask": (c_i32, [c_vp, c_i64, c_vp]),

@@ -122,7 +122,7 @@ def _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags, fdrop=None):
 
 
 def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_weights, weights_dtype, flags,
-                    fdrop=None):
+                    fdrop=None, save_stats=False):
     """One mi_attention_fwd call on flattened (F, L, B) operands."""
     global _last_kernel
     lib = _lib.load()
@@ -136,11 +136,21 @@ def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_we
     d.weights_dtype = alpha.code if alpha is not None else q.code
     kernel, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
     _lib.check(lib.mi_attention_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))
+    stats = None
+    if save_stats and out is not None and kernel.value == _lib.KERNEL_FLASH16 and fdrop is None:
+        # softmax row statistics for dot_product_attention_grad (what an AD rule keeps for its pullback)
+        nb = ctypes.c_size_t(0)
+        _lib.check(lib.mi_attention_stats_size(ctypes.byref(d), ctypes.byref(nb)))
+        stats = DeviceArray.empty((nb.value // 4,), "f32")
+        d.stats = stats.ptr
+        _lib.check(lib.mi_attention_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))   # saving them rules out split-kv
     wbuf, wsize = _get_workspace(ws.value)
     if wbuf is not None:
         d.workspace, d.workspace_bytes = wbuf.data_ptr(), wsize
     _lib.check(lib.mi_attention_fwd(ctypes.byref(d), _stream()))
     _last_kernel = kernel.value
+    if stats is not None:
+        out.saved_stats = stats
     return out, alpha
 
 
@@ -177,18 +187,20 @@ def _check_qkv(q, k, v, nheads):
 
 
 def dot_product_attention(q, k, v, bias=None, *, fdrop=identity, mask=None, nheads=1, return_weights=True,
-                          weights_dtype=None, _flags=0):
+                          weights_dtype=None, save_for_backward=False, _flags=0):
     """dot_product_attention(query, key, value, [bias]; [fdrop, mask, nheads])  (src/attention.jl:40-84).
 
     q (qk_dim, q_len, batch...), k (qk_dim, kv_len, batch...), v (v_dim, kv_len, batch...).
     Returns ``(x, alpha)``: x (v_dim, q_len, batch...), alpha (kv_len, q_len, nheads, batch...).
 
     Beyond the reference: ``return_weights=False`` skips materialising alpha (``None`` is returned
-    in its place) and ``weights_dtype="f32"`` asks for Float32 weights from 16-bit inputs."""
+    in its place), ``weights_dtype="f32"`` asks for Float32 weights from 16-bit inputs, and
+    ``save_for_backward=True`` keeps the softmax row statistics on the returned ``x`` (attribute
+    ``saved_stats``) so that ``dot_product_attention_grad(..., y=x)`` need not recompute them."""
     B, E, Ev, Lq, Lkv, bq = _check_qkv(q, k, v, nheads)
     if fdrop is identity or isinstance(fdrop, Dropout):
         x, alpha = _attention_call(q, k, v, bias, mask, nheads, B, E, Ev, Lq, Lkv, True, return_weights,
-                                   weights_dtype, _flags, fdrop if isinstance(fdrop, Dropout) else None)
+                                   weights_dtype, _flags, fdrop if isinstance(fdrop, Dropout) else None, save_for_backward)
     else:
         # alpha handed back is post-fdrop (src/attention.jl:126); the value product then runs as a
         # batched GEMM on the caller-visible weights, as src/attention.jl:96-98 does.
@@ -196,7 +208,10 @@ def dot_product_attention(q, k, v, bias=None, *, fdrop=identity, mask=None, nhea
                                    _flags)
         alpha = fdrop(alpha)
         x = _weights_times_values(alpha, v, nheads, B, Ev, Lq, Lkv)
+    stats = getattr(x, "saved_stats", None)
     x = x.reshape((Ev, Lq) + tuple(bq))
+    if stats is not None:
+        x.saved_stats = stats
     if alpha is not None:
         alpha = alpha.reshape((Lkv, Lq, nheads) + tuple(bq))
     return x, alpha
@@ -231,6 +246,8 @@ def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, m
         if y.dims != dy.dims or y.dtype != q.dtype:
             raise DimensionMismatch("y must have the size and element type of dy")
         d.fwd.out = y.ptr
+        if getattr(y, "saved_stats", None) is not None and dalpha is None and bias is None:
+            d.fwd.stats = y.saved_stats.ptr
     d.dout = dy.ptr
     if dalpha is not None:
         dalpha = _contig(dalpha, "dalpha")

@@ -32,8 +32,8 @@ def test_header_symbols_are_exported_and_bound(L):
 
 
 def test_struct_layout_matches_header(L):
-    # 6 x int32, 6 x int64, 6 pointers, 4 + 4 strides, workspace pointer + size, dropout (float, pad, u64)
-    assert ctypes.sizeof(L.mi_attn_desc) == 6 * 4 + 6 * 8 + 5 * 8 + 8 + 32 + 8 + 32 + 8 + 8 + 16
+    # 6 x int32, 6 x int64, 6 pointers, 4 + 4 strides, workspace pointer + size, dropout (float, pad, u64), stats
+    assert ctypes.sizeof(L.mi_attn_desc) == 6 * 4 + 6 * 8 + 5 * 8 + 8 + 32 + 8 + 32 + 8 + 8 + 16 + 8
     assert ctypes.sizeof(L.mi_attn_bwd_desc) == 8 + ctypes.sizeof(L.mi_attn_desc) + 8 * 8
     assert L.load().mi_version() == 100
 

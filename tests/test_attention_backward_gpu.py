@@ -136,6 +136,28 @@ def test_mfma_kernels_with_bias_input_but_no_bias_gradient(nn, oracle):
         assert rel_err(g.to_numpy(), r_) <= 1e-2
 
 
+@pytest.mark.parametrize("dtype,D,H,L,Lkv,causal", [("bf16", 128, 2, 300, 300, True), ("bf16", 128, 1, 513, 200, False),
+                                                    ("f16", 64, 2, 130, 130, True), ("f16", 64, 2, 64, 2500, False)])
+def test_statistics_saved_by_the_forward_call(nn, oracle, dtype, D, H, L, Lkv, causal):
+    """save_for_backward keeps the softmax row statistics of the forward call (both 16-bit forward
+    kernels write them); the gradient then skips its own statistics pass and must not change."""
+    rng = np.random.default_rng(L + Lkv)
+    E, B = D * H, 2
+    q, k, v, dy = (round_to(rng.standard_normal(s) * 0.5, dtype) for s in ((E, L, B), (E, Lkv, B), (E, Lkv, B), (E, L, B)))
+    Dv = nn.DeviceArray.from_numpy
+    dq_, dk_, dv_, ddy = Dv(q, dtype), Dv(k, dtype), Dv(v, dtype), Dv(dy, dtype)
+    mask = nn.make_causal_mask(dq_) if causal else None
+    y, _ = nn.dot_product_attention(dq_, dk_, dv_, mask=mask, nheads=H, return_weights=False, save_for_backward=True)
+    assert y.saved_stats is not None
+    y_plain, _ = nn.dot_product_attention(dq_, dk_, dv_, mask=mask, nheads=H, return_weights=False)
+    assert rel_err(y.to_numpy(), y_plain.to_numpy()) < 1e-2          # (the saving call never splits the key range)
+    with_stats = nn.dot_product_attention_grad(ddy, dq_, dk_, dv_, y=y, mask=mask, nheads=H)
+    assert nn.last_attention_bwd_kernel() == "flash16"
+    ref = oracle.attention_bwd_f64(q, k, v, dy, None, oracle.make_causal_mask(L) if causal else None, H)
+    for g, r_ in zip(with_stats[:3], ref[:3]):
+        assert np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05) <= 1e-2
+
+
 def test_mfma_and_generic_kernels_agree(nn):
     """Same call through both kernel families (the generic one forced by flag)."""
     rng = np.random.default_rng(9)
