@@ -18,6 +18,8 @@ bool attention_bwd_flash16_supports(const AttnBwdParams &bp) {
     if (!p.out || bp.dweights || bp.dbias) return false;
     if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.out) || !aligned16(bp.dout)) return false;
     if ((bp.dq && !aligned16(bp.dq)) || (bp.dk && !aligned16(bp.dk)) || (bp.dv && !aligned16(bp.dv))) return false;
+    // tiles are fetched with 32-bit byte offsets from the (batch, head) slice
+    if (p.Lq * p.E * 2 >= 2147483647LL || p.Lkv * p.E * 2 >= 2147483647LL) return false;
     const int64_t tiles = (p.Lq + 127) / 128 > (p.Lkv + 127) / 128 ? (p.Lq + 127) / 128 : (p.Lkv + 127) / 128;
     return tiles * p.H * p.B <= 2147483647LL;
 }
