@@ -234,6 +234,9 @@ EXTRA = {
     "bwd": "gradient of C3: causal bf16 (4096,4096,2) H=32 D=128, dq + dk + dv from dy and the forward result",
     "logsoftmax": "logsoftmax(x; dims=1), x (4096, 65536) f32 (1 GiB in, 1 GiB out)",
     "softmax_dims2": "softmax(x; dims=2), x (256, 4096, 128) bf16 (256 MiB in, 256 MiB out), reduction over the strided dim",
+    "softmax": "softmax(x; dims=1), x (1024, 131072) f32: the logits of C2 (512 MiB in, 512 MiB out)",
+    "batched_mul": "batched_mul(A, B), A (2048, 2048, 16), B (2048, 2048, 16) bf16",
+    "batched_mul_f32": "batched_mul(A, B), A (1024, 64, 128), B (64, 1024, 128) f32: the score product of C2",
 }
 
 
@@ -302,12 +305,40 @@ def measure_extra(key, steps, warmup, with_cpu):
             line["cpu_baseline"] = dict(value=flops / (dt * H * B) / 1e12, unit="TFLOP/s", cores=1, kind="port",
                                         sample=f"1 of {H * B} (head, batch) slices, forward + gradient oracle in Float64 on one thread "
                                                f"({dt:.1f} s), scaled by {H * B}x")
+    elif key.startswith("batched_mul"):
+        if key == "batched_mul":
+            dt_name, (m, kk, n, nb) = "bf16", (2048, 2048, 2048, 16)
+        else:
+            dt_name, (m, kk, n, nb) = "f32", (1024, 64, 1024, 128)
+        A, Bm = DA.empty((m, kk, nb), dt_name), DA.empty((kk, n, nb), dt_name)
+        C = DA.empty((m, n, nb), dt_name)
+        for sid, a in enumerate((A, Bm)):
+            _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, 11, sid, 1.0, None))
+        ms = _event_time(lib, _lib, lambda: nn.batched_mul_(C, A, Bm), steps, warmup)
+        flops = 2 * m * n * kk * nb
+        val = flops / (ms * 1e-3) / 1e12
+        line = dict(metric="batched_mul TFLOP/s", value=val, unit="TFLOP/s", dtype=dt_name,
+                    roofline=dict(bound="mfma", achieved=val, peak=PEAK[dt_name], unit="TFLOP/s", frac=val / PEAK[dt_name], traffic=None),
+                    config=dict(workload=EXTRA[key], kernel="batched_gemm_kernel"), flops_per_step=flops)
+        if with_cpu:
+            from oracle import oracle as O
+            ns = min(nb, 2 if key == "batched_mul" else 32)
+            rng = np.random.default_rng(0)
+            Ah = np.asfortranarray(rng.standard_normal((m, kk, ns), dtype=np.float32))
+            Bh = np.asfortranarray(rng.standard_normal((kk, n, ns), dtype=np.float32))
+            t0 = time.perf_counter()
+            O.batched_gemm(Ah, Bh, nthreads=cores)
+            dt = time.perf_counter() - t0
+            line["cpu_baseline"] = dict(value=2 * m * n * kk * ns / dt / 1e12, unit="TFLOP/s", cores=min(cores, ns), kind="port",
+                                        sample=f"{ns} of {nb} slices in Float32, one thread per slice as src/gemm.jl:121-123 ({dt:.1f} s)")
     else:
         if key == "logsoftmax":
             dims, dt_name, shape, op = 1, "f32", (4096, 65536), _lib.MI_LOGSOFTMAX
+        elif key == "softmax":
+            dims, dt_name, shape, op = 1, "f32", (1024, 131072), _lib.MI_SOFTMAX
         else:
             dims, dt_name, shape, op = 2, "bf16", (256, 4096, 128), _lib.MI_SOFTMAX
-        nsets = 2 if key == "logsoftmax" else 4          # rotate past the 256 MiB last-level cache
+        nsets = 2 if key in ("logsoftmax", "softmax") else 4          # rotate past the 256 MiB last-level cache
         xs = [DA.empty(shape, dt_name) for _ in range(nsets)]
         ys = [DA.empty(shape, dt_name) for _ in range(nsets)]
         for x in xs:
@@ -323,7 +354,8 @@ def measure_extra(key, steps, warmup, with_cpu):
         val = nbytes / (ms * 1e-3) / 1e9
         line = dict(metric=f"{key} GB/s", value=val, unit="GB/s", dtype=dt_name,
                     roofline=dict(bound="hbm", achieved=val, peak=HBM_PEAK, unit="GB/s", frac=val / HBM_PEAK, traffic=None),
-                    config=dict(workload=EXTRA[key], kernel="softmax_nd_kernel"), bytes_per_step=nbytes)
+                    config=dict(workload=EXTRA[key], kernel="softmax_dim1_kernel" if key == "softmax" else "softmax_nd_kernel"),
+                    bytes_per_step=nbytes)
         if with_cpu:
             from oracle import oracle as O
             small = (shape[0], shape[1] // 16) + shape[2:]
