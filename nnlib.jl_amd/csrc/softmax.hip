@@ -110,9 +110,90 @@ __global__ __launch_bounds__(256) void softmax_dim1_wave_kernel(const typename T
     }
 }
 
+// Columns of up to 64 * NCH * VEC elements whose rows can be moved in 16-byte pieces: one wavefront per
+// column, NCH pieces per lane held in registers, reductions by wavefront shuffles only (no LDS, no
+// barrier): one read and one write per element with four columns in flight per workgroup.
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void softmax_dim1_wave_vec_kernel(const typename T::type *x, typename T::type *y,
+                                                                     int64_t rows, int64_t cols) {
+    typedef typename T::type t;
+    constexpr int VEC = 16 / (int)sizeof(t);
+    const int lane = threadIdx.x & 63;
+    const int64_t nchunks = rows / VEC;
+    int64_t c = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t cstride = (int64_t)gridDim.x * 4;
+    for (; c < cols; c += cstride) {
+        const t *xc = x + c * rows;
+        t *yc = y + c * rows;
+        float v[NCH][VEC];
+        float m = MI_NEG_INF;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int64_t ch = lane + 64 * i;
+            if (ch < nchunks) {
+                const u32x4_t raw = *(const u32x4_t *)(xc + ch * VEC);
+                if constexpr (VEC == 4) {
+                    const floatx4_t f = __builtin_bit_cast(floatx4_t, raw);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) v[i][e] = f[e];
+                } else {
+                    const typename T::vec8 h = __builtin_bit_cast(typename T::vec8, raw);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) v[i][e] = T::to_f32(h[e]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) v[i][e] = MI_NEG_INF;
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; e++) m = fmaxf(m, v[i][e]);
+        }
+        m = mi_wave_max(m);
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NCH; i++)
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                // padding lanes hold -Inf: their term is 0 unless the whole column is -Inf (then NaN, as for real entries)
+                v[i][e] = (lane + 64 * i < nchunks) ? softmax_term(v[i][e], m) : 0.0f;
+                s += v[i][e];
+            }
+        s = mi_wave_sum(s);
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int64_t ch = lane + 64 * i;
+            if (ch < nchunks) {
+                if constexpr (VEC == 4) {
+                    floatx4_t f;
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) f[e] = v[i][e] / s;
+                    *(floatx4_t *)(yc + ch * VEC) = f;
+                } else {
+                    typename T::vec8 h;
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) h[e] = T::from_f32(v[i][e] / s);
+                    *(u32x4_t *)(yc + ch * VEC) = __builtin_bit_cast(u32x4_t, h);
+                }
+            }
+        }
+    }
+}
+
 template <typename T>
 static void launch_softmax(const void *x, void *y, int64_t rows, int64_t cols, hipStream_t st) {
     typedef typename T::type t;
+    constexpr int VEC = 16 / (int)sizeof(t);
+    const bool vec_ok = rows % VEC == 0 && ((((uintptr_t)x) | ((uintptr_t)y)) & 15) == 0;
+    if (vec_ok && rows > 256 && rows <= 64 * 8 * VEC) {
+        int64_t blocks = (cols + 3) / 4;
+        if (blocks > 262144) blocks = 262144;
+        const dim3 g((unsigned)blocks), b(256);
+        const int64_t nch = (rows / VEC + 63) / 64;
+        if (nch <= 2) hipLaunchKernelGGL((softmax_dim1_wave_vec_kernel<T, 2>), g, b, 0, st, (const t *)x, (t *)y, rows, cols);
+        else if (nch <= 4) hipLaunchKernelGGL((softmax_dim1_wave_vec_kernel<T, 4>), g, b, 0, st, (const t *)x, (t *)y, rows, cols);
+        else hipLaunchKernelGGL((softmax_dim1_wave_vec_kernel<T, 8>), g, b, 0, st, (const t *)x, (t *)y, rows, cols);
+        return;
+    }
     if (rows <= 256) {
         int64_t blocks = (cols + 3) / 4;
         if (blocks > 65536) blocks = 65536;
