@@ -15,6 +15,13 @@ int32_t launch_batched_gemm16(int32_t dtype, int transA, int transB, int64_t m, 
                               int64_t lda, int64_t sA, const void *B, int64_t ldb, int64_t sB, float beta, void *C, int64_t ldc,
                               int64_t sC, int64_t batch, hipStream_t st);
 
+// tiled Float32 fast path (batched_gemm32.hip)
+bool batched_gemm32_supports(int32_t dtype, int transA, int transB, int64_t m, int64_t n, int64_t k, const void *A, int64_t lda,
+                             int64_t sA, const void *B, int64_t ldb, int64_t sB);
+int32_t launch_batched_gemm32(int transA, int transB, int64_t m, int64_t n, int64_t k, float alpha, const void *A, int64_t lda,
+                              int64_t sA, const void *B, int64_t ldb, int64_t sB, float beta, void *C, int64_t ldc, int64_t sC,
+                              int64_t batch, hipStream_t st);
+
 namespace {
 
 constexpr int TM = 64, TN = 64;
@@ -221,6 +228,8 @@ MI_API int32_t mi_batched_gemm(int32_t dtype, char transA, char transB, int64_t 
     hipStream_t st = (hipStream_t)s;
     if (batched_gemm16_supports(dtype, ta, tb, m, n, k, A, lda, strideA, B, ldb, strideB))
         return launch_batched_gemm16(dtype, ta, tb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, st);
+    if (batched_gemm32_supports(dtype, ta, tb, m, n, k, A, lda, strideA, B, ldb, strideB))
+        return launch_batched_gemm32(ta, tb, m, n, k, alpha, A, lda, strideA, B, ldb, strideB, beta, C, ldc, strideC, batch, st);
     if (dtype == MI_F32) return launch<F32>(g, batch, st);
     if (dtype == MI_F16) return launch<F16>(g, batch, st);
     return launch<BF16>(g, batch, st);

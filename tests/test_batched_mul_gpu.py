@@ -187,12 +187,13 @@ def test_batched_vec_nd(nn):
 
 # ---- the tiled 16-bit kernel ---------------------------------------------------------------------------
 
-@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("dtype", ["bf16", "f16", "f32"])
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
-@pytest.mark.parametrize("m,n,k,nb", [(128, 128, 64, 2), (136, 200, 72, 3), (64, 264, 8, 1), (320, 72, 200, 2)])
+@pytest.mark.parametrize("m,n,k,nb", [(128, 128, 64, 2), (136, 200, 72, 3), (64, 264, 8, 1), (320, 72, 200, 2), (68, 132, 36, 2)])
 def test_tiled_kernel_all_layouts(nn, dtype, ta, tb, m, n, k, nb):
-    """Every N/T combination (lazy batched_transpose views), sizes that are multiples of 8 but not of the
-    128 x 128 x 64 tile, against the per-slice product in Float64 (test/batchedmul.jl:6-28)."""
+    """Every N/T combination (lazy batched_transpose views), sizes that are multiples of 8 (of 4 in the last
+    case: Float32 takes the tiled kernel, 16-bit types the small-tile one) but not of the 128 x 128 tile,
+    against the per-slice product in Float64 (test/batchedmul.jl:6-28)."""
     rng = np.random.default_rng(m + n + k)
     A = round_to(rng.standard_normal((k, m, nb) if ta else (m, k, nb)), dtype)
     B = round_to(rng.standard_normal((n, k, nb) if tb else (k, n, nb)), dtype)
@@ -203,18 +204,19 @@ def test_tiled_kernel_all_layouts(nn, dtype, ta, tb, m, n, k, nb):
     assert close(got, bmm(A, B, ta, tb), dtype)
 
 
-def test_tiled_kernel_alpha_beta_and_shared_operand(nn):
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_tiled_kernel_alpha_beta_and_shared_operand(nn, dtype):
     """test/ext_amdgpu/batched_mul.jl:15-19 (C .= pi; batched_mul!(C, A, B, 2, 3)) and the batch-1 operand of
     test/batchedmul.jl:104-106 at a size the tiled kernel takes."""
     rng = np.random.default_rng(5)
-    A = round_to(rng.standard_normal((192, 96, 4)), "bf16")
-    B = round_to(rng.standard_normal((96, 160, 1)), "bf16")
-    dA, dB = nn.DeviceArray.from_numpy(A, "bf16"), nn.DeviceArray.from_numpy(B, "bf16")
-    C0 = round_to(np.full((192, 160, 4), np.pi), "bf16")
-    dC = nn.DeviceArray.from_numpy(C0, "bf16")
+    A = round_to(rng.standard_normal((192, 96, 4)), dtype)
+    B = round_to(rng.standard_normal((96, 160, 1)), dtype)
+    dA, dB = nn.DeviceArray.from_numpy(A, dtype), nn.DeviceArray.from_numpy(B, dtype)
+    C0 = round_to(np.full((192, 160, 4), np.pi), dtype)
+    dC = nn.DeviceArray.from_numpy(C0, dtype)
     nn.batched_mul_(dC, dA, dB, 2.0, 3.0)
-    assert close(dC.to_numpy(), 2 * bmm(A, B) + 3 * C0, "bf16")
+    assert close(dC.to_numpy(), 2 * bmm(A, B) + 3 * C0, dtype)
     # beta = 0 overwrites NaN (BLAS semantics)
     dC.storage.fill_(float("nan"))
     nn.batched_mul_(dC, dA, dB)
-    assert close(dC.to_numpy(), bmm(A, B), "bf16")
+    assert close(dC.to_numpy(), bmm(A, B), dtype)
