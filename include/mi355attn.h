@@ -148,9 +148,10 @@ typedef struct mi_attn_desc {
     uint64_t dropout_seed;
     /* Optional: softmax row statistics saved for mi_attention_bwd (what an AD rule keeps between the
      * forward and the backward call).  NULL, or a buffer of mi_attention_stats_size() bytes, 16-byte
-     * aligned.  Written only by calls that mi_attention_plan() reports as MI_ATTN_KERNEL_FLASH16 (such
-     * calls then do not split the key range); other kernels leave it untouched.  Contents are private
-     * to the library.  In mi_attn_bwd_desc.fwd: pass the buffer a FLASH16 forward call of the same
+     * aligned.  Written only by calls that mi_attention_plan() reports as MI_ATTN_KERNEL_FLASH16 or
+     * MI_ATTN_KERNEL_FLASH32 (such calls then do not split the key range); other kernels leave it
+     * untouched.  Contents are private
+     * to the library.  In mi_attn_bwd_desc.fwd: pass the buffer such a forward call of the same
      * arguments filled (the backward call also writes into it), or NULL to have the statistics
      * recomputed. */
     float *stats;
@@ -171,8 +172,8 @@ int32_t mi_attention_stats_size(const mi_attn_desc *desc, size_t *bytes);
  * way the reference checks its gradients (test/attention.jl:70-76: against finite differences).
  *
  *   fwd      : the forward call (dtype, sizes, q, k, v, bias, mask, causal, flags).  fwd.out may
- *              hold the forward RESULT x; the MFMA kernels need it and the call falls back to the
- *              generic kernels without it.  fwd.weights and fwd.workspace are ignored.
+ *              hold the forward RESULT x; the MFMA kernels (all three dtypes, head dim 64 or 128)
+ *              need it and the call falls back to the generic kernels without it.  fwd.weights and fwd.workspace are ignored.
  *   dout     : (Ev, Lq, B) cotangent of x, `dtype`.
  *   dweights : NULL, or (Lkv, Lq, H, B) cotangent of the returned weights, `dtype`.
  *   dq, dk, dv : gradients with the shapes of q, k, v, `dtype`; any may be NULL (not computed).

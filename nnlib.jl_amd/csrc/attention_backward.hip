@@ -33,6 +33,10 @@ static int32_t choose_bwd(const mi_attn_bwd_desc *d, const AttnBwdParams &bp, si
         *ws = bp.have_stats ? 0 : attention_bwd_flash16_workspace(bp.p);
         return MI_ATTN_KERNEL_FLASH16;
     }
+    if (!(d->fwd.flags & MI_ATTN_FORCE_GENERIC) && attention_bwd_flash32_supports(bp)) {
+        *ws = bp.have_stats ? 0 : attention_stats_bytes(bp.p);
+        return MI_ATTN_KERNEL_FLASH32;
+    }
     if (bp.have_stats) {   // the generic kernels keep their own statistics, in their own layout
         *ws = attention_bwd_generic_workspace(bp.p);
         return MI_ATTN_KERNEL_GENERIC;
@@ -73,6 +77,7 @@ MI_API int32_t mi_attention_bwd(const mi_attn_bwd_desc *d, mi_stream s) {
                             d->workspace ? d->workspace_bytes : (size_t)0);
     if ((((uintptr_t)d->workspace) & 15) != 0) return mi_set_error(MI_EWORKSPACE, "mi_attention_bwd: workspace must be 16-byte aligned");
     if (kernel == MI_ATTN_KERNEL_FLASH16) return launch_attention_bwd_flash16(bp, st);
+    if (kernel == MI_ATTN_KERNEL_FLASH32) return launch_attention_bwd_flash32(bp, st);
     bp.stats = (float *)d->workspace;
     bp.have_stats = 0;
     return launch_attention_bwd_generic(bp, st);

@@ -1,0 +1,458 @@
+// Attention backward for Float32 inputs on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), head dim 64
+// or 128.  Same decomposition as the 16-bit kernels in attention_backward_flash16.inc (the chain AD
+// builds from src/attention.jl:86-127 through the rrule of batched_mul, src/batched/batchedmul.jl:96-110,
+// and _∇softmax!, src/softmax.jl:107-110):
+//
+//   kernel 1 (query tile stationary): row statistics (saved by the forward call, or a first pass over
+//            the keys), then dQ^T += K^T dS^T; statistics and delta go to the workspace
+//   kernel 2 (key tile stationary): S = Q K^T, dP = dO V^T against streamed query tiles,
+//            dV^T += dO^T P, dK^T += Q^T dS; for head dim 64 without bias / mask arrays it runs as a
+//            dV kernel and a dK kernel at two wavefronts per SIMD
+//
+// With one fp32 per register nothing is converted or transposed: the streamed tile is the A operand of
+// the first products through 16-byte LDS reads (contraction index permuted as in attention_flash32.hip:
+// k-step 4c+j of half-wave hh multiplies feature 8c + 4hh + j), the accumulator registers of P / dS are
+// the B operand of the second products as they stand, and the A operand of those is a plain 4-byte read
+// of tile[row][feature = lane].  Products and sums are true fp32.
+#include "flash_common.h"
+
+namespace {
+
+typedef F32 T;
+constexpr int BN = FLASH_BN;   // rows per streamed tile
+
+template <int D>
+struct Cfg {
+    static constexpr int KS = D + 4;                    // tile row stride (floats): conflict-free 16-byte row reads
+    static constexpr int TILEF = BN * KS;               // floats per tile
+    static constexpr int CHUNKS = BN * D / 4 / 256;     // 16-byte chunks per thread, tile and tensor
+    static constexpr int NDV = D / 32;
+    static constexpr size_t SMEM = sizeof(float) * (4 * TILEF + 2 * 3 * BN);   // two tensors + statistics, double buffered
+};
+
+__device__ inline floatx4_t ldg16f(const float *p, bool ok) {
+    const floatx4_t z = {0.f, 0.f, 0.f, 0.f};
+    return ok ? *(const floatx4_t *)p : z;
+}
+
+// Streams [BN][D] tiles of up to two row-major arrays through registers into double-buffered LDS tiles;
+// rows from `nrows` on read as zeros.
+template <int D>
+struct TileStream32 {
+    static constexpr int KS = Cfg<D>::KS, CHUNKS = Cfg<D>::CHUNKS;
+    const float *base1, *base2;   // base2 may be null
+    int64_t stride, nrows;
+    float *s1, *s2;
+    floatx4_t r1[CHUNKS], r2[CHUNKS];
+    __device__ void load(int64_t row0) {
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = threadIdx.x + 256 * u;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            const bool ok = row0 + row < nrows;
+            r1[u] = ldg16f(base1 + stride * (row0 + row) + col, ok);
+            if (base2) r2[u] = ldg16f(base2 + stride * (row0 + row) + col, ok);
+        }
+    }
+    __device__ void store(int buf) {
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = threadIdx.x + 256 * u;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            *(floatx4_t *)(s1 + (buf * BN + row) * KS + col) = r1[u];
+            if (base2) *(floatx4_t *)(s2 + (buf * BN + row) * KS + col) = r2[u];
+        }
+    }
+};
+
+// acc += tile rows [32kb, 32kb+32) (A operand) x stationary rows x (B operand), contraction over D
+template <int D>
+__device__ inline floatx16_t first_product(const float *tile, int kb, const float (&x)[D / 2], floatx16_t acc, int r, int hh) {
+    const float *t = tile + (32 * kb + r) * Cfg<D>::KS + 4 * hh;
+#pragma unroll
+    for (int c = 0; c < D / 8; c++) {
+        const floatx4_t k4 = *(const floatx4_t *)(t + 8 * c);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(k4[j], x[4 * c + j], acc, 0, 0, 0);
+    }
+    return acc;
+}
+
+// out[dvb] += tile^T (features x rows of block kb) x w (rows x stationary): register v of w belongs to tile row
+// 32kb + 8(v/4) + 4hh + v%4, which is also the contraction index the MFMA assigns to this half-wave
+template <int D>
+__device__ inline void second_product(const float *tile, int kb, const floatx16_t &w, floatx16_t (&out)[D / 32], int r, int hh) {
+    const float *t = tile + (32 * kb + 4 * hh) * Cfg<D>::KS + r;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const float *src = t + (8 * (v / 4) + (v % 4)) * Cfg<D>::KS;
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++) out[dvb] = __builtin_amdgcn_mfma_f32_32x32x2f32(src[32 * dvb], w[v], out[dvb], 0, 0, 0);
+    }
+}
+
+// stationary row in the permuted feature order of first_product
+template <int D>
+__device__ inline void load_stationary(float (&x)[D / 2], const float *row, bool ok, int hh) {
+#pragma unroll
+    for (int c = 0; c < D / 8; c++) {
+        const floatx4_t q4 = ldg16f(row + 8 * c + 4 * hh, ok);
+#pragma unroll
+        for (int j = 0; j < 4; j++) x[4 * c + j] = q4[j];
+    }
+}
+
+__device__ inline int64_t lq_pad(int64_t Lq) { return attention_stats_lq_pad(Lq); }
+
+// ---- kernel 1: statistics and dQ --------------------------------------------------------------------
+template <int D, bool CAUSAL, int EXTRAS, bool HAVE_STATS>
+__global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) void bwd32_dq_kernel(FlashArgs a, AttnBwdParams bp) {
+    constexpr int TILEF = Cfg<D>::TILEF, NDV = Cfg<D>::NDV;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
+    float *Ks = (float *)bwd_smem, *Vs = Ks + 2 * TILEF;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t hb = blockIdx.x % HB, qt = a.n_qtiles - 1 - blockIdx.x / HB;
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t i0 = qt * 128, iw = i0 + 32 * wave, qi = iw + r;
+    const bool qok = qi < p.Lq;
+
+    float qx[D / 2], dox[D / 2];
+    float delta = 0.0f;
+    {
+        const int64_t off = p.E * (qi + p.Lq * b) + D * h;   // E == Ev for these kernels
+        load_stationary<D>(qx, (const float *)p.q + off, qok, hh);
+        load_stationary<D>(dox, (const float *)bp.dout + off, qok, hh);
+        float ox[D / 2];
+        load_stationary<D>(ox, (const float *)p.out + off, qok, hh);
+#pragma unroll
+        for (int e = 0; e < D / 2; e++) delta = fmaf(ox[e], dox[e], delta);
+        delta += mi_swap32(delta);
+    }
+
+    int64_t kv_end = p.Lkv;
+    if (CAUSAL && i0 + 128 < kv_end) kv_end = i0 + 128;
+    const int n_tiles = (int)((kv_end + BN - 1) / BN);
+
+    TileStream32<D> ts;
+    ts.base1 = (const float *)p.k + p.E * (p.Lkv * b) + D * h;
+    ts.stride = p.E;
+    ts.nrows = p.Lkv;
+    ts.s1 = Ks;
+    ts.s2 = Vs;
+    floatx16_t unused_o[1][NDV];
+    float fm[1] = {MI_NEG_INF}, fl[1] = {0.0f};
+    const float cs = EXTRAS ? MI_LOG2E : a.c;
+    const int64_t plane = p.B * p.H * lq_pad(p.Lq), at = (b * p.H + h) * lq_pad(p.Lq) + qi;
+    if (HAVE_STATS) {
+        fm[0] = bp.stats[at] / cs;
+        fl[0] = bp.stats[plane + at];
+        if (hh == 0) bp.stats[2 * plane + at] = qok ? delta : 0.0f;
+    }
+
+    // pass 1: row maximum and row sum (K tiles only)
+    ts.base2 = nullptr;
+    if (!HAVE_STATS) {
+        ts.load(0);
+        ts.store(0);
+    }
+    __syncthreads();
+    for (int jt = 0; !HAVE_STATS && jt < n_tiles; jt++) {
+        const int buf = jt & 1;
+        const int64_t j0 = (int64_t)jt * BN;
+        if (jt + 1 < n_tiles) ts.load(j0 + BN);
+        if (!CAUSAL || j0 <= iw + 31) {
+            floatx16_t s[1][2] = {{(floatx16_t){0}, (floatx16_t){0}}};
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) s[0][kb] = first_product<D>(Ks + buf * TILEF, kb, qx, s[0][kb], r, hh);
+            flash_softmax_tile<T, 1, NDV, CAUSAL, EXTRAS, PHASE_STATS, float>(a, s, unused_o, fm, fl, b, h, iw, j0);
+        }
+        if (jt + 1 < n_tiles) ts.store(buf ^ 1);
+        __syncthreads();
+    }
+    if (!HAVE_STATS) {
+        fl[0] = 1.0f / (fl[0] + mi_swap32(fl[0]));   // all keys dropped: 1/0 = Inf, the weights become 0*Inf = NaN
+        if (hh == 0) {
+            // rows past Lq belong to the padding of the last tile: statistics that make their weights zero
+            bp.stats[at] = qok ? fm[0] * cs : 0.0f;
+            bp.stats[plane + at] = qok ? fl[0] : 0.0f;
+            bp.stats[2 * plane + at] = qok ? delta : 0.0f;
+        }
+    }
+    if (!bp.dq) return;
+
+    // pass 2: P, dP = V dO^T, dS = P (dP - delta), dQ^T += K^T dS^T
+    floatx16_t dq[NDV];
+#pragma unroll
+    for (int dvb = 0; dvb < NDV; dvb++) dq[dvb] = (floatx16_t){0};
+    ts.base2 = (const float *)p.v + p.Ev * (p.Lkv * b) + D * h;
+    ts.load(0);
+    __syncthreads();   // pass 1 may still be reading the tiles
+    ts.store(0);
+    __syncthreads();
+    const float m2 = fm[0] * cs, linv = fl[0];
+    for (int jt = 0; jt < n_tiles; jt++) {
+        const int buf = jt & 1;
+        const int64_t j0 = (int64_t)jt * BN;
+        if (jt + 1 < n_tiles) ts.load(j0 + BN);
+        if (!CAUSAL || j0 <= iw + 31) {
+            const float *kt = Ks + buf * TILEF, *vt = Vs + buf * TILEF;
+            if constexpr (EXTRAS == EXTRAS_NONE) {
+                const bool edge = (j0 + BN > p.Lkv) || (CAUSAL && j0 + BN - 1 > iw);
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+                    if (CAUSAL && j0 + 32 * kb > iw + 31) break;   // every key of this block is after every query of the wavefront
+                    floatx16_t sb = first_product<D>(kt, kb, qx, (floatx16_t){0}, r, hh);
+                    const floatx16_t dpb = first_product<D>(vt, kb, dox, (floatx16_t){0}, r, hh);
+                    int64_t lim = BN;
+                    if (edge) {
+                        lim = p.Lkv - j0;
+                        if (CAUSAL && qi - j0 + 1 < lim) lim = qi - j0 + 1;
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const int kvl = 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4);
+                        const float pw = (!edge || kvl < lim) ? mi_exp2(fmaf(sb[v], cs, -m2)) * linv : 0.0f;
+                        sb[v] = pw * (dpb[v] - delta);
+                    }
+                    second_product<D>(kt, kb, sb, dq, r, hh);
+                }
+            } else {
+                floatx16_t s[1][2] = {{(floatx16_t){0}, (floatx16_t){0}}};
+                floatx16_t dp[2];
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+                    s[0][kb] = first_product<D>(kt, kb, qx, s[0][kb], r, hh);
+                    dp[kb] = first_product<D>(vt, kb, dox, (floatx16_t){0}, r, hh);
+                }
+                flash_softmax_tile<T, 1, NDV, CAUSAL, EXTRAS, PHASE_FINAL, float>(a, s, unused_o, fm, fl, b, h, iw, j0);
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) s[0][kb][v] *= dp[kb][v] - delta;
+                    second_product<D>(kt, kb, s[0][kb], dq, r, hh);
+                }
+            }
+        }
+        if (jt + 1 < n_tiles) ts.store(buf ^ 1);
+        __syncthreads();
+    }
+    if (qok) {
+        float *dqrow = (float *)bp.dq + p.E * (qi + p.Lq * b) + D * h;
+#pragma unroll
+        for (int dvb = 0; dvb < NDV; dvb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                floatx4_t o4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o4[e] = dq[dvb][4 * g + e] * a.cn;
+                *(floatx4_t *)(dqrow + 32 * dvb + 8 * g + 4 * hh) = o4;
+            }
+    }
+}
+
+// ---- kernel 2: dK and dV ----------------------------------------------------------------------------
+enum { BWD_DV = 1, BWD_DK = 2 };
+template <int D, bool CAUSAL, int EXTRAS, int WHICH>
+__global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) void bwd32_dkdv_kernel(FlashArgs a, AttnBwdParams bp) {
+    constexpr int TILEF = Cfg<D>::TILEF, NDV = Cfg<D>::NDV;
+    constexpr bool DO_DV = (WHICH & BWD_DV) != 0, DO_DK = (WHICH & BWD_DK) != 0;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
+    float *Qs = (float *)bwd_smem, *dOs = Qs + 2 * TILEF;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t hb = blockIdx.x % HB, kt_idx = blockIdx.x / HB;   // with causal masks the early key tiles are the long ones
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t j0 = kt_idx * 128, jw = j0 + 32 * wave, kv = jw + r;
+    const bool kok = kv < p.Lkv;
+
+    float kx[D / 2], vx[DO_DK ? D / 2 : 1];
+    {
+        const int64_t off = p.E * (kv + p.Lkv * b) + D * h;
+        load_stationary<D>(kx, (const float *)p.k + off, kok, hh);
+        if constexpr (DO_DK) load_stationary<D>(vx, (const float *)p.v + off, kok, hh);
+    }
+    floatx16_t dk[NDV], dv[NDV];
+#pragma unroll
+    for (int dvb = 0; dvb < NDV; dvb++) dk[dvb] = dv[dvb] = (floatx16_t){0};
+
+    const int64_t plane = p.B * p.H * lq_pad(p.Lq);
+    // the row statistics of a query tile travel with it through LDS (48 threads x 4 floats)
+    const float *st_src = bp.stats + (b * p.H + h) * lq_pad(p.Lq) + (int64_t)(tid >> 4) * plane + 4 * (tid & 15);
+    float *st_lds = (float *)bwd_smem + 4 * TILEF;
+    floatx4_t st_reg = {0, 0, 0, 0};
+    const float *bias = (const float *)p.bias;
+    const int64_t boff = kv * p.bias_strides[0] + h * p.bias_strides[2] + b * p.bias_strides[3];
+    const int64_t moff = kv * p.mask_strides[0] + h * p.mask_strides[2] + b * p.mask_strides[3];
+    const float cs = EXTRAS ? MI_LOG2E : a.c;
+
+    TileStream32<D> ts;
+    ts.base1 = (const float *)p.q + p.E * (p.Lq * b) + D * h;
+    ts.base2 = (const float *)bp.dout + p.E * (p.Lq * b) + D * h;
+    ts.stride = p.E;
+    ts.nrows = p.Lq;
+    ts.s1 = Qs;
+    ts.s2 = dOs;
+    const int n_qt = (int)((p.Lq + BN - 1) / BN);
+    const int it0 = CAUSAL ? (int)(j0 / BN) : 0;   // query tiles before the first key of the workgroup see none of its keys
+    if (it0 < n_qt) {
+        ts.load((int64_t)it0 * BN);
+        ts.store(0);
+        if (tid < 48) *(floatx4_t *)(st_lds + 4 * tid) = *(const floatx4_t *)(st_src + (int64_t)it0 * BN);
+    }
+    __syncthreads();
+    for (int it = it0; it < n_qt; it++) {
+        const int buf = (it - it0) & 1;
+        const int64_t i0 = (int64_t)it * BN;
+        if (it + 1 < n_qt) {
+            ts.load(i0 + BN);
+            if (tid < 48) st_reg = *(const floatx4_t *)(st_src + i0 + BN);
+        }
+        if (!CAUSAL || i0 + BN - 1 >= jw) {
+            const float *qt = Qs + buf * TILEF, *dot = dOs + buf * TILEF;
+            const float *st = st_lds + buf * (3 * BN);
+            const bool diag = CAUSAL && i0 < jw + 32;   // some (query, key) pair of this tile has key > query
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                floatx16_t s = first_product<D>(qt, kb, kx, (floatx16_t){0}, r, hh);
+                floatx16_t dp = (floatx16_t){0};
+                if constexpr (DO_DK) dp = first_product<D>(dot, kb, vx, dp, r, hh);
+                // accumulator register 4g+e of this lane: query i0 + 32kb + 8g + 4hh + e, key kv
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int64_t qg = i0 + 32 * kb + 8 * g + 4 * hh;
+                    const int sq = 32 * kb + 8 * g + 4 * hh;
+                    const floatx4_t m4 = *(const floatx4_t *)(st + sq);
+                    const floatx4_t linv4 = *(const floatx4_t *)(st + BN + sq);
+                    floatx4_t delta4 = {0.0f, 0.0f, 0.0f, 0.0f};
+                    if (DO_DK) delta4 = *(const floatx4_t *)(st + 2 * BN + sq);
+                    if constexpr (EXTRAS == EXTRAS_NONE) {
+                        // rows past Lq carry statistics (0, 0, 0): their weights vanish; keys past Lkv only feed
+                        // accumulator columns that are never stored
+                        const int dq_ = (int)(jw - qg) + r;   // key index minus query index of element e = 0
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            float pw = mi_exp2(fmaf(s[4 * g + e], cs, -m4[e])) * linv4[e];
+                            if (diag) pw = dq_ - e > 0 ? 0.0f : pw;
+                            s[4 * g + e] = pw;
+                            if (DO_DK) dp[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
+                        }
+                        continue;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int64_t qi = qg + e;
+                        const bool in = kok && qi < p.Lq;
+                        float x = s[4 * g + e] * a.cn;
+                        if (bias && in) x += bias[boff + qi * p.bias_strides[1]];
+                        if (p.mask && in && !p.mask[moff + qi * p.mask_strides[1]]) x = MI_NEG_INF;
+                        if (diag && kv > qi) x = MI_NEG_INF;
+                        const float m = m4[e];
+                        float pw;
+                        if (m == MI_POS_INF) pw = x == MI_POS_INF ? linv4[e] : 0.0f;   // src/softmax.jl:74-75
+                        else pw = mi_exp2(fmaf(x, cs, m == MI_NEG_INF ? 0.0f : -m)) * linv4[e];
+                        pw = in ? pw : 0.0f;
+                        s[4 * g + e] = pw;
+                        if (DO_DK) dp[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
+                    }
+                }
+                if constexpr (DO_DV) second_product<D>(dot, kb, s, dv, r, hh);
+                if constexpr (DO_DK) second_product<D>(qt, kb, dp, dk, r, hh);
+            }
+        }
+        if (it + 1 < n_qt) {
+            ts.store(buf ^ 1);
+            if (tid < 48) *(floatx4_t *)(st_lds + (buf ^ 1) * (3 * BN) + 4 * tid) = st_reg;
+        }
+        __syncthreads();
+    }
+    if (kok) {
+        const int64_t off = p.E * (kv + p.Lkv * b) + D * h;
+#pragma unroll
+        for (int dvb = 0; dvb < NDV; dvb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                floatx4_t k4, v4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    k4[e] = dk[dvb][4 * g + e] * a.cn;
+                    v4[e] = dv[dvb][4 * g + e];
+                }
+                if (DO_DK && bp.dk) *(floatx4_t *)((float *)bp.dk + off + 32 * dvb + 8 * g + 4 * hh) = k4;
+                if (DO_DV && bp.dv) *(floatx4_t *)((float *)bp.dv + off + 32 * dvb + 8 * g + 4 * hh) = v4;
+            }
+    }
+}
+
+template <int D, bool CAUSAL, int EXTRAS>
+int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
+    const AttnParams &p = a.p;
+    constexpr size_t SMEM = Cfg<D>::SMEM;
+    // Two kernels (dV, then dK) where that buys two wavefronts per SIMD (head dim 64 without bias / mask
+    // arrays) or is needed to fit the register file at all (head dim 128: K, V, dK and dV of a lane are
+    // 256 registers before anything else); one pass otherwise.
+    constexpr bool SPLIT = (EXTRAS == EXTRAS_NONE && D == 64) || D == 128;
+    auto k1 = bp.have_stats ? bwd32_dq_kernel<D, CAUSAL, EXTRAS, true> : bwd32_dq_kernel<D, CAUSAL, EXTRAS, false>;
+    auto k2 = bwd32_dkdv_kernel<D, CAUSAL, EXTRAS, SPLIT ? BWD_DV : 3>;
+    auto k3 = bwd32_dkdv_kernel<D, CAUSAL, EXTRAS, SPLIT ? BWD_DK : 3>;
+    static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B)), dim3(256), SMEM, st, a, bp);
+    MI_LAUNCH_CHECK();
+    const dim3 g2((unsigned)(((p.Lkv + 127) / 128) * p.H * p.B));
+    if (SPLIT) {
+        if (bp.dv) hipLaunchKernelGGL(k2, g2, dim3(256), SMEM, st, a, bp);
+        if (bp.dk) hipLaunchKernelGGL(k3, g2, dim3(256), SMEM, st, a, bp);
+        MI_LAUNCH_CHECK();
+    } else if (bp.dk || bp.dv) {
+        hipLaunchKernelGGL(k2, g2, dim3(256), SMEM, st, a, bp);
+        MI_LAUNCH_CHECK();
+    }
+    return MI_OK;
+}
+
+template <int D>
+int32_t launch_d(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
+    const bool extras = bp.p.bias || bp.p.mask;
+    if (bp.p.causal) return extras ? launch_set<D, true, EXTRAS_DIRECT>(a, bp, st) : launch_set<D, true, EXTRAS_NONE>(a, bp, st);
+    return extras ? launch_set<D, false, EXTRAS_DIRECT>(a, bp, st) : launch_set<D, false, EXTRAS_NONE>(a, bp, st);
+}
+
+}  // namespace
+
+bool attention_bwd_flash32_supports(const AttnBwdParams &bp) {
+    const AttnParams &p = bp.p;
+    if (p.dtype != MI_F32) return false;
+    if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
+    // the kernels need the forward result (for delta), take no weight cotangent and give no bias gradient
+    if (!p.out || bp.dweights || bp.dbias) return false;
+    auto al = [](const void *x) { return (((uintptr_t)x) & 15) == 0; };
+    if (!al(p.q) || !al(p.k) || !al(p.v) || !al(p.out) || !al(bp.dout)) return false;
+    if ((bp.dq && !al(bp.dq)) || (bp.dk && !al(bp.dk)) || (bp.dv && !al(bp.dv))) return false;
+    const int64_t tiles = (p.Lq + 127) / 128 > (p.Lkv + 127) / 128 ? (p.Lq + 127) / 128 : (p.Lkv + 127) / 128;
+    return tiles * p.H * p.B <= 2147483647LL;
+}
+
+int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st) {
+    FlashArgs a;
+    a.p = bp.p;
+    a.p.weights = nullptr;
+    a.p.workspace = nullptr;
+    a.p.stats = nullptr;
+    a.cn = 1.0f / sqrtf((float)bp.p.D);
+    a.c = MI_LOG2E * a.cn;
+    a.n_qtiles = (int32_t)((bp.p.Lq + 127) / 128);
+    a.nsplit = 1;
+    a.tiles_per_split = 0;
+    flash_fill_vec_flags(a);
+    a.bias_lds = a.mask_lds = 0;
+    return bp.p.D == 64 ? launch_d<64>(a, bp, st) : launch_d<128>(a, bp, st);
+}

@@ -191,6 +191,7 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
                 const float l = f.l[qb] + mi_swap32(f.l[qb]);
                 inv = 1.0f / l;
             }
+            if (p.stats && hh == 0) flash_save_stats(p, b, h, qi, f.m[qb] * MI_LOG2E, WEIGHTS ? f.l[qb] : inv);
             if (qi < p.Lq) {
 #pragma unroll
                 for (int dvb = 0; dvb < D / 32; dvb++)

@@ -39,6 +39,8 @@ static inline size_t attention_stats_bytes(const AttnParams &p) {
 int32_t launch_attention_bwd_generic(const AttnBwdParams &bp, hipStream_t st);
 int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp, hipStream_t st);
 bool attention_bwd_flash16_supports(const AttnBwdParams &bp);
+int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st);
+bool attention_bwd_flash32_supports(const AttnBwdParams &bp);
 size_t attention_bwd_flash16_workspace(const AttnParams &p);
 size_t attention_bwd_generic_workspace(const AttnParams &p);
 int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_backward = false);

@@ -137,7 +137,7 @@ def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_we
     kernel, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
     _lib.check(lib.mi_attention_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))
     stats = None
-    if save_stats and out is not None and kernel.value == _lib.KERNEL_FLASH16 and fdrop is None:
+    if save_stats and out is not None and kernel.value in (_lib.KERNEL_FLASH16, _lib.KERNEL_FLASH32) and fdrop is None:
         # softmax row statistics for dot_product_attention_grad (what an AD rule keeps for its pullback)
         nb = ctypes.c_size_t(0)
         _lib.check(lib.mi_attention_stats_size(ctypes.byref(d), ctypes.byref(nb)))

@@ -105,6 +105,45 @@ def test_mfma_kernels(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, bias_k
          scale=0.4, expect="flash16" if bias_shape is None else "generic")
 
 
+F32_CASES = [
+    # D, H, Lq, Lkv, batch, mask_kind, saved statistics
+    (64, 2, 200, 200, (2,), "causal", False),
+    (64, 2, 130, 333, (1,), None, True),
+    (64, 1, 96, 160, (2,), "random", False),
+    (128, 2, 257, 257, (1,), "causal", True),
+    (128, 1, 100, 450, (2,), None, False),
+    (128, 1, 70, 130, (1,), "random", False),
+    (64, 3, 1, 300, (2,), None, False),
+]
+
+
+@pytest.mark.parametrize("D,H,Lq,Lkv,batch,mask_kind,saved", F32_CASES)
+def test_f32_mfma_kernels(nn, oracle, D, H, Lq, Lkv, batch, mask_kind, saved):
+    """Float32 inputs with head dim 64 or 128 take the fp32-MFMA gradient kernels (tolerance 1e-4 of the
+    gradient's scale), with and without the statistics saved by the forward call."""
+    rng = np.random.default_rng(D + Lq + Lkv)
+    E = D * H
+    q, k, v, dy = (rng.standard_normal(s).astype(np.float32) * sc for s, sc in
+                   (((E, Lq) + batch, 0.4), ((E, Lkv) + batch, 0.4), ((E, Lkv) + batch, 1.0), ((E, Lq) + batch, 1.0)))
+    Dv = nn.DeviceArray.from_numpy
+    dq_, dk_, dv_, ddy = Dv(q), Dv(k), Dv(v), Dv(dy)
+    mask = dmask = None
+    if mask_kind == "causal":
+        mask, dmask = oracle.make_causal_mask(Lq), nn.make_causal_mask(dq_)
+    elif mask_kind == "random":
+        mask = rng.random((Lkv, Lq)) < 0.8
+        mask[0] = True
+        dmask = Dv(mask)
+    y, _ = nn.dot_product_attention(dq_, dk_, dv_, mask=dmask, nheads=H, return_weights=False, save_for_backward=saved)
+    assert (getattr(y, "saved_stats", None) is not None) == saved
+    got = nn.dot_product_attention_grad(ddy, dq_, dk_, dv_, y=y, mask=dmask, nheads=H)
+    assert nn.last_attention_bwd_kernel() == "flash32"
+    ref = oracle.attention_bwd_f64(q, k, v, dy, None, mask, H)
+    for g, r_, name in zip(got[:3], ref[:3], ("dq", "dk", "dv")):
+        err = np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05)
+        assert err <= 1e-4, (name, err)
+
+
 def test_mfma_kernels_with_bias_input_but_no_bias_gradient(nn, oracle):
     """A bias changes the weights the MFMA kernels recompute; its own gradient needs the generic path, so
     here the bias gradient is not requested (C ABI level: dbias = NULL)."""
