@@ -232,6 +232,7 @@ def measure(key, steps, warmup, with_cpu):
 
 EXTRA = {
     "bwd": "gradient of C3: causal bf16 (4096,4096,2) H=32 D=128, dq + dk + dv from dy and the forward result",
+    "bwd_f32": "gradient of C2: causal f32 (1024,1024,8) H=16 D=64, dq + dk + dv from dy and the forward result",
     "logsoftmax": "logsoftmax(x; dims=1), x (4096, 65536) f32 (1 GiB in, 1 GiB out)",
     "softmax_dims2": "softmax(x; dims=2), x (256, 4096, 128) bf16 (256 MiB in, 256 MiB out), reduction over the strided dim",
     "softmax": "softmax(x; dims=1), x (1024, 131072) f32: the logits of C2 (512 MiB in, 512 MiB out)",
@@ -268,13 +269,14 @@ def measure_extra(key, steps, warmup, with_cpu):
     _lib.check(lib.mi_init(0))
     DA = nn.DeviceArray
     cores = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
-    if key == "bwd":
-        w = WORKLOADS["c3"]
+    if key in ("bwd", "bwd_f32"):
+        w = WORKLOADS["c3" if key == "bwd" else "c2"]
         E, L, B, H = w["E"], w["Lq"], w["B"], w["H"]
         D = E // H
-        arrs = [DA.empty((E, L, B), "bf16") for _ in range(4)]
+        dtn = w["dtype"]
+        arrs = [DA.empty((E, L, B), dtn) for _ in range(4)]
         for sid, a in enumerate(arrs):
-            _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, w["seed"], sid, 1.0, None))
+            _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, w["seed"], sid, w["scale"] if sid < 2 else 1.0, None))
         q, k, v, dy = arrs
         y, _ = nn.dot_product_attention(q, k, v, mask=nn.make_causal_mask(q), nheads=H, return_weights=False,
                                         save_for_backward=True)   # as an AD rule would: the pullback reuses the row statistics
@@ -282,7 +284,7 @@ def measure_extra(key, steps, warmup, with_cpu):
         d.struct_size = ctypes.sizeof(_lib.mi_attn_bwd_desc)
         nn.ops._fill_desc(d.fwd, q, k, v, None, nn.make_causal_mask(q), H, B, E, E, L, L, 0)
         d.fwd.out, d.dout, d.fwd.stats = y.ptr, dy.ptr, y.saved_stats.ptr
-        grads = [DA.empty((E, L, B), "bf16") for _ in range(3)]
+        grads = [DA.empty((E, L, B), dtn) for _ in range(3)]
         d.dq, d.dk, d.dv = (g.ptr for g in grads)
         kern, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
         _lib.check(lib.mi_attention_bwd_plan(ctypes.byref(d), ctypes.byref(kern), ctypes.byref(ws)))
@@ -292,19 +294,20 @@ def measure_extra(key, steps, warmup, with_cpu):
         # five products (S, dP, dV, dK, dQ) of 2*D FLOP per unmasked (query, key) pair
         flops = 10 * D * H * B * (L * (L + 1) // 2)
         val = flops / (ms * 1e-3) / 1e12
-        line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype="bf16",
-                    roofline=dict(bound="mfma", achieved=val, peak=PEAK["bf16"], unit="TFLOP/s", frac=val / PEAK["bf16"], traffic=None),
+        line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype=dtn,
+                    roofline=dict(bound="mfma", achieved=val, peak=PEAK[dtn], unit="TFLOP/s", frac=val / PEAK[dtn], traffic=None),
                     config=dict(workload=EXTRA[key], kernel=_lib.KERNEL_NAMES[kern.value]), flops_per_step=flops)
         if with_cpu:
             from oracle import oracle as O
             rng = np.random.default_rng(0)
-            a1 = [np.asfortranarray(rng.standard_normal((D, L, 1))) for _ in range(4)]
+            nh, nb = (4, 1) if key == "bwd" else (H, 2)          # a bounded sample of whole (head, batch) slices
+            a1 = [np.asfortranarray(rng.standard_normal((nh * D, L, nb))) for _ in range(4)]
             t0 = time.perf_counter()
-            O.attention_bwd_f64(a1[0], a1[1], a1[2], a1[3], None, O.make_causal_mask(L), 1)
+            O.attention_bwd_f64(a1[0], a1[1], a1[2], a1[3], None, O.make_causal_mask(L), nh)
             dt = time.perf_counter() - t0
-            line["cpu_baseline"] = dict(value=flops / (dt * H * B) / 1e12, unit="TFLOP/s", cores=1, kind="port",
-                                        sample=f"1 of {H * B} (head, batch) slices, forward + gradient oracle in Float64 on one thread "
-                                               f"({dt:.1f} s), scaled by {H * B}x")
+            line["cpu_baseline"] = dict(value=flops * nh * nb / (dt * H * B) / 1e12, unit="TFLOP/s", cores=1, kind="port",
+                                        sample=f"{nh * nb} of {H * B} (head, batch) slices, forward + gradient oracle in Float64 on one "
+                                               f"thread ({dt:.1f} s), scaled by {H * B / (nh * nb):g}x")
     elif key.startswith("batched_mul"):
         if key == "batched_mul":
             dt_name, (m, kk, n, nb) = "bf16", (2048, 2048, 2048, 16)
