@@ -40,34 +40,50 @@ __device__ inline typename T::vec4 lds_tr4(const char *p) {
     return __builtin_bit_cast(typename T::vec4, r);
 }
 
-// One operand tile.  X points at the slice; `rows` = extent along the operand's row index (m or n),
-// `ld` = leading dimension.  RM: element (row, kk) at X[row + kk*ld]; else at X[kk + row*ld].
+// One operand tile.  The slice is addressed through a buffer resource with 32-bit byte offsets, so that
+// loads need no branches (a piece outside the matrix gets an offset past the end of the resource and
+// reads as zeros) and the compiler can count outstanding loads exactly: loads run two stages ahead.
+// RM: element (row, kk) at X[row + kk*ld]; else at X[kk + row*ld].
 template <typename T, bool RM>
 struct Operand {
     typedef typename T::type t;
-    const t *X;
-    int64_t ld, rows, k, row0;
-    u32x4_t reg[4];
+    __amdgpu_buffer_rsrc_t rsrc;
+    int off[4];          // byte offset of this thread's four pieces at k0 = 0, or OOB for rows past the edge
+    int kstep;           // bytes per unit of k0
+    int64_t k;
+    u32x4_t regs[2][4];  // two stages in flight
+    static constexpr int OOB = 0x7fffffff;
 
-    // 1024 chunks of 16 bytes per tile, 4 per thread
-    __device__ void load(int64_t k0) {
-        const int tid = threadIdx.x;
+    __device__ void init(const t *X, int64_t ld, int64_t rows, int64_t k_, int64_t row0) {
+        k = k_;
+        const int64_t extent = RM ? (k_ - 1) * ld + rows : (rows - 1) * ld + k_;   // elements the slice spans
+        rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)X, 0, (int)(extent * 2), 0x00020000);
+        kstep = RM ? (int)(ld * 2) : 2;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const int c = tid + 256 * u;
-            u32x4_t z = {0, 0, 0, 0};
+            const int c = threadIdx.x + 256 * u;
             if (RM) {
-                const int kk = c >> 4, r8 = (c & 15) * 8;       // 16 chunks per k-row
-                const bool ok = k0 + kk < k && row0 + r8 < rows;
-                reg[u] = ok ? *(const u32x4_t *)(X + (row0 + r8) + (k0 + kk) * ld) : z;
+                const int kk = c >> 4, r8 = (c & 15) * 8;       // 16 pieces per k-row; kk >= k falls past the extent by itself
+                off[u] = row0 + r8 < rows ? (int)(((row0 + r8) + kk * ld) * 2) : OOB;
             } else {
-                const int r = c >> 3, k8 = (c & 7) * 8;         // 8 chunks per row
-                const bool ok = row0 + r < rows && k0 + k8 < k;
-                reg[u] = ok ? *(const u32x4_t *)(X + (k0 + k8) + (row0 + r) * ld) : z;
+                const int r = c >> 3, k8 = (c & 7) * 8;         // 8 pieces per row
+                off[u] = row0 + r < rows ? (int)((k8 + (row0 + r) * ld) * 2) : OOB;
             }
         }
     }
-    __device__ void store(char *tile) const {
+    __device__ void load(int set, int64_t k0) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            int o = off[u] == OOB ? OOB : off[u] + (int)k0 * kstep;
+            if (!RM) {   // a piece past k in a row-contiguous-in-k matrix would read the next row
+                const int k8 = ((threadIdx.x + 256 * u) & 7) * 8;
+                o = k0 + k8 < k ? o : OOB;
+            }
+            regs[set][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, o, 0, 0);
+        }
+    }
+    __device__ void store(int set, char *tile) const {
+        const u32x4_t (&reg)[4] = regs[set];
         const int tid = threadIdx.x;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -113,16 +129,9 @@ __global__ __launch_bounds__(256, 2) void gemm16_kernel(Gemm16Args g) {
 
     Operand<T, A_RM> a;
     Operand<T, B_RM> b;
-    a.X = (const t *)g.A + bz * g.sA;
-    a.ld = g.lda;
-    a.rows = g.m;
-    a.k = g.k;
-    a.row0 = (int64_t)blockIdx.x * TM;
-    b.X = (const t *)g.B + bz * g.sB;
-    b.ld = g.ldb;
-    b.rows = g.n;
-    b.k = g.k;
-    b.row0 = (int64_t)blockIdx.y * TN;
+    const int64_t m0 = (int64_t)blockIdx.x * TM, n0 = (int64_t)blockIdx.y * TN;
+    a.init((const t *)g.A + bz * g.sA, g.lda, g.m, g.k, m0);
+    b.init((const t *)g.B + bz * g.sB, g.ldb, g.n, g.k, n0);
 
     floatx16_t acc[2][2];   // [n block][m block]
 #pragma unroll
@@ -130,18 +139,23 @@ __global__ __launch_bounds__(256, 2) void gemm16_kernel(Gemm16Args g) {
 #pragma unroll
         for (int j = 0; j < 2; j++) acc[i][j] = (floatx16_t){0};
 
+    // Loads run two stages ahead of the MFMAs (one stage of 16 MFMAs per wavefront is far shorter than
+    // the latency of the loads behind it): stage it+1 sits in LDS or in register set (it+1)&1, stage
+    // it+2 is in flight into the other set.
     const int nk = (int)((g.k + KC - 1) / KC);
-    a.load(0);
-    b.load(0);
-    a.store(As);
-    b.store(Bs);
+    a.load(0, 0);
+    b.load(0, 0);
+    a.store(0, As);
+    b.store(0, Bs);
+    a.load(1, KC);
+    b.load(1, KC);
     __syncthreads();
-    for (int it = 0; it < nk; it++) {
+    auto stage = [&](int it, int set_next) {   // set_next = (it + 1) & 1, a compile-time constant at each call site
         const int buf = it & 1;
-        if (it + 1 < nk) {
-            a.load((int64_t)(it + 1) * KC);
-            b.load((int64_t)(it + 1) * KC);
-        }
+        // unconditional: past the last stage every piece is out of range and reads as zeros, and a load that is
+        // always issued lets the compiler wait for exactly the older set (vmcnt(8)) before the LDS stores below
+        a.load(set_next ^ 1, (int64_t)(it + 2) * KC);
+        b.load(set_next ^ 1, (int64_t)(it + 2) * KC);
         const char *at = As + buf * TILEB, *bt = Bs + buf * TILEB;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
@@ -157,23 +171,29 @@ __global__ __launch_bounds__(256, 2) void gemm16_kernel(Gemm16Args g) {
                 for (int j = 0; j < 2; j++) acc[i][j] = T::mfma32(bv[i], av[j], acc[i][j]);
         }
         if (it + 1 < nk) {
-            a.store(As + (buf ^ 1) * TILEB);
-            b.store(Bs + (buf ^ 1) * TILEB);
+            a.store(set_next, As + (buf ^ 1) * TILEB);
+            b.store(set_next, Bs + (buf ^ 1) * TILEB);
         }
         __syncthreads();
+    };
+    int it = 0;
+    for (; it + 1 < nk; it += 2) {
+        stage(it, 1);
+        stage(it + 1, 0);
     }
+    if (it < nk) stage(it, 1);
 
     // accumulator register v of lane (r, hh) of block (i, j): n = 32i + 8*(v/4) + 4*hh + v%4, m = 32j + r
     t *C = (t *)g.C + bz * g.sC;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        const int64_t mi = a.row0 + 64 * wm + 32 * j + r;
+        const int64_t mi = m0 + 64 * wm + 32 * j + r;
         if (mi >= g.m) continue;
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int64_t nj = b.row0 + 64 * wn + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
+                const int64_t nj = n0 + 64 * wn + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
                 if (nj < g.n) {
                     t *c = C + mi + nj * g.ldc;
                     float val = g.alpha * acc[i][j][v];
@@ -217,6 +237,9 @@ bool batched_gemm16_supports(int32_t dtype, int transA, int transB, int64_t m, i
     if (!al(A) || !al(B) || (lda & 7) || (ldb & 7) || (sA & 7) || (sB & 7)) return false;
     if ((transA ? k : m) & 7) return false;
     if ((transB ? n : k) & 7) return false;
+    // slices are addressed with 32-bit byte offsets
+    const int64_t extA = transA ? (m - 1) * lda + k : (k - 1) * lda + m, extB = transB ? (k - 1) * ldb + n : (n - 1) * ldb + k;
+    if (extA * 2 >= 2147483647LL || extB * 2 >= 2147483647LL) return false;
     return (n + TN - 1) / TN <= 65535;
 }
 
