@@ -120,27 +120,54 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     }
 }
 
-// one thread per output feature: merge the splits with the usual log-sum-exp rule
+// Merge of the splits with the usual log-sum-exp rule.  One workgroup per (256 features, batch): the
+// weights 2^(m_s - m) of every (head, split) pair are computed once into LDS, then each thread sums its
+// feature over the splits, eight independent loads at a time.
 template <typename T>
 __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
     const AttnParams &p = a.p;
+    __shared__ float wgt[4 * 1024];   // [heads of this workgroup <= 4][nsplit <= 1024]
+    __shared__ float inv_l[4];
     const int64_t b = blockIdx.y;
-    const int64_t f = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (f >= p.E) return;
-    const int64_t h = f / p.D;
+    const int64_t f0 = (int64_t)blockIdx.x * 256, f = f0 + threadIdx.x;
     const float *ws = (const float *)p.workspace;
     const float *wm = ws + (int64_t)p.B * a.nsplit * p.E;
     const float *wl = wm + (int64_t)p.B * a.nsplit * p.H;
-    float m = MI_NEG_INF;
-    for (int s = 0; s < a.nsplit; s++) m = fmaxf(m, wm[(b * a.nsplit + s) * p.H + h]);
-    float l = 0.0f, o = 0.0f;
-    for (int s = 0; s < a.nsplit; s++) {
-        const int64_t slot = b * a.nsplit + s;
-        const float w = mi_exp2((wm[slot * p.H + h] - m) * a.c);
-        l = fmaf(wl[slot * p.H + h], w, l);
-        o = fmaf(ws[slot * p.E + f], w, o);
+    const int64_t h0 = f0 / p.D;
+    const int nh = (int)(256 / p.D);                 // 2 or 4 heads per workgroup
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (wave < nh && h0 + wave < p.H) {
+        // one wavefront per head: maximum over the splits, then the weights and the total sum
+        const int64_t h = h0 + wave;
+        float m = MI_NEG_INF;
+        for (int s = lane; s < a.nsplit; s += 64) m = fmaxf(m, wm[(b * a.nsplit + s) * p.H + h]);
+        m = mi_wave_max(m);
+        float l = 0.0f;
+        for (int s = lane; s < a.nsplit; s += 64) {
+            const int64_t slot = b * a.nsplit + s;
+            const float w = mi_exp2((wm[slot * p.H + h] - m) * a.c);
+            wgt[wave * 1024 + s] = w;
+            l = fmaf(wl[slot * p.H + h], w, l);
+        }
+        l = mi_wave_sum(l);
+        if (lane == 0) inv_l[wave] = 1.0f / l;
     }
-    ((typename T::type *)p.out)[p.E * b + f] = T::from_f32(o / l);
+    __syncthreads();
+    if (f >= p.E) return;
+    const int hl = (int)(f / p.D - h0);
+    const float *src = ws + b * a.nsplit * p.E + f;
+    const float *w = wgt + hl * 1024;
+    float o = 0.0f;
+    int s = 0;
+    for (; s + 8 <= a.nsplit; s += 8) {
+        float x[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) x[u] = src[(int64_t)(s + u) * p.E];
+#pragma unroll
+        for (int u = 0; u < 8; u++) o = fmaf(x[u], w[s + u], o);
+    }
+    for (; s < a.nsplit; s++) o = fmaf(src[(int64_t)s * p.E], w[s], o);
+    ((typename T::type *)p.out)[p.E * b + f] = T::from_f32(o * inv_l[hl]);
 }
 
 int pick_nsplit(const AttnParams &p) {
