@@ -20,10 +20,23 @@
 
 namespace {
 
-constexpr int TM = 128, TN = 128, KC = 64;
-constexpr int RMAJ_ROWB = 256;                 // bytes per k-row of an RMAJ tile (128 rows x 2 bytes)
+constexpr int KC = 64;
 constexpr int KMAJ_ROWB = 136;                 // bytes per row of a KMAJ tile (64 k x 2 bytes + 8 pad: conflict-free 8-byte reads)
-constexpr int TILEB = 128 * KMAJ_ROWB;         // bytes reserved per tile and buffer (RMAJ needs 64*256 = 16384 <= 17408)
+
+// Two shapes: SMALL = 128 x 128 output tile, 4 wavefronts of 64 x 64 (2 x 2 MFMA blocks), two workgroups
+// per CU; LARGE = 256 x 256 tile, 8 wavefronts of 128 (m) x 64 (n) (4 x 2 blocks), one workgroup per CU:
+// twice the MFMAs per barrier, 3/4 of the LDS operand reads per MFMA and half the global and LDS-store
+// traffic per FLOP.  Both tiles are square, so A and B tiles have one size and every thread moves four
+// 16-byte pieces per tile and stage in either shape.
+template <bool LARGE>
+struct Shape {
+    static constexpr int TILE = LARGE ? 256 : 128;        // rows of an operand tile (m of A, n of B)
+    static constexpr int THREADS = LARGE ? 512 : 256;
+    static constexpr int WM = 2, WN = LARGE ? 4 : 2;      // wavefront grid
+    static constexpr int BM = LARGE ? 4 : 2, BNB = 2;     // 32 x 32 blocks per wavefront along m and n
+    static constexpr int RMAJ_ROWB = TILE * 2;            // bytes per k-row of an RMAJ tile
+    static constexpr int TILEB = TILE * KMAJ_ROWB;        // bytes reserved per tile and buffer (RMAJ needs 64 * RMAJ_ROWB, which is less)
+};
 
 struct Gemm16Args {
     const void *A, *B;
@@ -44,9 +57,11 @@ __device__ inline typename T::vec4 lds_tr4(const char *p) {
 // loads need no branches (a piece outside the matrix gets an offset past the end of the resource and
 // reads as zeros) and the compiler can count outstanding loads exactly: loads run two stages ahead.
 // RM: element (row, kk) at X[row + kk*ld]; else at X[kk + row*ld].
-template <typename T, bool RM>
+template <typename T, bool RM, bool LARGE>
 struct Operand {
     typedef typename T::type t;
+    static constexpr int THREADS = Shape<LARGE>::THREADS, RMAJ_ROWB = Shape<LARGE>::RMAJ_ROWB;
+    static constexpr int CPR = Shape<LARGE>::TILE / 8;   // 16-byte pieces per k-row of an RMAJ tile
     __amdgpu_buffer_rsrc_t rsrc;
     int off[4];          // byte offset of this thread's four pieces at k0 = 0, or OOB for rows past the edge
     int kstep;           // bytes per unit of k0
@@ -61,9 +76,9 @@ struct Operand {
         kstep = RM ? (int)(ld * 2) : 2;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const int c = threadIdx.x + 256 * u;
+            const int c = threadIdx.x + THREADS * u;
             if (RM) {
-                const int kk = c >> 4, r8 = (c & 15) * 8;       // 16 pieces per k-row; kk >= k falls past the extent by itself
+                const int kk = c / CPR, r8 = (c % CPR) * 8;     // kk >= k falls past the extent by itself
                 off[u] = row0 + r8 < rows ? (int)(((row0 + r8) + kk * ld) * 2) : OOB;
             } else {
                 const int r = c >> 3, k8 = (c & 7) * 8;         // 8 pieces per row
@@ -76,7 +91,7 @@ struct Operand {
         for (int u = 0; u < 4; u++) {
             int o = off[u] == OOB ? OOB : off[u] + (int)k0 * kstep;
             if (!RM) {   // a piece past k in a row-contiguous-in-k matrix would read the next row
-                const int k8 = ((threadIdx.x + 256 * u) & 7) * 8;
+                const int k8 = ((threadIdx.x + THREADS * u) & 7) * 8;
                 o = k0 + k8 < k ? o : OOB;
             }
             regs[set][u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, o, 0, 0);
@@ -87,9 +102,9 @@ struct Operand {
         const int tid = threadIdx.x;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const int c = tid + 256 * u;
+            const int c = tid + THREADS * u;
             if (RM) {
-                const int kk = c >> 4, chunk = c & 15;
+                const int kk = c / CPR, chunk = c % CPR;
                 *(u32x4_t *)(tile + kk * RMAJ_ROWB + ((chunk ^ rmaj_swz(kk)) << 4)) = reg[u];
             } else {
                 const int r = c >> 3, chunk = c & 7;
@@ -99,7 +114,7 @@ struct Operand {
             }
         }
     }
-    // MFMA operand of the 32-row block `blk` (0..3 within the tile) for k-step `ks` (0..3)
+    // MFMA operand of the 32-row block `blk` of the tile for k-step `ks` (0..3)
     __device__ static typename T::vec8 fetch(const char *tile, int blk, int ks, int lane) {
         const int hh = lane >> 5;
         if (RM) {
@@ -118,30 +133,32 @@ struct Operand {
     }
 };
 
-template <typename T, bool A_RM, bool B_RM>
-__global__ __launch_bounds__(256, 2) void gemm16_kernel(Gemm16Args g) {
+template <typename T, bool A_RM, bool B_RM, bool LARGE>
+__global__ __launch_bounds__(Shape<LARGE>::THREADS, LARGE ? 1 : 2) void gemm16_kernel(Gemm16Args g) {
     typedef typename T::type t;
+    typedef Shape<LARGE> S;
+    constexpr int TILEB = S::TILEB, BM = S::BM, BNB = S::BNB;
     extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
     char *As = (char *)gemm_smem, *Bs = As + 2 * TILEB;
     const int64_t bz = blockIdx.z;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave % S::WM, wn = wave / S::WM;
     const int r = lane & 31, hh = lane >> 5;
 
-    Operand<T, A_RM> a;
-    Operand<T, B_RM> b;
-    const int64_t m0 = (int64_t)blockIdx.x * TM, n0 = (int64_t)blockIdx.y * TN;
+    Operand<T, A_RM, LARGE> a;
+    Operand<T, B_RM, LARGE> b;
+    const int64_t m0 = (int64_t)blockIdx.x * S::TILE, n0 = (int64_t)blockIdx.y * S::TILE;
     a.init((const t *)g.A + bz * g.sA, g.lda, g.m, g.k, m0);
     b.init((const t *)g.B + bz * g.sB, g.ldb, g.n, g.k, n0);
 
-    floatx16_t acc[2][2];   // [n block][m block]
+    floatx16_t acc[BNB][BM];   // [n block][m block]
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < BNB; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = (floatx16_t){0};
+        for (int j = 0; j < BM; j++) acc[i][j] = (floatx16_t){0};
 
-    // Loads run two stages ahead of the MFMAs (one stage of 16 MFMAs per wavefront is far shorter than
-    // the latency of the loads behind it): stage it+1 sits in LDS or in register set (it+1)&1, stage
-    // it+2 is in flight into the other set.
+    // Loads run two stages ahead of the MFMAs (one stage of MFMAs is shorter than the latency of the loads
+    // behind it): stage it+1 sits in LDS or in register set (it+1)&1, stage it+2 is in flight into the
+    // other set.
     const int nk = (int)((g.k + KC - 1) / KC);
     a.load(0, 0);
     b.load(0, 0);
@@ -159,16 +176,15 @@ __global__ __launch_bounds__(256, 2) void gemm16_kernel(Gemm16Args g) {
         const char *at = As + buf * TILEB, *bt = Bs + buf * TILEB;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            typename T::vec8 av[2], bv[2];
+            typename T::vec8 av[BM], bv[BNB];
 #pragma unroll
-            for (int j = 0; j < 2; j++) {
-                av[j] = Operand<T, A_RM>::fetch(at, 2 * wm + j, ks, lane);
-                bv[j] = Operand<T, B_RM>::fetch(bt, 2 * wn + j, ks, lane);
-            }
+            for (int j = 0; j < BM; j++) av[j] = Operand<T, A_RM, LARGE>::fetch(at, BM * wm + j, ks, lane);
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < BNB; i++) bv[i] = Operand<T, B_RM, LARGE>::fetch(bt, BNB * wn + i, ks, lane);
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = T::mfma32(bv[i], av[j], acc[i][j]);
+            for (int i = 0; i < BNB; i++)
+#pragma unroll
+                for (int j = 0; j < BM; j++) acc[i][j] = T::mfma32(bv[i], av[j], acc[i][j]);
         }
         if (it + 1 < nk) {
             a.store(set_next, As + (buf ^ 1) * TILEB);
@@ -186,14 +202,14 @@ __global__ __launch_bounds__(256, 2) void gemm16_kernel(Gemm16Args g) {
     // accumulator register v of lane (r, hh) of block (i, j): n = 32i + 8*(v/4) + 4*hh + v%4, m = 32j + r
     t *C = (t *)g.C + bz * g.sC;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int64_t mi = m0 + 64 * wm + 32 * j + r;
+    for (int j = 0; j < BM; j++) {
+        const int64_t mi = m0 + 32 * BM * wm + 32 * j + r;
         if (mi >= g.m) continue;
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < BNB; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int64_t nj = n0 + 64 * wn + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
+                const int64_t nj = n0 + 32 * BNB * wn + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
                 if (nj < g.n) {
                     t *c = C + mi + nj * g.ldc;
                     float val = g.alpha * acc[i][j][v];
@@ -204,26 +220,35 @@ __global__ __launch_bounds__(256, 2) void gemm16_kernel(Gemm16Args g) {
     }
 }
 
-template <typename T, bool A_RM, bool B_RM>
+template <typename T, bool A_RM, bool B_RM, bool LARGE>
 int32_t launch_one(const Gemm16Args &g, int64_t nb, hipStream_t st) {
-    auto kern = gemm16_kernel<T, A_RM, B_RM>;
-    constexpr size_t smem = 4 * TILEB;
+    typedef Shape<LARGE> S;
+    auto kern = gemm16_kernel<T, A_RM, B_RM, LARGE>;
+    constexpr size_t smem = 4 * S::TILEB;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
     if (!attr_set) {
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    dim3 grid((unsigned)((g.m + TM - 1) / TM), (unsigned)((g.n + TN - 1) / TN), (unsigned)nb);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, g);
+    dim3 grid((unsigned)((g.m + S::TILE - 1) / S::TILE), (unsigned)((g.n + S::TILE - 1) / S::TILE), (unsigned)nb);
+    hipLaunchKernelGGL(kern, grid, dim3(S::THREADS), smem, st, g);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }
 
+template <typename T, bool LARGE>
+int32_t launch_l(const Gemm16Args &g, int transA, int transB, int64_t nb, hipStream_t st) {
+    const bool a_rm = !transA, b_rm = transB != 0;
+    if (a_rm) return b_rm ? launch_one<T, true, true, LARGE>(g, nb, st) : launch_one<T, true, false, LARGE>(g, nb, st);
+    return b_rm ? launch_one<T, false, true, LARGE>(g, nb, st) : launch_one<T, false, false, LARGE>(g, nb, st);
+}
+
 template <typename T>
 int32_t launch_t(const Gemm16Args &g, int transA, int transB, int64_t nb, hipStream_t st) {
-    const bool a_rm = !transA, b_rm = transB != 0;
-    if (a_rm) return b_rm ? launch_one<T, true, true>(g, nb, st) : launch_one<T, true, false>(g, nb, st);
-    return b_rm ? launch_one<T, false, true>(g, nb, st) : launch_one<T, false, false>(g, nb, st);
+    // the large tile when it still gives every CU a workgroup; the small one otherwise
+    const int64_t big = ((g.m + 255) / 256) * ((g.n + 255) / 256) * nb;
+    if (g.m >= 256 && g.n >= 256 && big >= 256) return launch_l<T, true>(g, transA, transB, nb, st);
+    return launch_l<T, false>(g, transA, transB, nb, st);
 }
 
 }  // namespace
@@ -240,7 +265,7 @@ bool batched_gemm16_supports(int32_t dtype, int transA, int transB, int64_t m, i
     // slices are addressed with 32-bit byte offsets
     const int64_t extA = transA ? (m - 1) * lda + k : (k - 1) * lda + m, extB = transB ? (k - 1) * ldb + n : (n - 1) * ldb + k;
     if (extA * 2 >= 2147483647LL || extB * 2 >= 2147483647LL) return false;
-    return (n + TN - 1) / TN <= 65535;
+    return (n + 127) / 128 <= 65535;
 }
 
 int32_t launch_batched_gemm16(int32_t dtype, int transA, int transB, int64_t m, int64_t n, int64_t k, float alpha, const void *A,

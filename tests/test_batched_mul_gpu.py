@@ -204,6 +204,22 @@ def test_tiled_kernel_all_layouts(nn, dtype, ta, tb, m, n, k, nb):
     assert close(got, bmm(A, B, ta, tb), dtype)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_large_tile_kernel(nn, dtype, ta, tb):
+    """Enough 256 x 256 tiles to fill the chip: the eight-wavefront shape of the 16-bit kernel, ragged in m, n
+    and k, with alpha and beta."""
+    rng = np.random.default_rng(17)
+    m, n, k, nb = 264, 520, 136, 48
+    A = round_to(rng.standard_normal((k, m, nb) if ta else (m, k, nb)), dtype)
+    B = round_to(rng.standard_normal((n, k, nb) if tb else (k, n, nb)), dtype)
+    C0 = round_to(rng.standard_normal((m, n, nb)), dtype)
+    dA, dB, dC = (nn.DeviceArray.from_numpy(x, dtype) for x in (A, B, C0))
+    T = nn.batched_transpose
+    nn.batched_mul_(dC, T(dA) if ta else dA, T(dB) if tb else dB, 0.5, 2.0)
+    assert close(dC.to_numpy(), 0.5 * bmm(A, B, ta, tb) + 2.0 * C0, dtype)
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 def test_tiled_kernel_alpha_beta_and_shared_operand(nn, dtype):
     """test/ext_amdgpu/batched_mul.jl:15-19 (C .= pi; batched_mul!(C, A, B, 2, 3)) and the batch-1 operand of
