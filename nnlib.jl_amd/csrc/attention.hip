@@ -10,6 +10,10 @@ int32_t launch_flash16_fast_bf16(const AttnParams &, hipStream_t);
 int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t);
 bool flash16_fast_supports_bf16(const AttnParams &);
 bool flash16_fast_supports_f16(const AttnParams &);
+int32_t launch_flash16_fast_bf16_d64(const AttnParams &, hipStream_t);
+int32_t launch_flash16_fast_f16_d64(const AttnParams &, hipStream_t);
+bool flash16_fast_supports_bf16_d64(const AttnParams &);
+bool flash16_fast_supports_f16_d64(const AttnParams &);
 
 #include "flash_common.h"
 
@@ -61,7 +65,7 @@ int32_t launch_flash_merge(const AttnParams &p, int nsplit, hipStream_t st) {
     return MI_OK;
 }
 
-// true when the call takes the software-pipelined head-dim-128 kernel (which never splits)
+// true when the call takes the software-pipelined kernel (which never splits)
 static bool takes_fast_path(const AttnParams &p);
 
 bool attention_flash16_supports(const AttnParams &p) {
@@ -75,12 +79,16 @@ bool attention_flash16_supports(const AttnParams &p) {
 }
 
 static bool takes_fast_path(const AttnParams &p) {
-    return (p.dtype == MI_BF16 && flash16_fast_supports_bf16(p)) || (p.dtype == MI_F16 && flash16_fast_supports_f16(p));
+    if (p.dtype == MI_BF16) return flash16_fast_supports_bf16(p) || flash16_fast_supports_bf16_d64(p);
+    if (p.dtype == MI_F16) return flash16_fast_supports_f16(p) || flash16_fast_supports_f16_d64(p);
+    return false;
 }
 
 int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
     if (p.dtype == MI_BF16 && flash16_fast_supports_bf16(p)) return launch_flash16_fast_bf16(p, st);
     if (p.dtype == MI_F16 && flash16_fast_supports_f16(p)) return launch_flash16_fast_f16(p, st);
+    if (p.dtype == MI_BF16 && flash16_fast_supports_bf16_d64(p)) return launch_flash16_fast_bf16_d64(p, st);
+    if (p.dtype == MI_F16 && flash16_fast_supports_f16_d64(p)) return launch_flash16_fast_f16_d64(p, st);
     if (p.dtype == MI_BF16) return p.D == 64 ? launch_flash16_bf16_d64(p, st) : launch_flash16_bf16_d128(p, st);
     return p.D == 64 ? launch_flash16_f16_d64(p, st) : launch_flash16_f16_d128(p, st);
 }

@@ -1,4 +1,4 @@
-// Instantiation of the software-pipelined head-dim-128 flash forward kernel for bf16.
+// Instantiation of the software-pipelined flash forward kernel (head dim 128) for bf16.
 #define FAST_T BF16
 #define FAST_ENTRY launch_flash16_fast_bf16
 #define FAST_SUPPORTS flash16_fast_supports_bf16

@@ -185,6 +185,13 @@ FLASH16_CASES = [
     ("f16", 128, 70, 336, 2, 2, dict(bias_shape=(336, 70, 2, 2), mask_shape=(336, 70, 1, 2))),
     ("bf16", 256, 150, 400, 1, 2, dict(bias_shape=(400, 150, 1, 1), mask_shape=(400, 1, 2, 1))),
     ("bf16", 128, 192, 192, 2, 2, dict(causal=True, bias_shape=(192, 192, 2, 1))),
+    # long enough for the steady-state loop of the software-pipelined kernel, head dims 64 and 128
+    ("bf16", 128, 300, 700, 1, 2, {}),
+    ("bf16", 128, 520, 520, 1, 2, dict(causal=True)),
+    ("f16", 64, 257, 1100, 2, 1, {}),
+    ("f16", 128, 600, 600, 1, 2, dict(causal=True)),
+    ("bf16", 256, 300, 700, 1, 2, {}),
+    ("f16", 256, 520, 520, 1, 2, dict(causal=True)),
 ]
 
 
