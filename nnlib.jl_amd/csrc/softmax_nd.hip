@@ -165,9 +165,10 @@ __global__ __launch_bounds__(256) void softmax_nd_kernel(const typename T::type 
 // ---- reductions over a strided dimension with wide rows ----------------------------------------------
 // inner is a multiple of VEC (16 bytes of elements) and every row starts 16-byte aligned: a thread owns
 // VEC consecutive `inner` positions and walks j in steps of TJ; TI threads side by side cover TI*VEC
-// positions, so a wavefront reads 64/TI rows of TI*16 contiguous bytes per load.  One pass finds the
-// maximum and the sum together (running maximum, sum rescaled when it grows), a second pass writes:
-// two reads and one write per element.
+// positions, so a wavefront reads 64/TI rows of TI*16 contiguous bytes per load.  Columns of up to 8192
+// elements (4096 for the gradients) are held in registers by a 512-thread workgroup: one read, one
+// write.  Longer ones are streamed: one pass finds the maximum and the sum together (running maximum,
+// sum rescaled when it grows), a second pass writes: two reads and one write per element.
 template <typename T, int VEC>
 struct VecIO {
     typedef typename T::type t;
@@ -215,6 +216,171 @@ __device__ inline void online_merge(float m2, float s2, float &m, float &s) {
     }
 }
 
+// Workgroups go to the 8 XCDs round-robin.  Tiles that are neighbours along `inner` share cache lines
+// of every row, so each XCD gets a contiguous range of tiles: a permutation of [0, 8*floor(n/8)), the
+// identity on the rest (2.05 -> 2.31 TB/s on a 256 x 4096 x 128 bf16 array reduced over dim 2).
+__device__ inline int64_t xcd_order(int64_t tile, int64_t n_tiles) {
+    const int64_t n8 = n_tiles >> 3;
+    return tile < 8 * n8 ? (tile & 7) * n8 + (tile >> 3) : tile;
+}
+
+// lanes with equal (lane & (TI-1)) hold slices of the same positions: butterfly within the wavefront,
+// then the eight wavefronts of a 512-thread workgroup through LDS (red: 8 * 64 * VEC floats)
+template <bool IS_MAX, int VEC>
+__device__ inline void reduce_slices_vec(float (&v)[VEC], int ti_log2, float *red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, ti = 1 << ti_log2;
+    for (int o = 32; o >= ti; o >>= 1) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            const float u = __shfl_xor(v[e], o, 64);
+            v[e] = IS_MAX ? fmaxf(v[e], u) : v[e] + u;
+        }
+    }
+    __syncthreads();  // previous use of `red`
+    if (lane < ti) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) red[(wave * 64 + lane) * VEC + e] = v[e];
+    }
+    __syncthreads();
+    const int il = lane & (ti - 1);
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        float r = red[il * VEC + e];
+#pragma unroll
+        for (int w = 1; w < 8; w++) {
+            const float u = red[(w * 64 + il) * VEC + e];
+            r = IS_MAX ? fmaxf(r, u) : r + u;
+        }
+        v[e] = r;
+    }
+}
+
+// Columns of up to NP * TJ elements (TJ = 512 / TI): the NP 16-byte pieces of a thread stay in registers
+// between the reduction and the result, so every element is read once and written once.  All loads are
+// issued before any arithmetic and are unconditional (threads without work read a valid dummy address).
+template <typename T, int OP, int VEC, int NP>
+__global__ __launch_bounds__(512) void softmax_nd_cached_kernel(const typename T::type *x, const typename T::type *x2,
+                                                                 typename T::type *y, Geometry g) {
+    typedef typename T::type t;
+    typedef VecIO<T, VEC> IO;
+    constexpr bool GRAD = OP >= OP_GRAD_SOFTMAX;
+    __shared__ float red[8 * 64 * VEC];
+    const int ti = 1 << g.ti_log2, tj = 512 >> g.ti_log2;
+    const int il = threadIdx.x & (ti - 1), js = threadIdx.x >> g.ti_log2;
+    const int64_t n_tiles = g.n_itiles * g.outer;
+    const int64_t step = g.inner * tj;   // elements between consecutive rows of one thread
+    for (int64_t tile0 = blockIdx.x; tile0 < n_tiles; tile0 += gridDim.x) {
+        const int64_t tile = xcd_order(tile0, n_tiles);
+        const int64_t o = tile / g.n_itiles, i = ((tile % g.n_itiles) * ti + il) * VEC;
+        const bool ok = i < g.inner;
+        const int nrows = ok && js < g.len ? (int)((g.len - js + tj - 1) / tj) : 0;   // <= NP (host)
+        const int64_t base = nrows ? i + g.inner * g.len * o + g.inner * js : g.inner * g.len * o;
+        const int last = nrows ? nrows - 1 : 0;
+        u32x4_t raw[NP], raw2[GRAD ? NP : 1];
+#pragma unroll
+        for (int u = 0; u < NP; u++) {
+            const int64_t at = base + step * (u < last ? u : last);
+            raw[u] = *(const u32x4_t *)(x + at);
+            if (GRAD) raw2[u] = *(const u32x4_t *)(x2 + at);
+        }
+        float m[VEC], sum[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            m[e] = MI_NEG_INF;
+            sum[e] = 0.0f;
+        }
+        if constexpr (GRAD) {
+#pragma unroll
+            for (int u = 0; u < NP; u++) {
+                if (u < nrows) {
+                    float v[VEC], v2[VEC];
+                    IO::unpack(raw[u], v);
+                    if (OP == OP_GRAD_SOFTMAX) IO::unpack(raw2[u], v2);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) sum[e] += OP == OP_GRAD_SOFTMAX ? v[e] * v2[e] : v[e];
+                }
+            }
+            reduce_slices_vec<false, VEC>(sum, g.ti_log2, red);
+#pragma unroll
+            for (int u = 0; u < NP; u++) {
+                if (u < nrows) {
+                    float v[VEC], v2[VEC], r[VEC];
+                    IO::unpack(raw[u], v);
+                    IO::unpack(raw2[u], v2);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++)
+                        r[e] = OP == OP_GRAD_SOFTMAX ? v2[e] * (v[e] - sum[e]) : v[e] - sum[e] * fast_exp(v2[e]);
+                    IO::store(y + base + step * u, r);
+                }
+            }
+            continue;
+        }
+        // forward ops: maximum, sum of exponentials, result, all from the registers
+#pragma unroll
+        for (int u = 0; u < NP; u++) {
+            if (u < nrows) {
+                float v[VEC];
+                IO::unpack(raw[u], v);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) m[e] = fmaxf(m[e], v[e]);
+            }
+        }
+        reduce_slices_vec<true, VEC>(m, g.ti_log2, red);
+        bool plain = true;   // finite maxima: no special cases
+#pragma unroll
+        for (int e = 0; e < VEC; e++) plain = plain && m[e] > MI_NEG_INF && m[e] < MI_POS_INF;
+        float c0[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) c0[e] = -m[e] * MI_LOG2E;
+#pragma unroll
+        for (int u = 0; u < NP; u++) {
+            if (u < nrows) {
+                float v[VEC];
+                IO::unpack(raw[u], v);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    if (plain) sum[e] += mi_exp2(fmaf(v[e], MI_LOG2E, c0[e]));
+                    else if (OP == OP_SOFTMAX) sum[e] += softmax_term(v[e], m[e]);
+                    else if (OP == OP_LOGSOFTMAX) sum[e] += fast_exp(logsoftmax_shift(v[e], m[e]));
+                    else sum[e] += fast_exp(v[e] - m[e]);   // logsumexp: no special cases (src/softmax.jl:202)
+                }
+            }
+        }
+        reduce_slices_vec<false, VEC>(sum, g.ti_log2, red);
+        if constexpr (OP == OP_LOGSUMEXP) {
+            if (ok && js == 0) {
+                float r[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; e++) r[e] = m[e] + logf(sum[e]);
+                IO::store(y + i + g.inner * o, r);
+            }
+            continue;
+        }
+        float c1[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            if (OP == OP_SOFTMAX) c1[e] = 1.0f / sum[e];
+            else {
+                c0[e] = logf(sum[e]);
+                c1[e] = -m[e] - c0[e];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NP; u++) {
+            if (u < nrows) {
+                float v[VEC], r[VEC];
+                IO::unpack(raw[u], v);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    if (OP == OP_SOFTMAX) r[e] = plain ? mi_exp2(fmaf(v[e], MI_LOG2E, c0[e])) * c1[e] : softmax_term(v[e], m[e]) / sum[e];
+                    else r[e] = plain ? v[e] + c1[e] : logsoftmax_shift(v[e], m[e]) - c0[e];
+                }
+                IO::store(y + base + step * u, r);
+            }
+        }
+    }
+}
+
 template <typename T, int OP, int VEC>
 __global__ __launch_bounds__(256) void softmax_nd_vec_kernel(const typename T::type *x, const typename T::type *x2,
                                                               typename T::type *y, Geometry g) {
@@ -227,7 +393,8 @@ __global__ __launch_bounds__(256) void softmax_nd_vec_kernel(const typename T::t
     const int il = threadIdx.x & (ti - 1), js = threadIdx.x >> g.ti_log2;
     const int64_t n_tiles = g.n_itiles * g.outer;
     const int64_t step = g.inner * tj;   // elements between consecutive rows of one thread
-    for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    for (int64_t tile0 = blockIdx.x; tile0 < n_tiles; tile0 += gridDim.x) {
+        const int64_t tile = xcd_order(tile0, n_tiles);
         const int64_t o = tile / g.n_itiles, i = ((tile % g.n_itiles) * ti + il) * VEC;
         const bool ok = i < g.inner;
         const int64_t base = i + g.inner * g.len * o + g.inner * js;
@@ -344,6 +511,20 @@ void launch_nd(const void *x, const void *x2, void *y, int64_t inner, int64_t le
     if (inner % VEC == 0 && inner >= 4 * VEC && len > 64 && al(x) && al(y) && (!x2 || al(x2))) {
         // wide rows and columns too long for the register cache of the scalar kernel
         const int64_t chunks = inner / VEC;
+        constexpr int NP = OP >= OP_GRAD_SOFTMAX ? 8 : 16;   // the gradients hold two arrays
+        if (len <= 512 * NP) {
+            // register-cached kernel: TI as wide as the column length allows (TJ * NP >= len)
+            g.ti_log2 = 0;
+            while ((1 << g.ti_log2) < 64 && ((int64_t)1 << g.ti_log2) < chunks && (int64_t)(512 >> (g.ti_log2 + 1)) * NP >= len)
+                g.ti_log2++;
+            while (g.ti_log2 > 0 && ((chunks + (1 << g.ti_log2) - 1) >> g.ti_log2) * outer < 1024) g.ti_log2--;
+            g.n_itiles = (chunks + (1 << g.ti_log2) - 1) >> g.ti_log2;
+            int64_t blocks = g.n_itiles * outer;
+            if (blocks > 262144) blocks = 262144;
+            hipLaunchKernelGGL((softmax_nd_cached_kernel<T, OP, VEC, NP>), dim3((unsigned)blocks), dim3(512), 0, st,
+                               (const t *)x, (const t *)x2, (t *)y, g);
+            return;
+        }
         g.ti_log2 = 0;
         while ((1 << g.ti_log2) < 64 && ((int64_t)1 << g.ti_log2) < chunks) g.ti_log2++;
         // enough workgroups to fill the chip, but rows of at least 64 contiguous bytes per wavefront load

@@ -47,7 +47,8 @@ def test_reference_values(nn):
 SHAPES = [((2, 2, 2, 2, 2), d) for d in (1, 2, 3, 4, 5)] + [
     ((5, 7), 2), ((3, 4), None), ((33, 65, 3), 2), ((64, 100, 5), 2), ((130, 17, 2), (2, 3)), ((7, 3000, 2), 2),
     ((1, 5000, 3), 2), ((300, 70, 2), 2), ((5000,), 1), ((70000,), None), ((4, 9, 6), (1, 2)), ((128, 40), 1),
-    ((9, 5), 3), ((256, 1000, 3), 2), ((96, 129, 2), 2), ((32, 70, 2, 2), (2, 3)), ((1024, 65), 2)]
+    ((9, 5), 3), ((256, 1000, 3), 2), ((96, 129, 2), 2), ((32, 70, 2, 2), (2, 3)), ((1024, 65), 2),
+    ((64, 9000, 2), 2), ((32, 5000, 2), 2), ((8, 8192, 1), 2), ((520, 300, 1), 2)]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
@@ -105,12 +106,13 @@ def test_errors(nn):
         nn.grad_softmax_(nn.DeviceArray.zeros((3, 2)), nn.DeviceArray.zeros((2, 3)), nn.DeviceArray.zeros((2, 3)))
 
 
+@pytest.mark.parametrize("length", [200, 9000], ids=["register-cached", "streamed"])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-def test_special_values_on_the_wide_row_kernel(nn, oracle, dtype):
-    """The one-pass maximum-and-sum of the strided kernel keeps the +-Inf / NaN rules of
-    src/softmax.jl:72-75, 140-144 wherever the special entry sits in the column."""
+def test_special_values_on_the_wide_row_kernel(nn, oracle, dtype, length):
+    """Both strided kernels (columns held in registers; longer columns with a one-pass maximum-and-sum)
+    keep the +-Inf / NaN rules of src/softmax.jl:72-75, 140-144 wherever the special entry sits."""
     rng = np.random.default_rng(11)
-    x = round_to(rng.standard_normal((64, 200, 2)), dtype)
+    x = round_to(rng.standard_normal((64, length, 2)), dtype)
     x[0, :, 0] = -np.inf                      # all -Inf: NaN
     x[1, 5, 0] = np.inf                       # one +Inf
     x[2, [3, 150], 0] = np.inf                # two +Inf: 0.5 each
