@@ -5,8 +5,9 @@
 //
 // Workgroup = 4 wavefronts (2 x 2), output tile 128 (m) x 128 (n), 64 x 64 per wavefront as 2 x 2
 // MFMA blocks of 32 x 32; k advances 64 per stage through double-buffered LDS tiles.
-// As in batched_gemm.hip the MFMA runs on the transposed problem (accumulator rows = n, columns = m),
-// so that the 32 lanes of a half-wave store 32 consecutive elements of a C column.
+// Accumulator rows = m, columns = n: a lane holds runs of 4 consecutive m of one C column, lanes l and
+// l + 32 complementary runs; they exchange halves and each lane stores 16 contiguous bytes (C rows that
+// cannot be written in aligned 16-byte pieces take element stores).
 //
 // An operand tile is kept in the orientation its memory has:
 //   RMAJ  contiguous along its row index (A with 'N', B with 'T'): tile [64 k][128 rows], chunks
@@ -43,6 +44,7 @@ struct Gemm16Args {
     void *C;
     int64_t m, n, k, lda, ldb, ldc, sA, sB, sC;
     float alpha, beta;
+    int32_t c_vec;   // C base, leading dimension, slice stride and m allow aligned 16-byte stores
 };
 
 __device__ inline int rmaj_swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(Shape<LARGE>::THREADS, LARGE ? 1 : 2) void gemm16_k
 #pragma unroll
             for (int i = 0; i < BNB; i++)
 #pragma unroll
-                for (int j = 0; j < BM; j++) acc[i][j] = T::mfma32(bv[i], av[j], acc[i][j]);
+                for (int j = 0; j < BM; j++) acc[i][j] = T::mfma32(av[j], bv[i], acc[i][j]);
         }
         if (it + 1 < nk) {
             a.store(set_next, As + (buf ^ 1) * TILEB);
@@ -199,22 +201,57 @@ __global__ __launch_bounds__(Shape<LARGE>::THREADS, LARGE ? 1 : 2) void gemm16_k
     }
     if (it < nk) stage(it, 1);
 
-    // accumulator register v of lane (r, hh) of block (i, j): n = 32i + 8*(v/4) + 4*hh + v%4, m = 32j + r
+    // accumulator register v of lane (r, hh) of block (i, j): m = 32j + 8*(v/4) + 4*hh + v%4, n = 32i + r
     t *C = (t *)g.C + bz * g.sC;
+    const bool vec_ok = g.c_vec != 0;   // C columns can be written in aligned 16-byte pieces
 #pragma unroll
-    for (int j = 0; j < BM; j++) {
-        const int64_t mi = m0 + 32 * BM * wm + 32 * j + r;
-        if (mi >= g.m) continue;
+    for (int i = 0; i < BNB; i++) {
+        const int64_t nj = n0 + 32 * BNB * wn + 32 * i + r;
+        t *ccol = C + (nj < g.n ? nj : 0) * g.ldc;
 #pragma unroll
-        for (int i = 0; i < BNB; i++)
+        for (int j = 0; j < BM; j++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int64_t nj = n0 + 32 * BNB * wn + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
-                if (nj < g.n) {
-                    t *c = C + mi + nj * g.ldc;
-                    float val = g.alpha * acc[i][j][v];
-                    if (g.beta != 0.0f) val += g.beta * T::to_f32(*c);
-                    *c = T::from_f32(val);
+            for (int gp = 0; gp < 2; gp++) {
+                // X: m = mb + 4hh .. +3 (v = 8gp ..), Y: m = mb + 8 + 4hh .. +3 (v = 8gp + 4 ..)
+                const int64_t mb = m0 + 32 * BM * wm + 32 * j + 16 * gp;
+                float xv[4], yv[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    xv[e] = g.alpha * acc[i][j][8 * gp + e];
+                    yv[e] = g.alpha * acc[i][j][8 * gp + 4 + e];
+                }
+                if (vec_ok) {
+                    if (g.beta != 0.0f && nj < g.n) {
+                        if (mb + 4 * hh < g.m) {
+                            const typename T::vec4 c4 = *(const typename T::vec4 *)(ccol + mb + 4 * hh);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) xv[e] += g.beta * T::to_f32(c4[e]);
+                        }
+                        if (mb + 8 + 4 * hh < g.m) {
+                            const typename T::vec4 c4 = *(const typename T::vec4 *)(ccol + mb + 8 + 4 * hh);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) yv[e] += g.beta * T::to_f32(c4[e]);
+                        }
+                    }
+                    typename T::vec4 xe, yo;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        xe[e] = T::from_f32(xv[e]);
+                        yo[e] = T::from_f32(yv[e]);
+                    }
+                    const u32x2_t x = __builtin_bit_cast(u32x2_t, xe), y = __builtin_bit_cast(u32x2_t, yo);
+                    uint32_t x0 = x[0], x1 = x[1], y0 = y[0], y1 = y[1];
+                    mi_pair_halves(x0, y0);   // every lane takes part; lanes outside C do not store
+                    mi_pair_halves(x1, y1);
+                    const u32x4_t piece = {x0, x1, y0, y1};
+                    if (nj < g.n && mb + 8 * hh < g.m) *(u32x4_t *)(ccol + mb + 8 * hh) = piece;   // m is a multiple of 8 here
+                } else if (nj < g.n) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int64_t mx = mb + 4 * hh + e, my = mx + 8;
+                        if (mx < g.m) ccol[mx] = T::from_f32(g.beta != 0.0f ? xv[e] + g.beta * T::to_f32(ccol[mx]) : xv[e]);
+                        if (my < g.m) ccol[my] = T::from_f32(g.beta != 0.0f ? yv[e] + g.beta * T::to_f32(ccol[my]) : yv[e]);
+                    }
                 }
             }
     }
@@ -275,7 +312,8 @@ int32_t launch_batched_gemm16(int32_t dtype, int transA, int transB, int64_t m, 
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {   // gridDim.z is limited to 65535: issue the batch in slabs
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         Gemm16Args g = {(const char *)A + es * b0 * sA, (const char *)B + es * b0 * sB, (char *)C + es * b0 * sC,
-                        m, n, k, lda, ldb, ldc, sA, sB, sC, alpha, beta};
+                        m, n, k, lda, ldb, ldc, sA, sB, sC, alpha, beta,
+                        (int32_t)((((uintptr_t)C) & 15) == 0 && (ldc & 7) == 0 && (sC & 7) == 0 && (m & 7) == 0)};
         const int32_t rc = dtype == MI_F16 ? launch_t<F16>(g, transA, transB, nb, st) : launch_t<BF16>(g, transA, transB, nb, st);
         if (rc != MI_OK) return rc;
     }

@@ -100,6 +100,16 @@ __device__ static inline float mi_swap32(float x) {
     return __shfl_xor(x, 32, 64);
 }
 
+// Lanes l < 32 and l + 32 of a wavefront hold complementary halves of two 8-byte pieces: in the MFMA
+// accumulator layout lane l holds elements 0-3 of piece X and of piece Y, lane l + 32 elements 4-7 of
+// both.  After the exchange lane l holds all of X and lane l + 32 all of Y, as (x, y) = (first half,
+// second half), so each lane can store 16 contiguous bytes.  One v_permlane32_swap per register.
+__device__ static inline void mi_pair_halves(uint32_t &x, uint32_t &y) {
+    auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);   // x[32..63] <-> y[0..31]
+    x = r[0];
+    y = r[1];
+}
+
 __device__ static inline float mi_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // max(a, b, c) as one instruction with no quieting of the inputs (fmaxf on MFMA results costs an extra
