@@ -165,13 +165,15 @@ int32_t mi_attention_fwd(const mi_attn_desc *desc, mi_stream stream);
 int32_t mi_attention_stats_size(const mi_attn_desc *desc, size_t *bytes);
 
 /*
- * Gradient of one dot_product_attention call (fdrop = identity).  The reference has no hand-written
+ * Gradient of one dot_product_attention call (fdrop = identity or fused dropout).  The reference has no hand-written
  * rule: reverse-mode AD walks src/attention.jl:86-127 backwards through the rrule of batched_mul
  * (src/batched/batchedmul.jl:96-110) and _∇softmax! (src/softmax.jl:107-110); this entry point is
  * that chain fused, never materialising the (Lkv, Lq, H, B) tensors.  Its results are checked the
  * way the reference checks its gradients (test/attention.jl:70-76: against finite differences).
  *
- *   fwd      : the forward call (dtype, sizes, q, k, v, bias, mask, causal, flags).  fwd.out may
+ *   fwd      : the forward call (dtype, sizes, q, k, v, bias, mask, causal, flags, and dropout_p /
+ *              dropout_seed when the forward call dropped weights: the keep decisions are redrawn
+ *              from the same stream, and the pullback of dropout multiplies by them).  fwd.out may
  *              hold the forward RESULT x; the MFMA kernels (all three dtypes, head dim 64 or 128)
  *              need it and the call falls back to the generic kernels without it.  fwd.weights and fwd.workspace are ignored.
  *   dout     : (Ev, Lq, B) cotangent of x, `dtype`.

@@ -142,8 +142,6 @@ int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_back
     p.causal = d->causal != 0;
     if (!(d->dropout_p >= 0.0f && d->dropout_p <= 1.0f))
         return mi_set_error(MI_EINVAL, "dropout expects a probability 0 <= p <= 1");   // src/dropout.jl:43
-    if (for_backward && d->dropout_p != 0.0f)
-        return mi_set_error(MI_EINVAL, "mi_attention_bwd: the gradient of a call with fused dropout is not available");
     p.drop_key = mi_stream_key(d->dropout_seed, MI_DROPOUT_STREAM);
     p.drop_thresh = mi_dropout_threshold(d->dropout_p);
     p.drop_scale = d->dropout_p < 1.0f ? 1.0f / (1.0f - d->dropout_p) : 0.0f;

@@ -230,7 +230,12 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-                    for (int v = 0; v < 16; v++) s[0][kb][v] *= dp[kb][v] - delta;
+                    for (int v = 0; v < 16; v++) {
+                        // fused dropout: the forward multiplied the weight by g (0 or 1/(1-p)), its pullback multiplies dP
+                        float dpv = dp[kb][v];
+                        if (bp.p.drop_thresh) dpv *= attention_drop_factor(bp.p, j0 + 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4), qi, h, b);
+                        s[0][kb][v] *= dpv - delta;
+                    }
                     second_product<D>(kt, kb, s[0][kb], dq, r, hh);
                 }
             }
@@ -354,8 +359,10 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
                         if (m == MI_POS_INF) pw = x == MI_POS_INF ? linv4[e] : 0.0f;   // src/softmax.jl:74-75
                         else pw = mi_exp2(fmaf(x, cs, m == MI_NEG_INF ? 0.0f : -m)) * linv4[e];
                         pw = in ? pw : 0.0f;
-                        s[4 * g + e] = pw;
-                        if (DO_DK) dp[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
+                        // fused dropout: the value product saw pw * gd, and the pullback multiplies dP by gd
+                        const float gd = bp.p.drop_thresh ? attention_drop_factor(bp.p, kv, qi, h, b) : 1.0f;
+                        s[4 * g + e] = pw * gd;
+                        if (DO_DK) dp[4 * g + e] = pw * (gd * dp[4 * g + e] - delta4[e]);
                     }
                 }
                 if constexpr (DO_DV) second_product<D>(dot, kb, s, dv, r, hh);
@@ -421,7 +428,7 @@ int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) 
 
 template <int D>
 int32_t launch_d(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
-    const bool extras = bp.p.bias || bp.p.mask;
+    const bool extras = bp.p.bias || bp.p.mask || bp.p.drop_thresh;
     if (bp.p.causal) return extras ? launch_set<D, true, EXTRAS_DIRECT>(a, bp, st) : launch_set<D, true, EXTRAS_NONE>(a, bp, st);
     return extras ? launch_set<D, false, EXTRAS_DIRECT>(a, bp, st) : launch_set<D, false, EXTRAS_NONE>(a, bp, st);
 }
@@ -454,5 +461,6 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st) {
     a.tiles_per_split = 0;
     flash_fill_vec_flags(a);
     a.bias_lds = a.mask_lds = 0;
+    a.p.drop_thresh = 0;   // the shared softmax step yields the weights before dropout; the kernels apply bp.p's dropout themselves
     return bp.p.D == 64 ? launch_d<64>(a, bp, st) : launch_d<128>(a, bp, st);
 }

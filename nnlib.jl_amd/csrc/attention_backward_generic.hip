@@ -4,9 +4,10 @@
 //
 // The reference has no hand-written rule for attention; AD reverses src/attention.jl:86-127 through
 // the rrule of batched_mul (src/batched/batchedmul.jl:96-110) and _∇softmax! (src/softmax.jl:107-110).
-// With a = softmax weights, da[j,i] = v_j . dx_i (+ dweights[j,i]), delta_i = sum_j a da,
+// With a = softmax weights, g = the factor fused dropout multiplied them by (1 without dropout: the
+// forward used and returned a g), da[j,i] = g (v_j . dx_i + dweights[j,i]), delta_i = sum_j a da,
 // ds = a (da - delta):
-//   dv_j = sum_i a[j,i] dx_i      dk_j = sum_i ds[j,i] q_i / sqrt(D)      dq_i = sum_j ds[j,i] k_j / sqrt(D)
+//   dv_j = sum_i a g [j,i] dx_i    dk_j = sum_i ds[j,i] q_i / sqrt(D)      dq_i = sum_j ds[j,i] k_j / sqrt(D)
 //   dbias += ds (summed over the dims the bias broadcasts along)
 //
 // Two kernels: one workgroup per query row (statistics m, l, delta into the workspace, and dq), then
@@ -67,11 +68,13 @@ __global__ __launch_bounds__(256) void bwd_generic_query_kernel(AttnBwdParams bp
         return s;
     };
     auto dalpha = [&](int64_t j) -> float {
+        const float g = attention_drop_factor(p, j, i, h, b);
+        if (g == 0.0f) return 0.0f;
         const t *vj = v + p.Ev * j;
         float s = 0.0f;
         for (int d = 0; d < p.Dv; d++) s = fmaf(T::to_f32(vj[d]), dxs[d], s);
         if (dw) s += T::to_f32(dw[j]);
-        return s;
+        return g * s;
     };
 
     float m = MI_NEG_INF;
@@ -156,15 +159,19 @@ __global__ __launch_bounds__(256) void bwd_generic_key_kernel(AttnBwdParams bp) 
                 s = MI_NEG_INF;
             if (p.causal && j > i) s = MI_NEG_INF;
             a = term(s, stats[3 * i]) / stats[3 * i + 1];
+            const float g = attention_drop_factor(p, j, i, h, b);
             if (a != 0.0f) {
-                const t *dxi = dx + p.Ev * i;
                 float da = 0.0f;
-                for (int d = 0; d < p.Dv; d++) da = fmaf(vs[d], T::to_f32(dxi[d]), da);
-                if (bp.dweights) da += T::to_f32(((const t *)bp.dweights)[j + p.Lkv * (i + p.Lq * (h + p.H * b))]);
-                ds = a * (da - stats[3 * i + 2]);
+                if (g != 0.0f) {
+                    const t *dxi = dx + p.Ev * i;
+                    for (int d = 0; d < p.Dv; d++) da = fmaf(vs[d], T::to_f32(dxi[d]), da);
+                    if (bp.dweights) da += T::to_f32(((const t *)bp.dweights)[j + p.Lkv * (i + p.Lq * (h + p.H * b))]);
+                }
+                ds = a * (g * da - stats[3 * i + 2]);
             } else if (a != a) {
                 ds = a;
             }
+            a *= g;   // the value product used the weights after dropout
             if (bp.dbias && ds != 0.0f)
                 atomicAdd(bp.dbias + j * p.bias_strides[0] + i * p.bias_strides[1] + h * p.bias_strides[2] + b * p.bias_strides[3], ds);
         }

@@ -19,6 +19,14 @@ struct AttnParams {
     float drop_scale;
 };
 
+#ifdef __HIPCC__
+// factor fused dropout multiplies weight (kv, q, h, b) by: 0 (dropped), drop_scale (kept), 1 without dropout
+__device__ inline float attention_drop_factor(const AttnParams &p, int64_t kv, int64_t q, int64_t h, int64_t b) {
+    if (p.drop_thresh == 0) return 1.0f;
+    return mi_dropout_keep(p.drop_key, (uint64_t)(kv + p.Lkv * (q + p.Lq * (h + p.H * b))), p.drop_thresh) ? p.drop_scale : 0.0f;
+}
+#endif
+
 // One backward call: the forward call it differentiates plus cotangents and gradient buffers.
 struct AttnBwdParams {
     AttnParams p;

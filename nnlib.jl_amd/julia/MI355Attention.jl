@@ -260,22 +260,26 @@ function dot_product_attention_scores(q::DeviceArray{T, 4}, k::DeviceArray{T, 4}
     return fdrop isa Dropout ? α : fdrop(α)
 end
 
-# Pullback of dot_product_attention(q, k, v, bias; mask, nheads) with fdrop = identity: returns
-# (dq, dk, dv, dbias) for the cotangent dy of the output (and optionally dα of the returned weights).
+# Pullback of dot_product_attention(q, k, v, bias; fdrop, mask, nheads) for fdrop = identity or the
+# Dropout(p, seed) the forward call got (the keep decisions repeat): returns (dq, dk, dv, dbias) for the
+# cotangent dy of the output (and optionally dα of the returned weights).
 # NNlib gets these from AD through src/attention.jl:86-127 (rrule of batched_mul,
-# src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110).  `y` is the forward result;
+# src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110; the pullback of dropout
+# multiplies by the mask it drew, src/dropout.jl:38-53).  `y` is the forward result;
 # passing it lets the MFMA kernels run.  A ChainRulesCore.rrule for DeviceArray arguments is three lines
 # on top of this function: call the forward, close over (q, k, v, bias, y), return this pullback.
 function ∇dot_product_attention(dy::DeviceArray{T, 3}, q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::DeviceArray{T, 3},
-                                bias = nothing; y = nothing, dα = nothing, mask = nothing, nheads = 1, stats = nothing) where {T <: MIFloat}
+                                bias = nothing; y = nothing, dα = nothing, mask = nothing, nheads = 1, stats = nothing,
+                                fdrop::Union{typeof(identity), Dropout} = identity) where {T <: MIFloat}
     E, Lq, B = size(q); Lkv = size(k, 2); Ev = size(v, 1)
     size(dy) == (Ev, Lq, B) || throw(DimensionMismatch("dy must have the size of the output $((Ev, Lq, B)), got $(size(dy))"))
     causal, mptr, mstr, bptr, bstr = mask_and_bias(T, bias, mask, (Lkv, Lq, nheads, B))
     dq, dk, dv = similar(q, T, size(q)), similar(k, T, size(k)), similar(v, T, size(v))
     dbias = bias === nothing ? nothing : DeviceArray{Float32}(undef, size(bias)...)
     dbias === nothing || check(ccall((:mi_fill_zero, libmi), Int32, (Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), dbias.ptr, sizeof(Float32) * length(dbias), C_NULL))
+    p, seed = fdrop isa Dropout ? (fdrop.p, fdrop.seed) : (0f0, UInt64(0))
     fwd = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0), E, Ev, Lq, Lkv, nheads, B,
-                   q.ptr, k.ptr, v.ptr, y === nothing ? C_NULL : y.ptr, C_NULL, bptr, bstr, mptr, mstr, C_NULL, 0, 0f0, UInt32(0), UInt64(0), stats === nothing ? C_NULL : stats.ptr)
+                   q.ptr, k.ptr, v.ptr, y === nothing ? C_NULL : y.ptr, C_NULL, bptr, bstr, mptr, mstr, C_NULL, 0, p, UInt32(0), seed, stats === nothing ? C_NULL : stats.ptr)
     mk(ws, wsbytes) = AttnBwdDesc(Int32(sizeof(AttnBwdDesc)), Int32(0), fwd, dy.ptr, dα === nothing ? C_NULL : dα.ptr, dq.ptr, dk.ptr,
                                   dv.ptr, dbias === nothing ? C_NULL : dbias.ptr, ws, wsbytes)
     need = Ref{Csize_t}(0)

@@ -225,12 +225,15 @@ def last_attention_bwd_kernel():
     return _lib.KERNEL_NAMES.get(_last_bwd_kernel)
 
 
-def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, mask=None, nheads=1, _flags=0):
-    """Pullback of ``dot_product_attention(q, k, v, bias; mask, nheads)`` with ``fdrop = identity``:
+def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, mask=None, nheads=1, fdrop=identity,
+                               _flags=0):
+    """Pullback of ``dot_product_attention(q, k, v, bias; fdrop, mask, nheads)`` for ``fdrop = identity`` or
+    a ``Dropout(p, seed)`` (the same object the forward call got, so that the keep decisions repeat):
     given the cotangent ``dy`` of the output (and optionally ``dalpha`` of the returned weights) it
     returns ``(dq, dk, dv, dbias)``; ``dbias`` is ``None`` without a bias and has the bias's size
     otherwise (Float32).  The reference gets the same values from AD through src/attention.jl:86-127
-    (rrule of batched_mul, src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110).
+    (rrule of batched_mul, src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110; the
+    pullback of dropout multiplies by the mask it drew, src/dropout.jl:38-53).
     ``y`` is the forward result; passing it lets the MFMA kernels run."""
     global _last_bwd_kernel
     B, E, Ev, Lq, Lkv, bq = _check_qkv(q, k, v, nheads)
@@ -240,7 +243,9 @@ def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, m
     lib = _lib.load()
     d = _lib.mi_attn_bwd_desc()
     d.struct_size = ctypes.sizeof(_lib.mi_attn_bwd_desc)
-    _fill_desc(d.fwd, q, k, v, bias, mask, nheads, B, E, Ev, Lq, Lkv, _flags)
+    if fdrop is not identity and not isinstance(fdrop, Dropout):
+        raise ArgumentError("the fused gradient takes fdrop = identity or a Dropout(p, seed)")
+    _fill_desc(d.fwd, q, k, v, bias, mask, nheads, B, E, Ev, Lq, Lkv, _flags, fdrop if isinstance(fdrop, Dropout) else None)
     if y is not None:
         y = _contig(y, "y")
         if y.dims != dy.dims or y.dtype != q.dtype:

@@ -16,6 +16,12 @@
  *
  * An optional cotangent of the returned weights is added to d_alpha (the forward returns (x, alpha)).
  *
+ * fdrop = dropout (src/attention.jl:126, src/dropout.jl:38-53) multiplies alpha elementwise by a fixed
+ * array g (0 where dropped, 1/(1-p) where kept) before the value product and before alpha is returned;
+ * its pullback multiplies the cotangent by the same g:
+ *   alpha_d = alpha .* g,  x = batched_mul(vt, alpha_d)  -> d_alpha = g .* (vt' * dx + d_returned)
+ * `keep_scale` is that g (NULL = identity).
+ *
  * Pinned by (tests/test_attention_backward_oracle.py): central finite differences of the forward
  * oracle (itself pinned by the golden vectors of test/attention.jl:25-34) for q, k, v and bias, on the
  * reference's own gradient-test shapes (test/attention.jl:70-76), with masks, causal masks and
@@ -29,13 +35,13 @@
 
 #define ORC_API __attribute__((visibility("default")))
 
-/* alpha: (Lkv, Lq, H, B) forward weights (from orc_attention_f64).
- * dout: (Ev, Lq, B); dweights: NULL or (Lkv, Lq, H, B).
+/* alpha: (Lkv, Lq, H, B) forward weights before dropout (from orc_attention_f64).
+ * dout: (Ev, Lq, B); dweights, keep_scale: NULL or (Lkv, Lq, H, B).
  * dq (E, Lq, B), dk (E, Lkv, B), dv (Ev, Lkv, B): overwritten.
  * dbias: NULL, or an array addressed with bias_strides (0 = broadcast dim, summed); ADDED into. */
 ORC_API void orc_attention_bwd_f64(const double *q, const double *k, const double *v,
                                    const double *alpha, const double *dout, const double *dweights,
-                                   const int64_t *bias_strides, int64_t E, int64_t Ev, int64_t Lq,
+                                   const double *keep_scale, const int64_t *bias_strides, int64_t E, int64_t Ev, int64_t Lq,
                                    int64_t Lkv, int64_t H, int64_t B, double *dq, double *dk,
                                    double *dv, double *dbias)
 {
@@ -56,12 +62,14 @@ ORC_API void orc_attention_bwd_f64(const double *q, const double *k, const doubl
                 for (int64_t j = 0; j < Lkv; j++) {
                     const double *vj = v + Dv * h + Ev * (j + Lkv * b);
                     double *dvj = dv + Dv * h + Ev * (j + Lkv * b);
+                    const double g = keep_scale ? keep_scale[j + Lkv * (i + Lq * (h + H * b))] : 1.0;
                     double s = 0.0;
                     for (int64_t d = 0; d < Dv; d++) {
-                        s += vj[d] * dx[d];      /* d_alpha = vt' * dx */
-                        dvj[d] += a[j] * dx[d];  /* dvt = dx * alpha'  */
+                        s += vj[d] * dx[d];          /* d_alpha_d = vt' * dx  */
+                        dvj[d] += a[j] * g * dx[d];  /* dvt = dx * alpha_d'   */
                     }
                     if (dweights) s += dweights[j + Lkv * (i + Lq * (h + H * b))];
+                    s *= g;                          /* pullback of alpha .* g */
                     da[j] = s;
                     dot += s * a[j];
                 }

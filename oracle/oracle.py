@@ -49,7 +49,7 @@ def lib():
         L.orc_nnlib_attention_f32.restype = None
         L.orc_attention_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp]
         L.orc_attention_f64.restype = None
-        L.orc_attention_bwd_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp, vp]
+        L.orc_attention_bwd_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp, vp]
         L.orc_attention_bwd_f64.restype = None
         for suf in ("f32", "f64"):
             getattr(L, "orc_softmax_nd_" + suf).argtypes = [ci, vp, vp, i64, i64, i64]
@@ -254,10 +254,11 @@ def scores4_f64(q4, k4, bias=None, mask=None):
     return _attention(q3, k3, None, bias, mask, H, np.float64, False, 1)[1]
 
 
-def attention_bwd_f64(q, k, v, dout, bias=None, mask=None, nheads=1, dweights=None):
+def attention_bwd_f64(q, k, v, dout, bias=None, mask=None, nheads=1, dweights=None, keep_scale=None):
     """Gradient of dot_product_attention with respect to q, k, v and bias, given the cotangent ``dout``
     of the output (and optionally ``dweights`` of the returned weights): the reverse of the op chain of
-    src/attention.jl:86-127.  Returns (dq, dk, dv, dbias); dbias has the shape of ``bias`` (None without)."""
+    src/attention.jl:86-127.  ``keep_scale``: the (Lkv, Lq, H, B) factor a dropout ``fdrop`` multiplied the
+    weights by (0 or 1/(1-p)).  Returns (dq, dk, dv, dbias); dbias has the shape of ``bias`` (None without)."""
     f8 = np.float64
     bshape = tuple(np.shape(q)[2:])
     q3, k3, v3, do3 = (_f(_flatten3(a), f8) for a in (q, k, v, dout))
@@ -267,17 +268,18 @@ def attention_bwd_f64(q, k, v, dout, bias=None, mask=None, nheads=1, dweights=No
     alpha = _f(alpha.reshape(Lkv, Lq, H, B, order="F"), f8)
     dq, dk, dv = (np.empty(a.shape, dtype=f8, order="F") for a in (q3, k3, v3))
     dw = None if dweights is None else _f(np.asarray(dweights).reshape(Lkv, Lq, H, B, order="F"), f8)
+    ks = None if keep_scale is None else _f(np.asarray(keep_scale).reshape(Lkv, Lq, H, B, order="F"), f8)
     db = bs = None
     if bias is not None:
         db = np.zeros(np.shape(bias), dtype=f8, order="F")
         bs = broadcast_strides(db.shape)
-    lib().orc_attention_bwd_f64(_ptr(q3), _ptr(k3), _ptr(v3), _ptr(alpha), _ptr(do3), _ptr(dw), bs,
+    lib().orc_attention_bwd_f64(_ptr(q3), _ptr(k3), _ptr(v3), _ptr(alpha), _ptr(do3), _ptr(dw), _ptr(ks), bs,
                                 E, Ev, Lq, Lkv, H, B, _ptr(dq), _ptr(dk), _ptr(dv), _ptr(db))
     return (dq.reshape(np.shape(q), order="F"), dk.reshape(np.shape(k), order="F"),
             dv.reshape(np.shape(v), order="F"), db)
 
 
-def numpy_attention_bwd(q, k, v, dout, bias=None, mask=None, nheads=1, dweights=None):
+def numpy_attention_bwd(q, k, v, dout, bias=None, mask=None, nheads=1, dweights=None, keep_scale=None):
     """Independent einsum statement of the same gradient (no C involved)."""
     f8 = np.float64
     q3, k3, v3, do3 = (_flatten3(np.asarray(a, dtype=f8)) for a in (q, k, v, dout))
@@ -291,7 +293,9 @@ def numpy_attention_bwd(q, k, v, dout, bias=None, mask=None, nheads=1, dweights=
     da = np.einsum("dhjb,dhib->jihb", v4, do4)
     if dweights is not None:
         da = da + np.asarray(dweights, dtype=f8).reshape(Lkv, Lq, H, B, order="F")
-    dv4 = np.einsum("jihb,dhib->dhjb", alpha, do4)
+    g = 1.0 if keep_scale is None else np.asarray(keep_scale, dtype=f8).reshape(Lkv, Lq, H, B, order="F")
+    dv4 = np.einsum("jihb,dhib->dhjb", alpha * g, do4)
+    da = da * g
     dl = alpha * (da - (alpha * da).sum(axis=0, keepdims=True))
     c = 1.0 / np.sqrt(f8(D))
     dq4 = c * np.einsum("jihb,dhjb->dhib", dl, k4)

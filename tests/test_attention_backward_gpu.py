@@ -11,7 +11,7 @@ TOL = {"f32": 1e-4, "f16": 1e-2, "bf16": 1e-2}
 
 
 def _run(nn, oracle, dtype, E, Ev, Lq, Lkv, batch, H, bias_shape=None, mask_kind=None, with_dalpha=False, flags=0,
-         seed=0, scale=1.0, expect=None, pass_y=True):
+         seed=0, scale=1.0, expect=None, pass_y=True, dropout=None, saved=False):
     rng = np.random.default_rng(seed)
     q = round_to(rng.standard_normal((E, Lq) + batch) * scale, dtype)
     k = round_to(rng.standard_normal((E, Lkv) + batch) * scale, dtype)
@@ -31,13 +31,19 @@ def _run(nn, oracle, dtype, E, Ev, Lq, Lkv, batch, H, bias_shape=None, mask_kind
     dq_, dk_, dv_ = D(q, dtype), D(k, dtype), D(v, dtype)
     dbias_ = None if bias is None else D(bias, dtype)
     y = None
+    fdrop, keep_scale = nn.identity, None
+    if dropout is not None:
+        p, dseed = dropout
+        fdrop = nn.Dropout(p, dseed)
+        keep_scale = oracle.dropout_keep_mask((Lkv, Lq, H) + batch, p, dseed) / (1.0 - p)
     if pass_y:
-        y, _ = nn.dot_product_attention(dq_, dk_, dv_, dbias_, mask=dmask, nheads=H, return_weights=False)
+        y, _ = nn.dot_product_attention(dq_, dk_, dv_, dbias_, mask=dmask, nheads=H, return_weights=False, fdrop=fdrop,
+                                        save_for_backward=saved)
     got = nn.dot_product_attention_grad(D(dy, dtype), dq_, dk_, dv_, dbias_, y=y, mask=dmask, nheads=H,
-                                        dalpha=None if da is None else D(da, dtype), _flags=flags)
+                                        dalpha=None if da is None else D(da, dtype), fdrop=fdrop, _flags=flags)
     if expect is not None:
         assert nn.last_attention_bwd_kernel() == expect, nn.last_attention_bwd_kernel()
-    ref = oracle.attention_bwd_f64(q, k, v, dy, bias, mask, H, da)
+    ref = oracle.attention_bwd_f64(q, k, v, dy, bias, mask, H, da, keep_scale=keep_scale)
     errs = []
     for g, r, name in zip(got, ref, ("dq", "dk", "dv", "dbias")):
         if r is None:
@@ -223,6 +229,61 @@ def test_fully_masked_query_gives_nan_gradients(nn):
     dq, dk = dq.to_numpy(), dk.to_numpy()
     assert np.isnan(dq[:, 2, 1]).all() and np.isfinite(dq[:, :, 0]).all() and np.isfinite(dq[:, [0, 1, 3], 1]).all()
     assert np.isnan(dk[:, :, 1]).all() and np.isfinite(dk[:, :, 0]).all()
+
+
+@pytest.mark.parametrize("dtype,E,H,Lq,Lkv,batch,mask_kind,bias_shape,with_dalpha,saved,expect", [
+    ("f32", 12, 2, 9, 7, (2,), None, (7, 9), True, False, "generic"),            # odd head dim, bias gradient, weight cotangent
+    ("f32", 12, 3, 6, 6, (1,), "causal", None, False, False, "generic"),
+    ("bf16", 128, 2, 150, 200, (2,), None, None, False, False, "flash16"),       # D = 64
+    ("bf16", 256, 2, 192, 192, (1,), "causal", None, False, True, "flash16"),    # D = 128, statistics from the forward call
+    ("f16", 256, 2, 70, 300, (2,), "random", None, False, False, "flash16"),
+    ("f16", 128, 2, 130, 130, (1,), "causal", (130, 130, 2, 1), False, False, "flash16"),
+    ("f32", 128, 2, 150, 200, (2,), None, None, False, True, "flash32"),         # D = 64
+    ("f32", 256, 2, 192, 192, (1,), "causal", None, False, False, "flash32"),    # D = 128
+    ("f32", 128, 2, 70, 300, (1,), "random", None, False, False, "flash32"),
+])
+def test_gradient_through_fused_dropout(nn, oracle, dtype, E, H, Lq, Lkv, batch, mask_kind, bias_shape, with_dalpha, saved,
+                                        expect):
+    """fdrop = Dropout(p, seed) in the forward call: the pullback redraws the same keep decisions
+    (src/attention.jl:126, src/dropout.jl:38-53; oracle pinned by finite differences with the mask held fixed)."""
+    if bias_shape is not None and expect != "generic":
+        # a bias input without a bias gradient: the MFMA kernels' bias path
+        _bias_input_case(nn, oracle, dtype, E, H, Lq, Lkv, batch, mask_kind, bias_shape, expect)
+        return
+    _run(nn, oracle, dtype, E, E, Lq, Lkv, batch, H, bias_shape=bias_shape, mask_kind=mask_kind, with_dalpha=with_dalpha,
+         expect=expect, dropout=(0.25, 4242), saved=saved, seed=5)
+
+
+def _bias_input_case(nn, oracle, dtype, E, H, Lq, Lkv, batch, mask_kind, bias_shape, expect):
+    rng = np.random.default_rng(17)
+    q, k, v, dy = (round_to(rng.standard_normal((E, L) + batch), dtype) for L in (Lq, Lkv, Lkv, Lq))
+    bias = round_to(rng.standard_normal(bias_shape) * 0.5, dtype)
+    mask = oracle.make_causal_mask(Lq) if mask_kind == "causal" else None
+    dmask = nn.make_causal_mask(nn.DeviceArray.zeros((1, Lq))) if mask_kind == "causal" else None
+    D = nn.DeviceArray.from_numpy
+    fdrop = nn.Dropout(0.25, 777)
+    g = oracle.dropout_keep_mask((Lkv, Lq, H) + batch, 0.25, 777) / 0.75
+    dq_, dk_, dv_, db_ = D(q, dtype), D(k, dtype), D(v, dtype), D(bias, dtype)
+    y, _ = nn.dot_product_attention(dq_, dk_, dv_, db_, mask=dmask, nheads=H, return_weights=False, fdrop=fdrop)
+    lib = nn._lib.load()
+    import ctypes
+    d = nn._lib.mi_attn_bwd_desc()
+    d.struct_size = ctypes.sizeof(nn._lib.mi_attn_bwd_desc)
+    B = int(np.prod(batch))
+    nn.ops._fill_desc(d.fwd, dq_, dk_, dv_, db_, dmask, H, B, E, E, Lq, Lkv, 0, fdrop)
+    ddy = D(dy, dtype)
+    d.fwd.out, d.dout = y.ptr, ddy.ptr
+    outs = [nn.DeviceArray.empty(a.shape, dtype) for a in (q, k, v)]
+    d.dq, d.dk, d.dv = (o.ptr for o in outs)
+    kern, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
+    nn._lib.check(lib.mi_attention_bwd_plan(ctypes.byref(d), ctypes.byref(kern), ctypes.byref(ws)))
+    assert nn._lib.KERNEL_NAMES[kern.value] == expect
+    wsbuf = nn.DeviceArray.empty((ws.value // 4 + 4,), "f32")
+    d.workspace, d.workspace_bytes = wsbuf.ptr, ws.value
+    nn._lib.check(lib.mi_attention_bwd(ctypes.byref(d), None))
+    ref = oracle.attention_bwd_f64(q, k, v, dy, bias, mask, H, keep_scale=g)
+    for o, r in zip(outs, ref[:3]):
+        assert np.abs(o.to_numpy() - r).max() / max(np.abs(r).max(), 0.05) <= TOL[dtype]
 
 
 def test_errors(nn):
