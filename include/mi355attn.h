@@ -252,10 +252,24 @@ int32_t mi_batched_gemm(int32_t dtype, char transA, char transB, int64_t m, int6
                         int64_t ldb, int64_t strideB, float beta, void *C, int64_t ldc,
                         int64_t strideC, int64_t batch, mi_stream stream);
 
+/* ComplexF32 batched_mul: C = alpha * op(A) * op(B) + beta * C per batch slice, complex alpha and beta.
+ * Arrays hold interleaved (re, im) Float32 pairs, as Julia stores ComplexF32.  Every operand is given
+ * by the ELEMENT strides of its (row, column, batch) indices AFTER op: op(A) is m x k, op(B) is k x n;
+ * conj_a / conj_b conjugate the operand.  'N' is (1, ld), 'T' is (ld, 1), 'C' is 'T' with conj: what the
+ * reference passes to cgemm (src/gemm.jl:31, flags chosen at src/batched/batchedmul.jl:261-296, 'C' for
+ * a BatchedAdjoint{<:Complex}); any other strides are the layouts it gives to batched_mul_generic!
+ * (src/batched/batchedmul.jl:306-325).  A batch stride of 0 shares one slice (src/gemm.jl:117-118).
+ * beta == 0 overwrites C without reading it. */
+int32_t mi_batched_mul_c32(int64_t m, int64_t n, int64_t k, float alpha_re, float alpha_im, const void *A,
+                           int64_t a_row_stride, int64_t a_col_stride, int64_t a_batch_stride, int32_t conj_a,
+                           const void *B, int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride,
+                           int32_t conj_b, float beta_re, float beta_im, void *C, int64_t c_row_stride,
+                           int64_t c_col_stride, int64_t c_batch_stride, int64_t batch, mi_stream stream);
+
 /* ---- materialising lazy views ------------------------------------------------------ */
 /* dst (contiguous column-major d0 x d1 x d2) = src read with element strides (s0, s1, s2): the copy(X)
  * the reference makes of a PermutedDimsArray / transposed view before a BLAS call cannot address it
- * (_copy_if_faster, src/batched/batchedmul.jl:76-83).  elem_bytes is 1, 2 or 4. */
+ * (_copy_if_faster, src/batched/batchedmul.jl:76-83).  elem_bytes is 1, 2, 4 or 8. */
 int32_t mi_strided_copy(void *dst, const void *src, int32_t elem_bytes, int64_t d0, int64_t d1, int64_t d2,
                         int64_t s0, int64_t s1, int64_t s2, mi_stream stream);
 

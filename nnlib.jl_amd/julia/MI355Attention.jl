@@ -11,7 +11,7 @@
 #   logsoftmax, logsoftmax!, logsumexp                             NNlib src/softmax.jl:133-147,200-203
 #   ∇softmax, ∇softmax!, ∇logsoftmax, ∇logsoftmax!                 NNlib src/softmax.jl:87-110,155-177
 #   batched_mul(A, B), batched_mul!(C, A, B, alpha, beta)          NNlib src/batched/batchedmul.jl:47-60,238-254
-#   batched_transpose, batched_adjoint                             NNlib src/batched/batchedadjtrans.jl:37-52
+#   batched_transpose, batched_adjoint (ComplexF32: BatchedAdjoint) NNlib src/batched/batchedadjtrans.jl:37-52
 #   batched_vec, matrix x 3-array forms of batched_mul             NNlib src/batched/batchedmul.jl:140-218
 #   Dropout(p, seed) as fdrop, dropout(x, p)                       NNlib src/dropout.jl:38-53
 #   ∇dot_product_attention, batched_mul_pullback                   what AD derives from src/attention.jl:86-127
@@ -83,7 +83,7 @@ function free!(a::DeviceArray)
     nothing
 end
 
-function DeviceArray(h::Array{T, N}) where {T <: Union{MIFloat, Bool}, N}
+function DeviceArray(h::Array{T, N}) where {T <: Union{MIFloat, Bool, ComplexF32}, N}
     d = DeviceArray{T}(undef, size(h)...)
     check(ccall((:mi_memcpy_h2d, libmi), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), d.ptr, h, sizeof(h), C_NULL))
     d
@@ -113,6 +113,16 @@ end
 batched_transpose(a::DeviceArray{T, 3}) where {T} =
     DeviceArray{T, 3}(a.ptr, (a.dims[2], a.dims[1], a.dims[3]), (a.strides[2], a.strides[1], a.strides[3]), a)
 batched_adjoint(a::DeviceArray{<:Real, 3}) = batched_transpose(a)
+
+# Complex arrays: the per-slice conjugate transpose is a wrapper, outermost as in the reference
+# (src/batched/batchedadjtrans.jl:23-52, src/batched/batchedmul.jl:234); the kernel reads it conjugated.
+struct BatchedAdjoint{T <: Complex} <: AbstractArray{T, 3}
+    parent::DeviceArray{T, 3}
+end
+batched_adjoint(a::DeviceArray{T, 3}) where {T <: Complex} = BatchedAdjoint{T}(a)
+batched_adjoint(a::BatchedAdjoint) = a.parent
+Base.size(a::BatchedAdjoint) = (size(a.parent, 2), size(a.parent, 1), size(a.parent, 3))
+Base.getindex(::BatchedAdjoint, I...) = error("scalar indexing of a device array is not supported")
 
 # ---- masks -----------------------------------------------------------------------------------------
 # make_causal_mask on a device array returns this lazy stand-in for triu(trues(len, len)); the kernel
@@ -401,6 +411,31 @@ function batched_mul!(C::DeviceArray{T, 3}, A::DeviceArray{T, 3}, B::DeviceArray
     GC.@preserve A B C gemm!(tA, tB, m, n, ka, Float32(α), A.ptr, lda, sA, B.ptr, ldb, sB, Float32(β), C.ptr,
                               max(strides(C)[2], m, 1), strides(C)[3], size(C, 3), T)
     C
+end
+
+# ComplexF32 (cgemm in the reference, src/gemm.jl:31): one strided kernel takes 'N', 'T', 'C' and every
+# permuted layout of A, B and C (the cases of src/batched/batchedmul.jl:261-296 and the generic fallback :306-325)
+const CArr = Union{DeviceArray{ComplexF32, 3}, BatchedAdjoint{ComplexF32}}
+operand(a::DeviceArray{ComplexF32, 3}) = (a.ptr, strides(a)[1], strides(a)[2], strides(a)[3], Int32(0))
+operand(a::BatchedAdjoint{ComplexF32}) = (a.parent.ptr, strides(a.parent)[2], strides(a.parent)[1], strides(a.parent)[3], Int32(1))
+function batched_mul!(C::DeviceArray{ComplexF32, 3}, A::CArr, B::CArr, α::Number = true, β::Number = false)
+    size(A, 3) == size(C, 3) || size(A, 3) == 1 || throw(DimensionMismatch("batch size mismatch: A != C"))
+    size(B, 3) == size(C, 3) || size(B, 3) == 1 || throw(DimensionMismatch("batch size mismatch: B != C"))
+    m, ka = size(A, 1), size(A, 2); kb, n = size(B, 1), size(B, 2)
+    (ka == kb && m == size(C, 1) && n == size(C, 2)) ||
+        throw(DimensionMismatch("A1 has size ($m,$ka), B1 has size ($kb,$n), C1 has size $(size(C)[1:2])"))
+    (pa, ar, ac, ab, ca), (pb, br, bc, bb, cb) = operand(A), operand(B)
+    al, be = ComplexF32(α), ComplexF32(β)
+    GC.@preserve A B C check(ccall((:mi_batched_mul_c32, libmi), Int32,
+        (Int64, Int64, Int64, Float32, Float32, Ptr{Cvoid}, Int64, Int64, Int64, Int32, Ptr{Cvoid}, Int64, Int64, Int64, Int32,
+         Float32, Float32, Ptr{Cvoid}, Int64, Int64, Int64, Int64, Ptr{Cvoid}),
+        m, n, ka, real(al), imag(al), pa, ar, ac, size(A, 3) == 1 ? 0 : ab, ca, pb, br, bc, size(B, 3) == 1 ? 0 : bb, cb,
+        real(be), imag(be), C.ptr, strides(C)[1], strides(C)[2], strides(C)[3], size(C, 3), C_NULL); shape_error = DimensionMismatch)
+    C
+end
+function batched_mul(A::CArr, B::CArr)
+    size(A, 3) == size(B, 3) || size(A, 3) == 1 || size(B, 3) == 1 || throw(DimensionMismatch("batch size mismatch: A != B"))
+    batched_mul!(DeviceArray{ComplexF32}(undef, size(A, 1), size(B, 2), max(size(A, 3), size(B, 3))), A, B)
 end
 
 # lazy PermutedDimsArray(A, perm) and matrix transpose: same memory, permuted size and strides

@@ -9,10 +9,10 @@ import torch
 
 from . import _lib
 
-_TORCH = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "bool": torch.uint8}
+_TORCH = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "bool": torch.uint8, "c64": torch.complex64}
 _CODE = {"f32": _lib.MI_F32, "f16": _lib.MI_F16, "bf16": _lib.MI_BF16}
 _NP2NAME = {np.dtype(np.float32): "f32", np.dtype(np.float16): "f16", np.dtype(np.bool_): "bool",
-            np.dtype(np.uint8): "bool"}
+            np.dtype(np.uint8): "bool", np.dtype(np.complex64): "c64", np.dtype(np.complex128): "c64"}
 
 
 def _require_gpu():
@@ -30,7 +30,8 @@ class DeviceArray:
     def __init__(self, storage, dims, dtype, strides=None, offset=0):
         self.storage = storage          # 1-D torch tensor that owns the memory
         self.dims = tuple(int(d) for d in dims)
-        self.dtype = dtype              # "f32" | "f16" | "bf16" | "bool"
+        self.dtype = dtype              # "f32" | "f16" | "bf16" | "bool" | "c64" (ComplexF32: batched_mul only)
+        self.conj = False               # set by batched_adjoint of a complex array: elements read conjugated
         if strides is None:
             strides, acc = [], 1
             for d in self.dims:
@@ -65,6 +66,8 @@ class DeviceArray:
         if dtype == "bool":
             flat = np.ascontiguousarray(a.astype(np.uint8).ravel(order="F"))
             t = torch.from_numpy(flat).cuda()
+        elif dtype == "c64":
+            t = torch.from_numpy(np.ascontiguousarray(a.astype(np.complex64).ravel(order="F"))).cuda()
         else:
             src = a.astype(np.float32) if a.dtype not in (np.float32, np.float16) else a
             flat = np.ascontiguousarray(src.ravel(order="F"))
@@ -106,7 +109,9 @@ class DeviceArray:
             dims = tuple(self.length // max(known, 1) if d == -1 else d for d in dims)
         assert self.is_contiguous(), "reshape needs a contiguous array"
         assert int(np.prod(dims, dtype=np.int64)) == self.length, "reshape must keep the element count"
-        return DeviceArray(self.storage, dims, self.dtype, None, self.offset)
+        out = DeviceArray(self.storage, dims, self.dtype, None, self.offset)
+        out.conj = self.conj
+        return out
 
     def permuted(self, *perm):
         """Lazy ``PermutedDimsArray(A, perm)`` (1-based ``perm`` as in Julia): same memory, permuted
@@ -114,13 +119,17 @@ class DeviceArray:
         if len(perm) == 1 and isinstance(perm[0], (tuple, list)):
             perm = tuple(perm[0])
         assert sorted(perm) == list(range(1, self.ndim + 1)), "perm must be a permutation of 1:ndims"
-        return DeviceArray(self.storage, [self.dims[p - 1] for p in perm], self.dtype,
-                           [self.strides[p - 1] for p in perm], self.offset)
+        out = DeviceArray(self.storage, [self.dims[p - 1] for p in perm], self.dtype,
+                          [self.strides[p - 1] for p in perm], self.offset)
+        out.conj = self.conj
+        return out
 
     def with_trailing(self, n):
         """Same memory viewed with ``n`` extra trailing dimensions of extent 1 (``reshape(A, size(A)..., 1)``
         for views whose strides must be kept)."""
-        return DeviceArray(self.storage, self.dims + (1,) * n, self.dtype, self.strides + (self.length,) * n, self.offset)
+        out = DeviceArray(self.storage, self.dims + (1,) * n, self.dtype, self.strides + (self.length,) * n, self.offset)
+        out.conj = self.conj
+        return out
 
     def copy(self):
         """Dense column-major copy (``copy(X)`` / ``permutedims``): materialises a lazy view of up to 3 dims."""
@@ -129,6 +138,8 @@ class DeviceArray:
         s = self.strides + (0,) * (3 - self.ndim)
         out = DeviceArray.empty(self.dims, self.dtype)
         _lib.check(_lib.load().mi_strided_copy(out.ptr, self.ptr, self.itemsize, d[0], d[1], d[2], s[0], s[1], s[2], None))
+        if self.conj:
+            out.storage.copy_(torch.conj_physical(out.storage))
         return out
 
     @property
@@ -141,11 +152,16 @@ class DeviceArray:
 
     @property
     def code(self):
+        if self.dtype not in _CODE:
+            raise _lib.ArgumentError(f"this operation takes Float32, Float16 or BFloat16 arrays, got {self.dtype}")
         return _CODE[self.dtype]
 
     # ---- host copies ---------------------------------------------------------------------
     def to_numpy(self):
         """Julia-shaped numpy array (Fortran order). bf16 comes back as float32, bool as bool."""
+        if self.conj:
+            plain = DeviceArray(self.storage, self.dims, self.dtype, self.strides, self.offset)
+            return np.conj(plain.to_numpy())
         if not self.is_contiguous():
             return self.copy().to_numpy()
         flat = self.storage[self.offset:self.offset + self.length]
@@ -168,11 +184,12 @@ class BatchedTranspose(DeviceArray):
         d, s = parent.dims, parent.strides
         super().__init__(parent.storage, (d[1], d[0], d[2]), parent.dtype, (s[1], s[0], s[2]), parent.offset)
         self.parent = parent
+        self.conj = parent.conj
 
 
 def batched_transpose(A):
     """batched_transpose(A) (src/batched/batchedadjtrans.jl:37-38); transposing twice unwraps."""
-    return A.parent if isinstance(A, BatchedTranspose) else BatchedTranspose(A)
+    return A.parent if type(A) is BatchedTranspose else BatchedTranspose(A)
 
 
 def transpose(M):
@@ -181,13 +198,28 @@ def transpose(M):
     return M.permuted(2, 1)
 
 
-adjoint = transpose
+def adjoint(M):
+    """Lazy conjugate transpose of a matrix (``M'``); equals ``transpose`` for the real element types."""
+    out = transpose(M)
+    if M.dtype == "c64":
+        out.conj = not M.conj
+    return out
+
+
+class BatchedAdjoint(BatchedTranspose):
+    """Lazy per-slice conjugate transpose of a complex 3-D array (src/batched/batchedadjtrans.jl:23-52)."""
+
+    def __init__(self, parent):
+        super().__init__(parent)
+        self.conj = not parent.conj
 
 
 def batched_adjoint(A):
-    """batched_adjoint(A): all element types here are real, so it equals batched_transpose
-    (src/batched/batchedadjtrans.jl:50-51)."""
-    return batched_transpose(A)
+    """batched_adjoint(A) (src/batched/batchedadjtrans.jl:50-51): the per-slice conjugate transpose; for the
+    real element types it equals batched_transpose.  Taking it twice unwraps."""
+    if A.dtype != "c64":
+        return batched_transpose(A)
+    return A.parent if isinstance(A, BatchedAdjoint) else BatchedAdjoint(A)
 
 
 class CausalMask:

@@ -463,6 +463,8 @@ def batched_mul_(C, A, B, alpha=1.0, beta=0.0):
         return C
     if not (A.dtype == B.dtype == C.dtype) or A.dtype == "bool":
         raise ArgumentError("batched_mul! needs one floating-point element type for A, B and C")
+    if A.dtype == "c64":
+        return _batched_mul_complex(C, A, B, alpha, beta)
     nb = C.dims[2]
     if A.dims[2] not in (nb, 1):
         raise DimensionMismatch("batch size mismatch: A != C")            # src/gemm.jl:99
@@ -485,6 +487,30 @@ def batched_mul_(C, A, B, alpha=1.0, beta=0.0):
     sB = 0 if B.dims[2] == 1 else sB
     _lib.check(_lib.load().mi_batched_gemm(C.code, tA, tB, m, n, ka, float(alpha), A.ptr, lda, sA, B.ptr, ldb, sB,
                                            float(beta), C.ptr, max(C.strides[1], m, 1), C.strides[2], nb, _stream()),
+               DimensionMismatch)
+    return C
+
+
+def _batched_mul_complex(C, A, B, alpha, beta):
+    """ComplexF32 operands: one strided kernel takes 'N', 'T', 'C' (a batched_adjoint) and every permuted
+    layout of A, B and C (src/batched/batchedmul.jl:261-296 and the generic fallback :306-325)."""
+    if C.conj:
+        raise ArgumentError("batched_mul! cannot write into a batched_adjoint")
+    nb = C.dims[2]
+    if A.dims[2] not in (nb, 1):
+        raise DimensionMismatch("batch size mismatch: A != C")            # src/gemm.jl:99
+    if B.dims[2] not in (nb, 1):
+        raise DimensionMismatch("batch size mismatch: B != C")            # src/gemm.jl:100
+    m, ka = A.dims[0], A.dims[1]
+    kb, n = B.dims[0], B.dims[1]
+    if ka != kb or m != C.dims[0] or n != C.dims[1]:                      # src/gemm.jl:106-108
+        raise DimensionMismatch(f"A1 has size ({m},{ka}), B1 has size ({kb},{n}), C1 has size {C.dims[:2]}")
+    al, be = complex(alpha), complex(beta)
+    sA = 0 if A.dims[2] == 1 else A.strides[2]                            # src/gemm.jl:117-118
+    sB = 0 if B.dims[2] == 1 else B.strides[2]
+    _lib.check(_lib.load().mi_batched_mul_c32(m, n, ka, al.real, al.imag, A.ptr, A.strides[0], A.strides[1], sA, int(A.conj),
+                                              B.ptr, B.strides[0], B.strides[1], sB, int(B.conj), be.real, be.imag,
+                                              C.ptr, C.strides[0], C.strides[1], C.strides[2], nb, _stream()),
                DimensionMismatch)
     return C
 
@@ -521,6 +547,8 @@ def batched_mul(A, B):
     if A.dtype != B.dtype:
         raise ArgumentError("batched_mul needs one element type for A and B")
     C = DeviceArray.empty((A.dims[0], B.dims[1], max(A.dims[2], B.dims[2])), A.dtype)
+    if A.dtype == "c64":
+        return batched_mul_(C, A, B)      # the complex kernel addresses every strided layout itself
     return batched_mul_(C, _copy_if_faster(A), _copy_if_faster(B))
 
 

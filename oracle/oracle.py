@@ -184,6 +184,20 @@ def grad_logsoftmax(dy, y, dims=1, dtype=np.float64):
     return grad_softmax(dy, y, dims, dtype, log=True)
 
 
+def per_slice_product(A, B, adjA=False, adjB=False, transA=False, transB=False):
+    """The reference's own oracle for batched_mul (bmm_test / bmm_adjtest, test/batchedmul.jl:6-28): the
+    ordinary matrix product slice by slice, in double precision (complex128 for complex inputs); a batch
+    extent of 1 is shared by every slice.  adj = conjugate transpose of each slice, trans = transpose."""
+    A, B = np.asarray(A), np.asarray(B)
+    wide = np.complex128 if (np.iscomplexobj(A) or np.iscomplexobj(B)) else np.float64
+    A, B = A.astype(wide), B.astype(wide)
+    op = lambda X, adj, tr: X.conj().T if adj else (X.T if tr else X)
+    nb = max(A.shape[2], B.shape[2])
+    out = [op(A[:, :, i if A.shape[2] > 1 else 0], adjA, transA) @ op(B[:, :, i if B.shape[2] > 1 else 0], adjB, transB)
+           for i in range(nb)]
+    return np.stack(out, axis=2)
+
+
 def batched_gemm(A, B, transA=False, transB=False, alpha=1.0, beta=0.0, C=None, dtype=np.float32, nthreads=1):
     """3-D column-major batched GEMM; a batch extent of 1 on A or B broadcasts."""
     A, B = _f(A, dtype), _f(B, dtype)

@@ -236,3 +236,78 @@ def test_tiled_kernel_alpha_beta_and_shared_operand(nn, dtype):
     dC.storage.fill_(float("nan"))
     nn.batched_mul_(dC, dA, dB)
     assert close(dC.to_numpy(), bmm(A, B), dtype)
+
+
+# ---- ComplexF32 (test/batchedmul.jl:51-59, 81-88, 99-119) -------------------------------------------
+
+def _crandn(rng, *shape):
+    return (rng.standard_normal(shape) + 1j * rng.standard_normal(shape)).astype(np.complex64)
+
+
+def _close(got, ref, tol=2e-5):
+    assert got.shape == ref.shape
+    assert np.abs(got - ref).max() <= tol * max(1.0, np.abs(ref).max())
+
+
+def test_complex_adjoints(nn, oracle):
+    """test/batchedmul.jl:51-59: batched_mul of complex arrays against the per-slice product, with
+    batched_adjoint on either side (the 'C' flag of src/batched/batchedmul.jl:268, 281)."""
+    rng = np.random.default_rng(0)
+    cA, cB, cC = _crandn(rng, 7, 5, 3), _crandn(rng, 5, 7, 3), _crandn(rng, 7, 6, 3)
+    D = nn.DeviceArray.from_numpy
+    dA, dB, dC = D(cA), D(cB), D(cC)
+    assert dA.dtype == "c64"
+    P = oracle.per_slice_product
+    _close(nn.batched_mul(dA, dB).to_numpy(), P(cA, cB))
+    _close(nn.batched_mul(nn.batched_adjoint(dA), nn.batched_adjoint(dB)).to_numpy(), P(cA, cB, adjA=True, adjB=True))
+    _close(nn.batched_mul(nn.batched_adjoint(dA), dC).to_numpy(), P(cA, cC, adjA=True))
+    _close(nn.batched_mul(dA, nn.batched_adjoint(dA)).to_numpy(), P(cA, cA, adjB=True))
+    # transposes without conjugation, and the double adjoint unwrapping
+    _close(nn.batched_mul(nn.batched_transpose(dA), dC).to_numpy(), P(cA, cC, transA=True))
+    assert nn.batched_adjoint(nn.batched_adjoint(dA)) is dA
+    _close(nn.batched_adjoint(dA).to_numpy(), np.conj(np.transpose(cA, (1, 0, 2))))
+    with pytest.raises(nn.ArgumentError):
+        nn.batched_mul(dA, D(np.ones((5, 7, 3), dtype=np.float32)))        # one element type for both
+
+
+@pytest.mark.parametrize("perm", [(1, 3, 2), (2, 1, 3), (3, 2, 1)])
+@pytest.mark.parametrize("adj", [False, True])
+def test_complex_permuted_dims_inputs(nn, oracle, perm, adj):
+    """test/batchedmul.jl:81-88 with ty = complex: lazily permuted operands, plain or under batched_adjoint."""
+    rng = np.random.default_rng(sum(perm) * 7 + adj)
+    A, B = _crandn(rng, 4, 4, 4), _crandn(rng, 4, 4, 4)
+    D = nn.DeviceArray.from_numpy
+    fun = nn.batched_adjoint if adj else (lambda x: x)
+    p0 = tuple(p - 1 for p in perm)
+    ref = oracle.per_slice_product(A, np.transpose(B, p0), adjA=adj)
+    _close(nn.batched_mul(fun(D(A)), D(B).permuted(*perm)).to_numpy(), ref)
+    ref = oracle.per_slice_product(np.transpose(A, p0), B, adjA=adj)
+    _close(nn.batched_mul(fun(D(A).permuted(*perm)), D(B)).to_numpy(), ref)
+
+
+def test_complex_alpha_beta_broadcast_and_permuted_output(nn, oracle):
+    """Five-argument form with complex alpha and beta (test/batchedmul.jl:99-101), a shared batch-1 operand
+    (:104-106), beta = 0 overwriting NaN, an output that is a lazily permuted array (:90-96), ragged tile edges."""
+    rng = np.random.default_rng(5)
+    A, B, C0 = _crandn(rng, 70, 33, 5), _crandn(rng, 33, 67, 1), _crandn(rng, 70, 67, 5)
+    D = nn.DeviceArray.from_numpy
+    al, be = 0.5 - 2.0j, 1.5 + 0.25j
+    C = D(C0)
+    assert nn.batched_mul_(C, D(A), D(B), al, be) is C
+    _close(C.to_numpy(), al * oracle.per_slice_product(A, B) + be * C0.astype(np.complex128), 5e-5)
+    Cn = D(np.full((70, 67, 5), np.nan + 0j, dtype=np.complex64))
+    nn.batched_mul_(Cn, D(A), D(B))
+    _close(Cn.to_numpy(), oracle.per_slice_product(A, B), 5e-5)
+    # output (70, 67, 5) as a permuted view of a (67, 5, 70) array
+    base = nn.DeviceArray.zeros((67, 5, 70), "c64")
+    out = base.permuted(3, 1, 2)
+    assert out.dims == (70, 67, 5)
+    nn.batched_mul_(out, D(A), D(B))
+    _close(np.transpose(base.to_numpy(), (2, 0, 1)), oracle.per_slice_product(A, B), 5e-5)
+    with pytest.raises(nn.DimensionMismatch):
+        nn.batched_mul_(nn.DeviceArray.zeros((70, 67, 4), "c64"), D(A), D(_crandn(rng, 33, 67, 5)))
+    # matrices on either side and the lazy adjoint of a matrix
+    M = _crandn(rng, 33, 9)
+    _close(nn.batched_mul(D(A), D(M)).to_numpy(), oracle.per_slice_product(A, M[:, :, None]), 5e-5)
+    M2 = _crandn(rng, 9, 70)
+    _close(nn.batched_mul(nn.adjoint(D(M2.conj().T.copy())), D(A)).to_numpy(), oracle.per_slice_product(M2[:, :, None], A), 5e-5)
