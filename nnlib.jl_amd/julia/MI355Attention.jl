@@ -405,7 +405,7 @@ function batched_mul!(C::DeviceArray{T, 3}, A::DeviceArray{T, 3}, B::DeviceArray
         return C
     end
     (tA, lda), (tB, ldb) = blas_layout(A), blas_layout(B)
-    strides(C)[1] == 1 || throw(ArgumentError("Unsupported array layout for batched mul.\n- Size: $(size(C))\n- Strides: $(strides(C))"))
+    (strides(C)[1] == 1 || size(C, 1) == 1) || throw(ArgumentError("Unsupported array layout for batched mul.\n- Size: $(size(C))\n- Strides: $(strides(C))"))
     sA = size(A, 3) == 1 ? 0 : strides(A)[3]          # src/gemm.jl:117-118
     sB = size(B, 3) == 1 ? 0 : strides(B)[3]
     GC.@preserve A B C gemm!(tA, tB, m, n, ka, Float32(α), A.ptr, lda, sA, B.ptr, ldb, sB, Float32(β), C.ptr,

@@ -481,7 +481,7 @@ def batched_mul_(C, A, B, alpha=1.0, beta=0.0):
         return C
     tA, lda, sA = _blas_layout(A, "A")
     tB, ldb, sB = _blas_layout(B, "B")
-    if C.strides[0] != 1:
+    if C.strides[0] != 1 and C.dims[0] > 1:   # the stride of an extent-1 dimension addresses nothing
         raise ArgumentError(f"Unsupported array layout for batched mul.\n- Size: {C.dims}\n- Strides: {C.strides}")
     sA = 0 if A.dims[2] == 1 else sA                                     # src/gemm.jl:117-118
     sB = 0 if B.dims[2] == 1 else sB

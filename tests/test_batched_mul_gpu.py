@@ -311,3 +311,55 @@ def test_complex_alpha_beta_broadcast_and_permuted_output(nn, oracle):
     _close(nn.batched_mul(D(A), D(M)).to_numpy(), oracle.per_slice_product(A, M[:, :, None]), 5e-5)
     M2 = _crandn(rng, 9, 70)
     _close(nn.batched_mul(nn.adjoint(D(M2.conj().T.copy())), D(A)).to_numpy(), oracle.per_slice_product(M2[:, :, None], A), 5e-5)
+
+
+# ---- trivial dimensions & unit strides (test/batchedmul.jl:125-160) ---------------------------------
+
+_WRAPS = ["identity", "batched_adjoint", "batched_transpose", "perm_12", "perm_23"]
+
+
+def _wrap(nn, kind, host, dev):
+    """(host array, device view) of tA(rand(sA..., 3)) for the reference's five wrappers."""
+    if kind == "identity":
+        return host, dev
+    if kind == "batched_adjoint":
+        return np.conj(np.transpose(host, (1, 0, 2))), nn.batched_adjoint(dev)
+    if kind == "batched_transpose":
+        return np.transpose(host, (1, 0, 2)), nn.batched_transpose(dev)
+    if kind == "perm_12":
+        return np.transpose(host, (1, 0, 2)), dev.permuted(2, 1, 3)
+    return np.transpose(host, (0, 2, 1)), dev.permuted(1, 3, 2)
+
+
+@pytest.mark.parametrize("complex_", [False, True], ids=["Float32", "ComplexF32"])
+def test_trivial_dimensions_and_unit_strides(nn, oracle, complex_):
+    """test/batchedmul.jl:125-160: every wrapper x every (1|3, 1|3) slice size on both sides, out of place and
+    in place with random alpha and beta, and into outputs that are themselves lazy transposes."""
+    rng = np.random.default_rng(2024 + complex_)
+    D = nn.DeviceArray.from_numpy
+    rnd = (lambda *s: _crandn(rng, *s)) if complex_ else (lambda *s: rng.standard_normal(s).astype(np.float32))
+    scal = (lambda: complex(rng.random(), rng.random())) if complex_ else (lambda: float(rng.random()))
+    ran = 0
+    for tA in _WRAPS:
+        for sA in [(1, 1), (1, 3), (3, 1), (3, 3)]:
+            for tB in _WRAPS:
+                for sB in [(1, 1), (1, 3), (3, 1), (3, 3)]:
+                    hA0, hB0 = rnd(*sA, 3), rnd(*sB, 3)
+                    hA, dA = _wrap(nn, tA, hA0, D(hA0))
+                    hB, dB = _wrap(nn, tB, hB0, D(hB0))
+                    if not (hA.shape[1] == hB.shape[0] and hA.shape[2] == hB.shape[2] == 3):
+                        continue
+                    assert dA.dims == hA.shape and dB.dims == hB.shape
+                    ref = oracle.per_slice_product(hA, hB)
+                    _close(nn.batched_mul(dA, dB).to_numpy(), ref, 1e-5)
+                    al, be = scal(), scal()
+                    hD = rnd(*ref.shape)
+                    want = al * ref + be * hD
+                    _close(nn.batched_mul_(D(hD), dA, dB, al, be).to_numpy(), want, 1e-5)
+                    # output that is a lazy transpose of a permuted copy: same values, other strides
+                    C2 = nn.batched_transpose(D(np.ascontiguousarray(np.transpose(hD, (1, 0, 2)))))
+                    assert C2.dims == ref.shape
+                    assert nn.batched_mul_(C2, dA, dB, al, be) is C2
+                    _close(C2.to_numpy(), want, 1e-5)
+                    ran += 1
+    assert ran > 100
