@@ -237,6 +237,11 @@ int32_t mi_logsumexp(int32_t dtype, const void *x, void *y, int64_t inner, int64
  * op = MI_LOGSOFTMAX: dx = dy - sum(dy)*exp(y)  (_∇logsoftmax!, src/softmax.jl:175-177) */
 int32_t mi_softmax_bwd(int32_t op, int32_t dtype, const void *dy, const void *y, void *dx,
                        int64_t inner, int64_t len, int64_t outer, mi_stream stream);
+/* Pullback of logsumexp (rrule at src/softmax.jl:205-212: dy .* tmp ./ sum(tmp)) given x and the forward
+ * RESULT lse: dx[i,j,o] = dy[i,o] * exp(x[i,j,o] - lse[i,o]); dy and lse are (inner, outer), x and dx
+ * (inner, len, outer).  A column whose lse is not finite gets NaN, as the reference's formula does. */
+int32_t mi_logsumexp_bwd(int32_t dtype, const void *dy, const void *x, const void *lse, void *dx,
+                         int64_t inner, int64_t len, int64_t outer, mi_stream stream);
 
 /* ---- batched GEMM ---------------------------------------------------------------- */
 /* C[:,:,b] = alpha * op(A[:,:,b]) * op(B[:,:,b]) + beta * C[:,:,b],  b in [0, batch).

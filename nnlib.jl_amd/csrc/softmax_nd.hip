@@ -560,7 +560,48 @@ int32_t dispatch(const char *name, int32_t dtype, const void *x, const void *x2,
     return MI_OK;
 }
 
+// pullback of logsumexp given its result: dx[i,j,o] = dy[i,o] * exp(x[i,j,o] - lse[i,o]), which is the
+// reference's dy .* tmp ./ sum(tmp) (src/softmax.jl:205-212) with tmp/sum(tmp) = exp(x - logsumexp).  A
+// column whose result is not finite gives NaN, as the reference's exp(x - max) does there.
+template <typename T>
+__global__ __launch_bounds__(256) void logsumexp_bwd_kernel(const typename T::type *dy, const typename T::type *x,
+                                                             const typename T::type *lse, typename T::type *dx,
+                                                             int64_t inner, int64_t len, int64_t outer) {
+    const int64_t n = inner * len * outer;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += stride) {
+        const int64_t i = idx % inner, o = idx / (inner * len);
+        const float z = T::to_f32(lse[i + inner * o]), g = T::to_f32(dy[i + inner * o]);
+        const bool finite = z > MI_NEG_INF && z < MI_POS_INF;   // false for NaN too
+        dx[idx] = T::from_f32(finite ? g * fast_exp(T::to_f32(x[idx]) - z) : __builtin_nanf(""));
+    }
+}
+
+template <typename T>
+void launch_logsumexp_bwd(const void *dy, const void *x, const void *lse, void *dx, int64_t inner, int64_t len, int64_t outer,
+                          hipStream_t st) {
+    typedef typename T::type t;
+    int64_t blocks = (inner * len * outer + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(logsumexp_bwd_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, st, (const t *)dy, (const t *)x,
+                       (const t *)lse, (t *)dx, inner, len, outer);
+}
+
 }  // namespace
+
+MI_API int32_t mi_logsumexp_bwd(int32_t dtype, const void *dy, const void *x, const void *lse, void *dx, int64_t inner,
+                                int64_t len, int64_t outer, mi_stream s) {
+    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_logsumexp_bwd: unknown dtype %d", dtype);
+    if (inner < 0 || len < 0 || outer < 0) return mi_set_error(MI_EINVAL, "mi_logsumexp_bwd: negative size");
+    if (inner == 0 || len == 0 || outer == 0) return MI_OK;
+    if (!dy || !x || !lse || !dx) return mi_set_error(MI_EINVAL, "mi_logsumexp_bwd: null pointer");
+    hipStream_t st = (hipStream_t)s;
+    if (dtype == MI_F32) launch_logsumexp_bwd<F32>(dy, x, lse, dx, inner, len, outer, st);
+    else if (dtype == MI_F16) launch_logsumexp_bwd<F16>(dy, x, lse, dx, inner, len, outer, st);
+    else launch_logsumexp_bwd<BF16>(dy, x, lse, dx, inner, len, outer, st);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
 
 MI_API int32_t mi_softmax(int32_t op, int32_t dtype, const void *x, void *y, int64_t inner, int64_t len, int64_t outer,
                           mi_stream s) {

@@ -356,6 +356,18 @@ function logsumexp(x::DeviceArray{T, N}; dims = :) where {T <: MIFloat, N}
     dims isa Colon ? Array(out)[] : out
 end
 
+# Pullback of logsumexp (rrule at src/softmax.jl:205-212): dy and lse are device arrays with the size of the
+# reduced result (for dims = : a 0-dimensional or one-element array holding the cotangent / the result).
+function ∇logsumexp(dy::DeviceArray{T}, x::DeviceArray{T}, lse::DeviceArray{T}; dims = :) where {T <: MIFloat}
+    inner, len, outer = reduction_geometry(size(x), dims)
+    length(dy) == length(lse) == inner * outer || throw(DimensionMismatch("dy and lse must have the size of logsumexp(x; dims)"))
+    dx = similar(x, T, size(x))
+    GC.@preserve dy x lse dx check(ccall((:mi_logsumexp_bwd, libmi), Int32,
+                                         (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
+                                         dtype_code(T), dy.ptr, x.ptr, lse.ptr, dx.ptr, inner, len, outer, C_NULL))
+    dx
+end
+
 function softmax_grad!(op::Int32, dx::DeviceArray{T}, dy::DeviceArray{T}, y::DeviceArray{T}, dims) where {T <: MIFloat}
     size(dx) == size(dy) == size(y) || throw(DimensionMismatch("dx, dy and y must have one size"))
     inner, len, outer = reduction_geometry(size(y), dims)

@@ -398,6 +398,23 @@ def logsumexp(x, *, dims=None):
     return out
 
 
+def grad_logsumexp(dy, x, *, dims=None, lse=None):
+    """Pullback of ``logsumexp(x; dims)`` (rrule at src/softmax.jl:205-212): ``dy`` has the size of the reduced
+    result; ``lse`` is that result when the caller kept it (recomputed otherwise)."""
+    if not isinstance(x, DeviceArray) or not isinstance(dy, DeviceArray):
+        raise _number_error("logsumexp")
+    x, dy = _contig(x, "x"), _contig(dy, "dy")
+    inner, n, outer, kept = _reduction_geometry(x.dims, dims)
+    if lse is None:
+        lse = logsumexp(x, dims=dims)
+    lse = _contig(lse, "lse")
+    if dy.length != inner * outer or lse.length != inner * outer or not (dy.dtype == lse.dtype == x.dtype):
+        raise DimensionMismatch(f"dy and lse must have the size {kept} of logsumexp(x; dims) and the element type of x")
+    dx = DeviceArray.empty(x.dims, x.dtype)
+    _lib.check(_lib.load().mi_logsumexp_bwd(x.code, dy.ptr, x.ptr, lse.ptr, dx.ptr, inner, n, outer, _stream()))
+    return dx
+
+
 def _softmax_grad(name, op, dx, dy, y, dims):
     dy, y, dx = _contig(dy, "dy"), _contig(y, "y"), _contig(dx, "dx")
     if not (dy.dims == y.dims == dx.dims):

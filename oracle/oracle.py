@@ -55,7 +55,8 @@ def lib():
             getattr(L, "orc_softmax_nd_" + suf).argtypes = [ci, vp, vp, i64, i64, i64]
             getattr(L, "orc_logsumexp_" + suf).argtypes = [vp, vp, i64, i64, i64]
             getattr(L, "orc_softmax_bwd_" + suf).argtypes = [ci, vp, vp, vp, i64, i64, i64]
-            for n in ("orc_softmax_nd_", "orc_logsumexp_", "orc_softmax_bwd_"):
+            getattr(L, "orc_logsumexp_bwd_" + suf).argtypes = [vp, vp, vp, i64, i64, i64]
+            for n in ("orc_softmax_nd_", "orc_logsumexp_", "orc_softmax_bwd_", "orc_logsumexp_bwd_"):
                 getattr(L, n + suf).restype = None
         _LIB = L
     return _LIB
@@ -169,6 +170,16 @@ def logsumexp(x, dims=None, dtype=np.float64):
     y = np.empty(kept, dtype=dtype, order="F")
     getattr(lib(), "orc_logsumexp_" + _suffix(dtype))(_ptr(x), _ptr(y), inner, n, outer)
     return y
+
+
+def grad_logsumexp(dy, x, dims=None, dtype=np.float64):
+    """Pullback of logsumexp(x; dims) (rrule, src/softmax.jl:205-212): dy has the size of the reduced result."""
+    x = _f(x, dtype)
+    inner, n, outer, kept = reduction_geometry(x.shape, dims)
+    dy = _f(np.asarray(dy, dtype=dtype).reshape(kept if kept else (1,), order="F"), dtype)
+    dx = np.empty_like(x, order="F")
+    getattr(lib(), "orc_logsumexp_bwd_" + _suffix(dtype))(_ptr(dy), _ptr(x), _ptr(dx), inner, n, outer)
+    return dx
 
 
 def grad_softmax(dy, y, dims=1, dtype=np.float64, log=False):

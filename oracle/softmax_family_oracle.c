@@ -71,6 +71,21 @@
                 y[i + inner * o] = m + LOG(s);                                                       \
             }                                                                                        \
     }                                                                                                \
+    /* pullback of logsumexp (rrule, src/softmax.jl:205-212): tmp = exp(x - max),                  \
+     * dx = dy .* tmp ./ sum(tmp).  dy: (inner, outer) */                                            \
+    ORC_API void orc_logsumexp_bwd_##SUF(const real *dy, const real *x, real *dx, int64_t inner,     \
+                                         int64_t len, int64_t outer)                                \
+    {                                                                                                \
+        for (int64_t o = 0; o < outer; o++)                                                          \
+            for (int64_t i = 0; i < inner; i++) {                                                    \
+                real m = (real)-INFINITY;                                                            \
+                for (int64_t j = 0; j < len; j++) m = x[AT(i, j, o)] > m ? x[AT(i, j, o)] : m;       \
+                real s = 0;                                                                          \
+                for (int64_t j = 0; j < len; j++) s += EXP(x[AT(i, j, o)] - m);                      \
+                for (int64_t j = 0; j < len; j++)                                                    \
+                    dx[AT(i, j, o)] = dy[i + inner * o] * EXP(x[AT(i, j, o)] - m) / s;               \
+            }                                                                                        \
+    }                                                                                                \
     /* op 0: dx = dy*y - y*sum(dy*y); op 1: dx = dy - sum(dy)*exp(y).  dx may alias dy */            \
     ORC_API void orc_softmax_bwd_##SUF(int op, const real *dy, const real *y, real *dx,             \
                                        int64_t inner, int64_t len, int64_t outer)                   \

@@ -135,3 +135,35 @@ def test_special_values_on_the_wide_row_kernel(nn, oracle, dtype, length):
         assert np.array_equal(np.isnan(got), np.isnan(ref)) and np.array_equal(np.isinf(got), np.isinf(ref))
         fin = np.isfinite(ref)
         assert np.abs(got[fin] - ref[fin]).max() <= tol * 10
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("shape,dims", [((3, 4), None), ((3, 4), 1), ((3, 4), 2), ((64, 100, 5), 2), ((33, 65, 3), (2, 3)),
+                                        ((5000,), 1), ((128, 40), 1)])
+def test_logsumexp_pullback(nn, oracle, dtype, shape, dims):
+    """Pullback of logsumexp (rrule at src/softmax.jl:205-212; the reference checks it with gradtest,
+    test/softmax.jl:126-128) against the oracle, with and without the saved forward result."""
+    rng = np.random.default_rng(abs(hash((shape, str(dims), 2))) % 2**31)
+    x = round_to(rng.standard_normal(shape) * 2, dtype)
+    ref_y = oracle.logsumexp(x, dims)
+    dy = round_to(rng.standard_normal(ref_y.shape if ref_y.shape else (1,)), dtype)
+    ref = oracle.grad_logsumexp(dy, x, dims)
+    dx_, dy_ = _dev(nn, x, dtype), _dev(nn, dy.reshape(ref_y.shape) if ref_y.shape else dy.reshape(()), dtype)
+    got = nn.grad_logsumexp(dy_, dx_, dims=dims).to_numpy()
+    assert got.shape == x.shape
+    assert np.abs(got - ref).max() <= TOL[dtype] * max(1.0, np.abs(ref).max())
+    lse = nn.logsumexp(dx_, dims=dims)
+    got2 = nn.grad_logsumexp(dy_, dx_, dims=dims, lse=lse).to_numpy()
+    assert np.array_equal(got, got2)
+
+
+def test_logsumexp_pullback_of_infinite_columns_is_nan(nn, oracle):
+    x = np.zeros((4, 3), dtype=np.float32)
+    x[:, 0] = -np.inf
+    x[1, 1] = np.inf
+    dy = np.ones((1, 3), dtype=np.float32)
+    with np.errstate(invalid="ignore"):
+        ref = oracle.grad_logsumexp(dy, x, 1)
+    got = nn.grad_logsumexp(_dev(nn, dy), _dev(nn, x), dims=1).to_numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    assert np.isnan(got[:, :2]).all() and np.allclose(got[:, 2], 0.25)

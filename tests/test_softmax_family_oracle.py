@@ -85,3 +85,25 @@ def test_gradients_by_finite_differences(oracle, dims, log):
         xm[idx] -= h
         num[idx] = ((f(xp) - f(xm)) * dy).sum() / (2 * h)
     assert np.abs(dx - num).max() < 1e-7
+
+
+@pytest.mark.parametrize("dims", [None, 1, 2])
+def test_logsumexp_pullback_against_finite_differences(oracle, dims):
+    """test/softmax.jl:126-128: gradtest(logsumexp, (3,4); dims = d) compares the rrule (src/softmax.jl:205-212)
+    with finite differences; here the finite differences are those of the forward oracle."""
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((3, 4))
+    y = oracle.logsumexp(x, dims)
+    dy = rng.standard_normal(y.shape if y.shape else (1,))
+    got = oracle.grad_logsumexp(dy, x, dims)
+    fd = np.zeros_like(x)
+    h = 1e-6
+    for idx in np.ndindex(x.shape):
+        xp, xm = x.copy(), x.copy()
+        xp[idx] += h
+        xm[idx] -= h
+        fd[idx] = ((oracle.logsumexp(xp, dims) - oracle.logsumexp(xm, dims)).reshape(dy.shape) * dy).sum() / (2 * h)
+    assert np.abs(got - fd).max() < 1e-8
+    # the gradient is softmax scaled by dy (the comment at src/softmax.jl:206)
+    scale = dy.reshape(y.shape) if y.shape else dy.reshape(())
+    assert np.abs(got - oracle.softmax(x, dims) * scale).max() < 1e-12
