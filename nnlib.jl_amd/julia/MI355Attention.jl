@@ -21,7 +21,7 @@
 module MI355Attention
 
 export DeviceArray, CausalMask, dot_product_attention, dot_product_attention_scores, make_causal_mask,
-       softmax, softmax!, logsoftmax, logsoftmax!, logsumexp, ∇softmax, ∇softmax!, ∇logsoftmax, ∇logsoftmax!,
+       softmax, softmax!, logsoftmax, logsoftmax!, logsumexp, ∇logsumexp, ∇softmax, ∇softmax!, ∇logsoftmax, ∇logsoftmax!,
        batched_mul, batched_mul!, batched_vec, batched_transpose, batched_adjoint, batched_mul_pullback,
        Dropout, dropout, ∇dot_product_attention
 
