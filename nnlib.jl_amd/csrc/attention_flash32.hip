@@ -37,7 +37,7 @@ __device__ inline floatx4_t ldg16f(const float *p, bool ok) {
 
 template <int D, int QB, bool CAUSAL, bool EXTRAS, int PHASE>
 __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *Ks, float *Vs, int64_t b, int64_t h,
-                                   int64_t iw, int n_tiles) {
+                                   int64_t iw, int n_tiles, unsigned wlds = 0) {
     constexpr int KS = Cfg<D>::KS, VS = Cfg<D>::VS, CHUNKS = Cfg<D>::CHUNKS;
     const AttnParams &p = a.p;
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hh = lane >> 5;
@@ -100,7 +100,8 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
                             s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(k4[j], f.q[qb][4 * c + j], s[qb][kb], 0, 0, 0);
                 }
 
-            flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0);
+            flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0,
+                                                                                                          FlashStaged<QB>(), 0, wlds);
 
             if (do_pv) {
                 // k-step v of key block kb multiplies key 32*kb + 8*(v/4) + 4*hh + v%4: exactly the key
@@ -177,7 +178,10 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
             const float l = f.l[qb] + mi_swap32(f.l[qb]);
             f.l[qb] = 1.0f / l;
         }
-        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_FINAL>(a, f, Ks, Vs, b, h, iw, n_tiles);
+        // weight tiles leave through a wavefront-private LDS region behind the K / V buffers
+        const unsigned wlds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem +
+                              (unsigned)Cfg<D>::SMEM + wave * FLASH_WSTAGE_BYTES;
+        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_FINAL>(a, f, Ks, Vs, b, h, iw, n_tiles, wlds);
         if (CAUSAL && p.weights) flash_zero_skipped_weights<QB, float>(a, b, h, iw, n_tiles);
     }
 
@@ -210,7 +214,7 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
 template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS>
 int32_t launch_one(const FlashArgs &a, hipStream_t st) {
     const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B;
-    constexpr size_t smem = Cfg<D>::SMEM;
+    constexpr size_t smem = Cfg<D>::SMEM + (WEIGHTS ? 4 * FLASH_WSTAGE_BYTES : 0);
     auto kern = flash32_kernel<D, QB, CAUSAL, EXTRAS, WEIGHTS>;
     static bool attr_set = false;
     if (!attr_set) {

@@ -22,7 +22,11 @@ struct FlashArgs {
     int32_t tiles_per_split;
     int32_t bias_lds;  // 16-bit kernels: bias / mask tiles may be staged through LDS with 16-byte DMA pieces
     int32_t mask_lds;
+    int32_t w_lds;     // weight rows start 16-byte aligned: tiles may be transposed through LDS and written as full lines
 };
+
+// Bytes of LDS per wavefront for the weight staging below: 16 query rows x 128 bytes.
+constexpr int FLASH_WSTAGE_BYTES = 2048;
 
 // Row statistics saved for the backward call: planes (maximum in log2 units, 1 / row sum, delta) of
 // [B*H][Lq rounded up to 128] floats; the forward kernels fill the first two.  Rows past Lq inside the
@@ -72,6 +76,7 @@ inline void flash_fill_vec_flags(FlashArgs &a) {
     a.mask_vec = p.mask && p.mask_strides[0] == 1 && mult4(p.mask_strides[1]) && mult4(p.mask_strides[2]) &&
                  mult4(p.mask_strides[3]) && mult4(p.Lkv) && (((uintptr_t)p.mask) & 3) == 0;
     a.w_vec = p.weights && mult4(p.Lkv) && (((uintptr_t)p.weights) & 15) == 0;
+    a.w_lds = p.weights && (p.Lkv * (int64_t)mi_dtype_size(p.weights_dtype)) % 16 == 0 && (((uintptr_t)p.weights) & 15) == 0;
     // LDS staging moves 16-byte pieces addressed with 32-bit byte offsets from the (head, batch) slice:
     // rows must start 16-byte aligned and the slice (plus one query tile of slack) must stay below 2 GiB.
     auto fits = [&](const int64_t *st, size_t elem) {
@@ -193,7 +198,8 @@ struct FlashStaged {
 template <typename T, int QB, int NDV, bool CAUSAL, int EXTRAS, int PHASE, typename TW>
 __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB][2], floatx16_t (&o)[QB][NDV],
                                           float (&fm)[QB], float (&fl)[QB], int64_t b, int64_t h, int64_t iw,
-                                          int64_t j0, const FlashStaged<QB> &sg = FlashStaged<QB>(), int stage = 0) {
+                                          int64_t j0, const FlashStaged<QB> &sg = FlashStaged<QB>(), int stage = 0,
+                                          unsigned wlds = 0) {
     const AttnParams &p = a.p;
     typedef typename T::type elem_t;
     constexpr int BN = FLASH_BN;
@@ -361,7 +367,55 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                 }
         }
 
-        if (PHASE == PHASE_FINAL && p.weights && qok) {
+        if (PHASE == PHASE_FINAL && p.weights && wlds != 0 && a.w_lds) {
+            // In the accumulator layout a lane holds runs of 4 keys of ONE query, so a direct store touches 32
+            // weight rows with 8 or 16 bytes each.  Instead the tile goes through a wavefront-private LDS region,
+            // 16 queries x 128 bytes at a time (64 keys of a 16-bit weight type, 32 keys of Float32), and comes
+            // back with 8 lanes per query row: every store instruction writes 8 full 128-byte lines.  Chunks are
+            // XOR-swizzled with the row pair (two rows share a bank span).  LDS operations of one wavefront
+            // complete in order, so no barrier is needed.
+            typedef __attribute__((address_space(3))) u32x4_t *lds16_t;
+            typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+            constexpr int EPC = 16 / (int)sizeof(TW);             // weights per 16-byte chunk
+            constexpr int NKB = sizeof(TW) == 4 ? 2 : 1;          // staging rounds per tile along the keys
+            TW *wbase = (TW *)p.weights + p.Lkv * (p.Lq * (h + p.H * b));
+#pragma unroll
+            for (int rk = 0; rk < NKB; rk++)
+#pragma unroll
+                for (int half = 0; half < 2; half++) {
+                    if ((r >> 4) == half) {
+                        const unsigned rowa = wlds + (unsigned)(r & 15) * 128u;
+                        const int sw = (r >> 1) & 7;
+                        if constexpr (sizeof(TW) == 2) {
+#pragma unroll
+                            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                                for (int g = 0; g < 4; g++) {
+                                    typedef TW tw4 __attribute__((ext_vector_type(4)));
+                                    tw4 t4;
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) t4[e] = (TW)s[qb][kb][4 * g + e];
+                                    *(lds8_t)(uintptr_t)(rowa + (unsigned)(((4 * kb + g) ^ sw) << 4) + 8u * hh) = __builtin_bit_cast(u32x2_t, t4);
+                                }
+                        } else {
+#pragma unroll
+                            for (int g = 0; g < 4; g++) {
+                                floatx4_t t4;
+#pragma unroll
+                                for (int e = 0; e < 4; e++) t4[e] = s[qb][rk][4 * g + e];
+                                *(lds16_t)(uintptr_t)(rowa + (unsigned)(((2 * g + hh) ^ sw) << 4)) = __builtin_bit_cast(u32x4_t, t4);
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 2; i++) {
+                        const int rr = (lane >> 3) + 8 * i, c = lane & 7;
+                        const u32x4_t piece = *(lds16_t)(uintptr_t)(wlds + (unsigned)rr * 128u + (unsigned)((c ^ ((rr >> 1) & 7)) << 4));
+                        const int64_t qrow = iw + 32 * qb + 16 * half + rr, kv0 = j0 + 32 * rk * (NKB - 1) + (int64_t)c * EPC;
+                        if (qrow < p.Lq && kv0 < p.Lkv) *(u32x4_t *)(wbase + p.Lkv * qrow + kv0) = piece;   // Lkv is a multiple of EPC here
+                    }
+                }
+        } else if (PHASE == PHASE_FINAL && p.weights && qok) {
             TW *w = (TW *)p.weights + p.Lkv * (qi + p.Lq * (h + p.H * b));
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
