@@ -209,6 +209,12 @@ int32_t mi_make_causal_mask(uint8_t *m, int64_t len, mi_stream stream);
  * place of Julia's RNG.  y may alias x.  0 <= p <= 1 (p = 1 zeroes everything). */
 int32_t mi_dropout(int32_t dtype, const void *x, void *y, int64_t n, float p, uint64_t seed,
                    mi_stream stream);
+/* dropout(x, p; dims) of src/dropout.jl:38-53 for dims other than `:`: one keep decision per index along the
+ * dimensions in dims_mask (bit d = dimension d + 1), shared along every other dimension, as the reference's
+ * random array has extent 1 there (_dropout_shape).  The decision is that of mi_dropout() at the column-major
+ * linear index within that smaller array.  sizes: ndim (<= 8) extents of x, a HOST array.  y may alias x. */
+int32_t mi_dropout_dims(int32_t dtype, const void *x, void *y, int32_t ndim, const int64_t *sizes,
+                        uint32_t dims_mask, float p, uint64_t seed, mi_stream stream);
 
 /* ---- softmax over the first dimension -------------------------------------------- */
 /* y[:, c] = softmax(x[:, c]) for a (rows, cols) column-major matrix; y may alias x

@@ -39,6 +39,28 @@ __global__ void dropout_kernel(const typename T::type *x, typename T::type *y, i
     for (; i < n; i += stride) y[i] = T::from_f32(mi_dropout_keep(key, (uint64_t)i, thresh) ? T::to_f32(x[i]) * scale : 0.0f);
 }
 
+// dropout(x, p; dims): one keep decision per index along `dims`, shared along every other dimension
+// (the random array has extent 1 there, _dropout_shape in src/dropout.jl).  mstride[d] is the stride of
+// dimension d in that array, 0 for the shared ones; its column-major linear index is the counter.
+struct DropDims {
+    int64_t size[8], mstride[8];
+    int32_t nd;
+};
+template <typename T>
+__global__ void dropout_dims_kernel(const typename T::type *x, typename T::type *y, int64_t n, DropDims g, uint64_t key,
+                                    uint32_t thresh, float scale) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        int64_t rest = i, at = 0;
+        for (int d = 0; d < g.nd; d++) {
+            at += (rest % g.size[d]) * g.mstride[d];
+            rest /= g.size[d];
+        }
+        y[i] = T::from_f32(mi_dropout_keep(key, (uint64_t)at, thresh) ? T::to_f32(x[i]) * scale : 0.0f);
+    }
+}
+
 template <typename TD, typename TS>
 __global__ void convert_kernel(typename TD::type *d, const typename TS::type *s, int64_t n) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -119,6 +141,36 @@ MI_API int32_t mi_dropout(int32_t dtype, const void *x, void *y, int64_t n, floa
     if (dtype == MI_F32) hipLaunchKernelGGL(dropout_kernel<F32>, g, b, 0, st, (const float *)x, (float *)y, n, key, thresh, scale);
     else if (dtype == MI_F16) hipLaunchKernelGGL(dropout_kernel<F16>, g, b, 0, st, (const _Float16 *)x, (_Float16 *)y, n, key, thresh, scale);
     else hipLaunchKernelGGL(dropout_kernel<BF16>, g, b, 0, st, (const __bf16 *)x, (__bf16 *)y, n, key, thresh, scale);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+MI_API int32_t mi_dropout_dims(int32_t dtype, const void *x, void *y, int32_t ndim, const int64_t *sizes, uint32_t dims_mask,
+                               float p, uint64_t seed, mi_stream s) {
+    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_dropout_dims: unknown dtype %d", dtype);
+    if (ndim < 0 || ndim > 8 || (ndim > 0 && !sizes)) return mi_set_error(MI_EINVAL, "mi_dropout_dims: 0 to 8 dimensions");
+    if (!(p >= 0.0f && p <= 1.0f)) return mi_set_error(MI_EINVAL, "dropout expects a probability 0 <= p <= 1");
+    DropDims g;
+    g.nd = ndim;
+    int64_t n = 1, ms = 1;
+    for (int d = 0; d < ndim; d++) {
+        if (sizes[d] < 0) return mi_set_error(MI_EINVAL, "mi_dropout_dims: negative size");
+        g.size[d] = sizes[d];
+        const bool own = (dims_mask >> d) & 1;
+        g.mstride[d] = own ? ms : 0;
+        if (own) ms *= sizes[d];
+        n *= sizes[d];
+    }
+    if (n == 0) return MI_OK;
+    if (!x || !y) return mi_set_error(MI_EINVAL, "mi_dropout_dims: null pointer");
+    const uint64_t key = mi_stream_key(seed, MI_DROPOUT_STREAM);
+    const uint32_t thresh = mi_dropout_threshold(p);
+    const float scale = p < 1.0f ? 1.0f / (1.0f - p) : 0.0f;
+    dim3 gr(grid_for(n)), b(256);
+    hipStream_t st = (hipStream_t)s;
+    if (dtype == MI_F32) hipLaunchKernelGGL(dropout_dims_kernel<F32>, gr, b, 0, st, (const float *)x, (float *)y, n, g, key, thresh, scale);
+    else if (dtype == MI_F16) hipLaunchKernelGGL(dropout_dims_kernel<F16>, gr, b, 0, st, (const _Float16 *)x, (_Float16 *)y, n, g, key, thresh, scale);
+    else hipLaunchKernelGGL(dropout_dims_kernel<BF16>, gr, b, 0, st, (const __bf16 *)x, (__bf16 *)y, n, g, key, thresh, scale);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }

@@ -167,12 +167,22 @@ struct Dropout
     end
 end
 (d::Dropout)(x::DeviceArray) = dropout(x, d.p; seed = d.seed)
-function dropout(x::DeviceArray{T}, p::Real; seed::Integer = 0) where {T <: MIFloat}
+function dropout(x::DeviceArray{T, N}, p::Real; seed::Integer = 0, dims = :) where {T <: MIFloat, N}
     0 <= p <= 1 || throw(ArgumentError("dropout expects a probability 0 <= p <= 1"))
     is_dense(x) || throw(ArgumentError("dropout needs a dense array"))
     y = similar(x, T, size(x))
-    GC.@preserve x y check(ccall((:mi_dropout, libmi), Int32, (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Float32, UInt64, Ptr{Cvoid}),
-                                 dtype_code(T), x.ptr, y.ptr, length(x), Float32(p), UInt64(seed), C_NULL))
+    if dims isa Colon
+        GC.@preserve x y check(ccall((:mi_dropout, libmi), Int32, (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Float32, UInt64, Ptr{Cvoid}),
+                                     dtype_code(T), x.ptr, y.ptr, length(x), Float32(p), UInt64(seed), C_NULL))
+    else
+        # one decision per index along dims, shared along the other dimensions (src/dropout.jl:38-53)
+        N <= 8 || throw(ArgumentError("dropout along dims takes arrays of up to 8 dimensions"))
+        mask = UInt32(sum(d -> 1 << (d - 1), filter(d -> d <= N, collect(dims)); init = 0))
+        sizes = collect(Int64, size(x))
+        GC.@preserve x y sizes check(ccall((:mi_dropout_dims, libmi), Int32,
+                                           (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int32, Ptr{Int64}, UInt32, Float32, UInt64, Ptr{Cvoid}),
+                                           dtype_code(T), x.ptr, y.ptr, Int32(N), sizes, mask, Float32(p), UInt64(seed), C_NULL))
+    end
     y
 end
 

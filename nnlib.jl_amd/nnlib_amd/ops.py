@@ -43,12 +43,20 @@ class Dropout:
 
 def dropout(x, p, *, seed=0, dims=None):
     """dropout(A, p; dims = :)  (src/dropout.jl:38-53): zero with probability p, else scale by 1/(1-p)."""
-    if dims is not None:
-        raise NotImplementedError("dropout along dims (one decision per slice) is not built")
     x = _contig(x, "x")
     if x.dtype == "bool":
         raise ArgumentError("dropout needs a floating-point array")
     out = DeviceArray.empty(x.dims, x.dtype)
+    if dims is not None:
+        ds = {int(d) for d in (dims if isinstance(dims, (tuple, list)) else (dims,))}
+        if not ds or min(ds) < 1:
+            raise ArgumentError(f"dims must be positive dimension numbers, got {dims}")
+        if x.ndim > 8:
+            raise ArgumentError("dropout along dims takes arrays of up to 8 dimensions")
+        mask = sum(1 << (d - 1) for d in ds if d <= x.ndim)
+        sizes = (ctypes.c_int64 * max(x.ndim, 1))(*x.dims)
+        _lib.check(_lib.load().mi_dropout_dims(x.code, x.ptr, out.ptr, x.ndim, sizes, mask, float(p), int(seed), _stream()))
+        return out
     _lib.check(_lib.load().mi_dropout(x.code, x.ptr, out.ptr, x.length, float(p), int(seed), _stream()))
     return out
 

@@ -86,3 +86,23 @@ def test_scores_with_fused_dropout_and_edge_probabilities(nn):
         nn.Dropout(1.5)
     with pytest.raises(nn.ArgumentError, match="probability"):
         nn.dropout(q, -0.1)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("shape,dims", [((6, 5), 1), ((6, 5), 2), ((4, 3, 5), (1, 3)), ((4, 3, 5), 2), ((3, 4, 2, 5), (2, 4)),
+                                        ((300, 70), 1), ((7,), 1), ((4, 3), (1, 2))])
+def test_dropout_along_dims(nn, oracle, dtype, shape, dims):
+    """dropout(x, p; dims) (src/dropout.jl:38-53): the random array has the extent of x along dims and 1 elsewhere,
+    so slices along the other dimensions share their decisions (the doctest: dims = 1 zeroes whole rows)."""
+    rng = np.random.default_rng(3)
+    x = round_to(rng.standard_normal(shape) + 3.0, dtype)
+    p, seed = 0.4, 11
+    got = nn.dropout(nn.DeviceArray.from_numpy(x, dtype), p, seed=seed, dims=dims).to_numpy()
+    ds = (dims,) if isinstance(dims, int) else dims
+    mshape = tuple(n if d + 1 in ds else 1 for d, n in enumerate(shape))
+    keep = oracle.dropout_keep_mask(mshape, p, seed)
+    ref = np.where(np.broadcast_to(keep, shape), x / (1 - p), 0.0)
+    assert np.array_equal(got == 0, ~np.broadcast_to(keep, shape))
+    assert np.abs(got - ref).max() <= (1e-6 if dtype == "f32" else 2e-2) * np.abs(ref).max()
+    if len(ds) == len(shape):     # every dimension owns its decisions: the same as dims = :
+        assert np.array_equal(got, nn.dropout(nn.DeviceArray.from_numpy(x, dtype), p, seed=seed).to_numpy())
