@@ -283,6 +283,10 @@ int32_t mi_batched_mul_c32(int64_t m, int64_t n, int64_t k, float alpha_re, floa
  * (_copy_if_faster, src/batched/batchedmul.jl:76-83).  elem_bytes is 1, 2, 4 or 8. */
 int32_t mi_strided_copy(void *dst, const void *src, int32_t elem_bytes, int64_t d0, int64_t d1, int64_t d2,
                         int64_t s0, int64_t s1, int64_t s2, mi_stream stream);
+/* The same for up to 8 dimensions: permutedims of an N-d array (what Base does for the reference when
+ * softmax and friends reduce over dimensions that are not neighbours).  sizes / strides: HOST arrays. */
+int32_t mi_strided_copy_nd(void *dst, const void *src, int32_t elem_bytes, int32_t ndim, const int64_t *sizes,
+                           const int64_t *strides, mi_stream stream);
 
 /* ---- reproducible inputs --------------------------------------------------------- */
 /* ptr[i] = dtype(scale * z_i), z_i ~ N(0,1) from a counter-based generator keyed by

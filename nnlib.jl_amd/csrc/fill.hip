@@ -85,6 +85,27 @@ __global__ void strided_copy_kernel(void *dst, const void *src, int64_t d0, int6
     }
 }
 
+// the same for up to 8 dimensions (permutedims of an N-d array)
+struct CopyDims {
+    int64_t size[8], stride[8];
+    int32_t nd;
+};
+template <int BYTES>
+__global__ void strided_copy_nd_kernel(void *dst, const void *src, int64_t n, CopyDims g) {
+    typedef typename std::conditional<BYTES == 8, uint64_t, typename std::conditional<BYTES == 4, uint32_t,
+            typename std::conditional<BYTES == 2, uint16_t, uint8_t>::type>::type>::type word;
+    int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; idx < n; idx += stride) {
+        int64_t rest = idx, at = 0;
+        for (int d = 0; d < g.nd; d++) {
+            at += (rest % g.size[d]) * g.stride[d];
+            rest /= g.size[d];
+        }
+        ((word *)dst)[idx] = ((const word *)src)[at];
+    }
+}
+
 // m[i + j*len] = (i <= j): reference src/attention.jl:145,149-153
 __global__ void causal_mask_kernel(uint8_t *m, int64_t len) {
     int64_t n = len * len;
@@ -211,6 +232,32 @@ MI_API int32_t mi_strided_copy(void *dst, const void *src, int32_t elem_bytes, i
     else if (elem_bytes == 4) hipLaunchKernelGGL(strided_copy_kernel<4>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
     else if (elem_bytes == 2) hipLaunchKernelGGL(strided_copy_kernel<2>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
     else hipLaunchKernelGGL(strided_copy_kernel<1>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+MI_API int32_t mi_strided_copy_nd(void *dst, const void *src, int32_t elem_bytes, int32_t ndim, const int64_t *sizes,
+                                  const int64_t *strides, mi_stream s) {
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
+        return mi_set_error(MI_EINVAL, "mi_strided_copy_nd: element size must be 1, 2, 4 or 8 bytes");
+    if (ndim < 0 || ndim > 8 || (ndim > 0 && (!sizes || !strides))) return mi_set_error(MI_EINVAL, "mi_strided_copy_nd: 0 to 8 dimensions");
+    CopyDims g;
+    g.nd = ndim;
+    int64_t n = 1;
+    for (int d = 0; d < ndim; d++) {
+        if (sizes[d] < 0 || strides[d] < 0) return mi_set_error(MI_EINVAL, "mi_strided_copy_nd: negative size or stride");
+        g.size[d] = sizes[d];
+        g.stride[d] = strides[d];
+        n *= sizes[d];
+    }
+    if (n == 0) return MI_OK;
+    if (!dst || !src) return mi_set_error(MI_EINVAL, "mi_strided_copy_nd: null pointer");
+    dim3 gr(grid_for(n)), b(256);
+    hipStream_t st = (hipStream_t)s;
+    if (elem_bytes == 8) hipLaunchKernelGGL(strided_copy_nd_kernel<8>, gr, b, 0, st, dst, src, n, g);
+    else if (elem_bytes == 4) hipLaunchKernelGGL(strided_copy_nd_kernel<4>, gr, b, 0, st, dst, src, n, g);
+    else if (elem_bytes == 2) hipLaunchKernelGGL(strided_copy_nd_kernel<2>, gr, b, 0, st, dst, src, n, g);
+    else hipLaunchKernelGGL(strided_copy_nd_kernel<1>, gr, b, 0, st, dst, src, n, g);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }

@@ -83,6 +83,7 @@ SIGNATURES = {
     "mi_batched_mul_c32": (c_i32, [c_i64, c_i64, c_i64, c_f32, c_f32, c_vp, c_i64, c_i64, c_i64, c_i32, c_vp, c_i64, c_i64, c_i64,
                                    c_i32, c_f32, c_f32, c_vp, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "mi_strided_copy": (c_i32, [c_vp, c_vp, c_i32, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_vp]),
+    "mi_strided_copy_nd": (c_i32, [c_vp, c_vp, c_i32, c_i32, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), c_vp]),
     "mi_randn_fill": (c_i32, [c_vp, c_i32, c_i64, c_u64, c_u64, c_f32, c_vp]),
     "mi_bernoulli_fill": (c_i32, [c_vp, c_i64, c_u64, c_u64, c_f32, c_vp]),
     "mi_convert": (c_i32, [c_vp, c_i32, c_vp, c_i32, c_i64, c_vp]),

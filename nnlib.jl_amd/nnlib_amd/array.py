@@ -132,12 +132,17 @@ class DeviceArray:
         return out
 
     def copy(self):
-        """Dense column-major copy (``copy(X)`` / ``permutedims``): materialises a lazy view of up to 3 dims."""
-        assert self.ndim <= 3, "copy of a strided view is built for up to 3 dimensions"
-        d = self.dims + (1,) * (3 - self.ndim)
-        s = self.strides + (0,) * (3 - self.ndim)
+        """Dense column-major copy (``copy(X)`` / ``permutedims``): materialises a lazy view of up to 8 dims."""
+        assert self.ndim <= 8, "copy of a strided view is built for up to 8 dimensions"
         out = DeviceArray.empty(self.dims, self.dtype)
-        _lib.check(_lib.load().mi_strided_copy(out.ptr, self.ptr, self.itemsize, d[0], d[1], d[2], s[0], s[1], s[2], None))
+        if self.ndim <= 3:
+            d = self.dims + (1,) * (3 - self.ndim)
+            s = self.strides + (0,) * (3 - self.ndim)
+            _lib.check(_lib.load().mi_strided_copy(out.ptr, self.ptr, self.itemsize, d[0], d[1], d[2], s[0], s[1], s[2], None))
+        else:
+            import ctypes
+            sizes, strides = (ctypes.c_int64 * self.ndim)(*self.dims), (ctypes.c_int64 * self.ndim)(*self.strides)
+            _lib.check(_lib.load().mi_strided_copy_nd(out.ptr, self.ptr, self.itemsize, self.ndim, sizes, strides, None))
         if self.conj:
             out.storage.copy_(torch.conj_physical(out.storage))
         return out

@@ -340,12 +340,36 @@ def _reduction_geometry(dims_of_x, dims):
     ds = [d for d in ds if d <= len(size)]       # trailing singleton dimensions reduce to themselves
     if not ds:
         return int(np.prod(size, dtype=np.int64)) if size else 1, 1, 1, size
-    if ds != list(range(ds[0], ds[-1] + 1)):
-        raise ArgumentError(f"dims = {dims}: only runs of adjacent dimensions are supported on device arrays")
+    if ds != list(range(ds[0], ds[-1] + 1)):   # callers route such sets through _nonadjacent_plan first
+        raise ArgumentError(f"dims = {dims}: a single kernel call reduces over a run of adjacent dimensions")
     lo, hi = ds[0] - 1, ds[-1]
     prod = lambda t: int(np.prod(t, dtype=np.int64)) if t else 1
     kept = size[:lo] + (1,) * (hi - lo) + size[hi:]
     return prod(size[:lo]), prod(size[lo:hi]), prod(size[hi:]), kept
+
+
+def _nonadjacent_plan(dims_of_x, dims):
+    """None when ``dims`` is ``None`` or a run of adjacent dimensions; otherwise ``(perm, inverse, k)``: the 1-based
+    permutation that brings the ``k`` reduced dimensions to the front (Base's reductions take any ``dims``; the
+    kernels take runs, so other sets go through ``permutedims`` there and back)."""
+    if dims is None:
+        return None
+    n = len(dims_of_x)
+    ds = sorted({int(d) for d in (dims if isinstance(dims, (tuple, list)) else (dims,))})
+    if not ds or ds[0] < 1:
+        raise ArgumentError(f"dims must be positive dimension numbers, got {dims}")
+    ds = [d for d in ds if d <= n]
+    if not ds or ds == list(range(ds[0], ds[-1] + 1)):
+        return None
+    perm = ds + [d for d in range(1, n + 1) if d not in ds]
+    inverse = [perm.index(d) + 1 for d in range(1, n + 1)]
+    return tuple(perm), tuple(inverse), len(ds)
+
+
+def _assign(out, y):
+    """out .= y for two dense arrays of one size and element type."""
+    out.storage[out.offset:out.offset + out.length].copy_(y.storage[y.offset:y.offset + y.length])
+    return out
 
 
 def _number_error(name):
@@ -363,6 +387,12 @@ def _softmax_like(name, op, out, x, dims):
         raise DimensionMismatch(f"output size {out.dims} differs from input size {x.dims}")
     if x.dtype == "bool" or out.dtype != x.dtype:
         raise ArgumentError(f"{name} needs floating-point input and output of one element type")
+    plan = _nonadjacent_plan(x.dims, dims)
+    if plan is not None:
+        perm, inverse, k = plan
+        xp = x.permuted(*perm).copy()
+        yp = _softmax_like(name, op, DeviceArray.empty(xp.dims, xp.dtype), xp, tuple(range(1, k + 1)))
+        return _assign(out, yp.permuted(*inverse).copy())
     inner, n, outer, _ = _reduction_geometry(x.dims, dims)
     _lib.check(_lib.load().mi_softmax(op, x.code, x.ptr, out.ptr, inner, n, outer, _stream()))
     return out
@@ -400,6 +430,10 @@ def logsumexp(x, *, dims=None):
     x = _contig(x, "x")
     if x.dtype == "bool":
         raise ArgumentError("logsumexp needs a floating-point array")
+    plan = _nonadjacent_plan(x.dims, dims)
+    if plan is not None:
+        perm, inverse, k = plan
+        return logsumexp(x.permuted(*perm).copy(), dims=tuple(range(1, k + 1))).permuted(*inverse).copy()
     inner, n, outer, kept = _reduction_geometry(x.dims, dims)
     out = DeviceArray.empty(kept, x.dtype)
     _lib.check(_lib.load().mi_logsumexp(x.code, x.ptr, out.ptr, inner, n, outer, _stream()))
@@ -412,6 +446,12 @@ def grad_logsumexp(dy, x, *, dims=None, lse=None):
     if not isinstance(x, DeviceArray) or not isinstance(dy, DeviceArray):
         raise _number_error("logsumexp")
     x, dy = _contig(x, "x"), _contig(dy, "dy")
+    plan = _nonadjacent_plan(x.dims, dims)
+    if plan is not None:
+        perm, inverse, k = plan
+        front = tuple(range(1, k + 1))
+        lp = None if lse is None else _contig(lse, "lse").permuted(*perm).copy()
+        return grad_logsumexp(dy.permuted(*perm).copy(), x.permuted(*perm).copy(), dims=front, lse=lp).permuted(*inverse).copy()
     inner, n, outer, kept = _reduction_geometry(x.dims, dims)
     if lse is None:
         lse = logsumexp(x, dims=dims)
@@ -429,6 +469,12 @@ def _softmax_grad(name, op, dx, dy, y, dims):
         raise DimensionMismatch(f"{name}: dx {dx.dims}, dy {dy.dims} and y {y.dims} must have one size")
     if y.dtype == "bool" or not (dy.dtype == y.dtype == dx.dtype):
         raise ArgumentError(f"{name} needs one floating-point element type for dx, dy and y")
+    plan = _nonadjacent_plan(y.dims, dims)
+    if plan is not None:
+        perm, inverse, k = plan
+        yp, dyp = y.permuted(*perm).copy(), dy.permuted(*perm).copy()
+        dxp = _softmax_grad(name, op, DeviceArray.empty(yp.dims, yp.dtype), dyp, yp, tuple(range(1, k + 1)))
+        return _assign(dx, dxp.permuted(*inverse).copy())
     inner, n, outer, _ = _reduction_geometry(y.dims, dims)
     _lib.check(_lib.load().mi_softmax_bwd(op, y.code, dy.ptr, y.ptr, dx.ptr, inner, n, outer, _stream()))
     return dx

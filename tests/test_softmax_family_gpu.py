@@ -106,8 +106,6 @@ def test_errors(nn):
         nn.logsoftmax(1.0)
     with pytest.raises(nn.ArgumentError, match="expects an array"):
         nn.logsumexp(1.0)
-    with pytest.raises(nn.ArgumentError, match="adjacent"):
-        nn.softmax(nn.DeviceArray.zeros((2, 3, 4)), dims=(1, 3))
     with pytest.raises(nn.DimensionMismatch):
         nn.grad_softmax_(nn.DeviceArray.zeros((3, 2)), nn.DeviceArray.zeros((2, 3)), nn.DeviceArray.zeros((2, 3)))
 
@@ -176,3 +174,38 @@ def test_logsumexp_pullback_of_infinite_columns_is_nan(nn, oracle):
     got = nn.grad_logsumexp(_dev(nn, dy), _dev(nn, x), dims=1).to_numpy()
     assert np.array_equal(np.isnan(got), np.isnan(ref))
     assert np.isnan(got[:, :2]).all() and np.allclose(got[:, 2], 0.25)
+
+
+@pytest.mark.parametrize("shape,dims", [((2, 3, 4), (1, 3)), ((3, 2, 4, 5), (2, 4)), ((3, 2, 4, 5), (1, 3, 4)), ((2, 2, 2, 2, 2), (1, 5))])
+def test_dims_that_are_not_neighbours(nn, oracle, shape, dims):
+    """Base's reductions take any dims tuple (src/softmax.jl:69-79 reduces with maximum / sum over dims); sets that
+    are not a run go through permutedims on the device.  Checked against the closed forms of test/softmax.jl:27-28
+    and against the adjacent-dims path on a host-permuted copy."""
+    rng = np.random.default_rng(len(shape) * 10 + len(dims))
+    x = rng.standard_normal(shape).astype(np.float32)
+    ax = tuple(d - 1 for d in dims)
+    e = np.exp(x.astype(np.float64))
+    sm = e / e.sum(axis=ax, keepdims=True)
+    d = _dev(nn, x)
+    assert np.abs(nn.softmax(d, dims=dims).to_numpy() - sm).max() < 1e-6
+    assert np.abs(nn.logsoftmax(d, dims=dims).to_numpy() - np.log(sm)).max() < 1e-5
+    lse = nn.logsumexp(d, dims=dims)
+    assert lse.dims == tuple(1 if i in ax else n for i, n in enumerate(shape))
+    assert np.abs(lse.to_numpy() - np.log(e.sum(axis=ax, keepdims=True))).max() < 1e-5
+    # gradients: against the oracle on a host-permuted copy whose reduced dims are the leading run
+    perm = list(ax) + [i for i in range(len(shape)) if i not in ax]
+    inv = np.argsort(perm)
+    front = tuple(range(1, len(dims) + 1))
+    dy = rng.standard_normal(shape).astype(np.float32)
+    y = sm.astype(np.float32)
+    ref = np.transpose(oracle.grad_softmax(np.transpose(dy, perm), np.transpose(y, perm), front), inv)
+    assert np.abs(nn.grad_softmax(_dev(nn, dy), _dev(nn, y), dims=dims).to_numpy() - ref).max() < 1e-5
+    ly = np.log(sm).astype(np.float32)
+    ref = np.transpose(oracle.grad_logsoftmax(np.transpose(dy, perm), np.transpose(ly, perm), front), inv)
+    assert np.abs(nn.grad_logsoftmax(_dev(nn, dy), _dev(nn, ly), dims=dims).to_numpy() - ref).max() < 1e-5
+    dl = rng.standard_normal(lse.dims).astype(np.float32)
+    assert np.abs(nn.grad_logsumexp(_dev(nn, dl), d, dims=dims).to_numpy() - dl * sm).max() < 1e-5
+    # in-place forms
+    out = nn.DeviceArray.zeros(shape)
+    assert nn.softmax_(out, d, dims=dims) is out
+    assert np.abs(out.to_numpy() - sm).max() < 1e-6
