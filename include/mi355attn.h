@@ -204,9 +204,11 @@ int32_t mi_attention_bwd(const mi_attn_bwd_desc *desc, mi_stream stream);
 int32_t mi_make_causal_mask(uint8_t *m, int64_t len, mi_stream stream);
 
 /* ---- dropout --------------------------------------------------------------------- */
-/* y[i] = keep_i ? x[i] / (1 - p) : 0 with keep_i ~ Bernoulli(1 - p) from the counter-based generator
- * keyed by (seed, i): dropout(x, p; dims = :) of src/dropout.jl:38-53 with a reproducible stream in
- * place of Julia's RNG.  y may alias x.  0 <= p <= 1 (p = 1 zeroes everything). */
+/* y[i] = keep_i ? x[i] / (1 - p) : 0 with keep_i ~ Bernoulli(1 - p) from a counter-based generator:
+ * dropout(x, p; dims = :) of src/dropout.jl:38-53 with a reproducible stream in place of Julia's RNG.
+ * The 64-bit word of counter i >> 2 (splitmix64 of a key derived from the seed) serves elements
+ * 4(i >> 2) .. +3 with 16 bits each; keep_i = (that field >= ceil(p * 65536)), so p has a resolution of
+ * 2^-16.  y may alias x.  0 <= p <= 1 (p = 1 zeroes everything). */
 int32_t mi_dropout(int32_t dtype, const void *x, void *y, int64_t n, float p, uint64_t seed,
                    mi_stream stream);
 /* dropout(x, p; dims) of src/dropout.jl:38-53 for dims other than `:`: one keep decision per index along the

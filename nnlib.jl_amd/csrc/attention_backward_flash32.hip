@@ -105,7 +105,8 @@ __device__ inline void load_stationary(float (&x)[D / 2], const float *row, bool
 __device__ inline int64_t lq_pad(int64_t Lq) { return attention_stats_lq_pad(Lq); }
 
 // ---- kernel 1: statistics and dQ --------------------------------------------------------------------
-template <int D, bool CAUSAL, int EXTRAS, bool HAVE_STATS>
+// DROP (per-element paths only): the forward call dropped weights; the kernels redraw the factor g.
+template <int D, bool CAUSAL, int EXTRAS, bool HAVE_STATS, bool DROP = false>
 __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) void bwd32_dq_kernel(FlashArgs a, AttnBwdParams bp) {
     constexpr int TILEF = Cfg<D>::TILEF, NDV = Cfg<D>::NDV;
     const AttnParams &p = a.p;
@@ -229,13 +230,18 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
                 flash_softmax_tile<T, 1, NDV, CAUSAL, EXTRAS, PHASE_FINAL, float>(a, s, unused_o, fm, fl, b, h, iw, j0);
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-                    for (int v = 0; v < 16; v++) {
+                    if (DROP) {
                         // fused dropout: the forward multiplied the weight by g (0 or 1/(1-p)), its pullback multiplies dP
-                        float dpv = dp[kb][v];
-                        if (bp.p.drop_thresh) dpv *= attention_drop_factor(bp.p, j0 + 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4), qi, h, b);
-                        s[0][kb][v] *= dpv - delta;
+#pragma unroll
+                        for (int g = 0; g < 4; g++) {
+                            float gf[4];
+                            attention_drop_factors_run4<false>(bp.p, (uint64_t)(p.Lkv * (qi + p.Lq * (h + p.H * b)) + 4 * hh + j0 + 32 * kb), g, gf);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) dp[kb][4 * g + e] *= gf[e];
+                        }
                     }
+#pragma unroll
+                    for (int v = 0; v < 16; v++) s[0][kb][v] *= dp[kb][v] - delta;
                     second_product<D>(kt, kb, s[0][kb], dq, r, hh);
                 }
             }
@@ -259,7 +265,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
 
 // ---- kernel 2: dK and dV ----------------------------------------------------------------------------
 enum { BWD_DV = 1, BWD_DK = 2 };
-template <int D, bool CAUSAL, int EXTRAS, int WHICH>
+template <int D, bool CAUSAL, int EXTRAS, int WHICH, bool DROP = false>
 __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) void bwd32_dkdv_kernel(FlashArgs a, AttnBwdParams bp) {
     constexpr int TILEF = Cfg<D>::TILEF, NDV = Cfg<D>::NDV;
     constexpr bool DO_DV = (WHICH & BWD_DV) != 0, DO_DK = (WHICH & BWD_DK) != 0;
@@ -360,7 +366,7 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
                         else pw = mi_exp2(fmaf(x, cs, m == MI_NEG_INF ? 0.0f : -m)) * linv4[e];
                         pw = in ? pw : 0.0f;
                         // fused dropout: the value product saw pw * gd, and the pullback multiplies dP by gd
-                        const float gd = bp.p.drop_thresh ? attention_drop_factor(bp.p, kv, qi, h, b) : 1.0f;
+                        const float gd = DROP ? attention_drop_factor(bp.p, kv, qi, h, b) : 1.0f;
                         s[4 * g + e] = pw * gd;
                         if (DO_DK) dp[4 * g + e] = pw * (gd * dp[4 * g + e] - delta4[e]);
                     }
@@ -393,7 +399,7 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
     }
 }
 
-template <int D, bool CAUSAL, int EXTRAS>
+template <int D, bool CAUSAL, int EXTRAS, bool DROP = false>
 int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
     const AttnParams &p = a.p;
     constexpr size_t SMEM = Cfg<D>::SMEM;
@@ -401,13 +407,13 @@ int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) 
     // arrays) or is needed to fit the register file at all (head dim 128: K, V, dK and dV of a lane are
     // 256 registers before anything else); one pass otherwise.
     constexpr bool SPLIT = (EXTRAS == EXTRAS_NONE && D == 64) || D == 128;
-    auto k1 = bp.have_stats ? bwd32_dq_kernel<D, CAUSAL, EXTRAS, true> : bwd32_dq_kernel<D, CAUSAL, EXTRAS, false>;
-    auto k2 = bwd32_dkdv_kernel<D, CAUSAL, EXTRAS, SPLIT ? BWD_DV : 3>;
-    auto k3 = bwd32_dkdv_kernel<D, CAUSAL, EXTRAS, SPLIT ? BWD_DK : 3>;
+    auto k1 = bp.have_stats ? bwd32_dq_kernel<D, CAUSAL, EXTRAS, true, DROP> : bwd32_dq_kernel<D, CAUSAL, EXTRAS, false, DROP>;
+    auto k2 = bwd32_dkdv_kernel<D, CAUSAL, EXTRAS, SPLIT ? BWD_DV : 3, DROP>;
+    auto k3 = bwd32_dkdv_kernel<D, CAUSAL, EXTRAS, SPLIT ? BWD_DK : 3, DROP>;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
     if (!attr_set) {
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, true, DROP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, false, DROP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         attr_set = true;
@@ -429,6 +435,8 @@ int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) 
 template <int D>
 int32_t launch_d(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
     const bool extras = bp.p.bias || bp.p.mask || bp.p.drop_thresh;
+    if (bp.p.drop_thresh)   // dropout runs on the per-element paths
+        return bp.p.causal ? launch_set<D, true, EXTRAS_DIRECT, true>(a, bp, st) : launch_set<D, false, EXTRAS_DIRECT, true>(a, bp, st);
     if (bp.p.causal) return extras ? launch_set<D, true, EXTRAS_DIRECT>(a, bp, st) : launch_set<D, true, EXTRAS_NONE>(a, bp, st);
     return extras ? launch_set<D, false, EXTRAS_DIRECT>(a, bp, st) : launch_set<D, false, EXTRAS_NONE>(a, bp, st);
 }

@@ -25,6 +25,43 @@ __device__ inline float attention_drop_factor(const AttnParams &p, int64_t kv, i
     if (p.drop_thresh == 0) return 1.0f;
     return mi_dropout_keep(p.drop_key, (uint64_t)(kv + p.Lkv * (q + p.Lq * (h + p.H * b))), p.drop_thresh) ? p.drop_scale : 0.0f;
 }
+
+// The same for the 16 accumulator registers of a lane that holds, for one query, the keys of a 32-key block
+// in runs of four: run g holds the weights at linear indices i0 + 8g + e (i0: the lane's first key of the block).
+// ALIGNED: Lkv is a multiple of 4, so a run is one hash group; otherwise each weight is looked up alone.
+template <bool ALIGNED>
+__device__ inline void attention_drop_factors_run4(const AttnParams &p, uint64_t i0, int g, float (&f)[4]) {
+    if (ALIGNED) {
+        const uint64_t bits = mi_dropout_group_bits(p.drop_key, (i0 + 8 * g) >> 2);
+#pragma unroll
+        for (int e = 0; e < 4; e++) f[e] = mi_dropout_keep_in(bits, e, p.drop_thresh) ? p.drop_scale : 0.0f;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) f[e] = mi_dropout_keep(p.drop_key, i0 + 8 * g + e, p.drop_thresh) ? p.drop_scale : 0.0f;
+    }
+}
+
+// The transposed case: a lane holds ONE key (kv; the four lanes of a quad hold kv = 4t .. 4t+3) and, in register
+// e of a run, query q0 + e.  Each lane hashes the group of query q0 + (lane & 3) and the quad exchanges the words,
+// so a quad still computes one hash per four weights.  f[e]: the factor of weight (kv, q0 + e).  Needs Lkv % 4 == 0.
+__device__ inline void attention_drop_factors_quad(const AttnParams &p, int64_t kv, int64_t q0, int64_t h, int64_t b, float (&f)[4]) {
+    const uint64_t col0 = (uint64_t)(kv + p.Lkv * (q0 + p.Lq * (h + p.H * b)));
+    {
+        const int sub = (int)(kv & 3);                         // == lane & 3 for the 32-aligned key blocks of the kernels
+        const uint64_t mine = mi_dropout_group_bits(p.drop_key, (col0 + (uint64_t)p.Lkv * (uint64_t)sub) >> 2);
+        const int lo = (int)(uint32_t)mine, hi = (int)(uint32_t)(mine >> 32);
+        // the word of quad lane E (quad_perm broadcast), of which a lane keeps its own 16-bit field
+#define MI_QUAD_FIELD(E)                                                                             \
+        {                                                                                            \
+            const int blo = __builtin_amdgcn_mov_dpp(lo, (E) * 0x55, 0xF, 0xF, true);                \
+            const int bhi = __builtin_amdgcn_mov_dpp(hi, (E) * 0x55, 0xF, 0xF, true);                \
+            const uint32_t word = (uint32_t)(sub < 2 ? blo : bhi);                                   \
+            f[E] = ((word >> (16 * (sub & 1))) & 0xFFFFu) >= p.drop_thresh ? p.drop_scale : 0.0f;    \
+        }
+        MI_QUAD_FIELD(0) MI_QUAD_FIELD(1) MI_QUAD_FIELD(2) MI_QUAD_FIELD(3)
+#undef MI_QUAD_FIELD
+    }
+}
 #endif
 
 // One backward call: the forward call it differentiates plus cotangents and gradient buffers.

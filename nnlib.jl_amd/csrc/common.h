@@ -132,17 +132,27 @@ __host__ __device__ static inline uint64_t mi_stream_key(uint64_t seed, uint64_t
     return mi_mix64(seed ^ (stream_id * 0xD1342543DE82EF95ull));
 }
 __host__ __device__ static inline uint64_t mi_counter_bits(uint64_t key, uint64_t i) {
+#ifdef MI_STUDY_FAKE_HASH
+    return key + i;
+#else
     return mi_mix64(key + i * 0x9E3779B97F4A7C15ull);
+#endif
 }
-// Dropout keep decision for element i: a 24-bit uniform u = bits[63:40] / 2^24 is kept when u >= p,
-// i.e. when its integer value reaches thresh = ceil(p * 2^24).
+// Dropout keep decisions: one 64-bit word serves the four elements i = 4g .. 4g+3 (the word of counter g),
+// 16 bits each: element i is kept when u = (bits(g) >> 16*(i & 3)) & 0xFFFF reaches thresh = ceil(p * 2^16).
+// The hash (two 64-bit multiplies) is by far the dearest part of a decision, and in the MFMA accumulator
+// layouts a lane, or a quad of lanes, holds four consecutive elements: one hash per four weights.
 #define MI_DROPOUT_STREAM 0x64726F70ull   // stream id reserved for dropout masks
 static inline uint32_t mi_dropout_threshold(float p) {
-    const double t = ceil((double)p * 16777216.0);
-    return t <= 0.0 ? 0u : (t >= 16777216.0 ? 16777216u : (uint32_t)t);
+    const double t = ceil((double)p * 65536.0);
+    return t <= 0.0 ? 0u : (t >= 65536.0 ? 65536u : (uint32_t)t);
+}
+__device__ static inline uint64_t mi_dropout_group_bits(uint64_t key, uint64_t group) { return mi_counter_bits(key, group); }
+__device__ static inline bool mi_dropout_keep_in(uint64_t bits, int sub, uint32_t thresh) {
+    return ((uint32_t)(bits >> (16 * sub)) & 0xFFFFu) >= thresh;
 }
 __device__ static inline bool mi_dropout_keep(uint64_t key, uint64_t i, uint32_t thresh) {
-    return (uint32_t)(mi_counter_bits(key, i) >> 40) >= thresh;
+    return mi_dropout_keep_in(mi_dropout_group_bits(key, i >> 2), (int)(i & 3), thresh);
 }
 
 // wavefront (64 lanes) reductions

@@ -358,12 +358,16 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
         // before the value product and before the weights are written, which are post-dropout.
         if (PHASE != PHASE_STATS && p.drop_thresh != 0) {
             const uint64_t row0 = (uint64_t)(p.Lkv * (qi + p.Lq * (h + p.H * b)) + j0 + 4 * hh);
+            const bool aligned = (p.Lkv & 3) == 0;   // every run of four keys of a lane is one hash group
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const bool keep = mi_dropout_keep(p.drop_key, row0 + (uint64_t)(32 * kb + 8 * (v / 4) + (v % 4)), p.drop_thresh);
-                    s[qb][kb][v] = keep ? s[qb][kb][v] * p.drop_scale : 0.0f;
+                for (int g = 0; g < 4; g++) {
+                    float f[4];
+                    if (aligned) attention_drop_factors_run4<true>(p, row0 + 32 * kb, g, f);
+                    else attention_drop_factors_run4<false>(p, row0 + 32 * kb, g, f);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) s[qb][kb][4 * g + e] *= f[e];
                 }
         }
 

@@ -119,14 +119,16 @@ def _mix64(z):
 
 def dropout_keep_mask(shape, p, seed):
     """Keep decisions (column-major linear index order) of the library's dropout stream: the published
-    definition restated in numpy: bits(i) = mix64(mix64(seed ^ stream*C) + i*G), u = bits >> 40 (24 bits),
-    keep = u >= ceil(p * 2^24).  The product's kernels must reproduce exactly this mask."""
+    definition restated in numpy: bits(g) = mix64(mix64(seed ^ stream*C) + g*G) serves the four elements
+    i = 4g .. 4g+3, u(i) = (bits(i >> 2) >> 16*(i & 3)) & 0xFFFF, keep = u >= ceil(p * 2^16).  The product's
+    kernels must reproduce exactly this mask."""
     n = int(np.prod(shape, dtype=np.int64))
+    i = np.arange(n, dtype=np.uint64)
     with np.errstate(over="ignore"):
         key = _mix64(np.array([seed], dtype=np.uint64) ^ (np.uint64(0x64726F70) * np.uint64(0xD1342543DE82EF95)))
-        bits = _mix64(key + np.arange(n, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15))
-    thresh = min(max(int(np.ceil(np.float32(p).astype(np.float64) * 16777216.0)), 0), 16777216)
-    keep = (bits >> np.uint64(40)).astype(np.int64) >= thresh
+        bits = _mix64(key + (i >> np.uint64(2)) * np.uint64(0x9E3779B97F4A7C15))
+    thresh = min(max(int(np.ceil(np.float32(p).astype(np.float64) * 65536.0)), 0), 65536)
+    keep = ((bits >> (np.uint64(16) * (i & np.uint64(3)))) & np.uint64(0xFFFF)).astype(np.int64) >= thresh
     return keep.reshape(shape, order="F")
 
 
