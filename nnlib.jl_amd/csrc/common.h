@@ -132,11 +132,7 @@ __host__ __device__ static inline uint64_t mi_stream_key(uint64_t seed, uint64_t
     return mi_mix64(seed ^ (stream_id * 0xD1342543DE82EF95ull));
 }
 __host__ __device__ static inline uint64_t mi_counter_bits(uint64_t key, uint64_t i) {
-#ifdef MI_STUDY_FAKE_HASH
-    return key + i;
-#else
     return mi_mix64(key + i * 0x9E3779B97F4A7C15ull);
-#endif
 }
 // Dropout keep decisions: one 64-bit word serves the four elements i = 4g .. 4g+3 (the word of counter g),
 // 16 bits each: element i is kept when u = (bits(g) >> 16*(i & 3)) & 0xFFFF reaches thresh = ceil(p * 2^16).
