@@ -65,7 +65,17 @@ int32_t launch_flash_merge(const AttnParams &p, int nsplit, hipStream_t st);
 enum { PHASE_ONLINE = 0, PHASE_STATS = 1, PHASE_FINAL = 2 };
 // how a kernel variant reads bias / mask: not at all, straight from global memory with arbitrary
 // strides, or from tiles staged through LDS (FlashStaged; every array present must qualify)
-enum { EXTRAS_NONE = 0, EXTRAS_DIRECT = 1, EXTRAS_STAGED = 2 };
+// EXTRAS_KEYMASK: no bias and a mask that does not depend on the query (a key-padding mask, query stride 0):
+// the scores stay raw dot products as with EXTRAS_NONE and dropped keys are set to -Inf from one mask byte per key.
+enum { EXTRAS_NONE = 0, EXTRAS_DIRECT = 1, EXTRAS_STAGED = 2, EXTRAS_KEYMASK = 3 };
+// true when the accumulators hold the reference's logits in natural units (bias added) rather than raw dot products
+constexpr bool flash_natural_units(int extras) { return extras == EXTRAS_DIRECT || extras == EXTRAS_STAGED; }
+// query-independent mask without bias whose bytes can be read four keys at a time (unit key stride, Lkv a
+// multiple of 4, 4-byte aligned slices): eligible for EXTRAS_KEYMASK
+inline bool flash_is_key_mask(const AttnParams &p) {
+    return p.mask && !p.bias && p.mask_strides[1] == 0 && p.mask_strides[0] == 1 && (p.Lkv & 3) == 0 &&
+           ((p.mask_strides[2] | p.mask_strides[3]) & 3) == 0 && (((uintptr_t)p.mask) & 3) == 0;
+}
 
 inline void flash_fill_vec_flags(FlashArgs &a) {
     const AttnParams &p = a.p;
@@ -142,7 +152,10 @@ struct FlashStaged {
         {   // set up unconditionally so that the resource words stay in scalar registers
             const int64_t s1 = p.bias_strides[1];
             const char *base = (const char *)p.bias + 2 * (h * p.bias_strides[2] + b * p.bias_strides[3]);
-            brs = flash_make_rsrc(base, (uint32_t)(2 * ((p.Lq - 1) * s1 + p.Lkv)));
+            // sizes are rounded up to whole dwords: the range check is per dword, and a row end that is not a
+            // multiple of 4 bytes (rows with stride 0 and any Lkv) would lose its last keys; the dword that
+            // holds the last valid byte lies in the same page, and keys past Lkv are dropped by the edge code
+            brs = flash_make_rsrc(base, (uint32_t)((2 * ((p.Lq - 1) * s1 + p.Lkv) + 3) & ~(int64_t)3));
 #pragma unroll
             for (int i = 0; i < 4 * QB; i++) {
                 const int row = 8 * i + (lane >> 3);
@@ -152,7 +165,7 @@ struct FlashStaged {
         {
             const int64_t s1 = p.mask_strides[1];
             const char *base = (const char *)p.mask + h * p.mask_strides[2] + b * p.mask_strides[3];
-            mrs = flash_make_rsrc(base, (uint32_t)((p.Lq - 1) * s1 + p.Lkv));
+            mrs = flash_make_rsrc(base, (uint32_t)(((p.Lq - 1) * s1 + p.Lkv + 3) & ~(int64_t)3));
 #pragma unroll
             for (int i = 0; i < 2 * QB; i++) {
                 const int row = 16 * i + (lane >> 2);
@@ -195,11 +208,24 @@ struct FlashStaged {
 // with m, l (and, ONLINE only, the output accumulators o) updated.
 //   T      element traits of the bias array
 //   NDV    number of 32-row blocks of the output accumulator
+// Key-mask bytes of a 64-key tile in the accumulator layout: word 4*kb + g holds the four bytes of keys
+// j0 + 32kb + 8g + 4hh .. +3 (nonzero = keep; keys past Lkv read as kept, the edge code drops them).  All lanes
+// of a half-wave read the same bytes.  Callers issue this before the QK^T MFMAs so that the loads are hidden.
+__device__ inline void flash_load_key_mask(const FlashArgs &a, int64_t b, int64_t h, int64_t j0, int hh, uint32_t (&w)[8]) {
+    const AttnParams &p = a.p;
+    const uint8_t *mk = p.mask + h * p.mask_strides[2] + b * p.mask_strides[3] + j0 + 4 * hh;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int off = 32 * (i >> 2) + 8 * (i & 3);
+        w[i] = j0 + 4 * hh + off < p.Lkv ? *(const uint32_t *)(mk + off) : 0x01010101u;   // Lkv is a multiple of 4
+    }
+}
+
 template <typename T, int QB, int NDV, bool CAUSAL, int EXTRAS, int PHASE, typename TW>
 __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB][2], floatx16_t (&o)[QB][NDV],
                                           float (&fm)[QB], float (&fl)[QB], int64_t b, int64_t h, int64_t iw,
                                           int64_t j0, const FlashStaged<QB> &sg = FlashStaged<QB>(), int stage = 0,
-                                          unsigned wlds = 0) {
+                                          unsigned wlds = 0, const uint32_t *key_mask = nullptr) {
     const AttnParams &p = a.p;
     typedef typename T::type elem_t;
     constexpr int BN = FLASH_BN;
@@ -286,6 +312,20 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                     }
                 }
         }
+        if (EXTRAS == EXTRAS_KEYMASK) {
+            // one mask byte per key, shared by every query
+            uint32_t own[8];
+            if (!key_mask) flash_load_key_mask(a, b, h, j0, hh, own);
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const uint32_t m4 = key_mask ? key_mask[4 * kb + g] : own[4 * kb + g];
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        s[qb][kb][4 * g + e] = ((m4 >> (8 * e)) & 0xFFu) ? s[qb][kb][4 * g + e] : MI_NEG_INF;
+                }
+        }
         if (EXTRAS != EXTRAS_DIRECT && edge) {
             // keys past the end of the sequence or, causal, after the query: tile-local limit per lane
             int64_t lim64 = p.Lkv - j0;
@@ -299,7 +339,8 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                     s[qb][kb][v] = kvl < lim ? s[qb][kb][v] : MI_NEG_INF;
                 }
         }
-        const float cs = EXTRAS ? MI_LOG2E : a.c;
+        constexpr bool NAT = flash_natural_units(EXTRAS);
+        const float cs = NAT ? MI_LOG2E : a.c;
 
         float pmul = 1.0f, msafe;
         bool pinf;  // the running maximum is +Inf: weights become the normalised indicator of the +Inf entries
@@ -314,7 +355,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             const float mnew = fmaxf(mold, mx);
             msafe = mnew == MI_NEG_INF ? 0.0f : mnew;
             float resc = mi_exp2((mold - msafe) * cs);
-            if (EXTRAS && mold == mnew) resc = 1.0f;  // also covers +Inf == +Inf
+            if (NAT && mold == mnew) resc = 1.0f;  // also covers +Inf == +Inf
             pinf = mnew == MI_POS_INF;
             fm[qb] = mnew;
             fl[qb] *= resc;
@@ -331,7 +372,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
         }
         // src/softmax.jl:74-75.  Only bias or an upstream overflow can produce +Inf logits, so the
         // per-element work sits behind a wavefront-uniform test.
-        if (EXTRAS && __builtin_expect(__builtin_amdgcn_ballot_w64(pinf) != 0, 0)) {
+        if (NAT && __builtin_expect(__builtin_amdgcn_ballot_w64(pinf) != 0, 0)) {
             if (pinf) {
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++)

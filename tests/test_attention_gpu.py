@@ -185,6 +185,10 @@ FLASH16_CASES = [
     ("f16", 128, 70, 336, 2, 2, dict(bias_shape=(336, 70, 2, 2), mask_shape=(336, 70, 1, 2))),
     ("bf16", 256, 150, 400, 1, 2, dict(bias_shape=(400, 150, 1, 1), mask_shape=(400, 1, 2, 1))),
     ("bf16", 128, 192, 192, 2, 2, dict(causal=True, bias_shape=(192, 192, 2, 1))),
+    # masks that do not depend on the query (key-padding masks): one mask byte per key, raw-score path
+    ("bf16", 256, 150, 400, 2, 2, dict(mask_shape=(400, 1, 1, 2))),
+    ("f16", 128, 70, 131, 2, 2, dict(mask_shape=(131,))),                 # unaligned length: byte loads
+    ("bf16", 128, 200, 520, 1, 2, dict(mask_shape=(520, 1, 2))),
     # long enough for the steady-state loop of the software-pipelined kernel, head dims 64 and 128
     ("bf16", 128, 300, 700, 1, 2, {}),
     ("bf16", 128, 520, 520, 1, 2, dict(causal=True)),
@@ -337,3 +341,30 @@ def test_plus_inf_logits(nn, oracle, dtype, E, Lkv, expect, weights):
     if weights:
         assert np.allclose(a, ar, atol=tol)
         assert a[3, 5, 0, 0] == 0.5 and a[Lkv - 2, 5, 1, 1] == 0.5 and a[70, 9, 0, 1] == 1.0 and a[1, 5, 0, 0] == 0.0
+
+
+@pytest.mark.parametrize("dtype,E,H", [("bf16", 256, 2), ("f16", 128, 2)])
+@pytest.mark.parametrize("weights", [False, True], ids=["noweights", "weights"])
+def test_key_padding_masks(nn, oracle, dtype, E, H, weights):
+    """Masks broadcast along the queries (batched sequences of different lengths): a padded tail, a dropped head
+    that spans the whole first tile, scattered keys, and one batch element with every key dropped (NaN, as
+    src/softmax.jl:73-75 gives for a fully masked column)."""
+    rng = np.random.default_rng(21)
+    Lq, Lkv, B = 140, 330, 4
+    q, k, v = (round_to(rng.standard_normal((E, L, B)), dtype) for L in (Lq, Lkv, Lkv))
+    mask = np.ones((Lkv, 1, 1, B), dtype=bool)
+    mask[250:, 0, 0, 0] = False            # padded tail
+    mask[:100, 0, 0, 1] = False            # the first tile and a half dropped
+    mask[:, 0, 0, 2] = rng.random(Lkv) < 0.5
+    mask[:, 0, 0, 3] = False               # nothing kept
+    y, a = _run(nn, q, k, v, dtype, None, mask, H, return_weights=weights, weights_dtype="f32" if weights else None)
+    assert nn.last_attention_kernel() == "flash16"
+    with np.errstate(invalid="ignore"):
+        yr, ar = oracle.nnlib_attention_f32(q, k, v, None, mask, H, nthreads=4)
+    assert np.isnan(y[:, :, 3]).all() and np.isnan(yr[:, :, 3]).all()
+    assert rel_err(y[:, :, :3], yr[:, :, :3]) <= TOL[dtype]
+    if weights:
+        assert np.isnan(a[..., 3]).all()
+        assert np.abs(a[..., :3] - ar[..., :3]).max() <= TOL[dtype]
+        keep = np.broadcast_to(mask, a.shape)[..., :3]
+        assert np.count_nonzero(a[..., :3][~keep]) == 0
