@@ -26,6 +26,11 @@ def _run(nn, oracle, dtype, E, Ev, Lq, Lkv, batch, H, bias_shape=None, mask_kind
         mask = rng.random((Lkv, Lq)) < 0.8
         mask[0] = True
         dmask = nn.DeviceArray.from_numpy(mask)
+    elif mask_kind == "keys":       # key-padding mask: no query dependence, one pattern per batch element
+        mask = rng.random((Lkv, 1, 1) + batch) < 0.7
+        mask[Lkv // 2, ...] = True
+        mask[:70, 0, 0, ..., -1] = False          # the first tile and a bit dropped for the last batch element
+        dmask = nn.DeviceArray.from_numpy(mask)
     da = round_to(rng.standard_normal((Lkv, Lq, H) + batch), dtype) if with_dalpha else None
     D = nn.DeviceArray.from_numpy
     dq_, dk_, dv_ = D(q, dtype), D(k, dtype), D(v, dtype)
@@ -284,6 +289,19 @@ def _bias_input_case(nn, oracle, dtype, E, H, Lq, Lkv, batch, mask_kind, bias_sh
     ref = oracle.attention_bwd_f64(q, k, v, dy, bias, mask, H, keep_scale=g)
     for o, r in zip(outs, ref[:3]):
         assert np.abs(o.to_numpy() - r).max() / max(np.abs(r).max(), 0.05) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype,D,H,Lq,Lkv,batch,saved,dropout", [
+    ("bf16", 128, 2, 192, 256, (2,), False, None),
+    ("bf16", 64, 2, 150, 200, (3,), True, None),
+    ("f16", 128, 1, 70, 328, (2,), False, (0.25, 99)),
+    ("f16", 64, 2, 257, 132, (2,), True, (0.25, 99)),
+])
+def test_key_padding_mask_on_the_lean_paths(nn, oracle, dtype, D, H, Lq, Lkv, batch, saved, dropout):
+    """A mask that does not depend on the query keeps the two-wavefront gradient kernels: one mask byte per key
+    (dQ: read per 32-key block; dK / dV: a lane's key is kept or dropped for the whole kernel)."""
+    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, batch, H, mask_kind="keys", expect="flash16", saved=saved, dropout=dropout,
+         seed=9)
 
 
 def test_errors(nn):
