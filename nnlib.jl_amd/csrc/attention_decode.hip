@@ -8,8 +8,11 @@
 // Each (segment, kv-split, batch) wavefront keeps an online-softmax state (m, l, o[8]) and writes it
 // to a workspace; a second small kernel merges the splits.
 //
-// Same arithmetic as the reference chain (src/attention.jl:112-127, fdrop = identity, no bias/mask):
+// Same arithmetic as the reference chain (src/attention.jl:112-127, fdrop = identity, no bias):
 //   s_j = sum_d k[d,j] * q[d] / sqrt(D),  a = softmax_j(s),  x[d] = sum_j a_j v[d,j].
+// An optional mask (src/attention.jl:133-138; with a single query every mask is a key mask, e.g. the context
+// lengths of a padded batch) costs one byte per key row and head: dropped keys get the score -Inf, a (head,
+// batch) pair with no key kept gives NaN like the reference.
 #include "common.h"
 #include "attention_params.h"
 
@@ -38,7 +41,7 @@ __device__ inline void unpack8(const u32x4_t &v, float *out, F16) {
 }
 
 // workspace layout: [B][nsplit][E] floats of o, then [B][nsplit][H] of m, then [B][nsplit][H] of l
-template <typename T, int D>
+template <typename T, int D, bool MASKED>
 __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     const AttnParams &p = a.p;
     typedef typename T::type t;
@@ -62,6 +65,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     float m = MI_NEG_INF, l = 0.0f;
     float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const u32x4_t zero = {0, 0, 0, 0};
+    // mask bytes of this lane's head: element (kv, 0, h, b)
+    const uint8_t *mrow = MASKED ? p.mask + (lane_ok ? f / D : 0) * p.mask_strides[2] + b * p.mask_strides[3] : nullptr;
 
     for (int64_t j = j_begin; j < j_end; j += ROWS) {
         u32x4_t kr[ROWS], vr[ROWS];
@@ -75,6 +80,9 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
             const bool ok = lane_ok && j + r < j_end;
             vr[r] = ok ? *(const u32x4_t *)(vb + p.E * (j + r)) : zero;
         }
+        bool keep[ROWS];
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) keep[r] = j + r < j_end && (!MASKED || mrow[(j + r) * p.mask_strides[0]] != 0);
         float s[ROWS];
         float mx = MI_NEG_INF;
 #pragma unroll
@@ -86,12 +94,14 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
             for (int e = 0; e < 8; e++) d = fmaf(kf[e], qf[e], d);
 #pragma unroll
             for (int off = 1; off < D / 8; off <<= 1) d += __shfl_xor(d, off, 64);
-            s[r] = j + r < j_end ? d : MI_NEG_INF;
+            s[r] = keep[r] ? d : MI_NEG_INF;
             mx = fmaxf(mx, s[r]);
         }
-        const float mnew = fmaxf(m, mx);      // finite: at least one row of the chunk is valid
-        const float resc = mi_exp2((m - mnew) * a.c);
+        float mnew = fmaxf(m, mx);            // finite without a mask: at least one row of the chunk is valid
+        const float mref = (MASKED && mnew == MI_NEG_INF) ? 0.0f : mnew;   // nothing kept so far: every term below is 0
+        const float resc = mi_exp2((m - mref) * a.c);
         m = mnew;
+        mnew = mref;
         l *= resc;
 #pragma unroll
         for (int e = 0; e < 8; e++) o[e] *= resc;
@@ -185,7 +195,7 @@ int pick_nsplit(const AttnParams &p) {
 
 bool attention_decode_supports(const AttnParams &p) {
     if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
-    if (p.Lq != 1 || p.weights || p.bias || p.mask || !p.out || p.drop_thresh) return false;
+    if (p.Lq != 1 || p.weights || p.bias || p.causal || !p.out || p.drop_thresh) return false;
     if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
     if (p.Lkv < 512) return false;   // short contexts: the tiled kernel is fine
     if (p.B > 65535) return false;
@@ -210,17 +220,21 @@ int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
         return mi_set_error(MI_EWORKSPACE, "decode workspace must be 16-byte aligned");
     dim3 grid((unsigned)((a.nseg + 3) / 4), (unsigned)a.nsplit, (unsigned)p.B);
     dim3 mgrid((unsigned)((p.E + 255) / 256), (unsigned)p.B);
+#define DECODE_LAUNCH(TT, DD)                                                                         \
+    {                                                                                                 \
+        if (p.mask) hipLaunchKernelGGL((decode_split_kernel<TT, DD, true>), grid, dim3(256), 0, st, a); \
+        else hipLaunchKernelGGL((decode_split_kernel<TT, DD, false>), grid, dim3(256), 0, st, a);       \
+    }
     if (p.dtype == MI_BF16) {
-        if (p.D == 128) hipLaunchKernelGGL((decode_split_kernel<BF16, 128>), grid, dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((decode_split_kernel<BF16, 64>), grid, dim3(256), 0, st, a);
+        if (p.D == 128) DECODE_LAUNCH(BF16, 128) else DECODE_LAUNCH(BF16, 64)
         MI_LAUNCH_CHECK();
         hipLaunchKernelGGL(decode_merge_kernel<BF16>, mgrid, dim3(256), 0, st, a);
     } else {
-        if (p.D == 128) hipLaunchKernelGGL((decode_split_kernel<F16, 128>), grid, dim3(256), 0, st, a);
-        else hipLaunchKernelGGL((decode_split_kernel<F16, 64>), grid, dim3(256), 0, st, a);
+        if (p.D == 128) DECODE_LAUNCH(F16, 128) else DECODE_LAUNCH(F16, 64)
         MI_LAUNCH_CHECK();
         hipLaunchKernelGGL(decode_merge_kernel<F16>, mgrid, dim3(256), 0, st, a);
     }
+#undef DECODE_LAUNCH
     MI_LAUNCH_CHECK();
     return MI_OK;
 }

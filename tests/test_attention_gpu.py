@@ -270,6 +270,30 @@ def test_decode_parity(nn, oracle, dtype, E, H, Lkv, B):
     _check(nn, oracle, rng, dtype, E, 1, Lkv, B, H, expect="decode", weights=False)
 
 
+@pytest.mark.parametrize("dtype,E,H,mask_shape", [("bf16", 512, 4, (1500, 1, 1, 3)), ("f16", 256, 4, (1500, 1, 4, 3)),
+                                                  ("bf16", 128, 2, (1500,))])
+def test_decode_with_context_length_masks(nn, oracle, dtype, E, H, mask_shape):
+    """A single query per (head, batch) with a mask: padded contexts of different lengths per batch element, a
+    pattern per head, one (head, batch) pair with nothing kept (NaN, src/softmax.jl:73-75)."""
+    rng = np.random.default_rng(5)
+    Lkv, B = 1500, 3
+    q, k, v = (round_to(rng.standard_normal((E, L, B)), dtype) for L in (1, Lkv, Lkv))
+    mask = rng.random(mask_shape) < 0.6
+    if len(mask_shape) == 4:
+        mask[900:, 0, :, 0] = False                  # context of 900 keys
+        mask[:700, 0, :, 1] = False                  # whole leading splits dropped
+        mask[:, 0, 0, 2] = False                     # nothing kept for (head 0 or all heads, batch 2)
+    y, _ = _run(nn, q, k, v, dtype, None, mask, H, return_weights=False)
+    assert nn.last_attention_kernel() == "decode"
+    with np.errstate(invalid="ignore"):
+        yr, _ = oracle.nnlib_attention_f32(q, k, v, None, mask, H, nthreads=4)
+    assert np.array_equal(np.isnan(y), np.isnan(yr))
+    if len(mask_shape) == 4:
+        assert np.isnan(y).any()
+    ok = ~np.isnan(yr)
+    assert np.abs(y[ok] - yr[ok]).max() / np.abs(yr[ok]).max() <= TOL[dtype]
+
+
 def test_decode_matches_flash16_on_device(nn):
     rng = np.random.default_rng(11)
     q = nn.DeviceArray.from_numpy(rng.standard_normal((512, 1, 2)).astype(np.float32), "bf16")
