@@ -15,7 +15,7 @@ bool attention_bwd_flash16_supports(const AttnBwdParams &bp) {
     if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
     if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
     // the kernels need the forward result (for delta), take no weight cotangent and give no bias gradient
-    if (!p.out || bp.dweights || bp.dbias) return false;
+    if (!p.out || bp.dweights) return false;   // a bias gradient is summed with atomics by the dQ kernel
     if (!aligned16(p.q) || !aligned16(p.k) || !aligned16(p.v) || !aligned16(p.out) || !aligned16(bp.dout)) return false;
     if ((bp.dq && !aligned16(bp.dq)) || (bp.dk && !aligned16(bp.dk)) || (bp.dv && !aligned16(bp.dv))) return false;
     // tiles are fetched with 32-bit byte offsets from the (batch, head) slice

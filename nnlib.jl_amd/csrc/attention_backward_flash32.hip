@@ -181,9 +181,10 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
             bp.stats[2 * plane + at] = qok ? delta : 0.0f;
         }
     }
-    if (!bp.dq) return;
+    if (!bp.dq && !bp.dbias) return;
 
     // pass 2: P, dP = V dO^T, dS = P (dP - delta), dQ^T += K^T dS^T
+    const unsigned dbias_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)bwd_smem + (unsigned)Cfg<D>::SMEM + wave * FLASH_WSTAGE_BYTES;
     floatx16_t dq[NDV];
 #pragma unroll
     for (int dvb = 0; dvb < NDV; dvb++) dq[dvb] = (floatx16_t){0};
@@ -242,6 +243,24 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
                     }
 #pragma unroll
                     for (int v = 0; v < 16; v++) s[0][kb][v] *= dp[kb][v] - delta;
+                if (bp.dbias) {
+                        // the bias adds to the logits, so its gradient is dS, summed over the dimensions it broadcasts
+                        // along (stride 0): Float32 atomics, one per weight that is not an exact zero
+                        float *db = bp.dbias + h * p.bias_strides[2] + b * p.bias_strides[3];
+                        const int64_t kv0 = j0 + 32 * kb;
+                        if (p.bias_strides[0] == 1) {
+                            const int64_t nq = p.Lq - iw, nk = p.Lkv - kv0;
+                            flash_atomic_add_block(dbias_lds, s[0][kb], db + kv0 + iw * p.bias_strides[1], p.bias_strides[1],
+                                                   (int)(nq > 32 ? 32 : nq), (int)(nk > 32 ? 32 : (nk < 0 ? 0 : nk)));
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; v++) {
+                                const int64_t kvv = kv0 + 8 * (v / 4) + 4 * hh + (v % 4);
+                                if (qok && kvv < p.Lkv && s[0][kb][v] != 0.0f)
+                                    atomicAdd(db + qi * p.bias_strides[1] + kvv * p.bias_strides[0], s[0][kb][v]);
+                            }
+                        }
+                    }
                     second_product<D>(kt, kb, s[0][kb], dq, r, hh);
                 }
             }
@@ -249,7 +268,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
         if (jt + 1 < n_tiles) ts.store(buf ^ 1);
         __syncthreads();
     }
-    if (qok) {
+    if (qok && bp.dq) {
         float *dqrow = (float *)bp.dq + p.E * (qi + p.Lq * b) + D * h;
 #pragma unroll
         for (int dvb = 0; dvb < NDV; dvb++)
@@ -403,6 +422,7 @@ template <int D, bool CAUSAL, int EXTRAS, bool DROP = false>
 int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
     const AttnParams &p = a.p;
     constexpr size_t SMEM = Cfg<D>::SMEM;
+    constexpr size_t SMEM_Q = SMEM + (EXTRAS == EXTRAS_NONE ? 0 : 4 * FLASH_WSTAGE_BYTES);   // the dQ kernel's staging for the bias gradient
     // Two kernels (dV, then dK) where that buys two wavefronts per SIMD (head dim 64 without bias / mask
     // arrays) or is needed to fit the register file at all (head dim 128: K, V, dK and dV of a lane are
     // 256 registers before anything else); one pass otherwise.
@@ -412,13 +432,13 @@ int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) 
     auto k3 = bwd32_dkdv_kernel<D, CAUSAL, EXTRAS, SPLIT ? BWD_DK : 3, DROP>;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
     if (!attr_set) {
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, true, DROP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, false, DROP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, true, DROP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_Q));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32_dq_kernel<D, CAUSAL, EXTRAS, false, DROP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_Q));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         attr_set = true;
     }
-    hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B)), dim3(256), SMEM, st, a, bp);
+    hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B)), dim3(256), SMEM_Q, st, a, bp);
     MI_LAUNCH_CHECK();
     const dim3 g2((unsigned)(((p.Lkv + 127) / 128) * p.H * p.B));
     if (SPLIT) {
@@ -448,7 +468,7 @@ bool attention_bwd_flash32_supports(const AttnBwdParams &bp) {
     if (p.dtype != MI_F32) return false;
     if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
     // the kernels need the forward result (for delta), take no weight cotangent and give no bias gradient
-    if (!p.out || bp.dweights || bp.dbias) return false;
+    if (!p.out || bp.dweights) return false;   // a bias gradient is summed with atomics by the dQ kernel
     auto al = [](const void *x) { return (((uintptr_t)x) & 15) == 0; };
     if (!al(p.q) || !al(p.k) || !al(p.v) || !al(p.out) || !al(bp.dout)) return false;
     if ((bp.dq && !al(bp.dq)) || (bp.dk && !al(bp.dk)) || (bp.dv && !al(bp.dv))) return false;

@@ -208,6 +208,61 @@ struct FlashStaged {
 // with m, l (and, ONLINE only, the output accumulators o) updated.
 //   T      element traits of the bias array
 //   NDV    number of 32-row blocks of the output accumulator
+// Orders a wavefront's LDS stores and loads around a cross-lane exchange: a compiler-level barrier (no instruction
+// is emitted; the LDS unit completes the operations of one wavefront in issue order).
+__device__ inline void flash_wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Adds a 32-key x 32-query block of Float32 values held in the MFMA accumulator layout (lane (r, hh): query row r
+// of the wavefront; register 4g + e: key 8g + 4hh + e of the block) to a Float32 array whose keys are contiguous:
+// dst points at (first key of the block, first query row of the wavefront), rows are qstride elements apart (0: every
+// query adds to the same row).  Straight from the registers one atomic instruction would touch 64 cache lines; the
+// block goes through the wavefront's FLASH_WSTAGE_BYTES LDS region 16 queries at a time and comes back with 8 lanes
+// per query row, so an instruction covers 8 rows of 128 contiguous bytes.  Exact zeros are skipped.
+__device__ inline void flash_atomic_add_block(unsigned wlds, const floatx16_t &v, float *dst, int64_t qstride, int nq, int nk) {
+    typedef __attribute__((address_space(3))) u32x4_t *lds16_t;
+    const int lane = threadIdx.x & 63, r = lane & 31, hh = lane >> 5;
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        if ((r >> 4) == half) {
+            const unsigned rowa = wlds + (unsigned)(r & 15) * 128u;
+            const int sw = (r >> 1) & 7;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                floatx4_t t4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) t4[e] = v[4 * g + e];
+                *(lds16_t)(uintptr_t)(rowa + (unsigned)(((2 * g + hh) ^ sw) << 4)) = __builtin_bit_cast(u32x4_t, t4);
+            }
+        }
+        // lanes exchange data through LDS: to the compiler a lane's loads below never alias its own stores above, so
+        // the order has to be pinned (the LDS itself completes a wavefront's operations in order)
+        flash_wave_lds_fence();
+        floatx4_t pieces[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int rr = (lane >> 3) + 8 * i, c = lane & 7;
+            pieces[i] = __builtin_bit_cast(floatx4_t, *(lds16_t)(uintptr_t)(wlds + (unsigned)rr * 128u + (unsigned)((c ^ ((rr >> 1) & 7)) << 4)));
+        }
+        flash_wave_lds_fence();
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int rr = (lane >> 3) + 8 * i, c = lane & 7;
+            const floatx4_t piece = pieces[i];
+            const int q = 16 * half + rr;
+            if (q < nq) {
+                float *row = dst + q * qstride + 4 * c;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (4 * c + e < nk && piece[e] != 0.0f) atomicAdd(row + e, piece[e]);
+            }
+        }
+    }
+}
+
 // Key-mask bytes of a 64-key tile in the accumulator layout: word 4*kb + g holds the four bytes of keys
 // j0 + 32kb + 8g + 4hh .. +3 (nonzero = keep; keys past Lkv read as kept, the edge code drops them).  All lanes
 // of a half-wave read the same bytes.  Callers issue this before the QK^T MFMAs so that the loads are hidden.
@@ -452,10 +507,18 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                             }
                         }
                     }
+                    flash_wave_lds_fence();   // a lane's loads never alias its own stores: the exchange has to be pinned
+                    u32x4_t pieces[2];
 #pragma unroll
                     for (int i = 0; i < 2; i++) {
                         const int rr = (lane >> 3) + 8 * i, c = lane & 7;
-                        const u32x4_t piece = *(lds16_t)(uintptr_t)(wlds + (unsigned)rr * 128u + (unsigned)((c ^ ((rr >> 1) & 7)) << 4));
+                        pieces[i] = *(lds16_t)(uintptr_t)(wlds + (unsigned)rr * 128u + (unsigned)((c ^ ((rr >> 1) & 7)) << 4));
+                    }
+                    flash_wave_lds_fence();
+#pragma unroll
+                    for (int i = 0; i < 2; i++) {
+                        const int rr = (lane >> 3) + 8 * i, c = lane & 7;
+                        const u32x4_t piece = pieces[i];
                         const int64_t qrow = iw + 32 * qb + 16 * half + rr, kv0 = j0 + 32 * rk * (NKB - 1) + (int64_t)c * EPC;
                         if (qrow < p.Lq && kv0 < p.Lkv) *(u32x4_t *)(wbase + p.Lkv * qrow + kv0) = piece;   // Lkv is a multiple of EPC here
                     }

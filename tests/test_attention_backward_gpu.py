@@ -113,7 +113,20 @@ def test_mfma_kernels(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, bias_k
     elif bias_kind == "row":
         bias_shape = (Lkv, 1)
     _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, batch, H, bias_shape=bias_shape, mask_kind=mask_kind, seed=Lq + Lkv,
-         scale=0.4, expect="flash16" if bias_shape is None else "generic")
+         scale=0.4, expect="flash16")
+
+
+@pytest.mark.parametrize("dtype,D,H,Lq,Lkv,batch,mask_kind,bias_shape,expect", [
+    ("f32", 64, 2, 130, 200, (2,), None, (200, 130, 2, 2), "flash32"),
+    ("f32", 128, 1, 96, 160, (2,), "random", (160, 96), "flash32"),          # broadcast over heads and batch: summed
+    ("bf16", 128, 2, 200, 200, (2,), "causal", (200, 200, 2, 1), "flash16"),
+    ("f16", 64, 2, 70, 300, (3,), None, (300, 1, 1, 3), "flash16"),          # one bias value per key and batch element
+])
+def test_bias_gradient_from_the_mfma_kernels(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, bias_shape, expect):
+    """The bias gradient is dS summed over the dims the bias broadcasts along; the dQ kernels add it with Float32
+    atomics (the reference gets it from the broadcast rule of `.+`, src/attention.jl:129-131)."""
+    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, batch, H, bias_shape=bias_shape, mask_kind=mask_kind, seed=Lq * 3 + Lkv,
+         scale=0.4, expect=expect)
 
 
 F32_CASES = [
