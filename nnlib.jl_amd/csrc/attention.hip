@@ -6,6 +6,8 @@ int32_t launch_flash16_bf16_d64(const AttnParams &, hipStream_t);
 int32_t launch_flash16_bf16_d128(const AttnParams &, hipStream_t);
 int32_t launch_flash16_f16_d64(const AttnParams &, hipStream_t);
 int32_t launch_flash16_f16_d128(const AttnParams &, hipStream_t);
+int32_t launch_flash16_bf16_d256(const AttnParams &, hipStream_t);
+int32_t launch_flash16_f16_d256(const AttnParams &, hipStream_t);
 int32_t launch_flash16_fast_bf16(const AttnParams &, hipStream_t);
 int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t);
 bool flash16_fast_supports_bf16(const AttnParams &);
@@ -70,7 +72,9 @@ static bool takes_fast_path(const AttnParams &p);
 
 bool attention_flash16_supports(const AttnParams &p) {
     if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
-    if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
+    // head dims: multiples of 8 (16-byte chunks) up to the 256-wide tiles; the tile width (64, 128 or 256) is the
+    // smallest that holds both, and what it has beyond them is zero-padded in flight
+    if (p.D < 8 || p.Dv < 8 || p.D > 256 || p.Dv > 256 || (p.D & 7) || (p.Dv & 7)) return false;
     if (!aligned16(p.q) || !aligned16(p.k) || (p.out && (!aligned16(p.v) || !aligned16(p.out)))) return false;
     // one workgroup per (query tile, head, batch) in a 1-D grid
     const int64_t tiles = (p.Lq + 127) / 128;
@@ -89,8 +93,10 @@ int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
     if (p.dtype == MI_F16 && flash16_fast_supports_f16(p)) return launch_flash16_fast_f16(p, st);
     if (p.dtype == MI_BF16 && flash16_fast_supports_bf16_d64(p)) return launch_flash16_fast_bf16_d64(p, st);
     if (p.dtype == MI_F16 && flash16_fast_supports_f16_d64(p)) return launch_flash16_fast_f16_d64(p, st);
-    if (p.dtype == MI_BF16) return p.D == 64 ? launch_flash16_bf16_d64(p, st) : launch_flash16_bf16_d128(p, st);
-    return p.D == 64 ? launch_flash16_f16_d64(p, st) : launch_flash16_f16_d128(p, st);
+    const int64_t dmax = p.D > p.Dv ? p.D : p.Dv;
+    if (p.dtype == MI_BF16)
+        return dmax <= 64 ? launch_flash16_bf16_d64(p, st) : dmax <= 128 ? launch_flash16_bf16_d128(p, st) : launch_flash16_bf16_d256(p, st);
+    return dmax <= 64 ? launch_flash16_f16_d64(p, st) : dmax <= 128 ? launch_flash16_f16_d128(p, st) : launch_flash16_f16_d256(p, st);
 }
 
 // Validation.  The first four conditions are the reference's ArgumentErrors

@@ -36,12 +36,13 @@ __device__ inline floatx4_t ldg16f(const float *p, bool ok) {
 }
 
 // Streams [BN][D] tiles of up to two row-major arrays through registers into double-buffered LDS tiles;
-// rows from `nrows` on read as zeros.
+// rows from `nrows` on and feature chunks from the head dim `dh` on (D is the tile width) read as zeros.
 template <int D>
 struct TileStream32 {
     static constexpr int KS = Cfg<D>::KS, CHUNKS = Cfg<D>::CHUNKS;
     const float *base1, *base2;   // base2 may be null
     int64_t stride, nrows;
+    int dh;
     float *s1, *s2;
     floatx4_t r1[CHUNKS], r2[CHUNKS];
     __device__ void load(int64_t row0) {
@@ -49,7 +50,7 @@ struct TileStream32 {
         for (int u = 0; u < CHUNKS; u++) {
             const int c = threadIdx.x + 256 * u;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-            const bool ok = row0 + row < nrows;
+            const bool ok = row0 + row < nrows && col < dh;
             r1[u] = ldg16f(base1 + stride * (row0 + row) + col, ok);
             if (base2) r2[u] = ldg16f(base2 + stride * (row0 + row) + col, ok);
         }
@@ -93,10 +94,10 @@ __device__ inline void second_product(const float *tile, int kb, const floatx16_
 
 // stationary row in the permuted feature order of first_product
 template <int D>
-__device__ inline void load_stationary(float (&x)[D / 2], const float *row, bool ok, int hh) {
+__device__ inline void load_stationary(float (&x)[D / 2], const float *row, bool ok, int hh, int dh) {
 #pragma unroll
     for (int c = 0; c < D / 8; c++) {
-        const floatx4_t q4 = ldg16f(row + 8 * c + 4 * hh, ok);
+        const floatx4_t q4 = ldg16f(row + 8 * c + 4 * hh, ok && 8 * c + 4 * hh < dh);
 #pragma unroll
         for (int j = 0; j < 4; j++) x[4 * c + j] = q4[j];
     }
@@ -122,11 +123,11 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
     float qx[D / 2], dox[D / 2];
     float delta = 0.0f;
     {
-        const int64_t off = p.E * (qi + p.Lq * b) + D * h;   // E == Ev for these kernels
-        load_stationary<D>(qx, (const float *)p.q + off, qok, hh);
-        load_stationary<D>(dox, (const float *)bp.dout + off, qok, hh);
+        const int64_t off = p.E * (qi + p.Lq * b) + p.D * h;   // E == Ev for these kernels
+        load_stationary<D>(qx, (const float *)p.q + off, qok, hh, (int)p.D);
+        load_stationary<D>(dox, (const float *)bp.dout + off, qok, hh, (int)p.D);
         float ox[D / 2];
-        load_stationary<D>(ox, (const float *)p.out + off, qok, hh);
+        load_stationary<D>(ox, (const float *)p.out + off, qok, hh, (int)p.D);
 #pragma unroll
         for (int e = 0; e < D / 2; e++) delta = fmaf(ox[e], dox[e], delta);
         delta += mi_swap32(delta);
@@ -137,7 +138,8 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
     const int n_tiles = (int)((kv_end + BN - 1) / BN);
 
     TileStream32<D> ts;
-    ts.base1 = (const float *)p.k + p.E * (p.Lkv * b) + D * h;
+    ts.base1 = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
+    ts.dh = (int)p.D;
     ts.stride = p.E;
     ts.nrows = p.Lkv;
     ts.s1 = Ks;
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
     floatx16_t dq[NDV];
 #pragma unroll
     for (int dvb = 0; dvb < NDV; dvb++) dq[dvb] = (floatx16_t){0};
-    ts.base2 = (const float *)p.v + p.Ev * (p.Lkv * b) + D * h;
+    ts.base2 = (const float *)p.v + p.Ev * (p.Lkv * b) + p.D * h;
     ts.load(0);
     __syncthreads();   // pass 1 may still be reading the tiles
     ts.store(0);
@@ -269,7 +271,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
         __syncthreads();
     }
     if (qok && bp.dq) {
-        float *dqrow = (float *)bp.dq + p.E * (qi + p.Lq * b) + D * h;
+        float *dqrow = (float *)bp.dq + p.E * (qi + p.Lq * b) + p.D * h;
 #pragma unroll
         for (int dvb = 0; dvb < NDV; dvb++)
 #pragma unroll
@@ -277,7 +279,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
                 floatx4_t o4;
 #pragma unroll
                 for (int e = 0; e < 4; e++) o4[e] = dq[dvb][4 * g + e] * a.cn;
-                *(floatx4_t *)(dqrow + 32 * dvb + 8 * g + 4 * hh) = o4;
+                if (32 * dvb + 8 * g + 4 * hh < p.D) *(floatx4_t *)(dqrow + 32 * dvb + 8 * g + 4 * hh) = o4;
             }
     }
 }
@@ -300,9 +302,9 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
 
     float kx[D / 2], vx[DO_DK ? D / 2 : 1];
     {
-        const int64_t off = p.E * (kv + p.Lkv * b) + D * h;
-        load_stationary<D>(kx, (const float *)p.k + off, kok, hh);
-        if constexpr (DO_DK) load_stationary<D>(vx, (const float *)p.v + off, kok, hh);
+        const int64_t off = p.E * (kv + p.Lkv * b) + p.D * h;
+        load_stationary<D>(kx, (const float *)p.k + off, kok, hh, (int)p.D);
+        if constexpr (DO_DK) load_stationary<D>(vx, (const float *)p.v + off, kok, hh, (int)p.D);
     }
     floatx16_t dk[NDV], dv[NDV];
 #pragma unroll
@@ -319,8 +321,9 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
     const float cs = EXTRAS ? MI_LOG2E : a.c;
 
     TileStream32<D> ts;
-    ts.base1 = (const float *)p.q + p.E * (p.Lq * b) + D * h;
-    ts.base2 = (const float *)bp.dout + p.E * (p.Lq * b) + D * h;
+    ts.base1 = (const float *)p.q + p.E * (p.Lq * b) + p.D * h;
+    ts.base2 = (const float *)bp.dout + p.E * (p.Lq * b) + p.D * h;
+    ts.dh = (int)p.D;
     ts.stride = p.E;
     ts.nrows = p.Lq;
     ts.s1 = Qs;
@@ -401,11 +404,12 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
         __syncthreads();
     }
     if (kok) {
-        const int64_t off = p.E * (kv + p.Lkv * b) + D * h;
+        const int64_t off = p.E * (kv + p.Lkv * b) + p.D * h;
 #pragma unroll
         for (int dvb = 0; dvb < NDV; dvb++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
+                if (32 * dvb + 8 * g + 4 * hh >= p.D) continue;
                 floatx4_t k4, v4;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -466,7 +470,8 @@ int32_t launch_d(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
 bool attention_bwd_flash32_supports(const AttnBwdParams &bp) {
     const AttnParams &p = bp.p;
     if (p.dtype != MI_F32) return false;
-    if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
+    // one head dim for q, k and v: a multiple of 4 (16-byte chunks) up to the 128-wide tiles
+    if (p.D != p.Dv || p.D < 4 || p.D > 128 || (p.D & 3)) return false;
     // the kernels need the forward result (for delta), take no weight cotangent and give no bias gradient
     if (!p.out || bp.dweights) return false;   // a bias gradient is summed with atomics by the dQ kernel
     auto al = [](const void *x) { return (((uintptr_t)x) & 15) == 0; };
@@ -490,5 +495,5 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st) {
     flash_fill_vec_flags(a);
     a.bias_lds = a.mask_lds = 0;
     a.p.drop_thresh = 0;   // the shared softmax step yields the weights before dropout; the kernels apply bp.p's dropout themselves
-    return bp.p.D == 64 ? launch_d<64>(a, bp, st) : launch_d<128>(a, bp, st);
+    return bp.p.D <= 64 ? launch_d<64>(a, bp, st) : launch_d<128>(a, bp, st);
 }

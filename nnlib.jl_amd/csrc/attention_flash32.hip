@@ -44,8 +44,10 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
     constexpr bool NEED_V = PHASE != PHASE_STATS;
     const bool do_pv = NEED_V && p.out != nullptr;
 
-    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + D * h;
-    const float *vbase = NEED_V && p.v ? (const float *)p.v + p.Ev * (p.Lkv * b) + D * h : nullptr;
+    // D is the tile width; the head dims p.D / p.Dv may be smaller (multiples of 4): the rest is loaded as zeros
+    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
+    const float *vbase = NEED_V && p.v ? (const float *)p.v + p.Ev * (p.Lkv * b) + p.Dv * h : nullptr;
+    const int dqk = (int)p.D, dv = (int)p.Dv;
 
     floatx4_t kreg[CHUNKS], vreg[CHUNKS];
     auto load_tile = [&](int jt) {
@@ -55,8 +57,8 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
             const int c = tid + 256 * u;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
             const bool ok = j0 + row < p.Lkv;
-            kreg[u] = ldg16f(kbase + p.E * (j0 + row) + col, ok);
-            if (NEED_V) vreg[u] = ldg16f(vbase + p.Ev * (j0 + row) + col, ok && do_pv);
+            kreg[u] = ldg16f(kbase + p.E * (j0 + row) + col, ok && col < dqk);
+            if (NEED_V) vreg[u] = ldg16f(vbase + p.Ev * (j0 + row) + col, ok && do_pv && col < dv);
         }
     };
     auto store_tile = [&](int buf) {
@@ -147,14 +149,14 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
     const int64_t i0 = qt * BM, iw = i0 + (int64_t)wave * 32 * QB;
 
     Frag32<D, QB> f;
-    const float *qbase = (const float *)p.q + p.E * (p.Lq * b) + D * h;
-    const float sq = sqrtf((float)D);
+    const float *qbase = (const float *)p.q + p.E * (p.Lq * b) + p.D * h;
+    const float sq = sqrtf((float)p.D);
 #pragma unroll
     for (int qb = 0; qb < QB; qb++) {
         const int64_t qi = iw + 32 * qb + r;
 #pragma unroll
         for (int c = 0; c < D / 8; c++) {
-            const floatx4_t q4 = ldg16f(qbase + p.E * qi + 8 * c + 4 * hh, qi < p.Lq);
+            const floatx4_t q4 = ldg16f(qbase + p.E * qi + 8 * c + 4 * hh, qi < p.Lq && 8 * c + 4 * hh < p.D);
             // the reference divides q by sqrt(D) before the product (src/attention.jl:118)
 #pragma unroll
             for (int j = 0; j < 4; j++) f.q[qb][4 * c + j] = q4[j] / sq;
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
     }
 
     if (p.out) {
-        float *obase = (float *)p.out + p.Ev * (p.Lq * b) + D * h;
+        float *obase = (float *)p.out + p.Ev * (p.Lq * b) + p.Dv * h;
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) {
             const int64_t qi = iw + 32 * qb + r;
@@ -204,7 +206,7 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
                         floatx4_t o4;
 #pragma unroll
                         for (int e = 0; e < 4; e++) o4[e] = f.o[qb][dvb][4 * g + e] * inv;
-                        *(floatx4_t *)(obase + p.Ev * qi + 32 * dvb + 8 * g + 4 * hh) = o4;
+                        if (32 * dvb + 8 * g + 4 * hh < p.Dv) *(floatx4_t *)(obase + p.Ev * qi + 32 * dvb + 8 * g + 4 * hh) = o4;
                     }
             }
         }
@@ -241,7 +243,8 @@ int32_t launch_d(const FlashArgs &a, hipStream_t st) {
 
 bool attention_flash32_supports(const AttnParams &p) {
     if (p.dtype != MI_F32) return false;
-    if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
+    // head dims: multiples of 4 (16-byte chunks) up to the 128-wide tiles; smaller ones are zero-padded in flight
+    if (p.D < 4 || p.Dv < 4 || p.D > 128 || p.Dv > 128 || (p.D & 3) || (p.Dv & 3)) return false;
     auto al = [](const void *x) { return (((uintptr_t)x) & 15) == 0; };
     if (!al(p.q) || !al(p.k) || (p.out && (!al(p.v) || !al(p.out)))) return false;
     const int64_t tiles = (p.Lq + 127) / 128;
@@ -257,5 +260,5 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     a.cn = 1.0f;
     a.n_qtiles = (int32_t)((p.Lq + 127) / 128);
     flash_fill_vec_flags(a);
-    return p.D == 64 ? launch_d<64, 1>(a, st) : launch_d<128, 1>(a, st);
+    return (p.D <= 64 && p.Dv <= 64) ? launch_d<64, 1>(a, st) : launch_d<128, 1>(a, st);
 }

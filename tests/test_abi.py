@@ -82,7 +82,12 @@ def test_plan_kernel_selection(L):
     assert K[_plan(L, _desc(L, dtype=L.MI_BF16, weights_dtype=L.MI_BF16, **big))[1]] == "flash16"
     assert K[_plan(L, _desc(L, **big))[1]] == "flash32"
     assert K[_plan(L, _desc(L, **big, flags=L.MI_ATTN_FORCE_GENERIC))[1]] == "generic"
-    assert K[_plan(L, _desc(L))[1]] == "generic"                     # head dim 4
+    assert K[_plan(L, _desc(L))[1]] == "flash32"                     # head dim 4: zero-padded into the 64-wide tiles
+    assert K[_plan(L, _desc(L, E=12, Ev=12))[1]] == "generic"        # head dim 6: rows are not whole 16-byte chunks
+    assert K[_plan(L, _desc(L, dtype=L.MI_BF16, weights_dtype=L.MI_BF16, **dict(big, E=3072, Ev=2560)))[1]] == "flash16"   # 96 / 80
+    assert K[_plan(L, _desc(L, dtype=L.MI_BF16, weights_dtype=L.MI_BF16, **dict(big, E=3200, Ev=3200)))[1]] == "generic"   # 100
+    assert K[_plan(L, _desc(L, dtype=L.MI_BF16, weights_dtype=L.MI_BF16, **dict(big, E=8192, Ev=6144)))[1]] == "flash16"   # 256 / 192
+    assert K[_plan(L, _desc(L, dtype=L.MI_BF16, weights_dtype=L.MI_BF16, **dict(big, E=8448, Ev=8448)))[1]] == "generic"   # 264
     rc, kern, ws = _plan(L, _desc(L, dtype=L.MI_BF16, weights_dtype=L.MI_BF16, E=4096, Ev=4096, H=32, Lq=1,
                                   Lkv=32768, B=16))
     assert rc == L.MI_OK and K[kern] == "decode" and ws > 0

@@ -100,12 +100,19 @@ MFMA_CASES = [
     ("f16", 128, 2, 64, 64, (1,), None, "row"),
     ("bf16", 128, 1, 1, 700, (3,), None, None),
     ("bf16", 64, 1, 500, 1, (1,), None, None),
+    # head dims below the 64- / 128-wide tiles (multiples of 8): zero-padded in flight
+    ("bf16", 96, 2, 200, 260, (2,), None, None),
+    ("f16", 32, 3, 257, 257, (1,), "causal", None),
+    ("bf16", 80, 2, 130, 333, (2,), "random", None),
+    ("f16", 40, 2, 96, 160, (2,), "random", "full"),
+    ("bf16", 112, 1, 300, 300, (1,), "causal", None),
+    ("f16", 8, 2, 70, 90, (2,), None, "row"),
 ]
 
 
 @pytest.mark.parametrize("dtype,D,H,Lq,Lkv,batch,mask_kind,bias_kind", MFMA_CASES)
 def test_mfma_kernels(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, bias_kind):
-    """bf16 / f16 inputs with head dim 64 or 128 take the MFMA kernels when the forward result is passed;
+    """bf16 / f16 inputs with head dims up to 128 (multiples of 8) take the MFMA kernels when the forward result is passed;
     tile-ragged lengths, causal and random masks, bias."""
     bias_shape = None
     if bias_kind == "full":
@@ -138,12 +145,16 @@ F32_CASES = [
     (128, 1, 100, 450, (2,), None, False),
     (128, 1, 70, 130, (1,), "random", False),
     (64, 3, 1, 300, (2,), None, False),
+    # head dims below the tile width (multiples of 4)
+    (96, 2, 230, 230, (1,), "causal", True),
+    (36, 2, 130, 333, (2,), None, False),
+    (4, 3, 70, 90, (2,), "random", False),
 ]
 
 
 @pytest.mark.parametrize("D,H,Lq,Lkv,batch,mask_kind,saved", F32_CASES)
 def test_f32_mfma_kernels(nn, oracle, D, H, Lq, Lkv, batch, mask_kind, saved):
-    """Float32 inputs with head dim 64 or 128 take the fp32-MFMA gradient kernels (tolerance 1e-4 of the
+    """Float32 inputs with head dims up to 128 (multiples of 4) take the fp32-MFMA gradient kernels (tolerance 1e-4 of the
     gradient's scale), with and without the statistics saved by the forward call."""
     rng = np.random.default_rng(D + Lq + Lkv)
     E = D * H
@@ -251,7 +262,9 @@ def test_fully_masked_query_gives_nan_gradients(nn):
 
 @pytest.mark.parametrize("dtype,E,H,Lq,Lkv,batch,mask_kind,bias_shape,with_dalpha,saved,expect", [
     ("f32", 12, 2, 9, 7, (2,), None, (7, 9), True, False, "generic"),            # odd head dim, bias gradient, weight cotangent
-    ("f32", 12, 3, 6, 6, (1,), "causal", None, False, False, "generic"),
+    ("f32", 18, 3, 6, 6, (1,), "causal", None, False, False, "generic"),
+    ("f32", 72, 3, 70, 70, (2,), "causal", None, False, False, "flash32"),       # D = 24 in 64-wide tiles
+    ("bf16", 192, 2, 150, 200, (2,), None, None, False, True, "flash16"),        # D = 96 in 128-wide tiles, lean dropout path
     ("bf16", 128, 2, 150, 200, (2,), None, None, False, False, "flash16"),       # D = 64
     ("bf16", 256, 2, 192, 192, (1,), "causal", None, False, True, "flash16"),    # D = 128, statistics from the forward call
     ("f16", 256, 2, 70, 300, (2,), "random", None, False, False, "flash16"),

@@ -196,6 +196,21 @@ FLASH16_CASES = [
     ("f16", 128, 600, 600, 1, 2, dict(causal=True)),
     ("bf16", 256, 300, 700, 1, 2, {}),
     ("f16", 256, 520, 520, 1, 2, dict(causal=True)),
+    # head dims below the 64- / 128-wide tiles (multiples of 8): zero-padded in flight
+    ("bf16", 192, 200, 333, 1, 2, {}),                                   # 96
+    ("f16", 64, 130, 130, 2, 2, dict(causal=True)),                      # 32
+    ("bf16", 160, 150, 400, 1, 2, dict(bias_shape=(400, 150, 2, 1), mask_shape=(400, 150))),   # 80, staged tiles
+    ("f16", 80, 70, 131, 2, 2, dict(bias_shape=(131, 70), mask_shape=(131, 70, 1, 2))),        # 40, unaligned strides
+    ("bf16", 96, 90, 200, 2, 2, dict(Ev=224)),                           # q, k: 48; v: 112
+    ("f16", 240, 64, 256, 1, 2, dict(Ev=48, causal=False, mask_shape=(256, 1, 1, 1))),   # q, k: 120; v: 24; key mask
+    ("bf16", 16, 40, 70, 3, 2, {}),                                      # 8
+    ("bf16", 224, 520, 520, 1, 2, dict(causal=True)),                    # 112, long
+    # head dims above 128 up to 256: 256-wide tiles, one workgroup per CU, bias / mask on the direct path
+    ("bf16", 512, 200, 333, 1, 2, {}),                                   # 256
+    ("f16", 384, 260, 260, 2, 2, dict(causal=True)),                     # 192
+    ("bf16", 320, 150, 400, 1, 2, dict(bias_shape=(400, 150, 2, 1), mask_shape=(400, 150))),   # 160
+    ("f16", 512, 70, 131, 2, 2, dict(Ev=144, mask_shape=(131, 1, 1, 2))),                      # q, k: 256; v: 72
+    ("bf16", 136, 100, 520, 1, 1, dict(Ev=256, mask_shape=(520,))),                            # q, k: 136; v: 256; key mask
 ]
 
 
@@ -209,9 +224,10 @@ def test_flash16_parity(nn, oracle, case, weights):
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 def test_generic_kernel_parity(nn, oracle, dtype):
-    """The generic kernel on a shape the MFMA kernels do not take (head dims 24 / 40)."""
+    """The generic kernel on a shape the MFMA kernels do not take (head dims 22 / 42: rows are not whole
+    16-byte chunks)."""
     rng = np.random.default_rng(7)
-    _check(nn, oracle, rng, dtype, 48, 37, 75, 2, 2, Ev=80, bias_shape=(75, 37, 2, 1), mask_shape=(75, 37),
+    _check(nn, oracle, rng, dtype, 44, 37, 75, 2, 2, Ev=84, bias_shape=(75, 37, 2, 1), mask_shape=(75, 37),
            expect="generic")
 
 
@@ -232,7 +248,7 @@ def test_fully_masked_column_is_nan(nn):
     """src/softmax.jl:73-75 gives exp(-Inf - -Inf) = NaN for an all-dropped column (by code reading;
     no reference test pins it).  Both kernel families must agree with that."""
     rng = np.random.default_rng(9)
-    for dtype, E, H, flags in (("f32", 16, 2, 0), ("bf16", 128, 1, 0)):
+    for dtype, E, H, flags in (("f32", 12, 2, 0), ("f32", 16, 2, 0), ("bf16", 128, 1, 0)):   # generic, flash32, flash16
         q = rng.standard_normal((E, 40, 1)).astype(np.float32)
         k = rng.standard_normal((E, 70, 1)).astype(np.float32)
         mask = np.ones((70, 40), bool)
@@ -251,6 +267,11 @@ FLASH32_CASES = [
     ("f32", 128, 70, 131, 2, 2, dict(bias_shape=(131, 70), mask_shape=(131, 70, 1, 2))),
     ("f32", 256, 96, 96, 1, 2, dict(causal=True, mask_shape=(96, 96))),
     ("f32", 64, 33, 65, 3, 1, {}),
+    # head dims below the tile width (multiples of 4)
+    ("f32", 192, 200, 333, 1, 2, {}),                                    # 96
+    ("f32", 72, 130, 130, 2, 2, dict(causal=True)),                      # 36
+    ("f32", 48, 70, 131, 2, 2, dict(Ev=160, bias_shape=(131, 70), mask_shape=(131, 70, 1, 2))),   # q, k: 24; v: 80
+    ("f32", 8, 40, 70, 3, 2, {}),                                        # 4
 ]
 
 
@@ -312,6 +333,9 @@ SPLIT_CASES = [
     ("bf16", 128, 2048, 2048, 1, 2, dict(causal=True)),            # head dim 64: general kernel, causal pieces
     ("bf16", 64, 70, 2500, 3, 1, {}),
     ("f16", 256, 130, 2100, 1, 2, dict(mask_shape=(2100, 130))),    # head dim 128 with a mask
+    ("bf16", 192, 130, 2100, 1, 2, dict(Ev=160, mask_shape=(2100, 130))),   # head dims 96 / 80 in 128-wide tiles
+    ("f16", 96, 70, 2500, 2, 2, {}),                                  # head dim 48 in 64-wide tiles
+    ("bf16", 256, 100, 2300, 2, 1, {}),                               # head dim 256
 ]
 
 
@@ -340,7 +364,7 @@ def test_split_kv_fully_masked_query(nn):
 
 
 @pytest.mark.parametrize("dtype,E,Lkv,expect", [("f32", 128, 136, "flash32"), ("f16", 128, 144, "flash16"),
-                                                ("bf16", 128, 131, "flash16"), ("f16", 48, 75, "generic")],
+                                                ("bf16", 128, 131, "flash16"), ("f16", 44, 75, "generic")],
                          ids=["flash32", "flash16-staged", "flash16-direct", "generic"])
 @pytest.mark.parametrize("weights", [False, True], ids=["noweights", "weights"])
 def test_plus_inf_logits(nn, oracle, dtype, E, Lkv, expect, weights):
