@@ -107,6 +107,11 @@ MFMA_CASES = [
     ("f16", 40, 2, 96, 160, (2,), "random", "full"),
     ("bf16", 112, 1, 300, 300, (1,), "causal", None),
     ("f16", 8, 2, 70, 90, (2,), None, "row"),
+    # head dims above 128 up to 256: 256-wide tiles, one workgroup per CU, dV and dK always in separate passes
+    ("bf16", 256, 1, 200, 260, (2,), None, None),
+    ("f16", 192, 2, 257, 257, (1,), "causal", None),
+    ("bf16", 160, 1, 130, 333, (2,), "random", None),
+    ("f16", 256, 1, 96, 160, (2,), "random", "full"),
 ]
 
 
@@ -265,6 +270,7 @@ def test_fully_masked_query_gives_nan_gradients(nn):
     ("f32", 18, 3, 6, 6, (1,), "causal", None, False, False, "generic"),
     ("f32", 72, 3, 70, 70, (2,), "causal", None, False, False, "flash32"),       # D = 24 in 64-wide tiles
     ("bf16", 192, 2, 150, 200, (2,), None, None, False, True, "flash16"),        # D = 96 in 128-wide tiles, lean dropout path
+    ("f16", 512, 2, 140, 140, (1,), "causal", None, False, False, "flash16"),    # D = 256
     ("bf16", 128, 2, 150, 200, (2,), None, None, False, False, "flash16"),       # D = 64
     ("bf16", 256, 2, 192, 192, (1,), "causal", None, False, True, "flash16"),    # D = 128, statistics from the forward call
     ("f16", 256, 2, 70, 300, (2,), "random", None, False, False, "flash16"),
