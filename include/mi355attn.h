@@ -84,8 +84,8 @@ int32_t mi_event_elapsed_ms(mi_event start, mi_event stop, float *ms);
 /* Which kernel family mi_attention_fwd picked (reported by mi_attention_plan). */
 enum {
     MI_ATTN_KERNEL_GENERIC = 0,  /* any shape / dtype, scalar FMA                        */
-    MI_ATTN_KERNEL_FLASH16 = 1,  /* f16 / bf16 MFMA flash forward, head dim 64 or 128    */
-    MI_ATTN_KERNEL_FLASH32 = 2,  /* f32 MFMA flash forward, head dim 64 or 128           */
+    MI_ATTN_KERNEL_FLASH16 = 1,  /* f16 / bf16 MFMA flash forward, head dims 8..256 (x8) */
+    MI_ATTN_KERNEL_FLASH32 = 2,  /* f32 MFMA flash forward, head dims 4..128 (x4)        */
     MI_ATTN_KERNEL_DECODE = 3    /* split-kv bandwidth-bound path for short queries      */
 };
 
@@ -174,7 +174,7 @@ int32_t mi_attention_stats_size(const mi_attn_desc *desc, size_t *bytes);
  *   fwd      : the forward call (dtype, sizes, q, k, v, bias, mask, causal, flags, and dropout_p /
  *              dropout_seed when the forward call dropped weights: the keep decisions are redrawn
  *              from the same stream, and the pullback of dropout multiplies by them).  fwd.out may
- *              hold the forward RESULT x; the MFMA kernels (all three dtypes, head dim 64 or 128)
+ *              hold the forward RESULT x; the MFMA kernels (f16 / bf16: head dim a multiple of 8 up to 256; f32: of 4 up to 128)
  *              need it and the call falls back to the generic kernels without it.  fwd.weights and fwd.workspace are ignored.
  *   dout     : (Ev, Lq, B) cotangent of x, `dtype`.
  *   dweights : NULL, or (Lkv, Lq, H, B) cotangent of the returned weights, `dtype`.
