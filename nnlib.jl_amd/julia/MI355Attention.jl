@@ -285,8 +285,9 @@ end
 # cotangent dy of the output (and optionally dα of the returned weights).
 # NNlib gets these from AD through src/attention.jl:86-127 (rrule of batched_mul,
 # src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110; the pullback of dropout
-# multiplies by the mask it drew, src/dropout.jl:38-53).  `y` is the forward result;
-# passing it lets the MFMA kernels run.  A ChainRulesCore.rrule for DeviceArray arguments is three lines
+# multiplies by the mask it drew, src/dropout.jl:38-53).  `y` is the forward result, which the MFMA kernels
+# need; without it (and without dα) one forward call recomputes it where those kernels can take the gradient.
+# A ChainRulesCore.rrule for DeviceArray arguments is three lines
 # on top of this function: call the forward, close over (q, k, v, bias, y), return this pullback.
 function ∇dot_product_attention(dy::DeviceArray{T, 3}, q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::DeviceArray{T, 3},
                                 bias = nothing; y = nothing, dα = nothing, mask = nothing, nheads = 1, stats = nothing,
@@ -298,8 +299,21 @@ function ∇dot_product_attention(dy::DeviceArray{T, 3}, q::DeviceArray{T, 3}, k
     dbias = bias === nothing ? nothing : DeviceArray{Float32}(undef, size(bias)...)
     dbias === nothing || check(ccall((:mi_fill_zero, libmi), Int32, (Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), dbias.ptr, sizeof(Float32) * length(dbias), C_NULL))
     p, seed = fdrop isa Dropout ? (fdrop.p, fdrop.seed) : (0f0, UInt64(0))
-    fwd = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0), E, Ev, Lq, Lkv, nheads, B,
-                   q.ptr, k.ptr, v.ptr, y === nothing ? C_NULL : y.ptr, C_NULL, bptr, bstr, mptr, mstr, C_NULL, 0, p, UInt32(0), seed, stats === nothing ? C_NULL : stats.ptr)
+    fwd_desc(yptr) = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0), E, Ev, Lq, Lkv, nheads, B,
+                              q.ptr, k.ptr, v.ptr, yptr, C_NULL, bptr, bstr, mptr, mstr, C_NULL, 0, p, UInt32(0), seed, stats === nothing ? C_NULL : stats.ptr)
+    if y === nothing && dα === nothing
+        # Without the forward result only the generic kernels can run (hundreds of times slower on the shapes the
+        # MFMA kernels take): ask the planner what it would pick with a result in place (dy stands in: the right
+        # size and alignment, and planning reads no memory); if that is an MFMA family, recompute the result.
+        kern = Ref{Int32}(0)
+        probe = AttnBwdDesc(Int32(sizeof(AttnBwdDesc)), Int32(0), fwd_desc(dy.ptr), dy.ptr, C_NULL, dq.ptr, dk.ptr, dv.ptr,
+                            dbias === nothing ? C_NULL : dbias.ptr, C_NULL, 0)
+        check(ccall((:mi_attention_bwd_plan, libmi), Int32, (Ref{AttnBwdDesc}, Ptr{Int32}, Ptr{Csize_t}), probe, kern, C_NULL))
+        if kern[] != 0      # MI_ATTN_KERNEL_GENERIC
+            y, _ = dot_product_attention(q, k, v, bias; fdrop, mask, nheads, return_weights = false)
+        end
+    end
+    fwd = fwd_desc(y === nothing ? C_NULL : y.ptr)
     mk(ws, wsbytes) = AttnBwdDesc(Int32(sizeof(AttnBwdDesc)), Int32(0), fwd, dy.ptr, dα === nothing ? C_NULL : dα.ptr, dq.ptr, dk.ptr,
                                   dv.ptr, dbias === nothing ? C_NULL : dbias.ptr, ws, wsbytes)
     need = Ref{Csize_t}(0)

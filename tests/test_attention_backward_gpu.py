@@ -237,6 +237,15 @@ def test_statistics_saved_by_the_forward_call(nn, oracle, dtype, D, H, L, Lkv, c
         assert np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05) <= 1e-2
 
 
+@pytest.mark.parametrize("dtype,D,expect", [("bf16", 96, "flash16"), ("f32", 64, "flash32"), ("f32", 6, "generic")])
+def test_forward_result_is_recomputed_when_missing(nn, oracle, dtype, D, expect):
+    """The MFMA gradient kernels need the forward result; a call without `y` runs one forward call first rather
+    than falling back to the generic kernels (which still take the shapes nothing else does)."""
+    _run(nn, oracle, dtype, 2 * D, 2 * D, 130, 200, (2,), 2, mask_kind="random", pass_y=False, expect=expect, seed=11, scale=0.5)
+    _run(nn, oracle, dtype, 2 * D, 2 * D, 150, 150, (1,), 2, mask_kind="causal", pass_y=False, expect=expect, seed=12, scale=0.5,
+         dropout=(0.2, 99))
+
+
 def test_mfma_and_generic_kernels_agree(nn):
     """Same call through both kernel families (the generic one forced by flag)."""
     rng = np.random.default_rng(9)
