@@ -123,6 +123,47 @@ __device__ inline i32x4_t flash_make_rsrc(const void *base, uint32_t bytes) {
     return rs;
 }
 
+// Streams [FLASH_BN][ROWB bytes] tiles of one row-major 16-bit array global -> LDS with 1 KiB DMA pieces: no staging
+// registers.  A piece (64 lanes x 16 bytes) covers 1024 / ROWB tile rows; lane l of piece i lands at chunk position
+// l % (ROWB / 16) of tile row i * (1024 / ROWB) + l / (ROWB / 16) and fetches the source chunk `position ^ swz(row)`,
+// which is how the consumers address the tile.  Each of the four wavefronts moves PIECES pieces per tile.
+// The buffer resource is rebuilt per tile with the tile's first row as its base (64-bit scalar arithmetic), so the
+// per-lane offsets are tile-local and arrays of any size work; rows past the end of the array lie outside the
+// resource and arrive as zeros, and so do chunks past the head dim `dh` (their lanes carry an offset of 2 GiB,
+// beyond the 2 GiB - 1 the resource size is clamped to).
+template <int ROWB>
+struct FlashTileDma {
+    static constexpr int TILEB = FLASH_BN * ROWB, RPP = 1024 / ROWB, PIECES = TILEB / 1024 / 4;
+    const char *base;          // element (row 0, first feature of the head) of this batch element
+    int64_t row_bytes, end;    // end: bytes from `base` to the end of the batch element's last row
+    unsigned lds;              // LDS byte address of this wavefront's first piece in buffer 0
+    int voff[PIECES];
+    template <typename SWZ>
+    __device__ void init(const void *base_, int64_t row_elems, int64_t nrows, int64_t head_off_elems, int dh, char *tiles, SWZ swz) {
+        const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        base = (const char *)base_;
+        row_bytes = row_elems * 2;
+        end = (nrows * row_elems - head_off_elems) * 2;
+        lds = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)tiles + wave * PIECES * 1024);   // wave-uniform: goes into M0
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const int row = (wave * PIECES + i) * RPP + lane / (ROWB / 16);
+            const int chunk = (lane % (ROWB / 16)) ^ swz(row);
+            voff[i] = 8 * chunk < dh ? row * (int)row_bytes + chunk * 16 : (int)0x80000000;
+        }
+    }
+    // start the copy of the tile whose first row is row0 into buffer `buf`
+    __device__ void load(int buf, int64_t row0) const {
+        const int64_t skip = row0 * row_bytes;
+        int64_t left = end - skip;
+        left = left < 0 ? 0 : (left > 0x7fffffffLL ? 0x7fffffffLL : left);
+        const i32x4_t rs = flash_make_rsrc(base + skip, (uint32_t)left);
+        const unsigned dst = __builtin_amdgcn_readfirstlane(lds + buf * TILEB);
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) flash_dma_1k(rs, dst + i * 1024, voff[i]);
+    }
+};
+
 // Bias / mask tiles of one wavefront staged through LDS (16-bit kernels).  A wavefront owns 32*QB query
 // rows; per kv tile it needs, for each of them, 64 bias elements (128 bytes) and 64 mask bytes.  Reading
 // those straight from global memory in the accumulator layout makes every load instruction touch 32
