@@ -23,6 +23,9 @@ struct FlashArgs {
     int32_t bias_lds;  // 16-bit kernels: bias / mask tiles may be staged through LDS with 16-byte DMA pieces
     int32_t mask_lds;
     int32_t w_lds;     // weight rows start 16-byte aligned: tiles may be transposed through LDS and written as full lines
+    // gradient kernels only: the launch covers batch elements [b0, b0 + nb), and the bias gradient may be summed
+    // without atomics (no two workgroups of one launch add to the same element)
+    int32_t b0, nb, dbias_plain;
 };
 
 // Bytes of LDS per wavefront for the weight staging below: 16 query rows x 128 bytes.
@@ -90,7 +93,7 @@ inline void flash_fill_vec_flags(FlashArgs &a) {
     // LDS staging moves 16-byte pieces addressed with 32-bit byte offsets from the (head, batch) slice:
     // rows must start 16-byte aligned and the slice (plus one query tile of slack) must stay below 2 GiB.
     auto fits = [&](const int64_t *st, size_t elem) {
-        const int64_t reach = ((p.Lq + 256) * st[1] + p.Lkv + FLASH_BN) * (int64_t)elem;
+        const int64_t reach = ((p.Lq + 256) * st[1] + p.Lkv + 128) * (int64_t)elem;   // tiles reach up to 127 keys past Lkv
         const int64_t per16 = 16 / (int64_t)elem;
         return st[0] == 1 && st[1] % per16 == 0 && st[2] % per16 == 0 && st[3] % per16 == 0 && reach < (int64_t)0x7fffffff;
     };
@@ -263,7 +266,10 @@ __device__ inline void flash_wave_lds_fence() {
 // query adds to the same row).  Straight from the registers one atomic instruction would touch 64 cache lines; the
 // block goes through the wavefront's FLASH_WSTAGE_BYTES LDS region 16 queries at a time and comes back with 8 lanes
 // per query row, so an instruction covers 8 rows of 128 contiguous bytes.  Exact zeros are skipped.
-__device__ inline void flash_atomic_add_block(unsigned wlds, const floatx16_t &v, float *dst, int64_t qstride, int nq, int nk) {
+// plain: no other workgroup running at the same time adds to these elements (the caller serialises the launches
+// that would), so the sum is a load, an add and a store instead of an atomic (Float32 atomics on one array from all
+// eight XCDs run at a small fraction of the store rate).
+__device__ inline void flash_atomic_add_block(unsigned wlds, const floatx16_t &v, float *dst, int64_t qstride, int nq, int nk, bool plain = false) {
     typedef __attribute__((address_space(3))) u32x4_t *lds16_t;
     const int lane = threadIdx.x & 63, r = lane & 31, hh = lane >> 5;
 #pragma unroll
@@ -296,6 +302,19 @@ __device__ inline void flash_atomic_add_block(unsigned wlds, const floatx16_t &v
             const int q = 16 * half + rr;
             if (q < nq) {
                 float *row = dst + q * qstride + 4 * c;
+                if (plain) {
+                    if (4 * c + 3 < nk && (((uintptr_t)row) & 15) == 0) {
+                        floatx4_t old = *(const floatx4_t *)row;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) old[e] += piece[e];
+                        *(floatx4_t *)row = old;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            if (4 * c + e < nk) row[e] += piece[e];
+                    }
+                    continue;
+                }
 #pragma unroll
                 for (int e = 0; e < 4; e++)
                     if (4 * c + e < nk && piece[e] != 0.0f) atomicAdd(row + e, piece[e]);

@@ -133,6 +133,11 @@ def test_mfma_kernels(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, bias_k
     ("f32", 128, 1, 96, 160, (2,), "random", (160, 96), "flash32"),          # broadcast over heads and batch: summed
     ("bf16", 128, 2, 200, 200, (2,), "causal", (200, 200, 2, 1), "flash16"),
     ("f16", 64, 2, 70, 300, (3,), None, (300, 1, 1, 3), "flash16"),          # one bias value per key and batch element
+    # plain (non-atomic) sums: own entries per query, head and batch element ...
+    ("bf16", 64, 2, 130, 200, (2,), "random", (200, 130, 2, 2), "flash16"),
+    # ... and entries shared by the batch elements, one launch per batch element (enough workgroups per launch)
+    ("bf16", 8, 16, 2048, 64, (3,), None, (64, 2048, 16, 1), "flash16"),
+    ("f16", 16, 16, 2048, 96, (2,), "random", (96, 2048, 16), "flash16"),
 ])
 def test_bias_gradient_from_the_mfma_kernels(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, bias_shape, expect):
     """The bias gradient is dS summed over the dims the bias broadcasts along; the dQ kernels add it with Float32
