@@ -70,7 +70,12 @@ enum { PHASE_ONLINE = 0, PHASE_STATS = 1, PHASE_FINAL = 2 };
 // strides, or from tiles staged through LDS (FlashStaged; every array present must qualify)
 // EXTRAS_KEYMASK: no bias and a mask that does not depend on the query (a key-padding mask, query stride 0):
 // the scores stay raw dot products as with EXTRAS_NONE and dropped keys are set to -Inf from one mask byte per key.
-enum { EXTRAS_NONE = 0, EXTRAS_DIRECT = 1, EXTRAS_STAGED = 2, EXTRAS_KEYMASK = 3 };
+// EXTRAS_MASKTILE: no bias and a dense mask whose tiles can be staged through LDS: raw dot products as with
+// EXTRAS_NONE, dropped entries set to -Inf from the staged mask bytes; only the mask half of the staging is allocated,
+// which keeps two workgroups per CU.
+enum { EXTRAS_NONE = 0, EXTRAS_DIRECT = 1, EXTRAS_STAGED = 2, EXTRAS_KEYMASK = 3, EXTRAS_MASKTILE = 4 };
+// variants that copy bias / mask tiles through LDS (FlashStaged), and the LDS bytes per wavefront they need
+constexpr bool flash_uses_staging(int extras) { return extras == EXTRAS_STAGED || extras == EXTRAS_MASKTILE; }
 // true when the accumulators hold the reference's logits in natural units (bias added) rather than raw dot products
 constexpr bool flash_natural_units(int extras) { return extras == EXTRAS_DIRECT || extras == EXTRAS_STAGED; }
 // query-independent mask without bias whose bytes can be read four keys at a time (unit key stride, Lkv a
@@ -179,6 +184,10 @@ template <int QB>
 struct FlashStaged {
     static constexpr int BIAS_STAGE = 32 * QB * 128, MASK_STAGE = 32 * QB * 64;  // bytes per stage
     static constexpr int BYTES_PER_WAVE = 2 * (BIAS_STAGE + MASK_STAGE);
+    static constexpr int BYTES_PER_WAVE_MASK_ONLY = 2 * MASK_STAGE;
+    static constexpr int bytes_per_wave(int extras) {
+        return extras == EXTRAS_STAGED ? BYTES_PER_WAVE : extras == EXTRAS_MASKTILE ? BYTES_PER_WAVE_MASK_ONLY : 0;
+    }
     bool bias = false, mask = false;
     i32x4_t brs, mrs;
     unsigned blds, mlds;                 // LDS byte addresses of the two-stage regions
@@ -187,12 +196,13 @@ struct FlashStaged {
     __device__ static int bias_swz(int row) { return (row >> 1) & 7; }
     __device__ static int mask_swz(int row) { return (row >> 2) & 3; }
 
-    __device__ void init(const FlashArgs &a, unsigned lds_wave_base, int lane, int64_t iw, int64_t h, int64_t b) {
+    // mask_only: the wavefront's region holds the two mask stages only (EXTRAS_MASKTILE)
+    __device__ void init(const FlashArgs &a, unsigned lds_wave_base, int lane, int64_t iw, int64_t h, int64_t b, bool mask_only = false) {
         const AttnParams &p = a.p;
-        bias = a.bias_lds;
+        bias = a.bias_lds && !mask_only;
         mask = a.mask_lds;
         blds = __builtin_amdgcn_readfirstlane(lds_wave_base);  // wave-uniform: goes into M0
-        mlds = blds + 2 * BIAS_STAGE;
+        mlds = mask_only ? blds : blds + 2 * BIAS_STAGE;
         {   // set up unconditionally so that the resource words stay in scalar registers
             const int64_t s1 = p.bias_strides[1];
             const char *base = (const char *)p.bias + 2 * (h * p.bias_strides[2] + b * p.bias_strides[3]);
@@ -425,6 +435,18 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                         float x = fmaf(s[qb][kb][4 * g + e], a.cn, bv[e]);
                         s[qb][kb][4 * g + e] = keep[e] ? x : MI_NEG_INF;
                     }
+                }
+        }
+        if (EXTRAS == EXTRAS_MASKTILE) {
+            const int row = 32 * qb + r;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const uint32_t m4 = sg.mask4(stage, row, 4 * kb + g, hh);
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        s[qb][kb][4 * g + e] = (m4 & (0xFFu << (8 * e))) ? s[qb][kb][4 * g + e] : MI_NEG_INF;
                 }
         }
         if (EXTRAS == EXTRAS_KEYMASK) {

@@ -189,6 +189,10 @@ FLASH16_CASES = [
     ("bf16", 256, 150, 400, 2, 2, dict(mask_shape=(400, 1, 1, 2))),
     ("f16", 128, 70, 131, 2, 2, dict(mask_shape=(131,))),                 # unaligned length: byte loads
     ("bf16", 128, 200, 520, 1, 2, dict(mask_shape=(520, 1, 2))),
+    # dense masks without bias whose rows start 16-byte aligned: mask tiles staged alone, raw-score path
+    ("bf16", 256, 150, 400, 2, 2, dict(mask_shape=(400, 150, 1, 2))),
+    ("f16", 128, 70, 336, 2, 2, dict(mask_shape=(336, 70))),
+    ("bf16", 192, 200, 208, 1, 2, dict(mask_shape=(208, 200, 2, 1))),     # head dim 96
     # long enough for the steady-state loop of the software-pipelined kernel, head dims 64 and 128
     ("bf16", 128, 300, 700, 1, 2, {}),
     ("bf16", 128, 520, 520, 1, 2, dict(causal=True)),
@@ -336,6 +340,7 @@ SPLIT_CASES = [
     ("bf16", 192, 130, 2100, 1, 2, dict(Ev=160, mask_shape=(2100, 130))),   # head dims 96 / 80 in 128-wide tiles
     ("f16", 96, 70, 2500, 2, 2, {}),                                  # head dim 48 in 64-wide tiles
     ("bf16", 256, 100, 2300, 2, 1, {}),                               # head dim 256
+    ("f16", 256, 130, 2112, 1, 2, dict(mask_shape=(2112, 130))),      # mask tiles staged alone
 ]
 
 
