@@ -2,6 +2,7 @@
 // per-(dtype, head dim) instantiations of attention_backward_flash16.inc.
 #include "common.h"
 #include "attention_params.h"
+#include "flash_common.h"
 
 int32_t launch_bwd_flash16_bf16_d64(const AttnBwdParams &, hipStream_t);
 int32_t launch_bwd_flash16_bf16_d128(const AttnBwdParams &, hipStream_t);
@@ -30,8 +31,60 @@ bool attention_bwd_flash16_supports(const AttnBwdParams &bp) {
 // three float planes [B*H][Lq rounded up to 128]: row maximum (log2 units), 1 / row sum, delta
 size_t attention_bwd_flash16_workspace(const AttnParams &p) { return attention_stats_bytes(p); }
 
-int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp, hipStream_t st) {
+// ---- dense masks packed into bits for the key-stationary kernels ----------------------------------------------
+// A dense mask without bias keeps the lean gradient kernels (raw scores, two wavefronts per SIMD).  The dQ kernel
+// stages the mask tiles through LDS as the forward kernel does; in the dK / dV kernels a lane owns one key and walks
+// the queries, so it wants the mask of (its key, the 64 queries of a tile) as one 64-bit word: a small kernel packs
+// those words once per call, [slice][query tile][key], slices being the distinct (head, batch) planes of the mask.
+static bool takes_mask_bits(const AttnParams &p) {
+    if (!p.mask || p.bias || p.D > 128 || flash_is_key_mask(p) || (p.Lkv & 3) != 0) return false;
+    FlashArgs a;
+    a.p = p;
+    a.p.weights = nullptr;
+    flash_fill_vec_flags(a);
+    return a.mask_lds != 0;   // the dQ kernel's staged mask tiles: unit key stride, 16-byte aligned rows
+}
+static int64_t mask_bits_slices(const AttnParams &p) { return (p.mask_strides[2] ? p.H : 1) * (p.mask_strides[3] ? p.B : 1); }
+static int64_t mask_bits_lkv_pad(const AttnParams &p) { return (p.Lkv + 255) / 256 * 256; }
+
+size_t attention_bwd_flash16_mask_bits_bytes(const AttnParams &p) {
+    if (!takes_mask_bits(p)) return 0;
+    return sizeof(uint64_t) * (size_t)(mask_bits_slices(p) * ((p.Lq + 63) / 64) * mask_bits_lkv_pad(p));
+}
+
+__global__ __launch_bounds__(256) void mask_bits_kernel(const uint8_t *mask, int64_t s0, int64_t s1, int64_t s2, int64_t s3, int64_t Lq,
+                                                        int64_t Lkv, int64_t lkv_pad, int64_t heads, uint64_t *out) {
+    const int64_t kv = (int64_t)blockIdx.x * 256 + threadIdx.x, qt = blockIdx.y, slice = blockIdx.z;
+    const int64_t h = slice % heads, b = slice / heads;   // heads == 1: the mask is shared by the heads (stride 0)
+    uint64_t word = 0;
+    if (kv < Lkv) {
+        const uint8_t *col = mask + kv * s0 + h * s2 + b * s3;
+#pragma unroll 8
+        for (int i = 0; i < 64; i++) {
+            const int64_t q = qt * 64 + i;
+            if (q < Lq && col[q * s1]) word |= (uint64_t)1 << i;
+        }
+    }
+    out[(slice * gridDim.y + qt) * lkv_pad + kv] = word;
+}
+
+int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp_in, hipStream_t st) {
+    AttnBwdParams bp = bp_in;
     const AttnParams &p = bp.p;
+    if (takes_mask_bits(p)) {
+        const int64_t nqt = (p.Lq + 63) / 64, pad = mask_bits_lkv_pad(p), slices = mask_bits_slices(p);
+        if (nqt > 65535 || slices > 65535) return mi_set_error(MI_ESHAPE, "attention gradient: mask packing supports at most 65535 query tiles and mask planes");
+        uint64_t *bits = (uint64_t *)((char *)bp.workspace + (bp.have_stats ? 0 : attention_bwd_flash16_workspace(p)));
+        const int64_t heads = p.mask_strides[2] ? p.H : 1;
+        hipLaunchKernelGGL(mask_bits_kernel, dim3((unsigned)(pad / 256), (unsigned)nqt, (unsigned)slices), dim3(256), 0, st, p.mask,
+                           p.mask_strides[0], p.mask_strides[1], p.mask_strides[2], p.mask_strides[3], p.Lq, p.Lkv, pad, heads, bits);
+        MI_LAUNCH_CHECK();
+        bp.mask_bits = bits;
+        bp.mb_h = p.mask_strides[2] ? 1 : 0;
+        bp.mb_b = p.mask_strides[3] ? heads : 0;
+        bp.mb_lkv_pad = pad;
+        bp.mb_nqt = nqt;
+    }
     if (p.dtype == MI_BF16)
         return p.D <= 64 ? launch_bwd_flash16_bf16_d64(bp, st) : p.D <= 128 ? launch_bwd_flash16_bf16_d128(bp, st) : launch_bwd_flash16_bf16_d256(bp, st);
     return p.D <= 64 ? launch_bwd_flash16_f16_d64(bp, st) : p.D <= 128 ? launch_bwd_flash16_f16_d128(bp, st) : launch_bwd_flash16_f16_d256(bp, st);

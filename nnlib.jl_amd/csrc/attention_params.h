@@ -73,6 +73,10 @@ struct AttnBwdParams {
     float *stats;      // per (query, head, batch) softmax statistics: the workspace, or the buffer a forward call saved
     int32_t have_stats; // the forward call already filled the first two planes of `stats`
     void *workspace;
+    // dense mask packed for the key-stationary gradient kernels: word [slice][query tile of 64][key] holds the mask
+    // bits of the tile's queries for that key; slice = h * mb_h + b * mb_b (0 where the mask is shared)
+    const uint64_t *mask_bits;
+    int64_t mb_h, mb_b, mb_lkv_pad, mb_nqt;
 };
 
 // size of the statistics planes shared by the forward kernels that save them and the backward kernels
@@ -87,6 +91,7 @@ bool attention_bwd_flash16_supports(const AttnBwdParams &bp);
 int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st);
 bool attention_bwd_flash32_supports(const AttnBwdParams &bp);
 size_t attention_bwd_flash16_workspace(const AttnParams &p);
+size_t attention_bwd_flash16_mask_bits_bytes(const AttnParams &p);   // 0 when the call does not take the packed-mask path
 size_t attention_bwd_generic_workspace(const AttnParams &p);
 int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_backward = false);
 

@@ -26,6 +26,10 @@ def _run(nn, oracle, dtype, E, Ev, Lq, Lkv, batch, H, bias_shape=None, mask_kind
         mask = rng.random((Lkv, Lq)) < 0.8
         mask[0] = True
         dmask = nn.DeviceArray.from_numpy(mask)
+    elif mask_kind in ("random_hb", "random_b"):   # a mask plane per (head, batch element) / per batch element
+        mask = rng.random((Lkv, Lq, H if mask_kind == "random_hb" else 1) + batch) < 0.8
+        mask[0] = True
+        dmask = nn.DeviceArray.from_numpy(mask)
     elif mask_kind == "keys":       # key-padding mask: no query dependence, one pattern per batch element
         mask = rng.random((Lkv, 1, 1) + batch) < 0.7
         mask[Lkv // 2, ...] = True
@@ -240,6 +244,20 @@ def test_statistics_saved_by_the_forward_call(nn, oracle, dtype, D, H, L, Lkv, c
     ref = oracle.attention_bwd_f64(q, k, v, dy, None, oracle.make_causal_mask(L) if causal else None, H)
     for g, r_ in zip(with_stats[:3], ref[:3]):
         assert np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05) <= 1e-2
+
+
+@pytest.mark.parametrize("dtype,D,H,Lq,Lkv,batch,mask_kind,saved,dropout", [
+    ("bf16", 128, 2, 200, 320, (2,), "random", False, None),
+    ("f16", 64, 2, 130, 208, (3,), "random_b", True, None),
+    ("bf16", 96, 2, 257, 272, (2,), "random_hb", True, None),
+    ("f16", 128, 1, 70, 400, (2,), "random", False, (0.25, 77)),
+    ("bf16", 32, 3, 300, 64, (1,), "random_hb", False, None),
+])
+def test_dense_mask_on_the_lean_paths(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, saved, dropout):
+    """A dense Bool mask without bias whose rows start 16-byte aligned: the dQ kernel reads staged mask tiles, the
+    dK / dV kernels 64-bit words packed by a small kernel first (one per key and query tile)."""
+    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, batch, H, mask_kind=mask_kind, expect="flash16", saved=saved, dropout=dropout,
+         seed=Lq + Lkv, scale=0.4)
 
 
 @pytest.mark.parametrize("dtype,D,expect", [("bf16", 96, "flash16"), ("f32", 64, "flash32"), ("f32", 6, "generic")])
