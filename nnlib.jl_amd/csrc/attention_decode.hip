@@ -13,6 +13,9 @@
 // An optional mask (src/attention.jl:133-138; with a single query every mask is a key mask, e.g. the context
 // lengths of a padded batch) costs one byte per key row and head: dropped keys get the score -Inf, a (head,
 // batch) pair with no key kept gives NaN like the reference.
+// When the caller wants the attention weights too (the reference always returns them), the first kernel also writes
+// the raw scores (Float32, 4 bytes per key and head: a few per mille of the K / V stream), the merge kernel leaves the
+// final maximum and 1 / sum per (head, batch), and a third, elementwise kernel turns the scores into weights.
 #include "common.h"
 #include "attention_params.h"
 
@@ -27,6 +30,8 @@ struct DecodeArgs {
     int32_t nsplit;
     int32_t rows_per_split;
     int32_t nseg;      // ceil(E / 512)
+    float *scores;     // weights requested: [B][H][Lkv] raw dot products (-Inf where masked), else null
+    float *final_ml;   // weights requested: [B][H][2] final maximum (raw units) and 1 / sum
 };
 
 __device__ inline void unpack8(const u32x4_t &v, float *out, BF16) {
@@ -41,11 +46,13 @@ __device__ inline void unpack8(const u32x4_t &v, float *out, F16) {
 }
 
 // workspace layout: [B][nsplit][E] floats of o, then [B][nsplit][H] of m, then [B][nsplit][H] of l
-template <typename T, int D, bool MASKED>
+template <typename T, int D, bool MASKED, bool SCORES>
 __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     const AttnParams &p = a.p;
     typedef typename T::type t;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int NH = SEG / D;                        // heads per wavefront
+    __shared__ float sc_lds[SCORES ? 4 * NH * 64 : 1]; // scores on their way out: [wavefront][head][64 keys]
     const int seg = blockIdx.x * 4 + wave;
     const int split = blockIdx.y;
     const int64_t b = blockIdx.z;
@@ -114,6 +121,33 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
 #pragma unroll
             for (int e = 0; e < 8; e++) o[e] = fmaf(pr, vf[e], o[e]);
         }
+        if (SCORES) {
+            // Scores leave in runs of 64 keys per head (256 contiguous bytes): written 32 bytes at a time, one piece per
+            // head and iteration, the scattered small writes cost the K / V stream a fifth of its rate.  The first lane
+            // of each head parks the 8 scores of this iteration in the wavefront's LDS rows; every 8th iteration the
+            // 64 lanes write one row per head.
+            const int slot8 = (int)(((j - j_begin) / ROWS) & 7);
+            if ((lane & (D / 8 - 1)) == 0) {
+                float *row = sc_lds + (wave * NH + lane / (D / 8)) * 64 + 8 * slot8;
+                *(floatx4_t *)row = (floatx4_t){s[0], s[1], s[2], s[3]};
+                *(floatx4_t *)(row + 4) = (floatx4_t){s[4], s[5], s[6], s[7]};
+            }
+            if (slot8 == 7 || j + ROWS >= j_end) {
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const int64_t jrun = j - 8 * slot8;     // first key of the run
+#pragma unroll
+                for (int hl = 0; hl < NH; hl++) {
+                    const int64_t h = (int64_t)seg * NH + hl;
+                    const float val = sc_lds[(wave * NH + hl) * 64 + lane];
+                    if (h < p.H && jrun + lane < j_end) a.scores[((int64_t)b * p.H + h) * p.Lkv + jrun + lane] = val;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            }
+        }
     }
     if (!lane_ok) return;
     float *ws = (float *)p.workspace;
@@ -160,7 +194,13 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
             l = fmaf(wl[slot * p.H + h], w, l);
         }
         l = mi_wave_sum(l);
-        if (lane == 0) inv_l[wave] = 1.0f / l;
+        if (lane == 0) {
+            inv_l[wave] = 1.0f / l;
+            if (a.final_ml) {   // a head belongs to exactly one workgroup of this kernel (256 is a multiple of the head dim)
+                a.final_ml[(b * p.H + h) * 2] = m;
+                a.final_ml[(b * p.H + h) * 2 + 1] = 1.0f / l;
+            }
+        }
     }
     __syncthreads();
     if (f >= p.E) return;
@@ -180,6 +220,20 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(DecodeArgs a) {
     ((typename T::type *)p.out)[p.E * b + f] = T::from_f32(o * inv_l[hl]);
 }
 
+// weights[kv, 0, h, b] = 2^((s - m) c) / l from the saved scores; a (head, batch) pair with every key masked has
+// s = m = -Inf and gets NaN, as the reference's softmax gives
+template <typename TW>
+__global__ __launch_bounds__(256) void decode_weights_kernel(DecodeArgs a, TW *weights) {
+    const AttnParams &p = a.p;
+    const int64_t hb = blockIdx.y, j = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const float m = a.final_ml[hb * 2], inv = a.final_ml[hb * 2 + 1];
+    const float *src = a.scores + hb * p.Lkv;
+    TW *dst = weights + hb * p.Lkv;
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+        if (j + e < p.Lkv) dst[j + e] = (TW)(mi_exp2((src[j + e] - m) * a.c) * inv);
+}
+
 int pick_nsplit(const AttnParams &p) {
     // enough wavefronts to cover the chip several times over, at least 256 rows per split
     const int64_t nseg = (p.E + SEG - 1) / SEG;
@@ -195,7 +249,8 @@ int pick_nsplit(const AttnParams &p) {
 
 bool attention_decode_supports(const AttnParams &p) {
     if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
-    if (p.Lq != 1 || p.weights || p.bias || p.causal || !p.out || p.drop_thresh) return false;
+    if (p.Lq != 1 || p.bias || p.causal || !p.out || p.drop_thresh || p.stats) return false;   // saved statistics: the tiled kernels write them
+    if (p.weights && p.H * p.B > 65535) return false;
     if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
     if (p.Lkv < 512) return false;   // short contexts: the tiled kernel is fine
     if (p.B > 65535) return false;
@@ -205,7 +260,8 @@ bool attention_decode_supports(const AttnParams &p) {
 
 size_t attention_decode_workspace(const AttnParams &p) {
     const size_t ns = (size_t)pick_nsplit(p);
-    return sizeof(float) * ns * (size_t)p.B * (size_t)(p.E + 2 * p.H);
+    // partial results of the splits, then (weights requested) the raw scores and the final statistics
+    return sizeof(float) * (ns * (size_t)p.B * (size_t)(p.E + 2 * p.H) + (p.weights ? (size_t)(p.Lkv * p.H * p.B + 2 * p.H * p.B) : 0));
 }
 
 int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
@@ -218,12 +274,23 @@ int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
     a.nseg = (int32_t)((p.E + SEG - 1) / SEG);
     if ((((uintptr_t)p.workspace) & 15) != 0)
         return mi_set_error(MI_EWORKSPACE, "decode workspace must be 16-byte aligned");
+    a.scores = a.final_ml = nullptr;
+    if (p.weights) {
+        // placed after the partial results, which are sized for pick_nsplit() splits (never fewer than a.nsplit)
+        a.scores = (float *)p.workspace + (size_t)pick_nsplit(p) * (size_t)p.B * (size_t)(p.E + 2 * p.H);
+        a.final_ml = a.scores + p.Lkv * p.H * p.B;
+    }
     dim3 grid((unsigned)((a.nseg + 3) / 4), (unsigned)a.nsplit, (unsigned)p.B);
     dim3 mgrid((unsigned)((p.E + 255) / 256), (unsigned)p.B);
-#define DECODE_LAUNCH(TT, DD)                                                                         \
-    {                                                                                                 \
-        if (p.mask) hipLaunchKernelGGL((decode_split_kernel<TT, DD, true>), grid, dim3(256), 0, st, a); \
-        else hipLaunchKernelGGL((decode_split_kernel<TT, DD, false>), grid, dim3(256), 0, st, a);       \
+#define DECODE_LAUNCH(TT, DD)                                                                                        \
+    {                                                                                                                \
+        if (p.weights) {                                                                                             \
+            if (p.mask) hipLaunchKernelGGL((decode_split_kernel<TT, DD, true, true>), grid, dim3(256), 0, st, a);     \
+            else hipLaunchKernelGGL((decode_split_kernel<TT, DD, false, true>), grid, dim3(256), 0, st, a);           \
+        } else {                                                                                                     \
+            if (p.mask) hipLaunchKernelGGL((decode_split_kernel<TT, DD, true, false>), grid, dim3(256), 0, st, a);    \
+            else hipLaunchKernelGGL((decode_split_kernel<TT, DD, false, false>), grid, dim3(256), 0, st, a);          \
+        }                                                                                                            \
     }
     if (p.dtype == MI_BF16) {
         if (p.D == 128) DECODE_LAUNCH(BF16, 128) else DECODE_LAUNCH(BF16, 64)
@@ -236,5 +303,12 @@ int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
     }
 #undef DECODE_LAUNCH
     MI_LAUNCH_CHECK();
+    if (p.weights) {
+        dim3 wgrid((unsigned)((p.Lkv + 1023) / 1024), (unsigned)(p.H * p.B));
+        if (p.weights_dtype == MI_F32) hipLaunchKernelGGL(decode_weights_kernel<float>, wgrid, dim3(256), 0, st, a, (float *)p.weights);
+        else if (p.dtype == MI_BF16) hipLaunchKernelGGL(decode_weights_kernel<__bf16>, wgrid, dim3(256), 0, st, a, (__bf16 *)p.weights);
+        else hipLaunchKernelGGL(decode_weights_kernel<_Float16>, wgrid, dim3(256), 0, st, a, (_Float16 *)p.weights);
+        MI_LAUNCH_CHECK();
+    }
     return MI_OK;
 }

@@ -289,10 +289,12 @@ def test_flash32_parity(nn, oracle, case, weights):
 
 @pytest.mark.parametrize("dtype,E,H,Lkv,B", [("bf16", 512, 4, 1500, 2), ("bf16", 256, 2, 4096, 3), ("f16", 512, 8, 777, 1),
                                              ("f16", 1024, 8, 2048, 2), ("bf16", 128, 1, 513, 1)])
-def test_decode_parity(nn, oracle, dtype, E, H, Lkv, B):
-    """Split-kv path for a single query per (head, batch)."""
+@pytest.mark.parametrize("weights", [False, True], ids=["noweights", "weights"])
+def test_decode_parity(nn, oracle, dtype, E, H, Lkv, B, weights):
+    """Split-kv path for a single query per (head, batch); with the weights returned (as the reference always does)
+    the raw scores are kept and normalised by a third kernel."""
     rng = np.random.default_rng(E + Lkv)
-    _check(nn, oracle, rng, dtype, E, 1, Lkv, B, H, expect="decode", weights=False)
+    _check(nn, oracle, rng, dtype, E, 1, Lkv, B, H, expect="decode", weights=weights)
 
 
 @pytest.mark.parametrize("dtype,E,H,mask_shape", [("bf16", 512, 4, (1500, 1, 1, 3)), ("f16", 256, 4, (1500, 1, 4, 3)),
@@ -308,26 +310,32 @@ def test_decode_with_context_length_masks(nn, oracle, dtype, E, H, mask_shape):
         mask[900:, 0, :, 0] = False                  # context of 900 keys
         mask[:700, 0, :, 1] = False                  # whole leading splits dropped
         mask[:, 0, 0, 2] = False                     # nothing kept for (head 0 or all heads, batch 2)
-    y, _ = _run(nn, q, k, v, dtype, None, mask, H, return_weights=False)
-    assert nn.last_attention_kernel() == "decode"
     with np.errstate(invalid="ignore"):
-        yr, _ = oracle.nnlib_attention_f32(q, k, v, None, mask, H, nthreads=4)
-    assert np.array_equal(np.isnan(y), np.isnan(yr))
-    if len(mask_shape) == 4:
-        assert np.isnan(y).any()
-    ok = ~np.isnan(yr)
-    assert np.abs(y[ok] - yr[ok]).max() / np.abs(yr[ok]).max() <= TOL[dtype]
+        yr, ar = oracle.nnlib_attention_f32(q, k, v, None, mask, H, nthreads=4)
+    for weights in (False, True):
+        y, a = _run(nn, q, k, v, dtype, None, mask, H, return_weights=weights, weights_dtype="f32" if weights else None)
+        assert nn.last_attention_kernel() == "decode"
+        assert np.array_equal(np.isnan(y), np.isnan(yr))
+        if len(mask_shape) == 4:
+            assert np.isnan(y).any()
+        ok = ~np.isnan(yr)
+        assert np.abs(y[ok] - yr[ok]).max() / np.abs(yr[ok]).max() <= TOL[dtype]
+        if weights:
+            assert np.array_equal(np.isnan(a), np.isnan(ar))
+            okw = ~np.isnan(ar)
+            assert np.abs(a[okw] - ar[okw]).max() <= TOL[dtype]
+            assert np.count_nonzero(a[okw & ~np.broadcast_to(mask.reshape(mask.shape + (1,) * (4 - mask.ndim)), a.shape)]) == 0
 
 
-def test_decode_matches_flash16_on_device(nn):
+def test_decode_matches_generic_on_device(nn):
     rng = np.random.default_rng(11)
     q = nn.DeviceArray.from_numpy(rng.standard_normal((512, 1, 2)).astype(np.float32), "bf16")
     k = nn.DeviceArray.from_numpy(rng.standard_normal((512, 3000, 2)).astype(np.float32), "bf16")
     v = nn.DeviceArray.from_numpy(rng.standard_normal((512, 3000, 2)).astype(np.float32), "bf16")
     y1, _ = nn.dot_product_attention(q, k, v, nheads=4, return_weights=False)
     assert nn.last_attention_kernel() == "decode"
-    y2, _ = nn.dot_product_attention(q, k, v, nheads=4, return_weights=True)   # weights force the tiled kernel
-    assert nn.last_attention_kernel() == "flash16"
+    y2, _ = nn.dot_product_attention(q, k, v, nheads=4, return_weights=False, _flags=nn._lib.MI_ATTN_FORCE_GENERIC)
+    assert nn.last_attention_kernel() == "generic"
     assert rel_err(y1.to_numpy(), y2.to_numpy()) < 1e-2
 
 
