@@ -114,9 +114,9 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
     extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
     float *Ks = (float *)bwd_smem, *Vs = Ks + 2 * TILEF;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
-    const int64_t HB = p.H * p.B;
+    const int64_t HB = p.H * a.nb;   // this launch's batch elements: [a.b0, a.b0 + a.nb)
     const int64_t hb = blockIdx.x % HB, qt = a.n_qtiles - 1 - blockIdx.x / HB;
-    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t h = hb % p.H, b = a.b0 + hb / p.H;
     const int64_t i0 = qt * 128, iw = i0 + 32 * wave, qi = iw + r;
     const bool qok = qi < p.Lq;
 
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
                         if (p.bias_strides[0] == 1) {
                             const int64_t nq = p.Lq - iw, nk = p.Lkv - kv0;
                             flash_atomic_add_block(dbias_lds, s[0][kb], db + kv0 + iw * p.bias_strides[1], p.bias_strides[1],
-                                                   (int)(nq > 32 ? 32 : nq), (int)(nk > 32 ? 32 : (nk < 0 ? 0 : nk)));
+                                                   (int)(nq > 32 ? 32 : nq), (int)(nk > 32 ? 32 : (nk < 0 ? 0 : nk)), a.dbias_plain != 0);
                         } else {
 #pragma unroll
                             for (int v = 0; v < 16; v++) {
@@ -442,7 +442,21 @@ int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) 
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         attr_set = true;
     }
-    hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B)), dim3(256), SMEM_Q, st, a, bp);
+    // Bias gradient without atomics where a workgroup owns the entries it adds to; entries shared by the batch
+    // elements are kept apart by one launch per batch element (the same rule as the 16-bit kernels)
+    FlashArgs a1 = a;
+    const bool own_rows = bp.dbias && p.bias_strides[0] == 1 && (p.bias_strides[1] != 0 || p.Lq == 1) && (p.bias_strides[2] != 0 || p.H == 1);
+    const bool per_batch = own_rows && p.bias_strides[3] == 0 && p.B > 1;
+    if (own_rows && (!per_batch || (int64_t)a.n_qtiles * p.H >= 256)) a1.dbias_plain = 1;
+    if (a1.dbias_plain && per_batch) {
+        a1.nb = 1;
+        for (int64_t b = 0; b < p.B; b++) {
+            a1.b0 = (int32_t)b;
+            hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H)), dim3(256), SMEM_Q, st, a1, bp);
+        }
+    } else {
+        hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B)), dim3(256), SMEM_Q, st, a1, bp);
+    }
     MI_LAUNCH_CHECK();
     const dim3 g2((unsigned)(((p.Lkv + 127) / 128) * p.H * p.B));
     if (SPLIT) {
@@ -492,6 +506,9 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st) {
     a.n_qtiles = (int32_t)((bp.p.Lq + 127) / 128);
     a.nsplit = 1;
     a.tiles_per_split = 0;
+    a.b0 = 0;
+    a.nb = (int32_t)bp.p.B;
+    a.dbias_plain = 0;
     flash_fill_vec_flags(a);
     a.bias_lds = a.mask_lds = 0;
     a.p.drop_thresh = 0;   // the shared softmax step yields the weights before dropout; the kernels apply bp.p's dropout themselves

@@ -142,6 +142,8 @@ def test_mfma_kernels(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, bias_k
     # ... and entries shared by the batch elements, one launch per batch element (enough workgroups per launch)
     ("bf16", 8, 16, 2048, 64, (3,), None, (64, 2048, 16, 1), "flash16"),
     ("f16", 16, 16, 2048, 96, (2,), "random", (96, 2048, 16), "flash16"),
+    ("f32", 64, 2, 130, 200, (2,), "random", (200, 130, 2, 2), "flash32"),
+    ("f32", 8, 16, 2048, 64, (3,), None, (64, 2048, 16, 1), "flash32"),
 ])
 def test_bias_gradient_from_the_mfma_kernels(nn, oracle, dtype, D, H, Lq, Lkv, batch, mask_kind, bias_shape, expect):
     """The bias gradient is dS summed over the dims the bias broadcasts along; the dQ kernels add it with Float32
