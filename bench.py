@@ -401,8 +401,8 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (heads and batches shard without communication; "
-                 "see DESIGN.md). Run with --gpus 1.")
+        sys.exit("bench.py: this build measures one GPU only ((head, batch) pairs are independent problems and shard "
+                 "without communication). Run with --gpus 1.")
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the attention path has no CPU fallback")
