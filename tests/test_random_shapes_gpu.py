@@ -50,3 +50,56 @@ def test_forward_and_gradient(nn, oracle, seed):
     for g, r_, name in zip(got[:3], ref[:3], ("dq", "dk", "dv")):
         err = np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05)
         assert err <= TOL[dtype], (name, err, dtype, D, H, B, Lq, Lkv, mask_kind, nn.last_attention_bwd_kernel())
+
+
+# ---- second sweep: head dims other than 64 / 128, bias shapes, mask kinds, dropout, returned weights -------------
+
+import os
+N_SEEDS = int(os.environ.get("MI355ATTN_SWEEP_SEEDS", "45"))   # raise for a longer one-off sweep
+DIMS16 = [8, 16, 24, 32, 40, 48, 64, 72, 80, 96, 112, 128, 136, 160, 192, 256]
+DIMS32 = [4, 12, 20, 32, 36, 64, 68, 96, 128]
+
+
+def _case2(seed):
+    rng = np.random.default_rng(5000 + seed)
+    dtype = ["bf16", "f16", "f32"][seed % 3]
+    dims = DIMS32 if dtype == "f32" else DIMS16
+    D, Dv = int(rng.choice(dims)), int(rng.choice(dims))
+    H, B = int(rng.integers(1, 4)), int(rng.integers(1, 3))
+    Lq = int(rng.choice([1, 31, 33, 64, 65, 127, 129, 200, 256, 300]))
+    mask_kind = [None, "causal", "random", "keys", "random_hb"][int(rng.integers(0, 5))]
+    aligned = bool(rng.integers(0, 2))   # rows of bias / mask start 16-byte aligned: the staged paths
+    Lkv = Lq if mask_kind == "causal" else int(rng.choice([48, 64, 112, 208, 320, 400] if aligned else [47, 65, 131, 333]))
+    if mask_kind == "keys" and Lkv < 100:   # the key-padding pattern of the gradient helper drops the first 70 keys of one batch element
+        Lkv += 256 if aligned else 255
+    bias_kind = [None, None, "full", "row", "shared"][int(rng.integers(0, 5))]
+    return rng, dtype, D, Dv, H, B, Lq, Lkv, mask_kind, bias_kind
+
+
+def _shapes(Lq, Lkv, H, B, mask_kind, bias_kind):
+    bias_shape = {None: None, "full": (Lkv, Lq, H, B), "row": (Lkv, 1), "shared": (Lkv, Lq)}[bias_kind]
+    mask_shape = {None: None, "causal": None, "random": (Lkv, Lq), "keys": (Lkv, 1, 1, B), "random_hb": (Lkv, Lq, H, B)}[mask_kind]
+    return bias_shape, mask_shape
+
+
+@pytest.mark.parametrize("seed", range(N_SEEDS))
+def test_forward_head_dims_bias_masks(nn, oracle, seed):
+    """Forward call against the oracle: head dims of q, k and of v drawn independently (zero-padded tiles), every
+    bias / mask layout the kernels tell apart, with and without the weights."""
+    from test_attention_gpu import _check
+    rng, dtype, D, Dv, H, B, Lq, Lkv, mask_kind, bias_kind = _case2(seed)
+    bias_shape, mask_shape = _shapes(Lq, Lkv, H, B, mask_kind, bias_kind)
+    _check(nn, oracle, rng, dtype, D * H, Lq, Lkv, B, H, Ev=Dv * H, causal=mask_kind == "causal", bias_shape=bias_shape,
+           mask_shape=mask_shape, scale=0.5, weights=bool(seed % 2))
+
+
+@pytest.mark.parametrize("seed", range(N_SEEDS))
+def test_gradient_head_dims_bias_masks(nn, oracle, seed):
+    """Gradient (with the bias gradient where there is a bias) against the float64 oracle over the same space, one
+    head dim for q, k and v, dropout in a quarter of the cases, saved statistics in half."""
+    from test_attention_backward_gpu import _run
+    rng, dtype, D, _, H, B, Lq, Lkv, mask_kind, bias_kind = _case2(seed)
+    bias_shape, _ = _shapes(Lq, Lkv, H, B, mask_kind, bias_kind)
+    dropout = (0.2, 17 + seed) if rng.integers(0, 4) == 0 else None
+    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, bias_shape=bias_shape, mask_kind=mask_kind, seed=seed, scale=0.4,
+         dropout=dropout, saved=bool(rng.integers(0, 2)))
