@@ -215,7 +215,7 @@ function mask_and_bias(::Type{T}, bias, mask, target::NTuple{4, Int}) where {T}
 end
 
 # `stats`: nothing, or a Float32 DeviceArray of mi_attention_stats_size bytes that receives the softmax
-# row statistics for ∇dot_product_attention (written by the 16-bit MFMA kernels only)
+# row statistics for ∇dot_product_attention (written by the MFMA flash kernels, with or without bias, mask and dropout)
 function attention_call(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v, bias, mask, H::Int; want_out::Bool,
                         want_weights::Bool, fdrop::Union{Nothing, Dropout} = nothing, stats = nothing) where {T <: MIFloat}
     E, Lq, B = size(q); Lkv = size(k, 2); Ev = v === nothing ? E : size(v, 1)

@@ -145,7 +145,7 @@ def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_we
     kernel, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
     _lib.check(lib.mi_attention_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))
     stats = None
-    if save_stats and out is not None and kernel.value in (_lib.KERNEL_FLASH16, _lib.KERNEL_FLASH32) and fdrop is None:
+    if save_stats and out is not None and kernel.value in (_lib.KERNEL_FLASH16, _lib.KERNEL_FLASH32):
         # softmax row statistics for dot_product_attention_grad (what an AD rule keeps for its pullback)
         nb = ctypes.c_size_t(0)
         _lib.check(lib.mi_attention_stats_size(ctypes.byref(d), ctypes.byref(nb)))
@@ -260,7 +260,7 @@ def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, m
         if y.dims != dy.dims or y.dtype != q.dtype:
             raise DimensionMismatch("y must have the size and element type of dy")
         d.fwd.out = y.ptr
-        if getattr(y, "saved_stats", None) is not None and dalpha is None and bias is None:
+        if getattr(y, "saved_stats", None) is not None and dalpha is None:
             d.fwd.stats = y.saved_stats.ptr
     d.dout = dy.ptr
     if dalpha is not None:
@@ -284,7 +284,7 @@ def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, m
         d.fwd.out = None
         if kernel.value != _lib.KERNEL_GENERIC:
             y, _ = dot_product_attention(q, k, v, bias, fdrop=fdrop, mask=mask, nheads=nheads, return_weights=False,
-                                         save_for_backward=bias is None, _flags=_flags)
+                                         save_for_backward=True, _flags=_flags)
             d.fwd.out = y.ptr
             if getattr(y, "saved_stats", None) is not None:
                 d.fwd.stats = y.saved_stats.ptr
