@@ -2,18 +2,19 @@
 #include "common.h"
 #include "attention_params.h"
 
-int32_t launch_flash16_bf16_d64(const AttnParams &, hipStream_t);
-int32_t launch_flash16_bf16_d128(const AttnParams &, hipStream_t);
-int32_t launch_flash16_f16_d64(const AttnParams &, hipStream_t);
-int32_t launch_flash16_f16_d128(const AttnParams &, hipStream_t);
-int32_t launch_flash16_bf16_d256(const AttnParams &, hipStream_t);
-int32_t launch_flash16_f16_d256(const AttnParams &, hipStream_t);
-int32_t launch_flash16_fast_bf16(const AttnParams &, hipStream_t);
-int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t);
+// kv_len: null, or per (head, batch) context lengths (FlashArgs::kv_len)
+int32_t launch_flash16_bf16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_bf16_d128(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_f16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_f16_d128(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_bf16_d256(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_f16_d256(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_fast_bf16(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
 bool flash16_fast_supports_bf16(const AttnParams &);
 bool flash16_fast_supports_f16(const AttnParams &);
-int32_t launch_flash16_fast_bf16_d64(const AttnParams &, hipStream_t);
-int32_t launch_flash16_fast_f16_d64(const AttnParams &, hipStream_t);
+int32_t launch_flash16_fast_bf16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_fast_f16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
 bool flash16_fast_supports_bf16_d64(const AttnParams &);
 bool flash16_fast_supports_f16_d64(const AttnParams &);
 
@@ -82,21 +83,87 @@ bool attention_flash16_supports(const AttnParams &p) {
     return true;
 }
 
-static bool takes_fast_path(const AttnParams &p) {
+static bool fast_kernel_fits(const AttnParams &p) {   // everything but the mask
     if (p.dtype == MI_BF16) return flash16_fast_supports_bf16(p) || flash16_fast_supports_bf16_d64(p);
     if (p.dtype == MI_F16) return flash16_fast_supports_f16(p) || flash16_fast_supports_f16_d64(p);
     return false;
 }
+static bool takes_fast_path(const AttnParams &p) { return !p.mask && fast_kernel_fits(p); }
 
-int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
-    if (p.dtype == MI_BF16 && flash16_fast_supports_bf16(p)) return launch_flash16_fast_bf16(p, st);
-    if (p.dtype == MI_F16 && flash16_fast_supports_f16(p)) return launch_flash16_fast_f16(p, st);
-    if (p.dtype == MI_BF16 && flash16_fast_supports_bf16_d64(p)) return launch_flash16_fast_bf16_d64(p, st);
-    if (p.dtype == MI_F16 && flash16_fast_supports_f16_d64(p)) return launch_flash16_fast_f16_d64(p, st);
+// ---- key-padding masks that are context lengths ------------------------------------------------------------------
+// Batches of sequences padded to one length carry a mask that keeps a prefix of the keys of each (head, batch) pair.
+// For such a pair the mask is just a shorter L_kv, which the software-pipelined kernel handles at full speed (and it
+// skips the padding instead of computing and discarding it).  Whether a mask is of that kind is only known on the
+// device, so: a small kernel measures every pair (length of the kept prefix, or 0 when the mask is anything else, an
+// empty one included), then BOTH forward kernels are launched and every (head, batch) pair is computed by exactly
+// one of them: the pipelined kernel takes the pairs with a length, the general kernel the others.
+static bool takes_length_path(const AttnParams &p) {
+    return flash_is_key_mask(p) && fast_kernel_fits(p) && flash_pick_nsplit(p, 128) == 1 && p.H * p.B <= 2147483647LL / 4;
+}
+static size_t length_path_workspace(const AttnParams &p) { return ((size_t)(p.H * p.B) * sizeof(int32_t) + 15) & ~(size_t)15; }
+
+__global__ __launch_bounds__(256) void key_mask_lengths_kernel(const uint8_t *mask, int64_t s2, int64_t s3, int64_t Lkv, int64_t H,
+                                                              int32_t *lens) {
+    const int64_t h = blockIdx.x % H, b = blockIdx.x / H;
+    const uint8_t *m = mask + h * s2 + b * s3;   // unit key stride, 4-byte aligned, Lkv a multiple of 4 (flash_is_key_mask)
+    int last = -1, count = 0;
+    for (int64_t j = 4 * (int64_t)threadIdx.x; j < Lkv; j += 4 * 256) {
+        const uint32_t w = *(const uint32_t *)(m + j);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if ((w >> (8 * e)) & 0xFFu) {
+                last = (int)j + e;
+                count++;
+            }
+    }
+    __shared__ int s_last[4], s_count[4];
+    for (int off = 32; off > 0; off >>= 1) {
+        const int o_last = __shfl_xor(last, off, 64);
+        last = o_last > last ? o_last : last;
+        count += __shfl_xor(count, off, 64);
+    }
+    if ((threadIdx.x & 63) == 0) {
+        s_last[threadIdx.x >> 6] = last;
+        s_count[threadIdx.x >> 6] = count;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int l = s_last[0], c = s_count[0];
+        for (int w = 1; w < 4; w++) {
+            l = s_last[w] > l ? s_last[w] : l;
+            c += s_count[w];
+        }
+        lens[blockIdx.x] = (c > 0 && c == l + 1) ? c : 0;
+    }
+}
+
+static int32_t launch_general16(const AttnParams &p, hipStream_t st, const int32_t *kv_len) {
     const int64_t dmax = p.D > p.Dv ? p.D : p.Dv;
     if (p.dtype == MI_BF16)
-        return dmax <= 64 ? launch_flash16_bf16_d64(p, st) : dmax <= 128 ? launch_flash16_bf16_d128(p, st) : launch_flash16_bf16_d256(p, st);
-    return dmax <= 64 ? launch_flash16_f16_d64(p, st) : dmax <= 128 ? launch_flash16_f16_d128(p, st) : launch_flash16_f16_d256(p, st);
+        return dmax <= 64 ? launch_flash16_bf16_d64(p, st, kv_len) : dmax <= 128 ? launch_flash16_bf16_d128(p, st, kv_len) : launch_flash16_bf16_d256(p, st, kv_len);
+    return dmax <= 64 ? launch_flash16_f16_d64(p, st, kv_len) : dmax <= 128 ? launch_flash16_f16_d128(p, st, kv_len) : launch_flash16_f16_d256(p, st, kv_len);
+}
+
+static int32_t launch_fast16(const AttnParams &p, hipStream_t st, const int32_t *kv_len) {
+    if (p.dtype == MI_BF16 && flash16_fast_supports_bf16(p)) return launch_flash16_fast_bf16(p, st, kv_len);
+    if (p.dtype == MI_F16 && flash16_fast_supports_f16(p)) return launch_flash16_fast_f16(p, st, kv_len);
+    if (p.dtype == MI_BF16) return launch_flash16_fast_bf16_d64(p, st, kv_len);
+    return launch_flash16_fast_f16_d64(p, st, kv_len);
+}
+
+int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
+    if (takes_length_path(p)) {
+        if (p.H * p.B > 2147483647LL) return mi_set_error(MI_ESHAPE, "attention: too many (head, batch) pairs");
+        int32_t *lens = (int32_t *)p.workspace;
+        hipLaunchKernelGGL(key_mask_lengths_kernel, dim3((unsigned)(p.H * p.B)), dim3(256), 0, st, p.mask, p.mask_strides[2],
+                           p.mask_strides[3], p.Lkv, p.H, lens);
+        MI_LAUNCH_CHECK();
+        int32_t rc = launch_fast16(p, st, lens);
+        if (rc != MI_OK) return rc;
+        return launch_general16(p, st, lens);
+    }
+    if (takes_fast_path(p)) return launch_fast16(p, st, nullptr);
+    return launch_general16(p, st, nullptr);
 }
 
 // Validation.  The first four conditions are the reference's ArgumentErrors
@@ -163,7 +230,8 @@ static int32_t choose(const mi_attn_desc *d, const AttnParams &p, size_t *ws) {
         return MI_ATTN_KERNEL_DECODE;
     }
     if (attention_flash16_supports(p)) {
-        if (!takes_fast_path(p)) *ws = flash_split_workspace(p, flash_pick_nsplit(p, 128));
+        if (takes_length_path(p)) *ws = length_path_workspace(p);   // one context length per (head, batch) pair
+        else if (!takes_fast_path(p)) *ws = flash_split_workspace(p, flash_pick_nsplit(p, 128));
         return MI_ATTN_KERNEL_FLASH16;
     }
     if (attention_flash32_supports(p)) return MI_ATTN_KERNEL_FLASH32;

@@ -26,6 +26,10 @@ struct FlashArgs {
     // gradient kernels only: the launch covers batch elements [b0, b0 + nb), and the bias gradient may be summed
     // without atomics (no two workgroups of one launch add to the same element)
     int32_t b0, nb, dbias_plain;
+    // forward kernels, key-padding masks that are context lengths: per (head, batch) pair [b * H + h] the number of
+    // leading keys kept when the mask keeps exactly a prefix (the software-pipelined kernel then treats it as that
+    // pair's L_kv and the general kernel leaves the pair alone), 0 otherwise (the general kernel applies the mask)
+    const int32_t *kv_len = nullptr;
 };
 
 // Bytes of LDS per wavefront for the weight staging below: 16 query rows x 128 bytes.

@@ -429,3 +429,30 @@ def test_key_padding_masks(nn, oracle, dtype, E, H, weights):
         assert np.abs(a[..., :3] - ar[..., :3]).max() <= TOL[dtype]
         keep = np.broadcast_to(mask, a.shape)[..., :3]
         assert np.count_nonzero(a[..., :3][~keep]) == 0
+
+
+@pytest.mark.parametrize("dtype,E,H,Lq,Lkv", [("bf16", 256, 2, 140, 332), ("f16", 128, 2, 300, 1100), ("bf16", 128, 1, 513, 2048)])
+@pytest.mark.parametrize("per_head", [False, True], ids=["per-batch", "per-head"])
+def test_context_length_masks(nn, oracle, dtype, E, H, Lq, Lkv, per_head):
+    """Key-padding masks that keep a prefix of the keys (padded batches): a device-side pass measures every (head,
+    batch) pair, the software-pipelined kernel computes the pairs whose mask is a context length as a shorter L_kv and
+    the general kernel the rest (scattered masks, an empty one: NaN).  Every pair must come from exactly one of them."""
+    rng = np.random.default_rng(Lq + Lkv)
+    B = 6
+    q, k, v = (round_to(rng.standard_normal((E, L, B)), dtype) for L in (Lq, Lkv, Lkv))
+    mask = np.ones((Lkv, 1, H if per_head else 1, B), dtype=bool)
+    mask[Lkv - 82:, 0, :, 0] = False            # context length Lkv - 82
+    mask[1:, 0, :, 1] = False                   # a single key
+    mask[:, 0, :, 3] = rng.random((Lkv, mask.shape[2])) < 0.5   # scattered: not a prefix
+    mask[:, 0, :, 4] = False                    # nothing kept
+    mask[:37, 0, :, 5] = False                  # a suffix is kept: not a prefix
+    if per_head:
+        mask[200:, 0, 0, 2] = False             # batch element 2: one head padded, the others full
+    y, _ = _run(nn, q, k, v, dtype, None, mask, H, return_weights=False)
+    assert nn.last_attention_kernel() == "flash16"
+    with np.errstate(invalid="ignore"):
+        yr, _ = oracle.nnlib_attention_f32(q, k, v, None, mask, H, nthreads=4)
+    assert np.isnan(y[:, :, 4]).all() and np.isnan(yr[:, :, 4]).all()
+    ok = [0, 1, 2, 3, 5]
+    assert not np.isnan(y[:, :, ok]).any()
+    assert rel_err(y[:, :, ok], yr[:, :, ok]) <= TOL[dtype]
