@@ -137,6 +137,14 @@ __global__ __launch_bounds__(256) void key_mask_lengths_kernel(const uint8_t *ma
     }
 }
 
+int32_t launch_key_mask_lengths(const AttnParams &p, int32_t *lens, hipStream_t st) {
+    if (p.H * p.B > 2147483647LL) return mi_set_error(MI_ESHAPE, "attention: too many (head, batch) pairs");
+    hipLaunchKernelGGL(key_mask_lengths_kernel, dim3((unsigned)(p.H * p.B)), dim3(256), 0, st, p.mask, p.mask_strides[2],
+                       p.mask_strides[3], p.Lkv, p.H, lens);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
 static int32_t launch_general16(const AttnParams &p, hipStream_t st, const int32_t *kv_len) {
     const int64_t dmax = p.D > p.Dv ? p.D : p.Dv;
     if (p.dtype == MI_BF16)
@@ -153,12 +161,10 @@ static int32_t launch_fast16(const AttnParams &p, hipStream_t st, const int32_t 
 
 int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
     if (takes_length_path(p)) {
-        if (p.H * p.B > 2147483647LL) return mi_set_error(MI_ESHAPE, "attention: too many (head, batch) pairs");
         int32_t *lens = (int32_t *)p.workspace;
-        hipLaunchKernelGGL(key_mask_lengths_kernel, dim3((unsigned)(p.H * p.B)), dim3(256), 0, st, p.mask, p.mask_strides[2],
-                           p.mask_strides[3], p.Lkv, p.H, lens);
-        MI_LAUNCH_CHECK();
-        int32_t rc = launch_fast16(p, st, lens);
+        int32_t rc = launch_key_mask_lengths(p, lens, st);
+        if (rc != MI_OK) return rc;
+        rc = launch_fast16(p, st, lens);
         if (rc != MI_OK) return rc;
         return launch_general16(p, st, lens);
     }

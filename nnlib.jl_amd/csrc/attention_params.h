@@ -77,6 +77,9 @@ struct AttnBwdParams {
     // bits of the tile's queries for that key; slice = h * mb_h + b * mb_b (0 where the mask is shared)
     const uint64_t *mask_bits;
     int64_t mb_h, mb_b, mb_lkv_pad, mb_nqt;
+    // key-padding mask measured on the device: per (head, batch) pair [b * H + h] the context length, or 0 when the
+    // mask of the pair is not a kept prefix; null when the call does not take that path
+    const int32_t *kv_len;
 };
 
 // size of the statistics planes shared by the forward kernels that save them and the backward kernels
@@ -92,6 +95,9 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st);
 bool attention_bwd_flash32_supports(const AttnBwdParams &bp);
 size_t attention_bwd_flash16_workspace(const AttnParams &p);
 size_t attention_bwd_flash16_mask_bits_bytes(const AttnParams &p);   // 0 when the call does not take the packed-mask path
+size_t attention_bwd_flash16_lengths_bytes(const AttnBwdParams &bp);  // 0 when the call does not take the context-length path
+// lens[b * H + h] = number of keys kept when the key-padding mask of the pair keeps exactly a prefix, else 0
+int32_t launch_key_mask_lengths(const AttnParams &p, int32_t *lens, hipStream_t st);
 size_t attention_bwd_generic_workspace(const AttnParams &p);
 int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_backward = false);
 

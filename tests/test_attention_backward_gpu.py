@@ -30,6 +30,16 @@ def _run(nn, oracle, dtype, E, Ev, Lq, Lkv, batch, H, bias_shape=None, mask_kind
         mask = rng.random((Lkv, Lq, H if mask_kind == "random_hb" else 1) + batch) < 0.8
         mask[0] = True
         dmask = nn.DeviceArray.from_numpy(mask)
+    elif mask_kind == "lengths":    # padded batch: context lengths per batch element, plus one scattered pattern
+        mask = np.ones((Lkv, 1, 1) + batch, dtype=bool)
+        nb = mask.shape[-1]
+        for i in range(nb):
+            if i % 3 == 1:
+                mask[Lkv - min(90, Lkv // 2):, ..., i] = False        # a padded tail
+            elif i % 3 == 2:
+                mask[..., i] = (rng.random(Lkv) < 0.6).reshape((Lkv, 1, 1) + (1,) * (len(batch) - 1))
+                mask[0, ..., i] = True
+        dmask = nn.DeviceArray.from_numpy(mask)
     elif mask_kind == "keys":       # key-padding mask: no query dependence, one pattern per batch element
         mask = rng.random((Lkv, 1, 1) + batch) < 0.7
         mask[Lkv // 2, ...] = True
@@ -259,6 +269,19 @@ def test_dense_mask_on_the_lean_paths(nn, oracle, dtype, D, H, Lq, Lkv, batch, m
     """A dense Bool mask without bias whose rows start 16-byte aligned: the dQ kernel reads staged mask tiles, the
     dK / dV kernels 64-bit words packed by a small kernel first (one per key and query tile)."""
     _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, batch, H, mask_kind=mask_kind, expect="flash16", saved=saved, dropout=dropout,
+         seed=Lq + Lkv, scale=0.4)
+
+
+@pytest.mark.parametrize("dtype,D,H,Lq,Lkv,B,causal_too,saved,dropout", [
+    ("bf16", 128, 2, 200, 332, 4, False, True, None),
+    ("f16", 64, 2, 300, 1100, 3, False, True, None),
+    ("bf16", 96, 1, 513, 520, 5, False, True, (0.2, 5)),
+    ("bf16", 128, 2, 200, 332, 4, False, False, None),      # no saved statistics: the key-mask kernels take every pair
+])
+def test_context_lengths_in_the_gradient(nn, oracle, dtype, D, H, Lq, Lkv, B, causal_too, saved, dropout):
+    """Key-padding masks with saved statistics: pairs whose mask keeps a prefix of the keys run the unmasked gradient
+    kernels on that many keys (the padding gets zero gradients), the others the key-mask kernels."""
+    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, mask_kind="lengths", expect="flash16", saved=saved, dropout=dropout,
          seed=Lq + Lkv, scale=0.4)
 
 
