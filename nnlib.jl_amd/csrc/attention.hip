@@ -240,7 +240,10 @@ static int32_t choose(const mi_attn_desc *d, const AttnParams &p, size_t *ws) {
         else if (!takes_fast_path(p)) *ws = flash_split_workspace(p, flash_pick_nsplit(p, 128));
         return MI_ATTN_KERNEL_FLASH16;
     }
-    if (attention_flash32_supports(p)) return MI_ATTN_KERNEL_FLASH32;
+    if (attention_flash32_supports(p)) {
+        *ws = attention_flash32_lengths_bytes(p);
+        return MI_ATTN_KERNEL_FLASH32;
+    }
     return MI_ATTN_KERNEL_GENERIC;
 }
 

@@ -36,7 +36,8 @@ __device__ inline floatx4_t ldg16f(const float *p, bool ok) {
 }
 
 template <int D, int QB, bool CAUSAL, bool EXTRAS, int PHASE>
-__device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *Ks, float *Vs, int64_t b, int64_t h,
+// kv_len: keys of this (head, batch) pair (L_kv, or a shorter context length)
+__device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *Ks, float *Vs, int64_t kv_len, int64_t b, int64_t h,
                                    int64_t iw, int n_tiles, unsigned wlds = 0) {
     constexpr int KS = Cfg<D>::KS, VS = Cfg<D>::VS, CHUNKS = Cfg<D>::CHUNKS;
     const AttnParams &p = a.p;
@@ -56,7 +57,7 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
         for (int u = 0; u < CHUNKS; u++) {
             const int c = tid + 256 * u;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
-            const bool ok = j0 + row < p.Lkv;
+            const bool ok = j0 + row < kv_len;
             kreg[u] = ldg16f(kbase + p.E * (j0 + row) + col, ok && col < dqk);
             if (NEED_V) vreg[u] = ldg16f(vbase + p.Ev * (j0 + row) + col, ok && do_pv && col < dv);
         }
@@ -103,7 +104,7 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
                 }
 
             flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0,
-                                                                                                          FlashStaged<QB>(), 0, wlds);
+                                                                                                          FlashStaged<QB>(), 0, wlds, nullptr, kv_len);
 
             if (do_pv) {
                 // k-step v of key block kb multiplies key 32*kb + 8*(v/4) + 4*hh + v%4: exactly the key
@@ -147,6 +148,15 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
     const int64_t qt = a.n_qtiles - 1 - id / HB;   // heaviest (latest) query tiles first
     const int64_t h = hb % p.H, b = hb / p.H;
     const int64_t i0 = qt * BM, iw = i0 + (int64_t)wave * 32 * QB;
+    // Key-padding masks measured on the device (FlashArgs::kv_len): a (head, batch) pair whose mask keeps a prefix of
+    // the keys is an unmasked problem with that many keys, which the variant without bias / mask code takes; the
+    // variant with it computes the other pairs.  Both are launched; every pair belongs to exactly one.
+    int64_t kv_len = p.Lkv;
+    if (a.kv_len) {
+        const int64_t len = a.kv_len[b * p.H + h];
+        if (EXTRAS == (len != 0)) return;
+        if (!EXTRAS) kv_len = len;
+    }
 
     Frag32<D, QB> f;
     const float *qbase = (const float *)p.q + p.E * (p.Lq * b) + p.D * h;
@@ -167,14 +177,14 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
         f.l[qb] = 0.0f;
     }
 
-    int64_t kv_end = p.Lkv;
+    int64_t kv_end = kv_len;
     if (CAUSAL && i0 + BM < kv_end) kv_end = i0 + BM;
     const int n_tiles = (int)((kv_end + BN - 1) / BN);
 
     if (!WEIGHTS) {
-        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_ONLINE>(a, f, Ks, Vs, b, h, iw, n_tiles);
+        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_ONLINE>(a, f, Ks, Vs, kv_len, b, h, iw, n_tiles);
     } else {
-        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_STATS>(a, f, Ks, Vs, b, h, iw, n_tiles);
+        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_STATS>(a, f, Ks, Vs, kv_len, b, h, iw, n_tiles);
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) {
             const float l = f.l[qb] + mi_swap32(f.l[qb]);
@@ -183,8 +193,9 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
         // weight tiles leave through a wavefront-private LDS region behind the K / V buffers
         const unsigned wlds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem +
                               (unsigned)Cfg<D>::SMEM + wave * FLASH_WSTAGE_BYTES;
-        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_FINAL>(a, f, Ks, Vs, b, h, iw, n_tiles, wlds);
+        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_FINAL>(a, f, Ks, Vs, kv_len, b, h, iw, n_tiles, wlds);
         if (CAUSAL && p.weights) flash_zero_skipped_weights<QB, float>(a, b, h, iw, n_tiles);
+        else if (p.weights && kv_len < p.Lkv) flash_zero_skipped_weights<QB, float>(a, b, h, iw, n_tiles, false);   // keys past the context length
     }
 
     if (p.out) {
@@ -229,8 +240,8 @@ int32_t launch_one(const FlashArgs &a, hipStream_t st) {
 }
 
 template <int D, int QB>
-int32_t launch_d(const FlashArgs &a, hipStream_t st) {
-    const bool extras = a.p.bias || a.p.mask, w = a.p.weights != nullptr;
+int32_t launch_d(const FlashArgs &a, hipStream_t st, bool extras) {
+    const bool w = a.p.weights != nullptr;
     if (a.p.causal) {
         if (extras) return w ? launch_one<D, QB, true, true, true>(a, st) : launch_one<D, QB, true, true, false>(a, st);
         return w ? launch_one<D, QB, true, false, true>(a, st) : launch_one<D, QB, true, false, false>(a, st);
@@ -240,6 +251,12 @@ int32_t launch_d(const FlashArgs &a, hipStream_t st) {
 }
 
 }  // namespace
+
+// context lengths of a key-padding mask, one per (head, batch) pair: workspace of the calls that take that path
+size_t attention_flash32_lengths_bytes(const AttnParams &p) {
+    if (!flash_is_key_mask(p) || p.H * p.B > 2147483647LL / 4) return 0;
+    return ((size_t)(p.H * p.B) * sizeof(int32_t) + 15) & ~(size_t)15;
+}
 
 bool attention_flash32_supports(const AttnParams &p) {
     if (p.dtype != MI_F32) return false;
@@ -260,5 +277,17 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     a.cn = 1.0f;
     a.n_qtiles = (int32_t)((p.Lq + 127) / 128);
     flash_fill_vec_flags(a);
-    return (p.D <= 64 && p.Dv <= 64) ? launch_d<64, 1>(a, st) : launch_d<128, 1>(a, st);
+    const bool narrow = p.D <= 64 && p.Dv <= 64;
+    if (attention_flash32_lengths_bytes(p) != 0) {
+        // key-padding mask: classify the (head, batch) pairs on the device, then launch both variants
+        int32_t *lens = (int32_t *)p.workspace;
+        int32_t rc = launch_key_mask_lengths(p, lens, st);
+        if (rc != MI_OK) return rc;
+        a.kv_len = lens;
+        rc = narrow ? launch_d<64, 1>(a, st, false) : launch_d<128, 1>(a, st, false);
+        if (rc != MI_OK) return rc;
+        return narrow ? launch_d<64, 1>(a, st, true) : launch_d<128, 1>(a, st, true);
+    }
+    const bool extras = p.bias || p.mask;
+    return narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
 }

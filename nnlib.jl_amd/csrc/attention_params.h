@@ -108,4 +108,5 @@ int32_t launch_attention_decode(const AttnParams &p, hipStream_t st);
 size_t attention_decode_workspace(const AttnParams &p);
 bool attention_flash16_supports(const AttnParams &p);
 bool attention_flash32_supports(const AttnParams &p);
+size_t attention_flash32_lengths_bytes(const AttnParams &p);
 bool attention_decode_supports(const AttnParams &p);

@@ -354,12 +354,15 @@ template <typename T, int QB, int NDV, bool CAUSAL, int EXTRAS, int PHASE, typen
 __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB][2], floatx16_t (&o)[QB][NDV],
                                           float (&fm)[QB], float (&fl)[QB], int64_t b, int64_t h, int64_t iw,
                                           int64_t j0, const FlashStaged<QB> &sg = FlashStaged<QB>(), int stage = 0,
-                                          unsigned wlds = 0, const uint32_t *key_mask = nullptr) {
+                                          unsigned wlds = 0, const uint32_t *key_mask = nullptr, int64_t kv_len = -1) {
     const AttnParams &p = a.p;
     typedef typename T::type elem_t;
     constexpr int BN = FLASH_BN;
     const int lane = threadIdx.x & 63, r = lane & 31, hh = lane >> 5;
-    const bool edge = (j0 + BN > p.Lkv) || (CAUSAL && j0 + BN - 1 > iw);
+    // kv_len >= 0: keys from kv_len on do not exist for this (head, batch) pair (a context length shorter than L_kv);
+    // the weights of such keys come out as exact zeros
+    const int64_t lkv = kv_len >= 0 ? kv_len : p.Lkv;
+    const bool edge = (j0 + BN > lkv) || (CAUSAL && j0 + BN - 1 > iw);
 #pragma unroll
     for (int qb = 0; qb < QB; qb++) {
         const int64_t qi = iw + 32 * qb + r;
@@ -469,7 +472,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
         }
         if (EXTRAS != EXTRAS_DIRECT && edge) {
             // keys past the end of the sequence or, causal, after the query: tile-local limit per lane
-            int64_t lim64 = p.Lkv - j0;
+            int64_t lim64 = lkv - j0;
             if (CAUSAL && qi - j0 + 1 < lim64) lim64 = qi - j0 + 1;
             const int lim = lim64 > BN ? BN : (lim64 < 0 ? 0 : (int)lim64);
 #pragma unroll
@@ -637,11 +640,13 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
 // Causal calls that return weights: keys after the last tile a wavefront visited are all dropped for
 // its queries; their weights are exact zeros, which still have to be written.
 template <int QB, typename TW>
-__device__ inline void flash_zero_skipped_weights(const FlashArgs &a, int64_t b, int64_t h, int64_t iw, int n_tiles) {
+// from_diag: the wavefront stopped at the tile that holds its last query's diagonal (causal); otherwise it visited
+// all n_tiles tiles
+__device__ inline void flash_zero_skipped_weights(const FlashArgs &a, int64_t b, int64_t h, int64_t iw, int n_tiles, bool from_diag = true) {
     const AttnParams &p = a.p;
     constexpr int BN = FLASH_BN;
     const int lane = threadIdx.x & 63;
-    int64_t kcov = ((iw + 32 * QB - 1) / BN + 1) * BN;
+    int64_t kcov = from_diag ? ((iw + 32 * QB - 1) / BN + 1) * BN : (int64_t)n_tiles * BN;
     if (kcov > (int64_t)n_tiles * BN) kcov = (int64_t)n_tiles * BN;
     for (int row = 0; row < 32 * QB; row++) {
         const int64_t qi = iw + row;

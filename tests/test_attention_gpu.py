@@ -431,7 +431,8 @@ def test_key_padding_masks(nn, oracle, dtype, E, H, weights):
         assert np.count_nonzero(a[..., :3][~keep]) == 0
 
 
-@pytest.mark.parametrize("dtype,E,H,Lq,Lkv", [("bf16", 256, 2, 140, 332), ("f16", 128, 2, 300, 1100), ("bf16", 128, 1, 513, 2048)])
+@pytest.mark.parametrize("dtype,E,H,Lq,Lkv", [("bf16", 256, 2, 140, 332), ("f16", 128, 2, 300, 1100), ("bf16", 128, 1, 513, 2048),
+                                              ("f32", 128, 2, 140, 332), ("f32", 72, 2, 300, 1100)])
 @pytest.mark.parametrize("per_head", [False, True], ids=["per-batch", "per-head"])
 def test_context_length_masks(nn, oracle, dtype, E, H, Lq, Lkv, per_head):
     """Key-padding masks that keep a prefix of the keys (padded batches): a device-side pass measures every (head,
@@ -448,11 +449,17 @@ def test_context_length_masks(nn, oracle, dtype, E, H, Lq, Lkv, per_head):
     mask[:37, 0, :, 5] = False                  # a suffix is kept: not a prefix
     if per_head:
         mask[200:, 0, 0, 2] = False             # batch element 2: one head padded, the others full
-    y, _ = _run(nn, q, k, v, dtype, None, mask, H, return_weights=False)
-    assert nn.last_attention_kernel() == "flash16"
     with np.errstate(invalid="ignore"):
-        yr, _ = oracle.nnlib_attention_f32(q, k, v, None, mask, H, nthreads=4)
-    assert np.isnan(y[:, :, 4]).all() and np.isnan(yr[:, :, 4]).all()
+        yr, ar = oracle.nnlib_attention_f32(q, k, v, None, mask, H, nthreads=4)
     ok = [0, 1, 2, 3, 5]
-    assert not np.isnan(y[:, :, ok]).any()
-    assert rel_err(y[:, :, ok], yr[:, :, ok]) <= TOL[dtype]
+    for weights in ((False, True) if dtype == "f32" else (False,)):   # Float32: the same path also returns the weights
+        y, a = _run(nn, q, k, v, dtype, None, mask, H, return_weights=weights)
+        assert nn.last_attention_kernel() == ("flash32" if dtype == "f32" else "flash16")
+        assert np.isnan(y[:, :, 4]).all() and np.isnan(yr[:, :, 4]).all()
+        assert not np.isnan(y[:, :, ok]).any()
+        assert rel_err(y[:, :, ok], yr[:, :, ok]) <= TOL[dtype]
+        if weights:
+            assert np.abs(a[..., ok] - ar[..., ok]).max() <= TOL[dtype]
+            keep = np.broadcast_to(mask, a.shape)[..., ok]
+            assert np.count_nonzero(a[..., ok][~keep]) == 0          # exact zeros past the context length
+            assert np.abs(a[..., ok].sum(axis=0) - 1).max() <= 1e-5
