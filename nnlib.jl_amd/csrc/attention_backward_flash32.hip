@@ -133,7 +133,16 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
         delta += mi_swap32(delta);
     }
 
-    int64_t kv_end = p.Lkv;
+    // Key-padding masks measured on the device (FlashArgs::kv_len): a (head, batch) pair whose mask keeps a prefix of
+    // the keys is an unmasked problem with that many keys (the kernels without mask code take it and leave the other
+    // pairs to the kernels with it, which are launched as well)
+    int64_t kv_len = p.Lkv;
+    if (a.kv_len) {
+        const int64_t len = a.kv_len[b * p.H + h];
+        if ((EXTRAS == EXTRAS_NONE) == (len == 0)) return;
+        if (EXTRAS == EXTRAS_NONE) kv_len = len;
+    }
+    int64_t kv_end = kv_len;
     if (CAUSAL && i0 + 128 < kv_end) kv_end = i0 + 128;
     const int n_tiles = (int)((kv_end + BN - 1) / BN);
 
@@ -141,7 +150,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
     ts.base1 = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
     ts.dh = (int)p.D;
     ts.stride = p.E;
-    ts.nrows = p.Lkv;
+    ts.nrows = kv_len;
     ts.s1 = Ks;
     ts.s2 = Vs;
     floatx16_t unused_o[1][NDV];
@@ -169,7 +178,8 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
             floatx16_t s[1][2] = {{(floatx16_t){0}, (floatx16_t){0}}};
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) s[0][kb] = first_product<D>(Ks + buf * TILEF, kb, qx, s[0][kb], r, hh);
-            flash_softmax_tile<T, 1, NDV, CAUSAL, EXTRAS, PHASE_STATS, float>(a, s, unused_o, fm, fl, b, h, iw, j0);
+            flash_softmax_tile<T, 1, NDV, CAUSAL, EXTRAS, PHASE_STATS, float>(a, s, unused_o, fm, fl, b, h, iw, j0, FlashStaged<1>(), 0, 0, nullptr,
+                                                                              kv_len);
         }
         if (jt + 1 < n_tiles) ts.store(buf ^ 1);
         __syncthreads();
@@ -203,7 +213,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
         if (!CAUSAL || j0 <= iw + 31) {
             const float *kt = Ks + buf * TILEF, *vt = Vs + buf * TILEF;
             if constexpr (EXTRAS == EXTRAS_NONE) {
-                const bool edge = (j0 + BN > p.Lkv) || (CAUSAL && j0 + BN - 1 > iw);
+                const bool edge = (j0 + BN > kv_len) || (CAUSAL && j0 + BN - 1 > iw);
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++) {
                     if (CAUSAL && j0 + 32 * kb > iw + 31) break;   // every key of this block is after every query of the wavefront
@@ -211,7 +221,7 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
                     const floatx16_t dpb = first_product<D>(vt, kb, dox, (floatx16_t){0}, r, hh);
                     int64_t lim = BN;
                     if (edge) {
-                        lim = p.Lkv - j0;
+                        lim = kv_len - j0;
                         if (CAUSAL && qi - j0 + 1 < lim) lim = qi - j0 + 1;
                     }
 #pragma unroll
@@ -299,12 +309,36 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
     const int64_t h = hb % p.H, b = hb / p.H;
     const int64_t j0 = kt_idx * 128, jw = j0 + 32 * wave, kv = jw + r;
     const bool kok = kv < p.Lkv;
+    // context lengths (see the dQ kernel): keys from the pair's length on get zero gradients, and a workgroup whose
+    // keys all lie there has nothing else to do
+    int64_t kv_len = p.Lkv;
+    if (a.kv_len) {
+        const int64_t len = a.kv_len[b * p.H + h];
+        if ((EXTRAS == EXTRAS_NONE) == (len == 0)) return;
+        if (EXTRAS == EXTRAS_NONE) kv_len = len;
+    }
+    const bool kvalid = EXTRAS == EXTRAS_NONE ? kv < kv_len : kok;
+    if (EXTRAS == EXTRAS_NONE && j0 >= kv_len) {
+        if (kok) {
+            const int64_t off = p.E * (kv + p.Lkv * b) + p.D * h;
+            const floatx4_t z4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int dvb = 0; dvb < NDV; dvb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    if (32 * dvb + 8 * g + 4 * hh >= p.D) continue;
+                    if (DO_DK && bp.dk) *(floatx4_t *)((float *)bp.dk + off + 32 * dvb + 8 * g + 4 * hh) = z4;
+                    if (DO_DV && bp.dv) *(floatx4_t *)((float *)bp.dv + off + 32 * dvb + 8 * g + 4 * hh) = z4;
+                }
+        }
+        return;
+    }
 
     float kx[D / 2], vx[DO_DK ? D / 2 : 1];
     {
         const int64_t off = p.E * (kv + p.Lkv * b) + p.D * h;
-        load_stationary<D>(kx, (const float *)p.k + off, kok, hh, (int)p.D);
-        if constexpr (DO_DK) load_stationary<D>(vx, (const float *)p.v + off, kok, hh, (int)p.D);
+        load_stationary<D>(kx, (const float *)p.k + off, kvalid, hh, (int)p.D);
+        if constexpr (DO_DK) load_stationary<D>(vx, (const float *)p.v + off, kvalid, hh, (int)p.D);
     }
     floatx16_t dk[NDV], dv[NDV];
 #pragma unroll
@@ -413,8 +447,8 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
                 floatx4_t k4, v4;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    k4[e] = dk[dvb][4 * g + e] * a.cn;
-                    v4[e] = dv[dvb][4 * g + e];
+                    k4[e] = (EXTRAS != EXTRAS_NONE || kvalid) ? dk[dvb][4 * g + e] * a.cn : 0.0f;
+                    v4[e] = (EXTRAS != EXTRAS_NONE || kvalid) ? dv[dvb][4 * g + e] : 0.0f;
                 }
                 if (DO_DK && bp.dk) *(floatx4_t *)((float *)bp.dk + off + 32 * dvb + 8 * g + 4 * hh) = k4;
                 if (DO_DV && bp.dv) *(floatx4_t *)((float *)bp.dv + off + 32 * dvb + 8 * g + 4 * hh) = v4;
@@ -472,6 +506,11 @@ int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) 
 
 template <int D>
 int32_t launch_d(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
+    if (a.kv_len) {   // key-padding mask measured on the device: both kernel sets, every (head, batch) pair in exactly one
+        const int32_t rc = bp.p.causal ? launch_set<D, true, EXTRAS_NONE>(a, bp, st) : launch_set<D, false, EXTRAS_NONE>(a, bp, st);
+        if (rc != MI_OK) return rc;
+        return bp.p.causal ? launch_set<D, true, EXTRAS_DIRECT>(a, bp, st) : launch_set<D, false, EXTRAS_DIRECT>(a, bp, st);
+    }
     const bool extras = bp.p.bias || bp.p.mask || bp.p.drop_thresh;
     if (bp.p.drop_thresh)   // dropout runs on the per-element paths
         return bp.p.causal ? launch_set<D, true, EXTRAS_DIRECT, true>(a, bp, st) : launch_set<D, false, EXTRAS_DIRECT, true>(a, bp, st);
@@ -480,6 +519,12 @@ int32_t launch_d(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
 }
 
 }  // namespace
+
+// context lengths of a key-padding mask (no dropout: that runs on the per-element paths), one per (head, batch) pair
+size_t attention_bwd_flash32_lengths_bytes(const AttnBwdParams &bp) {
+    if (bp.p.drop_thresh || !flash_is_key_mask(bp.p) || bp.p.H * bp.p.B > 2147483647LL / 4) return 0;
+    return ((size_t)(bp.p.H * bp.p.B) * sizeof(int32_t) + 15) & ~(size_t)15;
+}
 
 bool attention_bwd_flash32_supports(const AttnBwdParams &bp) {
     const AttnParams &p = bp.p;
@@ -512,5 +557,12 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st) {
     flash_fill_vec_flags(a);
     a.bias_lds = a.mask_lds = 0;
     a.p.drop_thresh = 0;   // the shared softmax step yields the weights before dropout; the kernels apply bp.p's dropout themselves
+    if (attention_bwd_flash32_lengths_bytes(bp) != 0) {
+        // the lengths follow the statistics planes when those live in the workspace too
+        int32_t *lens = (int32_t *)((char *)bp.workspace + (bp.have_stats ? 0 : attention_stats_bytes(bp.p)));
+        const int32_t rc = launch_key_mask_lengths(bp.p, lens, st);
+        if (rc != MI_OK) return rc;
+        a.kv_len = lens;
+    }
     return bp.p.D <= 64 ? launch_d<64>(a, bp, st) : launch_d<128>(a, bp, st);
 }

@@ -93,6 +93,7 @@ int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp, hipStream_t st);
 bool attention_bwd_flash16_supports(const AttnBwdParams &bp);
 int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st);
 bool attention_bwd_flash32_supports(const AttnBwdParams &bp);
+size_t attention_bwd_flash32_lengths_bytes(const AttnBwdParams &bp);
 size_t attention_bwd_flash16_workspace(const AttnParams &p);
 size_t attention_bwd_flash16_mask_bits_bytes(const AttnParams &p);   // 0 when the call does not take the packed-mask path
 size_t attention_bwd_flash16_lengths_bytes(const AttnBwdParams &bp);  // 0 when the call does not take the context-length path

@@ -277,12 +277,15 @@ def test_dense_mask_on_the_lean_paths(nn, oracle, dtype, D, H, Lq, Lkv, batch, m
     ("f16", 64, 2, 300, 1100, 3, False, True, None),
     ("bf16", 96, 1, 513, 520, 5, False, True, (0.2, 5)),
     ("bf16", 128, 2, 200, 332, 4, False, False, None),      # no saved statistics: the key-mask kernels take every pair
+    ("f32", 64, 2, 200, 332, 4, False, True, None),
+    ("f32", 96, 1, 300, 520, 3, False, False, None),        # Float32: also without saved statistics
+    ("f32", 36, 2, 130, 1100, 5, False, True, None),
 ])
 def test_context_lengths_in_the_gradient(nn, oracle, dtype, D, H, Lq, Lkv, B, causal_too, saved, dropout):
     """Key-padding masks with saved statistics: pairs whose mask keeps a prefix of the keys run the unmasked gradient
     kernels on that many keys (the padding gets zero gradients), the others the key-mask kernels."""
-    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, mask_kind="lengths", expect="flash16", saved=saved, dropout=dropout,
-         seed=Lq + Lkv, scale=0.4)
+    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, mask_kind="lengths", expect="flash32" if dtype == "f32" else "flash16",
+         saved=saved, dropout=dropout, seed=Lq + Lkv, scale=0.4)
 
 
 @pytest.mark.parametrize("dtype,D,expect", [("bf16", 96, "flash16"), ("f32", 64, "flash32"), ("f32", 6, "generic")])
