@@ -68,18 +68,18 @@ __global__ __launch_bounds__(256) void mask_bits_kernel(const uint8_t *mask, int
     out[(slice * gridDim.y + qt) * lkv_pad + kv] = word;
 }
 
-// Key-padding masks with saved statistics: the (head, batch) pairs are classified on the device and the pairs whose
-// mask is a context length run the unmasked kernels on that many keys (workgroups past it only write zeros).
+// Key-padding masks: the (head, batch) pairs are classified on the device and the pairs whose mask is a context
+// length run the unmasked kernels on that many keys (workgroups past it only write zeros).
 size_t attention_bwd_flash16_lengths_bytes(const AttnBwdParams &bp) {
-    if (!bp.have_stats || !flash_is_key_mask(bp.p)) return 0;
+    if (!flash_is_key_mask(bp.p) || bp.p.H * bp.p.B > 2147483647LL / 4) return 0;
     return ((size_t)(bp.p.H * bp.p.B) * sizeof(int32_t) + 15) & ~(size_t)15;
 }
 
 int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp_in, hipStream_t st) {
     AttnBwdParams bp = bp_in;
     const AttnParams &p = bp.p;
-    if (attention_bwd_flash16_lengths_bytes(bp) != 0) {   // have_stats and no packed mask bits: the lengths open the workspace
-        int32_t *lens = (int32_t *)bp.workspace;
+    if (attention_bwd_flash16_lengths_bytes(bp) != 0) {   // after the statistics planes when those live in the workspace (no packed mask bits here)
+        int32_t *lens = (int32_t *)((char *)bp.workspace + (bp.have_stats ? 0 : attention_bwd_flash16_workspace(p)));
         const int32_t rc = launch_key_mask_lengths(p, lens, st);
         if (rc != MI_OK) return rc;
         bp.kv_len = lens;

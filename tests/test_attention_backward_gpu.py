@@ -276,7 +276,7 @@ def test_dense_mask_on_the_lean_paths(nn, oracle, dtype, D, H, Lq, Lkv, batch, m
     ("bf16", 128, 2, 200, 332, 4, False, True, None),
     ("f16", 64, 2, 300, 1100, 3, False, True, None),
     ("bf16", 96, 1, 513, 520, 5, False, True, (0.2, 5)),
-    ("bf16", 128, 2, 200, 332, 4, False, False, None),      # no saved statistics: the key-mask kernels take every pair
+    ("bf16", 128, 2, 200, 332, 4, False, False, None),      # without saved statistics: the statistics pass walks the context length too
     ("f32", 64, 2, 200, 332, 4, False, True, None),
     ("f32", 96, 1, 300, 520, 3, False, False, None),        # Float32: also without saved statistics
     ("f32", 36, 2, 130, 1100, 5, False, True, None),
