@@ -3,12 +3,12 @@
 #include "attention_params.h"
 
 // kv_len: null, or per (head, batch) context lengths (FlashArgs::kv_len)
-int32_t launch_flash16_bf16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
-int32_t launch_flash16_bf16_d128(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
-int32_t launch_flash16_f16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
-int32_t launch_flash16_f16_d128(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
-int32_t launch_flash16_bf16_d256(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
-int32_t launch_flash16_f16_d256(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_bf16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
+int32_t launch_flash16_bf16_d128(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
+int32_t launch_flash16_f16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
+int32_t launch_flash16_f16_d128(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
+int32_t launch_flash16_bf16_d256(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
+int32_t launch_flash16_f16_d256(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
 int32_t launch_flash16_fast_bf16(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
 int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
 bool flash16_fast_supports_bf16(const AttnParams &);
@@ -98,7 +98,7 @@ static bool takes_fast_path(const AttnParams &p) { return !p.mask && fast_kernel
 // empty one included), then BOTH forward kernels are launched and every (head, batch) pair is computed by exactly
 // one of them: the pipelined kernel takes the pairs with a length, the general kernel the others.
 static bool takes_length_path(const AttnParams &p) {
-    return flash_is_key_mask(p) && fast_kernel_fits(p) && flash_pick_nsplit(p, 128) == 1 && p.H * p.B <= 2147483647LL / 4;
+    return flash_is_key_mask(p) && flash_pick_nsplit(p, 128) == 1 && p.H * p.B <= 2147483647LL / 4;
 }
 static size_t length_path_workspace(const AttnParams &p) { return ((size_t)(p.H * p.B) * sizeof(int32_t) + 15) & ~(size_t)15; }
 
@@ -145,11 +145,13 @@ int32_t launch_key_mask_lengths(const AttnParams &p, int32_t *lens, hipStream_t 
     return MI_OK;
 }
 
-static int32_t launch_general16(const AttnParams &p, hipStream_t st, const int32_t *kv_len) {
+static int32_t launch_general16(const AttnParams &p, hipStream_t st, const int32_t *kv_len, bool lv = false) {
     const int64_t dmax = p.D > p.Dv ? p.D : p.Dv;
     if (p.dtype == MI_BF16)
-        return dmax <= 64 ? launch_flash16_bf16_d64(p, st, kv_len) : dmax <= 128 ? launch_flash16_bf16_d128(p, st, kv_len) : launch_flash16_bf16_d256(p, st, kv_len);
-    return dmax <= 64 ? launch_flash16_f16_d64(p, st, kv_len) : dmax <= 128 ? launch_flash16_f16_d128(p, st, kv_len) : launch_flash16_f16_d256(p, st, kv_len);
+        return dmax <= 64    ? launch_flash16_bf16_d64(p, st, kv_len, lv)
+               : dmax <= 128 ? launch_flash16_bf16_d128(p, st, kv_len, lv)
+                             : launch_flash16_bf16_d256(p, st, kv_len, lv);
+    return dmax <= 64 ? launch_flash16_f16_d64(p, st, kv_len, lv) : dmax <= 128 ? launch_flash16_f16_d128(p, st, kv_len, lv) : launch_flash16_f16_d256(p, st, kv_len, lv);
 }
 
 static int32_t launch_fast16(const AttnParams &p, hipStream_t st, const int32_t *kv_len) {
@@ -164,7 +166,9 @@ int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
         int32_t *lens = (int32_t *)p.workspace;
         int32_t rc = launch_key_mask_lengths(p, lens, st);
         if (rc != MI_OK) return rc;
-        rc = launch_fast16(p, st, lens);
+        // pairs with a context length: the software-pipelined kernel where it fits the call, else the general kernel's
+        // variant without mask code (weights, dropout, other head dims); the other pairs: the key-mask variant
+        rc = fast_kernel_fits(p) ? launch_fast16(p, st, lens) : launch_general16(p, st, lens, true);
         if (rc != MI_OK) return rc;
         return launch_general16(p, st, lens);
     }

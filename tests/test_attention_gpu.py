@@ -452,8 +452,8 @@ def test_context_length_masks(nn, oracle, dtype, E, H, Lq, Lkv, per_head):
     with np.errstate(invalid="ignore"):
         yr, ar = oracle.nnlib_attention_f32(q, k, v, None, mask, H, nthreads=4)
     ok = [0, 1, 2, 3, 5]
-    for weights in ((False, True) if dtype == "f32" else (False,)):   # Float32: the same path also returns the weights
-        y, a = _run(nn, q, k, v, dtype, None, mask, H, return_weights=weights)
+    for weights in (False, True):   # with the weights: the general kernels' variant without mask code takes the pairs with a length
+        y, a = _run(nn, q, k, v, dtype, None, mask, H, return_weights=weights, weights_dtype="f32" if weights else None)
         assert nn.last_attention_kernel() == ("flash32" if dtype == "f32" else "flash16")
         assert np.isnan(y[:, :, 4]).all() and np.isnan(yr[:, :, 4]).all()
         assert not np.isnan(y[:, :, ok]).any()
