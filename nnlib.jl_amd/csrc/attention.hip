@@ -98,24 +98,20 @@ static bool takes_fast_path(const AttnParams &p) { return !p.mask && fast_kernel
 // empty one included), then BOTH forward kernels are launched and every (head, batch) pair is computed by exactly
 // one of them: the pipelined kernel takes the pairs with a length, the general kernel the others.
 static bool takes_length_path(const AttnParams &p) {
-    return flash_is_key_mask(p) && flash_pick_nsplit(p, 128) == 1 && p.H * p.B <= 2147483647LL / 4;
+    return flash_is_query_independent_mask(p) && flash_pick_nsplit(p, 128) == 1 && p.H * p.B <= 2147483647LL / 4;
 }
 static size_t length_path_workspace(const AttnParams &p) { return ((size_t)(p.H * p.B) * sizeof(int32_t) + 15) & ~(size_t)15; }
 
-__global__ __launch_bounds__(256) void key_mask_lengths_kernel(const uint8_t *mask, int64_t s2, int64_t s3, int64_t Lkv, int64_t H,
-                                                              int32_t *lens) {
+__global__ __launch_bounds__(256) void key_mask_lengths_kernel(const uint8_t *mask, int64_t s0, int64_t s2, int64_t s3, int64_t Lkv,
+                                                              int64_t H, int32_t *lens) {
     const int64_t h = blockIdx.x % H, b = blockIdx.x / H;
-    const uint8_t *m = mask + h * s2 + b * s3;   // unit key stride, 4-byte aligned, Lkv a multiple of 4 (flash_is_key_mask)
+    const uint8_t *m = mask + h * s2 + b * s3;   // one byte per key, any key stride and alignment
     int last = -1, count = 0;
-    for (int64_t j = 4 * (int64_t)threadIdx.x; j < Lkv; j += 4 * 256) {
-        const uint32_t w = *(const uint32_t *)(m + j);
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-            if ((w >> (8 * e)) & 0xFFu) {
-                last = (int)j + e;
-                count++;
-            }
-    }
+    for (int64_t j = threadIdx.x; j < Lkv; j += 256)
+        if (m[j * s0]) {
+            last = (int)j;
+            count++;
+        }
     __shared__ int s_last[4], s_count[4];
     for (int off = 32; off > 0; off >>= 1) {
         const int o_last = __shfl_xor(last, off, 64);
@@ -139,8 +135,8 @@ __global__ __launch_bounds__(256) void key_mask_lengths_kernel(const uint8_t *ma
 
 int32_t launch_key_mask_lengths(const AttnParams &p, int32_t *lens, hipStream_t st) {
     if (p.H * p.B > 2147483647LL) return mi_set_error(MI_ESHAPE, "attention: too many (head, batch) pairs");
-    hipLaunchKernelGGL(key_mask_lengths_kernel, dim3((unsigned)(p.H * p.B)), dim3(256), 0, st, p.mask, p.mask_strides[2],
-                       p.mask_strides[3], p.Lkv, p.H, lens);
+    hipLaunchKernelGGL(key_mask_lengths_kernel, dim3((unsigned)(p.H * p.B)), dim3(256), 0, st, p.mask, p.mask_strides[0],
+                       p.mask_strides[2], p.mask_strides[3], p.Lkv, p.H, lens);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }

@@ -37,7 +37,7 @@ size_t attention_bwd_flash16_workspace(const AttnParams &p) { return attention_s
 // the queries, so it wants the mask of (its key, the 64 queries of a tile) as one 64-bit word: a small kernel packs
 // those words once per call, [slice][query tile][key], slices being the distinct (head, batch) planes of the mask.
 static bool takes_mask_bits(const AttnParams &p) {
-    if (!p.mask || p.bias || p.D > 128 || flash_is_key_mask(p) || (p.Lkv & 3) != 0) return false;
+    if (!p.mask || p.bias || p.D > 128 || flash_is_query_independent_mask(p) || (p.Lkv & 3) != 0) return false;
     FlashArgs a;
     a.p = p;
     a.p.weights = nullptr;
@@ -71,7 +71,8 @@ __global__ __launch_bounds__(256) void mask_bits_kernel(const uint8_t *mask, int
 // Key-padding masks: the (head, batch) pairs are classified on the device and the pairs whose mask is a context
 // length run the unmasked kernels on that many keys (workgroups past it only write zeros).
 size_t attention_bwd_flash16_lengths_bytes(const AttnBwdParams &bp) {
-    if (!flash_is_key_mask(bp.p) || bp.p.H * bp.p.B > 2147483647LL / 4) return 0;
+    // with dropout the kernels without mask code need whole hash groups per run of four keys (Lkv a multiple of 4)
+    if (!flash_is_query_independent_mask(bp.p) || (bp.p.drop_thresh && (bp.p.Lkv & 3) != 0) || bp.p.H * bp.p.B > 2147483647LL / 4) return 0;
     return ((size_t)(bp.p.H * bp.p.B) * sizeof(int32_t) + 15) & ~(size_t)15;
 }
 

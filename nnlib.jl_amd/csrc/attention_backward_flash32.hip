@@ -522,7 +522,7 @@ int32_t launch_d(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
 
 // context lengths of a key-padding mask (no dropout: that runs on the per-element paths), one per (head, batch) pair
 size_t attention_bwd_flash32_lengths_bytes(const AttnBwdParams &bp) {
-    if (bp.p.drop_thresh || !flash_is_key_mask(bp.p) || bp.p.H * bp.p.B > 2147483647LL / 4) return 0;
+    if (bp.p.drop_thresh || !flash_is_query_independent_mask(bp.p) || bp.p.H * bp.p.B > 2147483647LL / 4) return 0;
     return ((size_t)(bp.p.H * bp.p.B) * sizeof(int32_t) + 15) & ~(size_t)15;
 }
 

@@ -254,7 +254,7 @@ int32_t launch_d(const FlashArgs &a, hipStream_t st, bool extras) {
 
 // context lengths of a key-padding mask, one per (head, batch) pair: workspace of the calls that take that path
 size_t attention_flash32_lengths_bytes(const AttnParams &p) {
-    if (!flash_is_key_mask(p) || p.H * p.B > 2147483647LL / 4) return 0;
+    if (!flash_is_query_independent_mask(p) || p.H * p.B > 2147483647LL / 4) return 0;
     return ((size_t)(p.H * p.B) * sizeof(int32_t) + 15) & ~(size_t)15;
 }
 

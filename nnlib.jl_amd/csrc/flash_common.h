@@ -84,6 +84,11 @@ constexpr bool flash_uses_staging(int extras) { return extras == EXTRAS_STAGED |
 constexpr bool flash_natural_units(int extras) { return extras == EXTRAS_DIRECT || extras == EXTRAS_STAGED; }
 // query-independent mask without bias whose bytes can be read four keys at a time (unit key stride, Lkv a
 // multiple of 4, 4-byte aligned slices): eligible for EXTRAS_KEYMASK
+// any mask without bias that does not depend on the query (a key-padding mask), whatever its strides: what the
+// device-side measurement of context lengths (FlashArgs::kv_len) applies to
+inline bool flash_is_query_independent_mask(const AttnParams &p) {
+    return p.mask && !p.bias && (p.mask_strides[1] == 0 || p.Lq == 1);
+}
 inline bool flash_is_key_mask(const AttnParams &p) {
     return p.mask && !p.bias && p.mask_strides[1] == 0 && p.mask_strides[0] == 1 && (p.Lkv & 3) == 0 &&
            ((p.mask_strides[2] | p.mask_strides[3]) & 3) == 0 && (((uintptr_t)p.mask) & 3) == 0;

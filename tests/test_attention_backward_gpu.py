@@ -280,6 +280,11 @@ def test_dense_mask_on_the_lean_paths(nn, oracle, dtype, D, H, Lq, Lkv, batch, m
     ("f32", 64, 2, 200, 332, 4, False, True, None),
     ("f32", 96, 1, 300, 520, 3, False, False, None),        # Float32: also without saved statistics
     ("f32", 36, 2, 130, 1100, 5, False, True, None),
+    # lengths that are not multiples of 4 (mask rows unaligned): the pairs without a length run the per-element paths
+    ("bf16", 128, 2, 200, 333, 4, False, True, None),
+    ("f16", 64, 1, 130, 1101, 3, False, False, None),
+    ("f32", 64, 2, 130, 333, 3, False, True, None),
+    ("bf16", 64, 2, 100, 333, 3, False, True, (0.2, 9)),    # with dropout the unaligned case stays on the per-element paths
 ])
 def test_context_lengths_in_the_gradient(nn, oracle, dtype, D, H, Lq, Lkv, B, causal_too, saved, dropout):
     """Key-padding masks with saved statistics: pairs whose mask keeps a prefix of the keys run the unmasked gradient

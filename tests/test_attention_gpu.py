@@ -432,7 +432,8 @@ def test_key_padding_masks(nn, oracle, dtype, E, H, weights):
 
 
 @pytest.mark.parametrize("dtype,E,H,Lq,Lkv", [("bf16", 256, 2, 140, 332), ("f16", 128, 2, 300, 1100), ("bf16", 128, 1, 513, 2048),
-                                              ("f32", 128, 2, 140, 332), ("f32", 72, 2, 300, 1100)])
+                                              ("f32", 128, 2, 140, 332), ("f32", 72, 2, 300, 1100),
+                                              ("bf16", 256, 2, 140, 333), ("f16", 64, 1, 513, 2049), ("f32", 128, 2, 140, 333)])
 @pytest.mark.parametrize("per_head", [False, True], ids=["per-batch", "per-head"])
 def test_context_length_masks(nn, oracle, dtype, E, H, Lq, Lkv, per_head):
     """Key-padding masks that keep a prefix of the keys (padded batches): a device-side pass measures every (head,
