@@ -95,6 +95,30 @@ def test_plan_kernel_selection(L):
     assert K[_plan(L, _desc(L, dtype=L.MI_BF16, weights_dtype=L.MI_BF16, **dict(big, q=0x1002)))[1]] == "generic"
 
 
+def test_plan_workspace_for_key_padding_masks(L):
+    """A mask without bias that does not depend on the query is measured on the device first (context lengths, one
+    Int32 per (head, batch) pair): the planner asks for that buffer, for 16-bit and Float32 calls, forward and gradient."""
+    big = dict(E=4096, Ev=4096, H=32, Lq=4096, Lkv=4096, B=2)
+    strides = (ctypes.c_int64 * 4)(1, 0, 0, 4096)                    # (Lkv, 1, 1, B)
+    lens_bytes = 32 * 2 * 4
+    for dt in (L.MI_BF16, L.MI_F32):
+        d = _desc(L, dtype=dt, weights_dtype=dt, mask=0x2000, **big)
+        d.mask_strides = strides
+        rc, kern, ws = _plan(L, d)
+        assert rc == L.MI_OK and ws == lens_bytes, (dt, ws)
+        dense = _desc(L, dtype=dt, weights_dtype=dt, mask=0x2000, **big)
+        dense.mask_strides = (ctypes.c_int64 * 4)(1, 4096, 0, 0)     # depends on the query: no lengths
+        assert _plan(L, dense)[2] == 0
+        b = L.mi_attn_bwd_desc()
+        b.struct_size = ctypes.sizeof(L.mi_attn_bwd_desc)
+        b.fwd = d
+        b.dout = b.dq = b.dk = b.dv = 0x3000
+        kern, ws = ctypes.c_int32(-1), ctypes.c_size_t(0)
+        assert L.load().mi_attention_bwd_plan(ctypes.byref(b), ctypes.byref(kern), ctypes.byref(ws)) == L.MI_OK
+        stats_bytes = 4 * 3 * 2 * 32 * 4096
+        assert ws.value == stats_bytes + lens_bytes, (dt, ws.value)   # statistics planes (none saved here), then the lengths
+
+
 def test_host_side_argument_checks_of_other_entry_points(L):
     lib = L.load()
     assert lib.mi_softmax_dim1(9, None, None, 4, 4, None) == L.MI_EDTYPE
