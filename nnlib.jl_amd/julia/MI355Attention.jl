@@ -20,7 +20,7 @@
 # (no Julia toolchain there); the Python mirror in nnlib_amd/ exercises the same entry points.
 module MI355Attention
 
-export DeviceArray, CausalMask, dot_product_attention, dot_product_attention_scores, make_causal_mask,
+export DeviceArray, CausalMask, CausalAnd, dot_product_attention, dot_product_attention_scores, make_causal_mask,
        softmax, softmax!, logsoftmax, logsoftmax!, logsumexp, ∇logsumexp, ∇softmax, ∇softmax!, ∇logsoftmax, ∇logsoftmax!,
        batched_mul, batched_mul!, batched_vec, batched_transpose, batched_adjoint, batched_mul_pullback,
        Dropout, dropout, ∇dot_product_attention
@@ -134,6 +134,18 @@ Base.size(m::CausalMask) = (m.len, m.len)
 Base.getindex(m::CausalMask, i::Int, j::Int) = i <= j
 make_causal_mask(x::DeviceArray; dims::Int = 2) = CausalMask(size(x, dims))
 
+# `make_causal_mask(x) .& padding` (a causal language model on a padded batch): the reference materialises the
+# product; here the causal half stays symbolic and the Bool array rides along, so that the kernels apply the causal
+# pattern from indices and read only the array (a key-padding mask of size (kv_len, 1, 1, batch) is then measured on
+# the device and becomes per-sequence context lengths).
+struct CausalAnd
+    len::Int
+    array::DeviceArray{Bool}
+end
+Base.Broadcast.broadcasted(::typeof(&), m::CausalMask, a::DeviceArray{Bool}) = CausalAnd(m.len, a)
+Base.Broadcast.broadcasted(::typeof(&), a::DeviceArray{Bool}, m::CausalMask) = CausalAnd(m.len, a)
+Base.Broadcast.materialize(m::CausalAnd) = m      # `.&` calls materialize on what broadcasted returned
+
 # ---- attention -------------------------------------------------------------------------------------
 # Mirror of `mi_attn_desc` (include/mi355attn.h); field order and sizes must match the header.
 struct AttnDesc
@@ -199,10 +211,12 @@ end
 function mask_and_bias(::Type{T}, bias, mask, target::NTuple{4, Int}) where {T}
     Lkv, Lq = target[1], target[2]
     causal, mptr, mstr = Int32(0), C_NULL, ntuple(_ -> Int64(0), 4)
-    if mask isa CausalMask
-        (mask.len == Lkv == Lq) || throw(DimensionMismatch("arrays could not be broadcast to a common size: mask has size $(size(mask)), attention scores have size $target"))
+    if mask isa CausalMask || mask isa CausalAnd
+        (mask.len == Lkv == Lq) || throw(DimensionMismatch("arrays could not be broadcast to a common size: mask has size $((mask.len, mask.len)), attention scores have size $target"))
         causal = Int32(1)
-    elseif mask !== nothing
+        mask = mask isa CausalAnd ? mask.array : nothing      # causal .& array: the flag and the array together
+    end
+    if mask !== nothing
         mask isa DeviceArray{Bool} || throw(ArgumentError("mask must be a Bool DeviceArray or a CausalMask"))
         mptr, mstr = mask.ptr, broadcast_strides(mask, target, "mask")
     end

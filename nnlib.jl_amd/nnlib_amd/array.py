@@ -247,3 +247,26 @@ class CausalMask:
 
     def to_numpy(self):
         return self.materialize().to_numpy()
+
+    def __and__(self, other):
+        """``make_causal_mask(x) .& padding`` in the reference materialises the product; here the causal half stays
+        symbolic and the Bool array (e.g. a key-padding mask of size (kv_len, 1, 1, batch)) rides along, so that the
+        kernels apply the causal pattern from indices and read only the array."""
+        if isinstance(other, CausalAnd):
+            return CausalAnd(self.length, other.array)
+        if not isinstance(other, DeviceArray) or other.dtype != "bool":
+            raise ArgumentError("a causal mask combines with a Bool DeviceArray")
+        return CausalAnd(self.length, other)
+
+    __rand__ = __and__
+
+
+class CausalAnd:
+    """Elementwise AND of the causal pattern with a Bool array, kept as the pair (see CausalMask.__and__)."""
+
+    def __init__(self, length, array):
+        self.length = int(length)
+        self.array = array
+
+    def materialize(self):
+        raise ArgumentError("materialise the two halves separately: CausalMask(length).materialize() and .array")

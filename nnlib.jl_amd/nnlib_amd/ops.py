@@ -11,7 +11,7 @@ import torch
 
 from . import _lib
 from ._lib import ArgumentError, DimensionMismatch
-from .array import BatchedTranspose, CausalMask, DeviceArray, batched_transpose
+from .array import BatchedTranspose, CausalAnd, CausalMask, DeviceArray, batched_transpose
 
 __all__ = ["dot_product_attention", "dot_product_attention_scores", "make_causal_mask", "softmax", "softmax_",
            "logsoftmax", "logsoftmax_", "logsumexp", "grad_softmax", "grad_softmax_", "grad_logsoftmax",
@@ -116,12 +116,13 @@ def _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags, fdrop=None):
         d.bias = bias.ptr
         d.bias_strides = (ctypes.c_int64 * 4)(*st)
     d.causal = 0
-    if isinstance(mask, CausalMask):
+    if isinstance(mask, (CausalMask, CausalAnd)):
         if mask.length != Lkv or mask.length != Lq:
-            raise DimensionMismatch(f"arrays could not be broadcast to a common size: mask has size {mask.dims}, "
+            raise DimensionMismatch(f"arrays could not be broadcast to a common size: mask has size {(mask.length, mask.length)}, "
                                     f"attention scores have size {target}")
         d.causal = 1
-    elif mask is not None:
+        mask = mask.array if isinstance(mask, CausalAnd) else None   # causal .& array: the flag and the array together
+    if mask is not None:
         if mask.dtype != "bool":
             raise ArgumentError("mask must be a Bool array")
         st = _broadcast_strides(mask, target, "mask")

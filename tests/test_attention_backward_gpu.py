@@ -427,3 +427,34 @@ def test_batched_mul_pullback(nn, oracle, shared):
         rB = rB.sum(axis=2, keepdims=True)
     assert dA.dims == rA.shape and dB.dims == rB.shape
     assert np.abs(dA.to_numpy() - rA).max() < 1e-4 and np.abs(dB.to_numpy() - rB).max() < 1e-4
+
+
+@pytest.mark.parametrize("dtype,D,H,L,B,saved", [("bf16", 128, 2, 300, 4, True), ("f16", 64, 2, 513, 3, False), ("f32", 64, 2, 200, 3, True),
+                                                 ("bf16", 96, 1, 333, 3, True)])
+def test_causal_and_padding_mask(nn, oracle, dtype, D, H, L, B, saved):
+    """`make_causal_mask(x) .& padding` (a causal language model on a padded batch): the causal half stays symbolic, the
+    key-padding array is measured on the device; forward output and gradients against the oracle with the dense product."""
+    rng = np.random.default_rng(L + D)
+    E = D * H
+    q, k, v, dy = (round_to(rng.standard_normal((E, L, B)) * sc, dtype) for sc in (0.4, 0.4, 1.0, 1.0))
+    pad = np.ones((L, 1, 1, B), dtype=bool)
+    pad[L - 77:, 0, 0, 1] = False                 # a padded tail
+    pad[:, 0, 0, 2] = rng.random(L) < 0.7         # scattered (not a context length)
+    pad[0, 0, 0, 2] = True
+    dense = oracle.make_causal_mask(L)[:, :, None, None] & pad
+    Dv = nn.DeviceArray.from_numpy
+    dq_, dk_, dv_, ddy = Dv(q, dtype), Dv(k, dtype), Dv(v, dtype), Dv(dy, dtype)
+    mask = nn.make_causal_mask(dq_) & Dv(pad)
+    assert isinstance(mask, nn.CausalAnd)
+    y, a = nn.dot_product_attention(dq_, dk_, dv_, mask=mask, nheads=H, weights_dtype="f32", save_for_backward=saved)
+    yr, ar = oracle.nnlib_attention_f32(q, k, v, None, dense, H, nthreads=4)
+    assert rel_err(y.to_numpy(), yr) <= TOL[dtype]
+    assert np.abs(a.to_numpy() - ar).max() <= TOL[dtype]
+    assert np.count_nonzero(a.to_numpy()[~np.broadcast_to(dense, ar.shape)]) == 0
+    y2, _ = nn.dot_product_attention(dq_, dk_, dv_, mask=mask, nheads=H, return_weights=False, save_for_backward=saved)
+    assert rel_err(y2.to_numpy(), yr) <= TOL[dtype]
+    got = nn.dot_product_attention_grad(ddy, dq_, dk_, dv_, y=y2, mask=mask, nheads=H)
+    ref = oracle.attention_bwd_f64(q, k, v, dy, None, dense, H)
+    for g, r_, name in zip(got[:3], ref[:3], ("dq", "dk", "dv")):
+        err = np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05)
+        assert err <= TOL[dtype], (name, err)
