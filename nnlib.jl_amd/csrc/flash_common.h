@@ -54,10 +54,7 @@ inline int flash_pick_nsplit(const AttnParams &p, int bm) {
     const int64_t wgs = ((p.Lq + bm - 1) / bm) * p.H * p.B;
     if (wgs >= 512 || p.Lkv < 2048) return 1;
     // aim at one resident round: two workgroups per CU on 256 CUs (measured best on the f16 cross-attention case)
-#ifndef FLASH_SPLIT_TARGET
-#define FLASH_SPLIT_TARGET 512
-#endif
-    int64_t n = (FLASH_SPLIT_TARGET + wgs - 1) / wgs;
+    int64_t n = (512 + wgs - 1) / wgs;
     const int64_t max_by_len = p.Lkv / 512;                 // at least 512 keys per piece
     if (n > max_by_len) n = max_by_len;
     if (n > 64) n = 64;
