@@ -1,10 +1,10 @@
-// Split-kv attention for a single query per (head, batch) ("decode" shape, Lq = 1), bf16 / f16.
+// Split-kv attention for a single query per (head, batch) ("decode" shape, Lq = 1), bf16 / f16 / Float32.
 //
 // The work is a stream over K and V: every byte is read once and used once, so the kernel is
 // organised around HBM, not around the matrix cores.  A kv row (all heads) is E contiguous elements;
-// a wavefront owns a 512-element segment of the row (4 heads at D = 128, 8 heads at D = 64), each
-// lane 8 consecutive features (one 16-byte load), and walks a contiguous range of kv rows.  The
-// dot product over a head is finished with a butterfly over the D/8 lanes that share the head.
+// a wavefront owns a 1 KiB segment of the row (512 16-bit features: 4 heads at D = 128, 8 heads at D = 64; half as
+// many in Float32), each lane one 16-byte load (8 or 4 consecutive features), and walks a contiguous range of kv
+// rows.  The dot product over a head is finished with a butterfly over the lanes that share the head.
 // Each (segment, kv-split, batch) wavefront keeps an online-softmax state (m, l, o[8]) and writes it
 // to a workspace; a second small kernel merges the splits.
 //
@@ -22,7 +22,9 @@
 namespace {
 
 constexpr int ROWS = 8;        // kv rows in flight per lane and tensor
-constexpr int SEG = 512;       // features per wavefront
+// features per lane (one 16-byte load) and per wavefront
+template <typename T> constexpr int epl() { return 16 / (int)sizeof(typename T::type); }
+template <typename T> constexpr int seg_width() { return 64 * epl<T>(); }
 
 struct DecodeArgs {
     AttnParams p;
@@ -44,6 +46,11 @@ __device__ inline void unpack8(const u32x4_t &v, float *out, F16) {
 #pragma unroll
     for (int e = 0; e < 8; e++) out[e] = (float)h[e];
 }
+__device__ inline void unpack8(const u32x4_t &v, float *out, F32) {   // four features
+    const floatx4_t h = __builtin_bit_cast(floatx4_t, v);
+#pragma unroll
+    for (int e = 0; e < 4; e++) out[e] = h[e];
+}
 
 // workspace layout: [B][nsplit][E] floats of o, then [B][nsplit][H] of m, then [B][nsplit][H] of l
 template <typename T, int D, bool MASKED, bool SCORES>
@@ -51,18 +58,19 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     const AttnParams &p = a.p;
     typedef typename T::type t;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int EPL = epl<T>(), SEG = seg_width<T>(), LPH = D / EPL;   // features per lane and wavefront, lanes per head
     constexpr int NH = SEG / D;                        // heads per wavefront
     __shared__ float sc_lds[SCORES ? 4 * NH * 64 : 1]; // scores on their way out: [wavefront][head][64 keys]
     const int seg = blockIdx.x * 4 + wave;
     const int split = blockIdx.y;
     const int64_t b = blockIdx.z;
-    const int64_t f = (int64_t)seg * SEG + lane * 8;   // first feature of this lane
-    const bool lane_ok = f < p.E;                      // E is a multiple of 8 (D is 64 or 128)
+    const int64_t f = (int64_t)seg * SEG + lane * EPL; // first feature of this lane
+    const bool lane_ok = f < p.E;                      // E is a multiple of EPL (D is 64 or 128)
     if (seg >= a.nseg) return;
 
     const t *kb = (const t *)p.k + p.E * p.Lkv * b + (lane_ok ? f : 0);
     const t *vb = (const t *)p.v + p.E * p.Lkv * b + (lane_ok ? f : 0);
-    float qf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float qf[EPL] = {};
     if (lane_ok) unpack8(*(const u32x4_t *)((const t *)p.q + p.E * b + f), qf, T());
 
     const int64_t j_begin = (int64_t)split * a.rows_per_split;
@@ -70,7 +78,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     if (j_end > p.Lkv) j_end = p.Lkv;
 
     float m = MI_NEG_INF, l = 0.0f;
-    float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float o[EPL] = {};
     const u32x4_t zero = {0, 0, 0, 0};
     // mask bytes of this lane's head: element (kv, 0, h, b)
     const uint8_t *mrow = MASKED ? p.mask + (lane_ok ? f / D : 0) * p.mask_strides[2] + b * p.mask_strides[3] : nullptr;
@@ -94,13 +102,13 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
         float mx = MI_NEG_INF;
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
-            float kf[8];
+            float kf[EPL];
             unpack8(kr[r], kf, T());
             float d = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; e++) d = fmaf(kf[e], qf[e], d);
+            for (int e = 0; e < EPL; e++) d = fmaf(kf[e], qf[e], d);
 #pragma unroll
-            for (int off = 1; off < D / 8; off <<= 1) d += __shfl_xor(d, off, 64);
+            for (int off = 1; off < LPH; off <<= 1) d += __shfl_xor(d, off, 64);
             s[r] = keep[r] ? d : MI_NEG_INF;
             mx = fmaxf(mx, s[r]);
         }
@@ -111,15 +119,15 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
         mnew = mref;
         l *= resc;
 #pragma unroll
-        for (int e = 0; e < 8; e++) o[e] *= resc;
+        for (int e = 0; e < EPL; e++) o[e] *= resc;
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
             const float pr = mi_exp2((s[r] - mnew) * a.c);
             l += pr;
-            float vf[8];
+            float vf[EPL];
             unpack8(vr[r], vf, T());
 #pragma unroll
-            for (int e = 0; e < 8; e++) o[e] = fmaf(pr, vf[e], o[e]);
+            for (int e = 0; e < EPL; e++) o[e] = fmaf(pr, vf[e], o[e]);
         }
         if (SCORES) {
             // Scores leave in runs of 64 keys per head (256 contiguous bytes): written 32 bytes at a time, one piece per
@@ -127,8 +135,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
             // of each head parks the 8 scores of this iteration in the wavefront's LDS rows; every 8th iteration the
             // 64 lanes write one row per head.
             const int slot8 = (int)(((j - j_begin) / ROWS) & 7);
-            if ((lane & (D / 8 - 1)) == 0) {
-                float *row = sc_lds + (wave * NH + lane / (D / 8)) * 64 + 8 * slot8;
+            if ((lane & (LPH - 1)) == 0) {
+                float *row = sc_lds + (wave * NH + lane / LPH) * 64 + 8 * slot8;
                 *(floatx4_t *)row = (floatx4_t){s[0], s[1], s[2], s[3]};
                 *(floatx4_t *)(row + 4) = (floatx4_t){s[4], s[5], s[6], s[7]};
             }
@@ -154,8 +162,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     const int64_t slot = b * a.nsplit + split;
     float *wo = ws + slot * p.E + f;
     *(floatx4_t *)wo = (floatx4_t){o[0], o[1], o[2], o[3]};
-    *(floatx4_t *)(wo + 4) = (floatx4_t){o[4], o[5], o[6], o[7]};
-    if ((lane & (D / 8 - 1)) == 0) {
+    if constexpr (EPL == 8) *(floatx4_t *)(wo + 4) = (floatx4_t){o[4], o[5], o[6], o[7]};
+    if ((lane & (LPH - 1)) == 0) {
         const int64_t h = f / D;
         float *wm = ws + (int64_t)p.B * a.nsplit * p.E;
         float *wl = wm + (int64_t)p.B * a.nsplit * p.H;
@@ -236,6 +244,7 @@ __global__ __launch_bounds__(256) void decode_weights_kernel(DecodeArgs a, TW *w
 
 int pick_nsplit(const AttnParams &p) {
     // enough wavefronts to cover the chip several times over, at least 256 rows per split
+    const int64_t SEG = p.dtype == MI_F32 ? seg_width<F32>() : seg_width<BF16>();
     const int64_t nseg = (p.E + SEG - 1) / SEG;
     int64_t want = 8192 / (nseg * p.B > 0 ? nseg * p.B : 1);
     int64_t maxs = (p.Lkv + 255) / 256;
@@ -248,7 +257,6 @@ int pick_nsplit(const AttnParams &p) {
 }  // namespace
 
 bool attention_decode_supports(const AttnParams &p) {
-    if (p.dtype != MI_F16 && p.dtype != MI_BF16) return false;
     if (p.Lq != 1 || p.bias || p.causal || !p.out || p.drop_thresh || p.stats) return false;   // saved statistics: the tiled kernels write them
     if (p.weights && p.H * p.B > 65535) return false;
     if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
@@ -271,6 +279,7 @@ int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
     a.nsplit = pick_nsplit(p);
     a.rows_per_split = (int32_t)((p.Lkv + a.nsplit - 1) / a.nsplit);
     a.nsplit = (int32_t)((p.Lkv + a.rows_per_split - 1) / a.rows_per_split);  // no empty split
+    const int64_t SEG = p.dtype == MI_F32 ? seg_width<F32>() : seg_width<BF16>();
     a.nseg = (int32_t)((p.E + SEG - 1) / SEG);
     if ((((uintptr_t)p.workspace) & 15) != 0)
         return mi_set_error(MI_EWORKSPACE, "decode workspace must be 16-byte aligned");
@@ -296,6 +305,10 @@ int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
         if (p.D == 128) DECODE_LAUNCH(BF16, 128) else DECODE_LAUNCH(BF16, 64)
         MI_LAUNCH_CHECK();
         hipLaunchKernelGGL(decode_merge_kernel<BF16>, mgrid, dim3(256), 0, st, a);
+    } else if (p.dtype == MI_F32) {
+        if (p.D == 128) DECODE_LAUNCH(F32, 128) else DECODE_LAUNCH(F32, 64)
+        MI_LAUNCH_CHECK();
+        hipLaunchKernelGGL(decode_merge_kernel<F32>, mgrid, dim3(256), 0, st, a);
     } else {
         if (p.D == 128) DECODE_LAUNCH(F16, 128) else DECODE_LAUNCH(F16, 64)
         MI_LAUNCH_CHECK();

@@ -288,7 +288,8 @@ def test_flash32_parity(nn, oracle, case, weights):
 
 
 @pytest.mark.parametrize("dtype,E,H,Lkv,B", [("bf16", 512, 4, 1500, 2), ("bf16", 256, 2, 4096, 3), ("f16", 512, 8, 777, 1),
-                                             ("f16", 1024, 8, 2048, 2), ("bf16", 128, 1, 513, 1)])
+                                             ("f16", 1024, 8, 2048, 2), ("bf16", 128, 1, 513, 1),
+                                             ("f32", 512, 4, 1500, 2), ("f32", 256, 4, 2048, 3), ("f32", 64, 1, 777, 1)])
 @pytest.mark.parametrize("weights", [False, True], ids=["noweights", "weights"])
 def test_decode_parity(nn, oracle, dtype, E, H, Lkv, B, weights):
     """Split-kv path for a single query per (head, batch); with the weights returned (as the reference always does)
@@ -298,7 +299,7 @@ def test_decode_parity(nn, oracle, dtype, E, H, Lkv, B, weights):
 
 
 @pytest.mark.parametrize("dtype,E,H,mask_shape", [("bf16", 512, 4, (1500, 1, 1, 3)), ("f16", 256, 4, (1500, 1, 4, 3)),
-                                                  ("bf16", 128, 2, (1500,))])
+                                                  ("bf16", 128, 2, (1500,)), ("f32", 256, 2, (1500, 1, 2, 3))])
 def test_decode_with_context_length_masks(nn, oracle, dtype, E, H, mask_shape):
     """A single query per (head, batch) with a mask: padded contexts of different lengths per batch element, a
     pattern per head, one (head, batch) pair with nothing kept (NaN, src/softmax.jl:73-75)."""
