@@ -62,6 +62,8 @@ int32_t launch_flash_merge(const AttnParams &p, int nsplit, hipStream_t st) {
     const float *ws = (const float *)p.workspace;
     if (p.dtype == MI_BF16)
         hipLaunchKernelGGL(flash_merge_kernel<BF16>, grid, dim3(256), 0, st, ws, (__bf16 *)p.out, nsplit, p.B, p.Lq, p.Ev, p.H);
+    else if (p.dtype == MI_F32)
+        hipLaunchKernelGGL(flash_merge_kernel<F32>, grid, dim3(256), 0, st, ws, (float *)p.out, nsplit, p.B, p.Lq, p.Ev, p.H);
     else
         hipLaunchKernelGGL(flash_merge_kernel<F16>, grid, dim3(256), 0, st, ws, (_Float16 *)p.out, nsplit, p.B, p.Lq, p.Ev, p.H);
     MI_LAUNCH_CHECK();
@@ -241,7 +243,8 @@ static int32_t choose(const mi_attn_desc *d, const AttnParams &p, size_t *ws) {
         return MI_ATTN_KERNEL_FLASH16;
     }
     if (attention_flash32_supports(p)) {
-        *ws = attention_flash32_lengths_bytes(p);
+        const int nsplit = attention_flash32_nsplit(p);
+        *ws = nsplit > 1 ? flash_split_workspace(p, nsplit) : attention_flash32_lengths_bytes(p);
         return MI_ATTN_KERNEL_FLASH32;
     }
     return MI_ATTN_KERNEL_GENERIC;

@@ -38,7 +38,7 @@ __device__ inline floatx4_t ldg16f(const float *p, bool ok) {
 template <int D, int QB, bool CAUSAL, bool EXTRAS, int PHASE>
 // kv_len: keys of this (head, batch) pair (L_kv, or a shorter context length)
 __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *Ks, float *Vs, int64_t kv_len, int64_t b, int64_t h,
-                                   int64_t iw, int n_tiles, unsigned wlds = 0) {
+                                   int64_t iw, int n_tiles, unsigned wlds = 0, int jt0 = 0) {
     constexpr int KS = Cfg<D>::KS, VS = Cfg<D>::VS, CHUNKS = Cfg<D>::CHUNKS;
     const AttnParams &p = a.p;
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hh = lane >> 5;
@@ -72,14 +72,14 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
         }
     };
 
-    if (n_tiles <= 0) return;
-    load_tile(0);
+    if (n_tiles <= jt0) return;
+    load_tile(jt0);
     __syncthreads();
     store_tile(0);
     __syncthreads();
 
-    for (int jt = 0; jt < n_tiles; jt++) {
-        const int buf = jt & 1;
+    for (int jt = jt0; jt < n_tiles; jt++) {
+        const int buf = (jt - jt0) & 1;
         const int64_t j0 = (int64_t)jt * BN;
         if (jt + 1 < n_tiles) load_tile(jt + 1);
 
@@ -143,7 +143,8 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
     const int64_t HB = p.H * p.B;
-    const int64_t id = blockIdx.x;
+    const int split = (int)(blockIdx.x % a.nsplit);   // split-kv: this workgroup's piece of the key range
+    const int64_t id = blockIdx.x / a.nsplit;
     const int64_t hb = id % HB;
     const int64_t qt = a.n_qtiles - 1 - id / HB;   // heaviest (latest) query tiles first
     const int64_t h = hb % p.H, b = hb / p.H;
@@ -182,7 +183,38 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
     const int n_tiles = (int)((kv_end + BN - 1) / BN);
 
     if (!WEIGHTS) {
-        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_ONLINE>(a, f, Ks, Vs, kv_len, b, h, iw, n_tiles);
+        int jt0 = 0, jt1 = n_tiles;
+        if (a.nsplit > 1) {
+            jt0 = split * a.tiles_per_split;
+            if (jt0 + a.tiles_per_split < jt1) jt1 = jt0 + a.tiles_per_split;
+        }
+        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_ONLINE>(a, f, Ks, Vs, kv_len, b, h, iw, jt1, 0, jt0);
+        if (a.nsplit > 1) {
+            // partial result of this key piece for flash_merge_kernel: unnormalised o, row maximum (log2 units), row sum
+            float *wo = (float *)p.workspace + ((int64_t)split * p.B + b) * p.Lq * p.Ev + p.Dv * h;
+            float *wml = (float *)p.workspace + (int64_t)a.nsplit * p.B * p.Lq * p.Ev + (((int64_t)split * p.B + b) * p.H + h) * p.Lq * 2;
+#pragma unroll
+            for (int qb = 0; qb < QB; qb++) {
+                const int64_t qi = iw + 32 * qb + r;
+                const float l = f.l[qb] + mi_swap32(f.l[qb]);
+                if (qi < p.Lq) {
+#pragma unroll
+                    for (int dvb = 0; dvb < D / 32; dvb++)
+#pragma unroll
+                        for (int g = 0; g < 4; g++) {
+                            floatx4_t o4;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) o4[e] = f.o[qb][dvb][4 * g + e];
+                            if (32 * dvb + 8 * g + 4 * hh < p.Dv) *(floatx4_t *)(wo + p.Ev * qi + 32 * dvb + 8 * g + 4 * hh) = o4;
+                        }
+                    if (hh == 0) {
+                        wml[2 * qi] = f.m[qb] * MI_LOG2E;
+                        wml[2 * qi + 1] = l;
+                    }
+                }
+            }
+            return;
+        }
     } else {
         run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_STATS>(a, f, Ks, Vs, kv_len, b, h, iw, n_tiles);
 #pragma unroll
@@ -226,7 +258,7 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
 
 template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS>
 int32_t launch_one(const FlashArgs &a, hipStream_t st) {
-    const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B;
+    const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B * a.nsplit;
     constexpr size_t smem = Cfg<D>::SMEM + (WEIGHTS ? 4 * FLASH_WSTAGE_BYTES : 0);
     auto kern = flash32_kernel<D, QB, CAUSAL, EXTRAS, WEIGHTS>;
     static bool attr_set = false;
@@ -251,6 +283,11 @@ int32_t launch_d(const FlashArgs &a, hipStream_t st, bool extras) {
 }
 
 }  // namespace
+
+int attention_flash32_nsplit(const AttnParams &p) {
+    if (flash_is_query_independent_mask(p) || p.Lq > 65535 || p.B > 65535) return 1;   // context lengths instead / merge kernel's grid limits
+    return flash_pick_nsplit(p, 128);
+}
 
 // context lengths of a key-padding mask, one per (head, batch) pair: workspace of the calls that take that path
 size_t attention_flash32_lengths_bytes(const AttnParams &p) {
@@ -278,6 +315,18 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     a.n_qtiles = (int32_t)((p.Lq + 127) / 128);
     flash_fill_vec_flags(a);
     const bool narrow = p.D <= 64 && p.Dv <= 64;
+    // split-kv as in the 16-bit kernel: few (query tile, head, batch) workgroups and a long key range (calls that
+    // measure context lengths are not split: the planner gives their workspace to the lengths)
+    a.nsplit = attention_flash32_nsplit(p);
+    if (a.nsplit > 1) {
+        const int64_t n_tiles = (p.Lkv + BN - 1) / BN;
+        a.tiles_per_split = (int32_t)((n_tiles + a.nsplit - 1) / a.nsplit);
+        if ((((uintptr_t)p.workspace) & 15) != 0) return mi_set_error(MI_EWORKSPACE, "attention workspace must be 16-byte aligned");
+        const bool extras = p.bias || p.mask;
+        const int32_t rc = narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
+        if (rc != MI_OK) return rc;
+        return launch_flash_merge(p, a.nsplit, st);
+    }
     if (attention_flash32_lengths_bytes(p) != 0) {
         // key-padding mask: classify the (head, batch) pairs on the device, then launch both variants
         int32_t *lens = (int32_t *)p.workspace;

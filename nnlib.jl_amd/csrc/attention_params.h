@@ -110,4 +110,5 @@ size_t attention_decode_workspace(const AttnParams &p);
 bool attention_flash16_supports(const AttnParams &p);
 bool attention_flash32_supports(const AttnParams &p);
 size_t attention_flash32_lengths_bytes(const AttnParams &p);
+int attention_flash32_nsplit(const AttnParams &p);   // pieces the key range is cut into (1: no split)
 bool attention_decode_supports(const AttnParams &p);

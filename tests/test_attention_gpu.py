@@ -350,6 +350,12 @@ SPLIT_CASES = [
     ("f16", 96, 70, 2500, 2, 2, {}),                                  # head dim 48 in 64-wide tiles
     ("bf16", 256, 100, 2300, 2, 1, {}),                               # head dim 256
     ("f16", 256, 130, 2112, 1, 2, dict(mask_shape=(2112, 130))),      # mask tiles staged alone
+    # Float32: the same split + merge
+    ("f32", 128, 100, 3000, 1, 2, dict(bias_shape=(3000, 100, 2, 1), mask_shape=(3000, 100))),
+    ("f32", 64, 70, 2500, 3, 1, {}),
+    ("f32", 256, 130, 2100, 1, 2, dict(mask_shape=(2100, 130))),
+    ("f32", 72, 300, 4096, 1, 2, dict(Ev=160)),                       # head dims 36 / 80
+    ("f32", 128, 2048, 2048, 1, 2, dict(causal=True)),
 ]
 
 
@@ -360,7 +366,7 @@ def test_split_kv_parity(nn, oracle, case):
     dtype, E, Lq, Lkv, B, H, kw = case
     rng = np.random.default_rng(hash((E, Lq, Lkv, B, H, 7)) % 2**32)
     import ctypes
-    _check(nn, oracle, rng, dtype, E, Lq, Lkv, B, H, expect="flash16", weights=False, **kw)
+    _check(nn, oracle, rng, dtype, E, Lq, Lkv, B, H, expect="flash32" if dtype == "f32" else "flash16", weights=False, **kw)
     from nnlib_amd import ops
     assert ops._workspace is not None and ops._workspace.numel() > 0      # the split path was taken
 
