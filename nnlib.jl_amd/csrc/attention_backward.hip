@@ -24,6 +24,8 @@ static int32_t validate_bwd(const mi_attn_bwd_desc *d, AttnBwdParams *out) {
     bp.workspace = d->workspace;
     bp.mask_bits = nullptr;
     bp.kv_len = nullptr;
+    bp.dq_partial = nullptr;
+    bp.dq_nsplit = 1;
     bp.mb_h = bp.mb_b = bp.mb_lkv_pad = bp.mb_nqt = 0;
     bp.have_stats = d->fwd.stats != nullptr;
     bp.stats = bp.have_stats ? d->fwd.stats : (float *)d->workspace;
@@ -34,7 +36,7 @@ static int32_t validate_bwd(const mi_attn_bwd_desc *d, AttnBwdParams *out) {
 static int32_t choose_bwd(const mi_attn_bwd_desc *d, const AttnBwdParams &bp, size_t *ws) {
     if (!(d->fwd.flags & MI_ATTN_FORCE_GENERIC) && attention_bwd_flash16_supports(bp)) {
         *ws = (bp.have_stats ? 0 : attention_bwd_flash16_workspace(bp.p)) + attention_bwd_flash16_mask_bits_bytes(bp.p) +
-              attention_bwd_flash16_lengths_bytes(bp);
+              attention_bwd_flash16_lengths_bytes(bp) + attention_bwd_flash16_dq_partial_bytes(bp);
         return MI_ATTN_KERNEL_FLASH16;
     }
     if (!(d->fwd.flags & MI_ATTN_FORCE_GENERIC) && attention_bwd_flash32_supports(bp)) {

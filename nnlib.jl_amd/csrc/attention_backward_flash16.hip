@@ -76,9 +76,48 @@ size_t attention_bwd_flash16_lengths_bytes(const AttnBwdParams &bp) {
     return ((size_t)(bp.p.H * bp.p.B) * sizeof(int32_t) + 15) & ~(size_t)15;
 }
 
+// ---- dQ kernel split over the keys ---------------------------------------------------------------------------
+// The dQ kernel has one workgroup per (query tile, head, batch): cross-attention with few queries and many keys
+// leaves most of the chip idle (32 workgroups for 128 queries, 16 heads, 2 batch elements).  With saved statistics
+// every key piece is independent, so the key range is cut like the forward kernel's and the Float32 partial sums are
+// added up by dq_merge_kernel.
+int attention_bwd_flash16_dq_nsplit(const AttnBwdParams &bp) {
+    const AttnParams &p = bp.p;
+    if (!bp.have_stats || !bp.dq || p.causal) return 1;
+    const int64_t wgs = ((p.Lq + 127) / 128) * p.H * p.B;
+    if (wgs >= 256 || p.Lkv < 2048) return 1;
+    int64_t n = (512 + wgs - 1) / wgs;
+    if (n > p.Lkv / 512) n = p.Lkv / 512;
+    if (n > 32) n = 32;
+    return n < 2 ? 1 : (int)n;
+}
+size_t attention_bwd_flash16_dq_partial_bytes(const AttnBwdParams &bp) {
+    const int n = attention_bwd_flash16_dq_nsplit(bp);
+    return n > 1 ? sizeof(float) * (size_t)n * (size_t)(bp.p.B * bp.p.Lq * bp.p.E) : 0;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void dq_merge_kernel(const float *ws, typename T::type *dq, int nsplit, int64_t n) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;   // E is a multiple of 8: whole groups of 4
+    if (i >= n) return;
+    floatx4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s = 0; s < nsplit; s++) {
+        const floatx4_t v = *(const floatx4_t *)(ws + (int64_t)s * n + i);
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[e] += v[e];
+    }
+    typename T::vec4 r;
+#pragma unroll
+    for (int e = 0; e < 4; e++) r[e] = T::from_f32(acc[e]);
+    *(typename T::vec4 *)(dq + i) = r;
+}
+
 int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp_in, hipStream_t st) {
     AttnBwdParams bp = bp_in;
     const AttnParams &p = bp.p;
+    bp.dq_nsplit = attention_bwd_flash16_dq_nsplit(bp);
+    if (bp.dq_nsplit > 1)   // implies saved statistics: the workspace holds [packed mask bits][lengths][these partial sums]
+        bp.dq_partial = (float *)((char *)bp.workspace + attention_bwd_flash16_mask_bits_bytes(p) + attention_bwd_flash16_lengths_bytes(bp));
     if (attention_bwd_flash16_lengths_bytes(bp) != 0) {   // after the statistics planes when those live in the workspace (no packed mask bits here)
         int32_t *lens = (int32_t *)((char *)bp.workspace + (bp.have_stats ? 0 : attention_bwd_flash16_workspace(p)));
         const int32_t rc = launch_key_mask_lengths(p, lens, st);
@@ -99,7 +138,16 @@ int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp_in, hipStream_t st)
         bp.mb_lkv_pad = pad;
         bp.mb_nqt = nqt;
     }
+    int32_t rc;
     if (p.dtype == MI_BF16)
-        return p.D <= 64 ? launch_bwd_flash16_bf16_d64(bp, st) : p.D <= 128 ? launch_bwd_flash16_bf16_d128(bp, st) : launch_bwd_flash16_bf16_d256(bp, st);
-    return p.D <= 64 ? launch_bwd_flash16_f16_d64(bp, st) : p.D <= 128 ? launch_bwd_flash16_f16_d128(bp, st) : launch_bwd_flash16_f16_d256(bp, st);
+        rc = p.D <= 64 ? launch_bwd_flash16_bf16_d64(bp, st) : p.D <= 128 ? launch_bwd_flash16_bf16_d128(bp, st) : launch_bwd_flash16_bf16_d256(bp, st);
+    else
+        rc = p.D <= 64 ? launch_bwd_flash16_f16_d64(bp, st) : p.D <= 128 ? launch_bwd_flash16_f16_d128(bp, st) : launch_bwd_flash16_f16_d256(bp, st);
+    if (rc != MI_OK || bp.dq_nsplit <= 1) return rc;
+    const int64_t n = p.B * p.Lq * p.E;
+    const dim3 grid((unsigned)((n / 4 + 255) / 256));
+    if (p.dtype == MI_BF16) hipLaunchKernelGGL(dq_merge_kernel<BF16>, grid, dim3(256), 0, st, bp.dq_partial, (__bf16 *)bp.dq, bp.dq_nsplit, n);
+    else hipLaunchKernelGGL(dq_merge_kernel<F16>, grid, dim3(256), 0, st, bp.dq_partial, (_Float16 *)bp.dq, bp.dq_nsplit, n);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
 }

@@ -80,6 +80,10 @@ struct AttnBwdParams {
     // key-padding mask measured on the device: per (head, batch) pair [b * H + h] the context length, or 0 when the
     // mask of the pair is not a kept prefix; null when the call does not take that path
     const int32_t *kv_len;
+    // dQ kernel split over the keys (few query tiles, many keys; calls with saved statistics): Float32 partial sums
+    // [piece][B][Lq][E], summed by a small kernel; dq_nsplit = 1 and null otherwise
+    float *dq_partial;
+    int32_t dq_nsplit;
 };
 
 // size of the statistics planes shared by the forward kernels that save them and the backward kernels
@@ -97,6 +101,8 @@ size_t attention_bwd_flash32_lengths_bytes(const AttnBwdParams &bp);
 size_t attention_bwd_flash16_workspace(const AttnParams &p);
 size_t attention_bwd_flash16_mask_bits_bytes(const AttnParams &p);   // 0 when the call does not take the packed-mask path
 size_t attention_bwd_flash16_lengths_bytes(const AttnBwdParams &bp);  // 0 when the call does not take the context-length path
+int attention_bwd_flash16_dq_nsplit(const AttnBwdParams &bp);         // pieces the dQ kernel's key range is cut into (1: no split)
+size_t attention_bwd_flash16_dq_partial_bytes(const AttnBwdParams &bp);
 // lens[b * H + h] = number of keys kept when the key-padding mask of the pair keeps exactly a prefix, else 0
 int32_t launch_key_mask_lengths(const AttnParams &p, int32_t *lens, hipStream_t st);
 size_t attention_bwd_generic_workspace(const AttnParams &p);

@@ -458,3 +458,19 @@ def test_causal_and_padding_mask(nn, oracle, dtype, D, H, L, B, saved):
     for g, r_, name in zip(got[:3], ref[:3], ("dq", "dk", "dv")):
         err = np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05)
         assert err <= TOL[dtype], (name, err)
+
+
+@pytest.mark.parametrize("dtype,D,H,Lq,Lkv,B,mask_kind,bias_kind,dropout", [
+    ("bf16", 128, 2, 100, 2304, 1, None, None, None),
+    ("f16", 64, 2, 130, 4096, 2, "random", None, None),        # dense mask tiles
+    ("bf16", 96, 1, 64, 2500, 2, "random", None, None),        # unaligned: per-element path
+    ("bf16", 64, 2, 200, 2304, 2, "lengths", None, None),      # context lengths: both kernel sets write their pairs' pieces
+    ("f16", 128, 1, 70, 2048, 2, None, "full", None),          # bias and its gradient
+    ("bf16", 64, 2, 100, 2304, 1, None, None, (0.2, 3)),
+])
+def test_dq_split_over_the_keys(nn, oracle, dtype, D, H, Lq, Lkv, B, mask_kind, bias_kind, dropout):
+    """Few queries, many keys, saved statistics: the dQ kernel's key range is cut into pieces whose Float32 partial sums a
+    small kernel adds up."""
+    bias_shape = (Lkv, Lq, H, B) if bias_kind == "full" else None
+    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, mask_kind=mask_kind, bias_shape=bias_shape, expect="flash16", saved=True,
+         dropout=dropout, seed=Lq + Lkv, scale=0.4)
