@@ -40,7 +40,8 @@ static int32_t choose_bwd(const mi_attn_bwd_desc *d, const AttnBwdParams &bp, si
         return MI_ATTN_KERNEL_FLASH16;
     }
     if (!(d->fwd.flags & MI_ATTN_FORCE_GENERIC) && attention_bwd_flash32_supports(bp)) {
-        *ws = (bp.have_stats ? 0 : attention_stats_bytes(bp.p)) + attention_bwd_flash32_lengths_bytes(bp);
+        *ws = (bp.have_stats ? 0 : attention_stats_bytes(bp.p)) + attention_bwd_flash32_lengths_bytes(bp) +
+              attention_bwd_flash16_dq_partial_bytes(bp);
         return MI_ATTN_KERNEL_FLASH32;
     }
     if (bp.have_stats) {   // the generic kernels keep their own statistics, in their own layout

@@ -144,10 +144,14 @@ int32_t launch_attention_bwd_flash16(const AttnBwdParams &bp_in, hipStream_t st)
     else
         rc = p.D <= 64 ? launch_bwd_flash16_f16_d64(bp, st) : p.D <= 128 ? launch_bwd_flash16_f16_d128(bp, st) : launch_bwd_flash16_f16_d256(bp, st);
     if (rc != MI_OK || bp.dq_nsplit <= 1) return rc;
-    const int64_t n = p.B * p.Lq * p.E;
+    return launch_dq_merge(p.dtype, bp.dq_partial, bp.dq, bp.dq_nsplit, p.B * p.Lq * p.E, st);
+}
+
+int32_t launch_dq_merge(int32_t dtype, const float *partial, void *dq, int nsplit, int64_t n, hipStream_t st) {
     const dim3 grid((unsigned)((n / 4 + 255) / 256));
-    if (p.dtype == MI_BF16) hipLaunchKernelGGL(dq_merge_kernel<BF16>, grid, dim3(256), 0, st, bp.dq_partial, (__bf16 *)bp.dq, bp.dq_nsplit, n);
-    else hipLaunchKernelGGL(dq_merge_kernel<F16>, grid, dim3(256), 0, st, bp.dq_partial, (_Float16 *)bp.dq, bp.dq_nsplit, n);
+    if (dtype == MI_BF16) hipLaunchKernelGGL(dq_merge_kernel<BF16>, grid, dim3(256), 0, st, partial, (__bf16 *)dq, nsplit, n);
+    else if (dtype == MI_F16) hipLaunchKernelGGL(dq_merge_kernel<F16>, grid, dim3(256), 0, st, partial, (_Float16 *)dq, nsplit, n);
+    else hipLaunchKernelGGL(dq_merge_kernel<F32>, grid, dim3(256), 0, st, partial, (float *)dq, nsplit, n);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }

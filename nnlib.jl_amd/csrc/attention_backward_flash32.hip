@@ -115,7 +115,9 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
     float *Ks = (float *)bwd_smem, *Vs = Ks + 2 * TILEF;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
     const int64_t HB = p.H * a.nb;   // this launch's batch elements: [a.b0, a.b0 + a.nb)
-    const int64_t hb = blockIdx.x % HB, qt = a.n_qtiles - 1 - blockIdx.x / HB;
+    const int split = (int)(blockIdx.x % a.nsplit);   // piece of the key range (a.nsplit > 1: calls with saved statistics only)
+    const int64_t bid = blockIdx.x / a.nsplit;
+    const int64_t hb = bid % HB, qt = a.n_qtiles - 1 - bid / HB;
     const int64_t h = hb % p.H, b = a.b0 + hb / p.H;
     const int64_t i0 = qt * 128, iw = i0 + 32 * wave, qi = iw + r;
     const bool qok = qi < p.Lq;
@@ -201,15 +203,20 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
 #pragma unroll
     for (int dvb = 0; dvb < NDV; dvb++) dq[dvb] = (floatx16_t){0};
     ts.base2 = (const float *)p.v + p.Ev * (p.Lkv * b) + p.D * h;
-    ts.load(0);
+    int jt0 = 0, jt1 = n_tiles;
+    if (a.nsplit > 1) {
+        jt0 = split * a.tiles_per_split;
+        if (jt0 + a.tiles_per_split < jt1) jt1 = jt0 + a.tiles_per_split;
+    }
+    ts.load((int64_t)jt0 * BN);
     __syncthreads();   // pass 1 may still be reading the tiles
     ts.store(0);
     __syncthreads();
     const float m2 = fm[0] * cs, linv = fl[0];
-    for (int jt = 0; jt < n_tiles; jt++) {
-        const int buf = jt & 1;
+    for (int jt = jt0; jt < jt1; jt++) {
+        const int buf = (jt - jt0) & 1;
         const int64_t j0 = (int64_t)jt * BN;
-        if (jt + 1 < n_tiles) ts.load(j0 + BN);
+        if (jt + 1 < jt1) ts.load(j0 + BN);
         if (!CAUSAL || j0 <= iw + 31) {
             const float *kt = Ks + buf * TILEF, *vt = Vs + buf * TILEF;
             if constexpr (EXTRAS == EXTRAS_NONE) {
@@ -281,7 +288,9 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
         __syncthreads();
     }
     if (qok && bp.dq) {
-        float *dqrow = (float *)bp.dq + p.E * (qi + p.Lq * b) + p.D * h;
+        // one piece of the key range (a.nsplit > 1): its share of dQ goes to the workspace for the merge kernel
+        float *dqrow = a.nsplit > 1 ? bp.dq_partial + ((int64_t)split * p.B * p.Lq + qi + p.Lq * b) * p.E + p.D * h
+                                    : (float *)bp.dq + p.E * (qi + p.Lq * b) + p.D * h;
 #pragma unroll
         for (int dvb = 0; dvb < NDV; dvb++)
 #pragma unroll
@@ -479,6 +488,10 @@ int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) 
     // Bias gradient without atomics where a workgroup owns the entries it adds to; entries shared by the batch
     // elements are kept apart by one launch per batch element (the same rule as the 16-bit kernels)
     FlashArgs a1 = a;
+    if (bp.dq_nsplit > 1) {   // the dQ kernel's key range in pieces (the dK / dV kernels below keep a.nsplit = 1)
+        a1.nsplit = bp.dq_nsplit;
+        a1.tiles_per_split = (int32_t)(((p.Lkv + BN - 1) / BN + bp.dq_nsplit - 1) / bp.dq_nsplit);
+    }
     const bool own_rows = bp.dbias && p.bias_strides[0] == 1 && (p.bias_strides[1] != 0 || p.Lq == 1) && (p.bias_strides[2] != 0 || p.H == 1);
     const bool per_batch = own_rows && p.bias_strides[3] == 0 && p.B > 1;
     if (own_rows && (!per_batch || (int64_t)a.n_qtiles * p.H >= 256)) a1.dbias_plain = 1;
@@ -486,10 +499,10 @@ int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) 
         a1.nb = 1;
         for (int64_t b = 0; b < p.B; b++) {
             a1.b0 = (int32_t)b;
-            hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H)), dim3(256), SMEM_Q, st, a1, bp);
+            hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * a1.nsplit)), dim3(256), SMEM_Q, st, a1, bp);
         }
     } else {
-        hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B)), dim3(256), SMEM_Q, st, a1, bp);
+        hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B * a1.nsplit)), dim3(256), SMEM_Q, st, a1, bp);
     }
     MI_LAUNCH_CHECK();
     const dim3 g2((unsigned)(((p.Lkv + 127) / 128) * p.H * p.B));
@@ -540,7 +553,12 @@ bool attention_bwd_flash32_supports(const AttnBwdParams &bp) {
     return tiles * p.H * p.B <= 2147483647LL;
 }
 
-int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st) {
+int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp_in, hipStream_t st) {
+    AttnBwdParams bp = bp_in;
+    // few queries, many keys, saved statistics: the dQ kernel's key range in pieces (the 16-bit kernels' rule); the
+    // workspace then holds [context lengths][partial sums]
+    bp.dq_nsplit = attention_bwd_flash16_dq_nsplit(bp);
+    if (bp.dq_nsplit > 1) bp.dq_partial = (float *)((char *)bp.workspace + attention_bwd_flash32_lengths_bytes(bp));
     FlashArgs a;
     a.p = bp.p;
     a.p.weights = nullptr;
@@ -564,5 +582,7 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp, hipStream_t st) {
         if (rc != MI_OK) return rc;
         a.kv_len = lens;
     }
-    return bp.p.D <= 64 ? launch_d<64>(a, bp, st) : launch_d<128>(a, bp, st);
+    const int32_t rc = bp.p.D <= 64 ? launch_d<64>(a, bp, st) : launch_d<128>(a, bp, st);
+    if (rc != MI_OK || bp.dq_nsplit <= 1) return rc;
+    return launch_dq_merge(MI_F32, bp.dq_partial, bp.dq, bp.dq_nsplit, bp.p.B * bp.p.Lq * bp.p.E, st);
 }

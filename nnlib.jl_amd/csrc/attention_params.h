@@ -102,7 +102,9 @@ size_t attention_bwd_flash16_workspace(const AttnParams &p);
 size_t attention_bwd_flash16_mask_bits_bytes(const AttnParams &p);   // 0 when the call does not take the packed-mask path
 size_t attention_bwd_flash16_lengths_bytes(const AttnBwdParams &bp);  // 0 when the call does not take the context-length path
 int attention_bwd_flash16_dq_nsplit(const AttnBwdParams &bp);         // pieces the dQ kernel's key range is cut into (1: no split)
-size_t attention_bwd_flash16_dq_partial_bytes(const AttnBwdParams &bp);
+size_t attention_bwd_flash16_dq_partial_bytes(const AttnBwdParams &bp);   // the same rule serves the Float32 kernels
+// dq[i] = sum over the pieces of partial[piece][i], i < n (a multiple of 4), converted to `dtype`
+int32_t launch_dq_merge(int32_t dtype, const float *partial, void *dq, int nsplit, int64_t n, hipStream_t st);
 // lens[b * H + h] = number of keys kept when the key-padding mask of the pair keeps exactly a prefix, else 0
 int32_t launch_key_mask_lengths(const AttnParams &p, int32_t *lens, hipStream_t st);
 size_t attention_bwd_generic_workspace(const AttnParams &p);

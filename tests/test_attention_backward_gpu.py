@@ -467,10 +467,14 @@ def test_causal_and_padding_mask(nn, oracle, dtype, D, H, L, B, saved):
     ("bf16", 64, 2, 200, 2304, 2, "lengths", None, None),      # context lengths: both kernel sets write their pairs' pieces
     ("f16", 128, 1, 70, 2048, 2, None, "full", None),          # bias and its gradient
     ("bf16", 64, 2, 100, 2304, 1, None, None, (0.2, 3)),
+    ("f32", 64, 2, 100, 2304, 1, None, None, None),
+    ("f32", 128, 1, 130, 2500, 2, "random", None, None),
+    ("f32", 36, 2, 200, 2304, 2, "lengths", None, None),
+    ("f32", 64, 1, 70, 2048, 2, None, "full", None),
 ])
 def test_dq_split_over_the_keys(nn, oracle, dtype, D, H, Lq, Lkv, B, mask_kind, bias_kind, dropout):
     """Few queries, many keys, saved statistics: the dQ kernel's key range is cut into pieces whose Float32 partial sums a
     small kernel adds up."""
     bias_shape = (Lkv, Lq, H, B) if bias_kind == "full" else None
-    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, mask_kind=mask_kind, bias_shape=bias_shape, expect="flash16", saved=True,
-         dropout=dropout, seed=Lq + Lkv, scale=0.4)
+    _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, mask_kind=mask_kind, bias_shape=bias_shape,
+         expect="flash32" if dtype == "f32" else "flash16", saved=True, dropout=dropout, seed=Lq + Lkv, scale=0.4)
