@@ -27,7 +27,7 @@ HBM_BOUND = ("c4", "c5")                                # workloads priced again
 # --pmc WRITE_SIZE in separate runs of this script and scaled by what the same counters read for the
 # 1 GiB copy of --workload copy (factors 2.000 and 1.000); the runs are summarised under profiles/.
 MIB = 1 << 20
-MEASURED_TRAFFIC = {"c2": (304.7 + 544.0) * MIB, "c3": (448.1 + 64.0) * MIB, "c4": (438.7 + 16.5) * MIB,
+MEASURED_TRAFFIC = {"c2": (335.5 + 544.0) * MIB, "c3": (429.3 + 64.0) * MIB, "c4": (419.0 + 16.5) * MIB,
                     "c5": (8192.5 + 16.5) * MIB}
 ROTATE_BYTES = 1 << 30                                  # input sets rotated until they cover 4x the last-level cache
 
