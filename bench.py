@@ -238,6 +238,7 @@ EXTRA = {
     "softmax": "softmax(x; dims=1), x (1024, 131072) f32: the logits of C2 (512 MiB in, 512 MiB out)",
     "batched_mul": "batched_mul(A, B), A (2048, 2048, 16), B (2048, 2048, 16) bf16",
     "batched_mul_f32": "batched_mul(A, B), A (1024, 64, 128), B (64, 1024, 128) f32: the score product of C2",
+    "batched_mul_c32": "batched_mul(A, B), A and B (1024, 1024, 16) ComplexF32, 8 real FLOP per complex multiply-add",
 }
 
 
@@ -311,19 +312,26 @@ def measure_extra(key, steps, warmup, with_cpu):
     elif key.startswith("batched_mul"):
         if key == "batched_mul":
             dt_name, (m, kk, n, nb) = "bf16", (2048, 2048, 2048, 16)
+        elif key == "batched_mul_c32":
+            dt_name, (m, kk, n, nb) = "c64", (1024, 1024, 1024, 16)
         else:
             dt_name, (m, kk, n, nb) = "f32", (1024, 64, 1024, 128)
         A, Bm = DA.empty((m, kk, nb), dt_name), DA.empty((kk, n, nb), dt_name)
         C = DA.empty((m, n, nb), dt_name)
         for sid, a in enumerate((A, Bm)):
-            _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, 11, sid, 1.0, None))
+            if dt_name == "c64":   # a complex array is filled as twice as many Float32 values
+                _lib.check(lib.mi_randn_fill(a.ptr, _lib.MI_F32, 2 * a.length, 11, sid, 1.0, None))
+            else:
+                _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, 11, sid, 1.0, None))
         ms = _event_time(lib, _lib, lambda: nn.batched_mul_(C, A, Bm), steps, warmup)
-        flops = 2 * m * n * kk * nb
+        flops = (8 if dt_name == "c64" else 2) * m * n * kk * nb
         val = flops / (ms * 1e-3) / 1e12
+        peak = PEAK["f32"] if dt_name == "c64" else PEAK[dt_name]
         line = dict(metric="batched_mul TFLOP/s", value=val, unit="TFLOP/s", dtype=dt_name,
-                    roofline=dict(bound="mfma", achieved=val, peak=PEAK[dt_name], unit="TFLOP/s", frac=val / PEAK[dt_name], traffic=None),
-                    config=dict(workload=EXTRA[key], kernel="batched_gemm_kernel"), flops_per_step=flops)
-        if with_cpu:
+                    roofline=dict(bound="mfma", achieved=val, peak=peak, unit="TFLOP/s", frac=val / peak, traffic=None),
+                    config=dict(workload=EXTRA[key], kernel="gemm_c32_kernel" if dt_name == "c64" else "batched_gemm_kernel"),
+                    flops_per_step=flops)
+        if with_cpu and dt_name != "c64":
             from oracle import oracle as O
             ns = min(nb, 2 if key == "batched_mul" else 32)
             rng = np.random.default_rng(0)

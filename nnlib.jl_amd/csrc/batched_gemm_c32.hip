@@ -5,8 +5,13 @@
 // batched_mul_generic! (src/batched/batchedmul.jl:306-325: PermutedDimsArray inputs and outputs, an
 // adjoint of a non-unit-stride parent) in one kernel, without copies.
 //
-// 64 x 64 output tile per 256-thread workgroup, 4 x 4 complex results per thread, k in steps of 16
-// through LDS; scalar complex multiply-adds in Float32 (4 real FMAs each).
+// 64 x 64 output tile per 256-thread workgroup, k in steps of 16 through LDS, products on the Float32
+// matrix cores (v_mfma_f32_32x32x2_f32).  A complex product is a real one of twice the size: with C, A
+// and B viewed as real arrays whose rows (for B: whose k) alternate real and imaginary parts,
+//   C'[2i+p, j] = sum_k  A^[2i+p, 2k] * Br[k, j] + A^[2i+p, 2k+1] * Bi[k, j],
+//   A^[2i, 2k] = Ar   A^[2i, 2k+1] = -Ai   A^[2i+1, 2k] = Ai   A^[2i+1, 2k+1] = Ar,
+// i.e. 8 real FLOP per complex multiply-add, the same count as the scalar form.  A^ is never stored: a
+// lane picks the part it needs from the complex tile in LDS and flips its sign.
 #include "common.h"
 
 namespace {
@@ -20,25 +25,22 @@ struct CGemmArgs {
     float alpha_re, alpha_im, beta_re, beta_im;
 };
 
-__device__ inline float2 cmul(float2 a, float2 b) { return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x); }
-__device__ inline void cfma(float2 a, float2 b, float2 &c) {
-    c.x = fmaf(a.x, b.x, c.x);
-    c.x = fmaf(-a.y, b.y, c.x);
-    c.y = fmaf(a.x, b.y, c.y);
-    c.y = fmaf(a.y, b.x, c.y);
-}
-
 __global__ __launch_bounds__(256) void gemm_c32_kernel(CGemmArgs g) {
-    constexpr int TM = 64, TK = 16;
+    constexpr int TM = 64, TK = 16, LD = 2 * (TM + 1);   // LD: floats per k row of a tile
     __shared__ float2 As[TK][TM + 1], Bs[TK][TM + 1];
-    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int tid = threadIdx.x;
     const int64_t m0 = (int64_t)blockIdx.x * TM, n0 = (int64_t)blockIdx.y * TM, bz = blockIdx.z;
     const float2 *A = g.A + bz * g.a_bs, *B = g.B + bz * g.b_bs;
-    float2 acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = make_float2(0.0f, 0.0f);
+    // Each wavefront owns 16 complex rows (32 real rows) x 64 columns: two 32 x 32 blocks, computed
+    // transposed (first MFMA operand from B) so that the lanes of an accumulator register run along m.
+    const int lane = tid & 63, wr = tid >> 6, l = lane & 31, h = lane >> 5, part = l & 1;
+    const int a_word = 2 * (16 * wr + (l >> 1)) + (part != h);          // which float of the complex A element
+    const uint32_t a_sign = (part == 0 && h == 1) ? 0x80000000u : 0u;   // A^[2i, 2k+1] = -Ai
+    const int b_word = 2 * l + h;                                        // real part for k' even, imaginary for odd
+    const float *Af = (const float *)&As[0][0], *Bf = (const float *)&Bs[0][0];
+    floatx16_t acc[2];
+    acc[0] = (floatx16_t){0};
+    acc[1] = (floatx16_t){0};
     // consecutive threads walk the unit-stride direction of each operand where there is one
     const bool a_rows_fast = g.a_rs <= g.a_cs, b_rows_fast = g.b_cs <= g.b_rs;   // for B the "row" of the tile is n
     for (int64_t k0 = 0; k0 < g.k; k0 += TK) {
@@ -59,35 +61,30 @@ __global__ __launch_bounds__(256) void gemm_c32_kernel(CGemmArgs g) {
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < TK; kk++) {
-            float2 a[4], b[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) a[i] = As[kk][tx + 16 * i];
-#pragma unroll
-            for (int j = 0; j < 4; j++) b[j] = Bs[kk][ty + 16 * j];
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) cfma(a[i], b[j], acc[i][j]);
+            const float a = __uint_as_float(__float_as_uint(Af[kk * LD + a_word]) ^ a_sign);
+            const float b0 = Bf[kk * LD + b_word], b1 = Bf[kk * LD + 64 + b_word];
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(b0, a, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(b1, a, acc[1], 0, 0, 0);
         }
         __syncthreads();
     }
-    float2 *C = g.C + bz * g.c_bs;
-    const float2 alpha = make_float2(g.alpha_re, g.alpha_im), beta = make_float2(g.beta_re, g.beta_im);
-    const bool have_beta = beta.x != 0.0f || beta.y != 0.0f;   // beta = 0 overwrites (a NaN in C does not spread), as BLAS does
+    // acc[jb][r]: column n0 + 32*jb + 8*(r/4) + 4*h + r%4, complex row m0 + 16*wr + l/2, real (part 0) or
+    // imaginary (part 1) component; the other component sits in the neighbouring lane
+    float *C = (float *)(g.C + bz * g.c_bs);
+    const float other_alpha = part ? g.alpha_im : -g.alpha_im, other_beta = part ? g.beta_im : -g.beta_im;
+    const bool have_beta = g.beta_re != 0.0f || g.beta_im != 0.0f;   // beta = 0 overwrites (a NaN in C does not spread), as BLAS does
+    const int64_t mi = m0 + 16 * wr + (l >> 1);
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int jb = 0; jb < 2; jb++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int64_t mi = m0 + tx + 16 * i, nj = n0 + ty + 16 * j;
+        for (int r = 0; r < 16; r++) {
+            const float mine = acc[jb][r], other = __shfl_xor(mine, 1, 64);
+            float out = fmaf(g.alpha_re, mine, other_alpha * other);
+            const int64_t nj = n0 + 32 * jb + 8 * (r >> 2) + 4 * h + (r & 3);
             if (mi < g.m && nj < g.n) {
-                float2 *c = C + mi * g.c_rs + nj * g.c_cs;
-                float2 r = cmul(alpha, acc[i][j]);
-                if (have_beta) {
-                    const float2 old = cmul(beta, *c);
-                    r.x += old.x;
-                    r.y += old.y;
-                }
-                *c = r;
+                float *c = C + 2 * (mi * g.c_rs + nj * g.c_cs);
+                if (have_beta) out += fmaf(g.beta_re, c[part], other_beta * c[part ^ 1]);
+                c[part] = out;
             }
         }
 }
