@@ -200,7 +200,10 @@ struct VecIO {
 
 // running (maximum, sum of exponentials against it); the special cases keep the reference's results:
 // nothing but -Inf so far contributes no terms, a +Inf maximum counts the +Inf entries (src/softmax.jl:72-75)
+// A NaN entry becomes the maximum and stays it (no comparison replaces it), which turns every later term and
+// the results of the whole column into NaN, as the reference's maximum does (src/softmax.jl:69-70).
 __device__ inline void online_add(float x, float &m, float &s) {
+    if (x != x) m = x;
     if (x > m) {
         s = (m == MI_NEG_INF) ? 0.0f : s * fast_exp(m - x);
         m = x;
@@ -208,6 +211,7 @@ __device__ inline void online_add(float x, float &m, float &s) {
     if (m != MI_NEG_INF) s += softmax_term(x, m);
 }
 __device__ inline void online_merge(float m2, float s2, float &m, float &s) {
+    if (m2 != m2) m = m2;
     if (m2 > m) {
         s = (m == MI_NEG_INF) ? s2 : s2 + s * fast_exp(m - m2);
         m = m2;

@@ -141,6 +141,40 @@ def test_special_values_on_the_wide_row_kernel(nn, oracle, dtype, length):
         assert np.abs(got[fin] - ref[fin]).max() <= tol * 10
 
 
+@pytest.mark.parametrize("length", [200, 9000, 20000], ids=["register-cached", "streamed", "streamed-long"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_nan_poisons_its_whole_column_wherever_it_sits(nn, oracle, dtype, length):
+    """src/softmax.jl:69-70: a NaN becomes the column maximum, so the whole column is NaN.  In the streamed kernel
+    every thread keeps a running (maximum, sum) of its own rows: the NaN is put in a thread's very first row, right
+    after a run of -Inf entries, in the middle, and in the last row."""
+    rng = np.random.default_rng(12)
+    x = round_to(rng.standard_normal((64, length, 2)), dtype)
+    x[0, 0, 0] = np.nan                        # first row of the first slice
+    x[1, 1, 0] = np.nan                        # first row of the second slice
+    run = min(300, length // 2)
+    x[2, :run, 0] = -np.inf
+    x[2, run, 0] = np.nan                      # after a leading run of -Inf
+    x[3, length // 2 + 7, 0] = np.nan
+    x[4, length - 1, 0] = np.nan
+    x[5, 63, 1] = np.nan
+    x[5, 64:128, 1] = -np.inf
+    x[6, :, 1] = -np.inf
+    x[6, 17, 1] = np.nan                       # NaN among nothing but -Inf
+    d = _dev(nn, x, dtype)
+    poisoned = np.zeros((64, 2), bool)
+    poisoned[[0, 1, 2, 3, 4], 0] = True
+    poisoned[[5, 6], 1] = True
+    with np.errstate(invalid="ignore"):
+        for fn, ref in ((nn.softmax, oracle.softmax(x, 2)), (nn.logsoftmax, oracle.logsoftmax(x, 2))):
+            got = fn(d, dims=2).to_numpy()
+            assert np.array_equal(np.isnan(ref), np.broadcast_to(poisoned[:, None, :], ref.shape))   # the oracle agrees
+            assert np.array_equal(np.isnan(got), np.isnan(ref))
+            fin = np.isfinite(ref)
+            assert np.abs(got[fin] - ref[fin]).max() <= TOL[dtype] * max(1.0, np.abs(ref[fin]).max())
+        got, ref = nn.logsumexp(d, dims=2).to_numpy(), oracle.logsumexp(x, 2)
+        assert np.array_equal(np.isnan(got).reshape(64, 2), poisoned) and np.array_equal(np.isnan(ref).reshape(64, 2), poisoned)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("shape,dims", [((3, 4), None), ((3, 4), 1), ((3, 4), 2), ((64, 100, 5), 2), ((33, 65, 3), (2, 3)),
                                         ((5000,), 1), ((128, 40), 1)])
