@@ -164,6 +164,18 @@ int32_t mi_attention_workspace_size(const mi_attn_desc *desc, size_t *bytes);
 int32_t mi_attention_fwd(const mi_attn_desc *desc, mi_stream stream);
 int32_t mi_attention_stats_size(const mi_attn_desc *desc, size_t *bytes);
 
+/* mi_attention_fwd for callers that cannot allocate device memory: code under stream (graph) capture, serving loops
+ * and harnesses that forbid it.  No counterpart in the reference.  Same arguments and results as mi_attention_fwd,
+ * except that desc.workspace / workspace_bytes are ignored: the partial results of split-kv calls, the raw scores of
+ * single-query calls that return weights and the context lengths of key-padding masks go into an array of
+ * MI_ATTN_STATIC_WORKSPACE_BYTES that is part of the library's device image (each GPU the library runs on holds one
+ * copy until the process ends).  A call whose mi_attention_workspace_size() exceeds that returns MI_EWORKSPACE.  The
+ * call allocates and frees nothing.  All calls on one GPU share the array: calls that may run at the same time on one
+ * GPU (different streams) race and must be ordered by the caller.  mi_init(device) looks the array's address up for
+ * that device; without it the first call on a device does. */
+#define MI_ATTN_STATIC_WORKSPACE_BYTES (32u << 20)
+int32_t mi_attention_fwd_static(const mi_attn_desc *desc, mi_stream stream);
+
 /*
  * Gradient of one dot_product_attention call (fdrop = identity or fused dropout).  The reference has no hand-written
  * rule: reverse-mode AD walks src/attention.jl:86-127 backwards through the rrule of batched_mul

@@ -1,6 +1,7 @@
 // mi_attention_fwd: validation (mirrors the reference's argument checks) and kernel selection.
 #include "common.h"
 #include "attention_params.h"
+#include <mutex>
 
 // kv_len: null, or per (head, batch) context lengths (FlashArgs::kv_len)
 int32_t launch_flash16_bf16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
@@ -275,7 +276,39 @@ MI_API int32_t mi_attention_workspace_size(const mi_attn_desc *d, size_t *bytes)
     return mi_attention_plan(d, nullptr, bytes);
 }
 
-MI_API int32_t mi_attention_fwd(const mi_attn_desc *d, mi_stream s) {
+// ---- the forward call on a workspace that lives in the library's own device image ------------------------------
+// For callers that cannot allocate device memory (under stream capture, in loops that must not touch the allocator):
+// the split-kv partials, raw single-query scores and context lengths go into a file-scope device array instead of a
+// caller-provided workspace.  Every GPU the library runs on holds its own copy of the array at its own address, which
+// hipGetSymbolAddress reports for the device that is current; in host code the array's name is not that address.
+static __device__ __align__(256) unsigned char scratch[MI_ATTN_STATIC_WORKSPACE_BYTES];
+
+#define MI_MAX_DEVICES 64
+static void *g_scratch_ptr[MI_MAX_DEVICES];   // per device: address of `scratch` there, null = not asked yet
+static std::mutex g_scratch_lock;
+
+// Address of `scratch` on the current device (asked once per device).
+int32_t attention_static_scratch(void **out) {
+    int dev = -1;
+    MI_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MI_MAX_DEVICES) return mi_set_error(MI_EINVAL, "mi_attention_fwd_static: device %d is beyond the %d this library tracks", dev, MI_MAX_DEVICES);
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        MI_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return mi_set_error(MI_EHIP, "mi_attention_fwd_static: the device image holds no workspace array");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return MI_OK;
+}
+
+static int32_t attention_forward(const mi_attn_desc *d, mi_stream s, bool static_workspace);
+
+MI_API int32_t mi_attention_fwd(const mi_attn_desc *d, mi_stream s) { return attention_forward(d, s, false); }
+MI_API int32_t mi_attention_fwd_static(const mi_attn_desc *d, mi_stream s) { return attention_forward(d, s, true); }
+
+static int32_t attention_forward(const mi_attn_desc *d, mi_stream s, bool static_workspace) {
     AttnParams p;
     int32_t rc = attention_validate(d, &p);
     if (rc != MI_OK) return rc;
@@ -288,7 +321,17 @@ MI_API int32_t mi_attention_fwd(const mi_attn_desc *d, mi_stream s) {
     }
     size_t ws = 0;
     const int32_t kernel = choose(d, p, &ws);
-    if (ws > 0 && (!d->workspace || d->workspace_bytes < ws))
+    if (static_workspace) {
+        // every kernel writes what it later reads of the workspace, so what an earlier call left there needs no clearing
+        if (ws > MI_ATTN_STATIC_WORKSPACE_BYTES)
+            return mi_set_error(MI_EWORKSPACE, "mi_attention_fwd_static: this call needs a workspace of %zu bytes, the built-in one has %zu; "
+                                "use mi_attention_fwd with a caller-provided workspace", ws, (size_t)MI_ATTN_STATIC_WORKSPACE_BYTES);
+        p.workspace = nullptr;
+        if (ws > 0) {
+            rc = attention_static_scratch(&p.workspace);
+            if (rc != MI_OK) return rc;
+        }
+    } else if (ws > 0 && (!d->workspace || d->workspace_bytes < ws))
         return mi_set_error(MI_EWORKSPACE, "mi_attention_fwd: workspace of %zu bytes required, %zu given", ws,
                             d->workspace ? d->workspace_bytes : (size_t)0);
     switch (kernel) {

@@ -2,6 +2,8 @@
 #include "common.h"
 #include <string.h>
 
+int32_t attention_static_scratch(void **out);   // attention.hip
+
 static thread_local char g_err[512] = "";
 
 int32_t mi_set_error(int32_t code, const char *fmt, ...) {
@@ -34,7 +36,8 @@ MI_API int32_t mi_init(int32_t device) {
     if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
         return mi_set_error(MI_EHIP, "mi_init: device %d is %s; this library carries gfx950 code only",
                             device, p.gcnArchName);
-    return MI_OK;
+    void *scratch = nullptr;   // look the built-in attention workspace of this device up now, not inside a later call
+    return attention_static_scratch(&scratch);
 }
 
 MI_API int32_t mi_device_name(char *buf, size_t buflen) {

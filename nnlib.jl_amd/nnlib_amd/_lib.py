@@ -14,6 +14,7 @@ MI_F32, MI_F16, MI_BF16 = 0, 1, 2
 KERNEL_GENERIC, KERNEL_FLASH16, KERNEL_FLASH32, KERNEL_DECODE = 0, 1, 2, 3
 KERNEL_NAMES = {0: "generic", 1: "flash16", 2: "flash32", 3: "decode"}
 MI_ATTN_FORCE_GENERIC = 1
+MI_ATTN_STATIC_WORKSPACE_BYTES = 32 << 20
 MI_SOFTMAX, MI_LOGSOFTMAX = 0, 1
 
 c_i32, c_i64, c_u64, c_f32 = ctypes.c_int32, ctypes.c_int64, ctypes.c_uint64, ctypes.c_float
@@ -67,6 +68,7 @@ SIGNATURES = {
     "mi_attention_plan": (c_i32, [ctypes.POINTER(mi_attn_desc), ctypes.POINTER(c_i32), ctypes.POINTER(c_sz)]),
     "mi_attention_workspace_size": (c_i32, [ctypes.POINTER(mi_attn_desc), ctypes.POINTER(c_sz)]),
     "mi_attention_fwd": (c_i32, [ctypes.POINTER(mi_attn_desc), c_vp]),
+    "mi_attention_fwd_static": (c_i32, [ctypes.POINTER(mi_attn_desc), c_vp]),
     "mi_attention_stats_size": (c_i32, [ctypes.POINTER(mi_attn_desc), ctypes.POINTER(c_sz)]),
     "mi_attention_bwd_plan": (c_i32, [ctypes.POINTER(mi_attn_bwd_desc), ctypes.POINTER(c_i32), ctypes.POINTER(c_sz)]),
     "mi_attention_bwd": (c_i32, [ctypes.POINTER(mi_attn_bwd_desc), c_vp]),
