@@ -67,6 +67,23 @@ def algorithmic_work(w):
     return flops, nbytes
 
 
+PREHEAT_S = 1.0     # seconds of the same launches before the counted warm-up (0 = none)
+
+
+def preheat(step, sync):
+    """Time-based pre-heat: the same launch back to back for PREHEAT_S seconds, so that the counted warm-up and
+    the timed steps run at the clocks of a sustained run rather than on a GPU coming out of idle.  Returns the
+    milliseconds spent.  `--steps` and `--warmup` keep their meaning."""
+    if PREHEAT_S <= 0:
+        return 0.0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < PREHEAT_S:
+        for _ in range(10):
+            step()
+        sync()
+    return (time.perf_counter() - t0) * 1e3
+
+
 class Runner:
     """Owns the device buffers of one workload and launches it through the C ABI."""
 
@@ -139,6 +156,7 @@ class Runner:
         e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
         _lib.check(lib.mi_event_create(ctypes.byref(e0)))
         _lib.check(lib.mi_event_create(ctypes.byref(e1)))
+        self.preheat_ms = preheat(self.step, lambda: _lib.check(lib.mi_device_sync()))
         for _ in range(warmup):
             self.step()
         _lib.check(lib.mi_device_sync())
@@ -214,7 +232,7 @@ def measure(key, steps, warmup, with_cpu):
     else:
         pk = PEAK[w["dtype"]]
         roof = dict(bound="mfma", achieved=tflops, peak=pk, unit="TFLOP/s", frac=tflops / pk, traffic=MEASURED_TRAFFIC.get(key))
-    res = dict(workload=w["name"], kernel=r.kernel, ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, gbps=gbps,
+    res = dict(workload=w["name"], kernel=r.kernel, preheat_ms=r.preheat_ms, ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, gbps=gbps,
                flops_per_step=flops, bytes_per_step=nbytes, roofline=roof)
     if with_cpu:
         c = cpu_baseline(key)
@@ -246,6 +264,7 @@ def _event_time(lib, _lib, fn, steps, warmup):
     e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
     _lib.check(lib.mi_event_create(ctypes.byref(e0)))
     _lib.check(lib.mi_event_create(ctypes.byref(e1)))
+    preheat(fn, lambda: _lib.check(lib.mi_device_sync()))
     for _ in range(warmup):
         fn()
     _lib.check(lib.mi_device_sync())
@@ -406,8 +425,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + sorted(EXTRA) + ["copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--preheat", type=float, default=1.0, help="seconds of untimed launches before the counted warm-up")
     ap.add_argument("--no-decode", action="store_true", help="skip the secondary decode measurement")
     args = ap.parse_args()
+    globals()["PREHEAT_S"] = args.preheat
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only ((head, batch) pairs are independent problems and shard "
                  "without communication). Run with --gpus 1.")
@@ -427,7 +448,7 @@ def main():
         "value": main_res["tflops"] if prefill else main_res["gbps"],
         "unit": "TFLOP/s" if prefill else "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": main_res["ms_per_step"],
+        "ms_per_step": main_res["ms_per_step"], "preheat_ms": main_res["preheat_ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": main_res["workload"], "kernel": main_res["kernel"], "E": w["E"], "Lq": w["Lq"],
