@@ -5,8 +5,8 @@
 
 A "step" is one dot_product_attention call on synthetic inputs that are already resident in HBM.
 The default workload is C3 (bf16 causal prefill, head dim 128, L = 4096), the configuration the
-prefill target is quoted on; the decode workload C5 is measured in the same run and reported under
-"decode" in the same JSON line.  Timing is by HIP events on the stream the kernels are launched on.
+prefill target is quoted on; the other four configurations are measured in the same run and reported under
+"configs" in the same JSON line (C5, the decode target, also under "decode").  Timing is by HIP events on the stream the kernels are launched on.
 """
 import argparse
 import ctypes
@@ -23,12 +23,30 @@ sys.path.insert(0, os.path.join(ROOT, "nnlib.jl_amd"))
 PEAK = {"bf16": 2516.0, "f16": 2516.0, "f32": 157.3}   # dense MFMA TFLOP/s
 HBM_PEAK = 8000.0                                       # GB/s
 HBM_BOUND = ("c4", "c5")                                # workloads priced against the HBM roofline
-# HBM bytes per launch of each workload's dominant kernel, read with rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE in separate runs of this script and scaled by what the same counters read for the
-# 1 GiB copy of --workload copy (factors 2.000 and 1.000); the runs are summarised under profiles/.
+# HBM bytes per launch of each workload's dominant kernel are not measured by this script: they come from
+# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of it, summarised in the file below (which also gives the
+# commands and the copy-kernel calibration), and are read from there so that the figure and its source travel together.
 MIB = 1 << 20
-MEASURED_TRAFFIC = {"c2": (335.5 + 544.0) * MIB, "c3": (429.3 + 64.0) * MIB, "c4": (419.0 + 16.5) * MIB,
-                    "c5": (8192.5 + 16.5) * MIB}
+TRAFFIC_FILE = os.path.join("profiles", "hbm_traffic_fetch_write_size.md")
+DOMINANT_KERNEL = {"c1": "flash32_kernel", "c2": "flash32_kernel", "c3": "flash16_fast_kernel", "c4": "flash16_kernel",
+                   "c5": "decode_split_kernel"}
+
+
+def measured_traffic(key):
+    """(bytes per launch, source) of the workload's dominant kernel from the tracked rocprofv3 summary: the row of
+    its table whose first column is the workload and whose kernel name contains DOMINANT_KERNEL[key]; read MiB +
+    written MiB.  (None, None) when the file has no such row."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 6 and cells[0] == key and DOMINANT_KERNEL.get(key, "\0") in cells[1]:
+                    return (float(cells[4]) + float(cells[5])) * MIB, TRAFFIC_FILE
+    except (OSError, ValueError):
+        pass
+    return None, None
+
+
 ROTATE_BYTES = 1 << 30                                  # input sets rotated until they cover 4x the last-level cache
 
 # name -> description of BASELINE.json's configs
@@ -175,47 +193,58 @@ class Runner:
         return ms.value / steps, wall_ms
 
 
-def cpu_baseline(key, budget_s=15.0):
-    """The CPU oracle (NNlib's op sequence restated in C, Float32, NNlib's thread policy) timed on a
-    bounded sample of the same workload: whole (head, batch) slices of it, as many as fit in about
-    `budget_s` seconds (sized from a one-slice-per-thread trial run), scaled to the whole job."""
+def cpu_baseline(runner, budget_s=10.0):
+    """The CPU oracle (NNlib's op sequence restated in C, Float32, NNlib's thread policy) timed on a bounded sample
+    of the same workload: whole (head, batch) slices of the tensors the GPU was timed on (copied to the host and
+    widened to Float32, as the reference's CPU path would see them), as many as fit in about `budget_s` seconds
+    (sized from a one-slice-per-thread trial run), scaled to the whole job.  The GEMM slices run on the host's BLAS
+    sgemm_ when SciPy's can be bound (what the reference calls, src/gemm.jl:141-149), else on the oracle's own kernel;
+    `sample` says which."""
     import numpy as np
     from oracle import oracle as O
-    w = WORKLOADS[key]
+    w = runner.w
     E, Lq, Lkv, B, H = w["E"], w["Lq"], w["Lkv"], w["B"], w["H"]
     D = E // H
     cores = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
-    rng = np.random.default_rng(w["seed"] & 0xFFFF)
-    f32 = np.float32
+    O.lib()
+    blas = O.use_host_blas()
     mask = None
-    if w.get("mask"):
-        mask = rng.random((Lkv, Lq)) < 0.9
+    if runner.mask is not None:
+        mask = np.asfortranarray(runner.mask.storage.view(Lq, Lkv).cpu().numpy().T.astype(bool))
     if w["causal"]:
         mask = O.make_causal_mask(Lq)
-    O.lib()
+
+    def host(arr, L, nh, nb):      # heads 0..nh-1 of batch elements 0..nb-1 of an (E, L, B) device array
+        t = arr.storage.view(B, L, E)[:nb, :, :nh * D].float().cpu().numpy()
+        return np.asfortranarray(t.transpose(2, 1, 0))
 
     def run(nh, nb):
-        q = np.asfortranarray(rng.standard_normal((nh * D, Lq, nb), dtype=f32) * f32(w["scale"]))
-        k = np.asfortranarray(rng.standard_normal((nh * D, Lkv, nb), dtype=f32) * f32(w["scale"]))
-        v = np.asfortranarray(rng.standard_normal((nh * D, Lkv, nb), dtype=f32))
-        bias = f32(0.5) * rng.standard_normal((Lkv, Lq, nh, nb), dtype=f32) if w.get("bias") else None
+        q, k, v = host(runner.q, Lq, nh, nb), host(runner.k, Lkv, nh, nb), host(runner.v, Lkv, nh, nb)
+        bias = None
+        if runner.bias is not None:
+            t = runner.bias.storage.view(B, H, Lq, Lkv)[:nb, :nh].float().cpu().numpy()
+            bias = np.asfortranarray(t.transpose(3, 2, 1, 0))
         t0 = time.perf_counter()
         O.nnlib_attention_f32(q, k, v, bias, mask, nh, nthreads=cores)
         return time.perf_counter() - t0
 
-    trial_h = min(H, cores)
-    t_trial = run(trial_h, 1)
-    slices = H * B
-    want = int(max(trial_h, min(slices, trial_h * budget_s / max(t_trial, 1e-6))))
-    nh = min(H, want)
-    nb = max(1, min(B, want // nh))
-    dt = run(nh, nb) if nh * nb > trial_h else t_trial
-    n = nh * nb if nh * nb > trial_h else trial_h
+    try:
+        trial_h = min(H, cores)
+        t_trial = run(trial_h, 1)
+        slices = H * B
+        want = int(max(trial_h, min(slices, trial_h * budget_s / max(t_trial, 1e-6))))
+        nh = min(H, want)
+        nb = max(1, min(B, want // nh))
+        dt = run(nh, nb) if nh * nb > trial_h else t_trial
+        n = nh * nb if nh * nb > trial_h else trial_h
+    finally:
+        O.use_host_blas(False)
     flops, nbytes = algorithmic_work(w)
     full_s = dt * slices / n
+    gemm = f"GEMM slices by {blas}" if blas else "GEMM slices by the oracle's own 8x16 SGEMM kernel (no BLAS could be bound)"
     return dict(seconds_sample=dt, seconds_full_job=full_s, cores=cores,
-                sample=f"{n} of {slices} (head, batch) slices of the same workload ({dt:.1f} s), Float32, "
-                       f"{cores} threads over batch slices (NNlib's policy), scaled by {slices / n:.3g}x",
+                sample=f"{n} of {slices} (head, batch) slices of the tensors the GPU was timed on ({dt:.1f} s), Float32, "
+                       f"{cores} threads over batch slices (NNlib's policy), {gemm}, scaled by {slices / n:.3g}x",
                 tflops=flops / full_s / 1e12, gbps=nbytes / full_s / 1e9)
 
 
@@ -227,15 +256,18 @@ def measure(key, steps, warmup, with_cpu):
     tflops = flops / (ms * 1e-3) / 1e12
     gbps = nbytes / (ms * 1e-3) / 1e9
     hbm_bound = key in HBM_BOUND
+    traffic, source = measured_traffic(key)
     if hbm_bound:
-        roof = dict(bound="hbm", achieved=gbps, peak=HBM_PEAK, unit="GB/s", frac=gbps / HBM_PEAK, traffic=MEASURED_TRAFFIC.get(key))
+        roof = dict(bound="hbm", achieved=gbps, peak=HBM_PEAK, unit="GB/s", frac=gbps / HBM_PEAK, traffic=traffic,
+                    traffic_source=source)
     else:
         pk = PEAK[w["dtype"]]
-        roof = dict(bound="mfma", achieved=tflops, peak=pk, unit="TFLOP/s", frac=tflops / pk, traffic=MEASURED_TRAFFIC.get(key))
+        roof = dict(bound="mfma", achieved=tflops, peak=pk, unit="TFLOP/s", frac=tflops / pk, traffic=traffic,
+                    traffic_source=source, hbm_frac=gbps / HBM_PEAK)
     res = dict(workload=w["name"], kernel=r.kernel, preheat_ms=r.preheat_ms, ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, gbps=gbps,
                flops_per_step=flops, bytes_per_step=nbytes, roofline=roof)
     if with_cpu:
-        c = cpu_baseline(key)
+        c = cpu_baseline(r)
         if hbm_bound:
             res["cpu_baseline"] = dict(value=c["gbps"], unit="GB/s", cores=c["cores"], kind="port", sample=c["sample"],
                                        seconds_sample=c["seconds_sample"])
@@ -459,15 +491,24 @@ def main():
     if "cpu_baseline" in main_res:
         line["cpu_baseline"] = main_res["cpu_baseline"]
     if args.workload == "c3" and not args.no_decode:
-        dsteps = max(5, min(args.steps, 50))
-        dec = measure("c5", dsteps, min(args.warmup, 10), not args.no_cpu)
-        line["decode"] = {"metric": "attention GB/s (decode)", "value": dec["gbps"], "unit": "GB/s",
-                          "ms_per_step": dec["ms_per_step"], "steps": dsteps, "dtype": "bf16",
-                          "config": {"workload": dec["workload"], "kernel": dec["kernel"]},
-                          "roofline": dec["roofline"]}
-        if "cpu_baseline" in dec:
-            line["decode"]["cpu_baseline"] = dec["cpu_baseline"]
+        # the other four configurations of BASELINE.json in the same line: C5 (the decode target) also under "decode"
+        line["configs"] = {}
+        for key in ("c1", "c2", "c4", "c5"):
+            ksteps = max(5, min(args.steps, 50))
+            res = measure(key, ksteps, min(args.warmup, 10), not args.no_cpu)
+            hbm = key in HBM_BOUND
+            entry = {"metric": "attention GB/s" if hbm else "attention TFLOP/s", "value": res["gbps"] if hbm else res["tflops"],
+                     "unit": "GB/s" if hbm else "TFLOP/s", "ms_per_step": res["ms_per_step"], "steps": ksteps,
+                     "dtype": WORKLOADS[key]["dtype"], "config": {"workload": res["workload"], "kernel": res["kernel"]},
+                     "roofline": res["roofline"], "flops_per_step": res["flops_per_step"], "bytes_per_step": res["bytes_per_step"]}
+            if "cpu_baseline" in res:
+                entry["cpu_baseline"] = res["cpu_baseline"]
+            line["configs"][key] = entry
+        dec = dict(line["configs"]["c5"])
+        dec["metric"] = "attention GB/s (decode)"
+        line["decode"] = dec
     print(json.dumps(line))
+    sys.stdout.flush()
 
 
 if __name__ == "__main__":

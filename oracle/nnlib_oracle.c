@@ -70,11 +70,31 @@ static inline float op_at(const float *X, int64_t ld, int trans, int64_t r, int6
     return trans ? X[c + r * ld] : X[r + c * ld];
 }
 
+/*
+ * Optional: a BLAS sgemm_ (Fortran interface) to run the slices with, as the reference does
+ * (ccall of sgemm_ through libblastrampoline, src/gemm.jl:141-149).  Unset (NULL) = the kernel
+ * above.  The benchmark's CPU baseline sets it when the host has a BLAS; the parity tests leave
+ * it unset, so parity never depends on a library's rounding.
+ */
+typedef void (*sgemm_fn)(const char *, const char *, const int *, const int *, const int *,
+                         const float *, const float *, const int *, const float *, const int *,
+                         const float *, float *, const int *);
+static sgemm_fn g_sgemm = NULL;
+ORC_API void orc_set_sgemm(void *fn) { g_sgemm = (sgemm_fn)fn; }
+ORC_API int orc_has_sgemm(void) { return g_sgemm != NULL; }
+
 /* trans flags: 0 = 'N', 1 = 'T'. */
 static void sgemm_slice(int transA, int transB, int64_t m, int64_t n, int64_t k, float alpha,
                         const float *A, int64_t lda, const float *B, int64_t ldb, float beta,
                         float *C, int64_t ldc)
 {
+    if (g_sgemm && m > 0 && n > 0 && m < 2147483647 && n < 2147483647 && k < 2147483647 &&
+        lda < 2147483647 && ldb < 2147483647 && ldc < 2147483647) {
+        const char ta = transA ? 'T' : 'N', tb = transB ? 'T' : 'N';
+        const int mi = (int)m, ni = (int)n, ki = (int)k, la = (int)lda, lb = (int)ldb, lc = (int)ldc;
+        g_sgemm(&ta, &tb, &mi, &ni, &ki, &alpha, A, &la, B, &lb, &beta, C, &lc);
+        return;
+    }
     /* reference BLAS semantics: beta == 0 overwrites C without reading it */
     for (int64_t j = 0; j < n; j++)
         for (int64_t i = 0; i < m; i++) {

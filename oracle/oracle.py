@@ -58,8 +58,46 @@ def lib():
             getattr(L, "orc_logsumexp_bwd_" + suf).argtypes = [vp, vp, vp, i64, i64, i64]
             for n in ("orc_softmax_nd_", "orc_logsumexp_", "orc_softmax_bwd_", "orc_logsumexp_bwd_"):
                 getattr(L, n + suf).restype = None
+        L.orc_set_sgemm.argtypes = [vp]
+        L.orc_set_sgemm.restype = None
+        L.orc_has_sgemm.restype = ci
         _LIB = L
     return _LIB
+
+
+def use_host_blas(enable=True):
+    """Run the Float32 GEMM slices of ``batched_gemm`` / ``nnlib_attention_f32`` with the host's BLAS ``sgemm_``, as
+    the reference does (src/gemm.jl:141-149), instead of the oracle's own kernel.  The routine is the one SciPy
+    ships (``scipy.linalg.cython_blas``: OpenBLAS), pinned to one BLAS thread as src/gemm.jl:152-155 pins it inside
+    its threaded loop.  Used by the benchmark's CPU baseline only; parity tests keep the oracle's own kernel.
+    Returns a description of the BLAS in use, or None when none could be bound (the own kernel stays)."""
+    L = lib()
+    if not enable:
+        L.orc_set_sgemm(None)
+        return None
+    try:
+        from scipy.linalg import cython_blas
+        cap = cython_blas.__pyx_capi__["sgemm"]
+        api = ctypes.pythonapi
+        api.PyCapsule_GetName.restype, api.PyCapsule_GetName.argtypes = ctypes.c_char_p, [ctypes.py_object]
+        api.PyCapsule_GetPointer.restype, api.PyCapsule_GetPointer.argtypes = ctypes.c_void_p, [ctypes.py_object, ctypes.c_char_p]
+        fn = api.PyCapsule_GetPointer(cap, api.PyCapsule_GetName(cap))
+        if not fn:
+            return None
+        desc = "SciPy's BLAS sgemm_"
+        try:
+            import threadpoolctl
+            threadpoolctl.threadpool_limits(1, user_api="blas")
+            info = [i for i in threadpoolctl.threadpool_info() if i.get("user_api") == "blas"]
+            if info:
+                desc = f"{info[0].get('internal_api', 'blas')} {info[0].get('version', '')} sgemm_ (SciPy's), 1 BLAS thread"
+        except Exception:
+            pass
+        L.orc_set_sgemm(fn)
+        return desc
+    except Exception:
+        L.orc_set_sgemm(None)
+        return None
 
 
 def _f(a, dt):
