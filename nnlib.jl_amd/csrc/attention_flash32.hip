@@ -90,18 +90,20 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
             for (int qb = 0; qb < QB; qb++)
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++) s[qb][kb] = (floatx16_t){0};
+            // the two key blocks alternate, so that consecutive MFMAs never wait for each other's accumulator
             const float *kt = Ks + (buf * BN + r) * KS + 4 * hh;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int c = 0; c < D / 8; c++) {
+                const floatx4_t k4a = *(const floatx4_t *)(kt + 8 * c);
+                const floatx4_t k4b = *(const floatx4_t *)(kt + 32 * KS + 8 * c);
 #pragma unroll
-                for (int c = 0; c < D / 8; c++) {
-                    const floatx4_t k4 = *(const floatx4_t *)(kt + kb * 32 * KS + 8 * c);
+                for (int j = 0; j < 4; j++)
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-#pragma unroll
-                        for (int qb = 0; qb < QB; qb++)
-                            s[qb][kb] = __builtin_amdgcn_mfma_f32_32x32x2f32(k4[j], f.q[qb][4 * c + j], s[qb][kb], 0, 0, 0);
-                }
+                    for (int qb = 0; qb < QB; qb++) {
+                        s[qb][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(k4a[j], f.q[qb][4 * c + j], s[qb][0], 0, 0, 0);
+                        s[qb][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(k4b[j], f.q[qb][4 * c + j], s[qb][1], 0, 0, 0);
+                    }
+            }
 
             flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0,
                                                                                                           FlashStaged<QB>(), 0, wlds, nullptr, kv_len);

@@ -650,6 +650,20 @@ __device__ inline void flash_zero_skipped_weights(const FlashArgs &a, int64_t b,
     const int lane = threadIdx.x & 63;
     int64_t kcov = from_diag ? ((iw + 32 * QB - 1) / BN + 1) * BN : (int64_t)n_tiles * BN;
     if (kcov > (int64_t)n_tiles * BN) kcov = (int64_t)n_tiles * BN;
+    if (kcov >= p.Lkv) return;
+    constexpr int EPC = 16 / (int)sizeof(TW);   // weights per 16-byte store
+    if (a.w_lds) {
+        // rows start 16-byte aligned and hold a whole number of 16-byte pieces (kcov is a multiple of 64 keys): a
+        // store instruction clears 1 KiB of a row
+        const u32x4_t z = {0, 0, 0, 0};
+        for (int row = 0; row < 32 * QB; row++) {
+            const int64_t qi = iw + row;
+            if (qi >= p.Lq) break;
+            TW *w = (TW *)p.weights + p.Lkv * (qi + p.Lq * (h + p.H * b));
+            for (int64_t kv = kcov + (int64_t)lane * EPC; kv < p.Lkv; kv += 64 * EPC) *(u32x4_t *)(w + kv) = z;
+        }
+        return;
+    }
     for (int row = 0; row < 32 * QB; row++) {
         const int64_t qi = iw + row;
         if (qi >= p.Lq) break;
