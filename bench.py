@@ -20,7 +20,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "nnlib.jl_amd"))
 
-PEAK = {"bf16": 2516.0, "f16": 2516.0, "f32": 157.3}   # dense MFMA TFLOP/s
+PEAK = {"bf16": 2516.0, "f16": 2516.0, "f32": 157.3, "f64": 78.6}   # dense MFMA TFLOP/s
 HBM_PEAK = 8000.0                                       # GB/s
 HBM_BOUND = ("c4", "c5")                                # workloads priced against the HBM roofline
 # HBM bytes per launch of each workload's dominant kernel are not measured by this script: they come from
@@ -289,6 +289,7 @@ EXTRA = {
     "batched_mul": "batched_mul(A, B), A (2048, 2048, 16), B (2048, 2048, 16) bf16",
     "batched_mul_f32": "batched_mul(A, B), A (1024, 64, 128), B (64, 1024, 128) f32: the score product of C2",
     "batched_mul_c32": "batched_mul(A, B), A and B (1024, 1024, 16) ComplexF32, 8 real FLOP per complex multiply-add",
+    "batched_mul_f64": "batched_mul(A, B), A (1024, 1024, 32), B (1024, 1024, 32) Float64",
 }
 
 
@@ -365,6 +366,8 @@ def measure_extra(key, steps, warmup, with_cpu):
             dt_name, (m, kk, n, nb) = "bf16", (2048, 2048, 2048, 16)
         elif key == "batched_mul_c32":
             dt_name, (m, kk, n, nb) = "c64", (1024, 1024, 1024, 16)
+        elif key == "batched_mul_f64":
+            dt_name, (m, kk, n, nb) = "f64", (1024, 1024, 1024, 32)
         else:
             dt_name, (m, kk, n, nb) = "f32", (1024, 64, 1024, 128)
         A, Bm = DA.empty((m, kk, nb), dt_name), DA.empty((kk, n, nb), dt_name)
@@ -372,6 +375,10 @@ def measure_extra(key, steps, warmup, with_cpu):
         for sid, a in enumerate((A, Bm)):
             if dt_name == "c64":   # a complex array is filled as twice as many Float32 values
                 _lib.check(lib.mi_randn_fill(a.ptr, _lib.MI_F32, 2 * a.length, 11, sid, 1.0, None))
+            elif dt_name == "f64":   # Float32 values widened (the generator has no Float64 stream)
+                tmp = DA.empty(a.dims, "f32")
+                _lib.check(lib.mi_randn_fill(tmp.ptr, tmp.code, tmp.length, 11, sid, 1.0, None))
+                a.storage.copy_(tmp.storage.double())
             else:
                 _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, 11, sid, 1.0, None))
         ms = _event_time(lib, _lib, lambda: nn.batched_mul_(C, A, Bm), steps, warmup)
@@ -380,9 +387,9 @@ def measure_extra(key, steps, warmup, with_cpu):
         peak = PEAK["f32"] if dt_name == "c64" else PEAK[dt_name]
         line = dict(metric="batched_mul TFLOP/s", value=val, unit="TFLOP/s", dtype=dt_name,
                     roofline=dict(bound="mfma", achieved=val, peak=peak, unit="TFLOP/s", frac=val / peak, traffic=None),
-                    config=dict(workload=EXTRA[key], kernel="gemm_c32_kernel" if dt_name == "c64" else "batched_gemm_kernel"),
+                    config=dict(workload=EXTRA[key], kernel={"c64": "gemm_c32_kernel", "f64": "gemm64_kernel"}.get(dt_name, "batched_gemm_kernel")),
                     flops_per_step=flops)
-        if with_cpu and dt_name != "c64":
+        if with_cpu and dt_name not in ("c64", "f64"):
             from oracle import oracle as O
             ns = min(nb, 2 if key == "batched_mul" else 32)
             rng = np.random.default_rng(0)

@@ -50,7 +50,11 @@ enum {
 };
 
 /* ---- element types --------------------------------------------------------------- */
-enum { MI_F32 = 0, MI_F16 = 1, MI_BF16 = 2 };
+enum {
+    MI_F32 = 0, MI_F16 = 1, MI_BF16 = 2,
+    /* taken by mi_batched_gemm_f64 / mi_batched_mul_generic only (every other entry point answers MI_EDTYPE) */
+    MI_F64 = 3, MI_C64 = 4 /* ComplexF32 */, MI_C128 = 5 /* ComplexF64 */, MI_I32 = 6, MI_I64 = 7
+};
 
 typedef void *mi_stream; /* a hipStream_t */
 typedef void *mi_event;  /* a hipEvent_t  */
@@ -291,10 +295,33 @@ int32_t mi_batched_mul_c32(int64_t m, int64_t n, int64_t k, float alpha_re, floa
                            int32_t conj_b, float beta_re, float beta_im, void *C, int64_t c_row_stride,
                            int64_t c_col_stride, int64_t c_batch_stride, int64_t batch, mi_stream stream);
 
+/* Float64 batched_mul!: the same call as mi_batched_gemm for the element type the reference hands to dgemm_
+ * (src/gemm.jl:27-32, 141-149; ext/NNlibAMDGPUExt/batched_mul.jl:22 lists Float64 among the rocBLAS types), on the
+ * fp64 matrix cores.  alpha and beta are doubles; beta == 0 overwrites C without reading it. */
+int32_t mi_batched_gemm_f64(char transA, char transB, int64_t m, int64_t n, int64_t k, double alpha, const void *A,
+                            int64_t lda, int64_t strideA, const void *B, int64_t ldb, int64_t strideB, double beta,
+                            void *C, int64_t ldc, int64_t strideC, int64_t batch, mi_stream stream);
+
+/* batched_mul_generic! (src/batched/batchedmul.jl:306-325): what the reference falls back to when no BLAS routine
+ * takes the call: element types that differ between A, B and C (test/batchedmul.jl:41-73: Float64 x Float32,
+ * integers, complex x real), Int32 / Int64, ComplexF64, and layouts that are neither 'N' nor 'T'.  Operands are
+ * given by their element types and by the ELEMENT strides of the (row, column, batch) indices after op, as in
+ * mi_batched_mul_c32; conj_a / conj_b conjugate a complex operand.  dtype_c is the promoted type (Julia's
+ * promote_type of the two): A and B are converted to it element by element and the arithmetic is that type's
+ * (integer products and sums wrap like Julia's).  dtype_c: MI_F32, MI_F64, MI_I32, MI_I64, MI_C64 or MI_C128.
+ * alpha_im / beta_im must be 0 for a real C, alpha and beta integers for an integer C.  A batch stride of 0
+ * shares one slice; beta == 0 overwrites C without reading it. */
+int32_t mi_batched_mul_generic(int32_t dtype_c, int32_t dtype_a, int32_t dtype_b, int64_t m, int64_t n, int64_t k,
+                               double alpha_re, double alpha_im, const void *A, int64_t a_row_stride,
+                               int64_t a_col_stride, int64_t a_batch_stride, int32_t conj_a, const void *B,
+                               int64_t b_row_stride, int64_t b_col_stride, int64_t b_batch_stride, int32_t conj_b,
+                               double beta_re, double beta_im, void *C, int64_t c_row_stride, int64_t c_col_stride,
+                               int64_t c_batch_stride, int64_t batch, mi_stream stream);
+
 /* ---- materialising lazy views ------------------------------------------------------ */
 /* dst (contiguous column-major d0 x d1 x d2) = src read with element strides (s0, s1, s2): the copy(X)
  * the reference makes of a PermutedDimsArray / transposed view before a BLAS call cannot address it
- * (_copy_if_faster, src/batched/batchedmul.jl:76-83).  elem_bytes is 1, 2, 4 or 8. */
+ * (_copy_if_faster, src/batched/batchedmul.jl:76-83).  elem_bytes is 1, 2, 4, 8 or 16. */
 int32_t mi_strided_copy(void *dst, const void *src, int32_t elem_bytes, int64_t d0, int64_t d1, int64_t d2,
                         int64_t s0, int64_t s1, int64_t s2, mi_stream stream);
 /* The same for up to 8 dimensions: permutedims of an N-d array (what Base does for the reference when

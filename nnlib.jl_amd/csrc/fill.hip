@@ -74,8 +74,8 @@ __global__ void convert_kernel(typename TD::type *d, const typename TS::type *s,
 template <int BYTES>
 __global__ void strided_copy_kernel(void *dst, const void *src, int64_t d0, int64_t d1, int64_t d2, int64_t s0, int64_t s1,
                                     int64_t s2) {
-    typedef typename std::conditional<BYTES == 8, uint64_t, typename std::conditional<BYTES == 4, uint32_t,
-            typename std::conditional<BYTES == 2, uint16_t, uint8_t>::type>::type>::type word;
+    typedef typename std::conditional<BYTES == 16, u32x4_t, typename std::conditional<BYTES == 8, uint64_t, typename std::conditional<BYTES == 4, uint32_t,
+            typename std::conditional<BYTES == 2, uint16_t, uint8_t>::type>::type>::type>::type word;
     const int64_t n = d0 * d1 * d2;
     int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -92,8 +92,8 @@ struct CopyDims {
 };
 template <int BYTES>
 __global__ void strided_copy_nd_kernel(void *dst, const void *src, int64_t n, CopyDims g) {
-    typedef typename std::conditional<BYTES == 8, uint64_t, typename std::conditional<BYTES == 4, uint32_t,
-            typename std::conditional<BYTES == 2, uint16_t, uint8_t>::type>::type>::type word;
+    typedef typename std::conditional<BYTES == 16, u32x4_t, typename std::conditional<BYTES == 8, uint64_t, typename std::conditional<BYTES == 4, uint32_t,
+            typename std::conditional<BYTES == 2, uint16_t, uint8_t>::type>::type>::type>::type word;
     int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; idx < n; idx += stride) {
@@ -220,15 +220,16 @@ MI_API int32_t mi_convert(void *dst, int32_t dd, const void *src, int32_t ds, in
 
 MI_API int32_t mi_strided_copy(void *dst, const void *src, int32_t elem_bytes, int64_t d0, int64_t d1, int64_t d2, int64_t s0,
                                int64_t s1, int64_t s2, mi_stream s) {
-    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
-        return mi_set_error(MI_EINVAL, "mi_strided_copy: element size must be 1, 2, 4 or 8 bytes");
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8 && elem_bytes != 16)
+        return mi_set_error(MI_EINVAL, "mi_strided_copy: element size must be 1, 2, 4, 8 or 16 bytes");
     if (d0 < 0 || d1 < 0 || d2 < 0 || s0 < 0 || s1 < 0 || s2 < 0) return mi_set_error(MI_EINVAL, "mi_strided_copy: negative size or stride");
     const int64_t n = d0 * d1 * d2;
     if (n == 0) return MI_OK;
     if (!dst || !src) return mi_set_error(MI_EINVAL, "mi_strided_copy: null pointer");
     dim3 g(grid_for(n)), b(256);
     hipStream_t st = (hipStream_t)s;
-    if (elem_bytes == 8) hipLaunchKernelGGL(strided_copy_kernel<8>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
+    if (elem_bytes == 16) hipLaunchKernelGGL(strided_copy_kernel<16>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
+    else if (elem_bytes == 8) hipLaunchKernelGGL(strided_copy_kernel<8>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
     else if (elem_bytes == 4) hipLaunchKernelGGL(strided_copy_kernel<4>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
     else if (elem_bytes == 2) hipLaunchKernelGGL(strided_copy_kernel<2>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
     else hipLaunchKernelGGL(strided_copy_kernel<1>, g, b, 0, st, dst, src, d0, d1, d2, s0, s1, s2);
@@ -238,8 +239,8 @@ MI_API int32_t mi_strided_copy(void *dst, const void *src, int32_t elem_bytes, i
 
 MI_API int32_t mi_strided_copy_nd(void *dst, const void *src, int32_t elem_bytes, int32_t ndim, const int64_t *sizes,
                                   const int64_t *strides, mi_stream s) {
-    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8)
-        return mi_set_error(MI_EINVAL, "mi_strided_copy_nd: element size must be 1, 2, 4 or 8 bytes");
+    if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4 && elem_bytes != 8 && elem_bytes != 16)
+        return mi_set_error(MI_EINVAL, "mi_strided_copy_nd: element size must be 1, 2, 4, 8 or 16 bytes");
     if (ndim < 0 || ndim > 8 || (ndim > 0 && (!sizes || !strides))) return mi_set_error(MI_EINVAL, "mi_strided_copy_nd: 0 to 8 dimensions");
     CopyDims g;
     g.nd = ndim;
@@ -254,7 +255,8 @@ MI_API int32_t mi_strided_copy_nd(void *dst, const void *src, int32_t elem_bytes
     if (!dst || !src) return mi_set_error(MI_EINVAL, "mi_strided_copy_nd: null pointer");
     dim3 gr(grid_for(n)), b(256);
     hipStream_t st = (hipStream_t)s;
-    if (elem_bytes == 8) hipLaunchKernelGGL(strided_copy_nd_kernel<8>, gr, b, 0, st, dst, src, n, g);
+    if (elem_bytes == 16) hipLaunchKernelGGL(strided_copy_nd_kernel<16>, gr, b, 0, st, dst, src, n, g);
+    else if (elem_bytes == 8) hipLaunchKernelGGL(strided_copy_nd_kernel<8>, gr, b, 0, st, dst, src, n, g);
     else if (elem_bytes == 4) hipLaunchKernelGGL(strided_copy_nd_kernel<4>, gr, b, 0, st, dst, src, n, g);
     else if (elem_bytes == 2) hipLaunchKernelGGL(strided_copy_nd_kernel<2>, gr, b, 0, st, dst, src, n, g);
     else hipLaunchKernelGGL(strided_copy_nd_kernel<1>, gr, b, 0, st, dst, src, n, g);

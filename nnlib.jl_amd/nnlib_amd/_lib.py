@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("MI355ATTN_LIB") or os.path.normpath(os.path.join(_HERE, "..", "lib", "libmi355attn.so"))
 
 MI_OK, MI_EINVAL, MI_EDTYPE, MI_ESHAPE, MI_EHIP, MI_ENOMEM, MI_EWORKSPACE = range(7)
-MI_F32, MI_F16, MI_BF16 = 0, 1, 2
+MI_F32, MI_F16, MI_BF16, MI_F64, MI_C64, MI_C128, MI_I32, MI_I64 = range(8)
 KERNEL_GENERIC, KERNEL_FLASH16, KERNEL_FLASH32, KERNEL_DECODE = 0, 1, 2, 3
 KERNEL_NAMES = {0: "generic", 1: "flash16", 2: "flash32", 3: "decode"}
 MI_ATTN_FORCE_GENERIC = 1
@@ -82,6 +82,11 @@ SIGNATURES = {
                                 c_vp, c_i64, c_i64, c_f32, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "mi_dropout_dims": (c_i32, [c_i32, c_vp, c_vp, c_i32, ctypes.POINTER(c_i64), ctypes.c_uint32, c_f32, c_u64, c_vp]),
     "mi_logsumexp_bwd": (c_i32, [c_i32, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
+    "mi_batched_gemm_f64": (c_i32, [ctypes.c_char, ctypes.c_char, c_i64, c_i64, c_i64, ctypes.c_double, c_vp, c_i64, c_i64,
+                                    c_vp, c_i64, c_i64, ctypes.c_double, c_vp, c_i64, c_i64, c_i64, c_vp]),
+    "mi_batched_mul_generic": (c_i32, [c_i32, c_i32, c_i32, c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_double, c_vp, c_i64, c_i64, c_i64,
+                                       c_i32, c_vp, c_i64, c_i64, c_i64, c_i32, ctypes.c_double, ctypes.c_double, c_vp, c_i64, c_i64,
+                                       c_i64, c_i64, c_vp]),
     "mi_batched_mul_c32": (c_i32, [c_i64, c_i64, c_i64, c_f32, c_f32, c_vp, c_i64, c_i64, c_i64, c_i32, c_vp, c_i64, c_i64, c_i64,
                                    c_i32, c_f32, c_f32, c_vp, c_i64, c_i64, c_i64, c_i64, c_vp]),
     "mi_strided_copy": (c_i32, [c_vp, c_vp, c_i32, c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_vp]),

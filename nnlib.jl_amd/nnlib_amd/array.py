@@ -9,10 +9,20 @@ import torch
 
 from . import _lib
 
-_TORCH = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "bool": torch.uint8, "c64": torch.complex64}
+_TORCH = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "bool": torch.uint8, "c64": torch.complex64,
+          "f64": torch.float64, "c128": torch.complex128, "i32": torch.int32, "i64": torch.int64}
 _CODE = {"f32": _lib.MI_F32, "f16": _lib.MI_F16, "bf16": _lib.MI_BF16}
+# element type codes of the batched_mul entry points, which also take Float64, integers and complex numbers
+_CODE_ANY = dict(_CODE, f64=_lib.MI_F64, c64=_lib.MI_C64, c128=_lib.MI_C128, i32=_lib.MI_I32, i64=_lib.MI_I64)
+_NP = {"f32": np.float32, "f16": np.float16, "bf16": np.float32, "c64": np.complex64, "f64": np.float64, "c128": np.complex128,
+       "i32": np.int32, "i64": np.int64}
+# Default element type for a host array.  NumPy's default float is Float64 where the Julia code this mirrors has
+# Float32 arrays: a float64 host array becomes Float32 unless dtype="f64" is asked for.  Integers and complex128 keep
+# their width (complex128 -> ComplexF64: nothing is narrowed silently).
 _NP2NAME = {np.dtype(np.float32): "f32", np.dtype(np.float16): "f16", np.dtype(np.bool_): "bool",
-            np.dtype(np.uint8): "bool", np.dtype(np.complex64): "c64", np.dtype(np.complex128): "c64"}
+            np.dtype(np.uint8): "bool", np.dtype(np.complex64): "c64", np.dtype(np.complex128): "c128",
+            np.dtype(np.int32): "i32", np.dtype(np.int64): "i64"}
+COMPLEX = ("c64", "c128")
 
 
 def _require_gpu():
@@ -30,7 +40,7 @@ class DeviceArray:
     def __init__(self, storage, dims, dtype, strides=None, offset=0):
         self.storage = storage          # 1-D torch tensor that owns the memory
         self.dims = tuple(int(d) for d in dims)
-        self.dtype = dtype              # "f32" | "f16" | "bf16" | "bool" | "c64" (ComplexF32: batched_mul only)
+        self.dtype = dtype              # "f32" | "f16" | "bf16" | "bool"; batched_mul also takes "f64", "i32", "i64", "c64", "c128"
         self.conj = False               # set by batched_adjoint of a complex array: elements read conjugated
         if strides is None:
             strides, acc = [], 1
@@ -66,8 +76,8 @@ class DeviceArray:
         if dtype == "bool":
             flat = np.ascontiguousarray(a.astype(np.uint8).ravel(order="F"))
             t = torch.from_numpy(flat).cuda()
-        elif dtype == "c64":
-            t = torch.from_numpy(np.ascontiguousarray(a.astype(np.complex64).ravel(order="F"))).cuda()
+        elif dtype in ("c64", "c128", "f64", "i32", "i64"):
+            t = torch.from_numpy(np.ascontiguousarray(a.astype(_NP[dtype]).ravel(order="F"))).cuda()
         else:
             src = a.astype(np.float32) if a.dtype not in (np.float32, np.float16) else a
             flat = np.ascontiguousarray(src.ravel(order="F"))
@@ -161,6 +171,13 @@ class DeviceArray:
             raise _lib.ArgumentError(f"this operation takes Float32, Float16 or BFloat16 arrays, got {self.dtype}")
         return _CODE[self.dtype]
 
+    @property
+    def code_any(self):
+        """Element type code for the batched_mul entry points (every numeric element type)."""
+        if self.dtype not in _CODE_ANY:
+            raise _lib.ArgumentError(f"batched_mul takes numeric arrays, got {self.dtype}")
+        return _CODE_ANY[self.dtype]
+
     # ---- host copies ---------------------------------------------------------------------
     def to_numpy(self):
         """Julia-shaped numpy array (Fortran order). bf16 comes back as float32, bool as bool."""
@@ -206,7 +223,7 @@ def transpose(M):
 def adjoint(M):
     """Lazy conjugate transpose of a matrix (``M'``); equals ``transpose`` for the real element types."""
     out = transpose(M)
-    if M.dtype == "c64":
+    if M.dtype in COMPLEX:
         out.conj = not M.conj
     return out
 
@@ -222,7 +239,7 @@ class BatchedAdjoint(BatchedTranspose):
 def batched_adjoint(A):
     """batched_adjoint(A) (src/batched/batchedadjtrans.jl:50-51): the per-slice conjugate transpose; for the
     real element types it equals batched_transpose.  Taking it twice unwraps."""
-    if A.dtype != "c64":
+    if A.dtype not in COMPLEX:
         return batched_transpose(A)
     return A.parent if isinstance(A, BatchedAdjoint) else BatchedAdjoint(A)
 

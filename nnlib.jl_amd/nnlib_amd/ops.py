@@ -547,10 +547,15 @@ def batched_mul_(C, A, B, alpha=1.0, beta=0.0):
         C3 = C.reshape(C.dims[0], C.dims[1], -1)
         batched_mul_(C3, A.reshape(A.dims[0], A.dims[1], -1), B.reshape(B.dims[0], B.dims[1], -1), alpha, beta)
         return C
-    if not (A.dtype == B.dtype == C.dtype) or A.dtype == "bool":
-        raise ArgumentError("batched_mul! needs one floating-point element type for A, B and C")
-    if A.dtype == "c64":
+    if "bool" in (A.dtype, B.dtype, C.dtype):
+        raise ArgumentError("batched_mul! needs numeric arrays")
+    if A.dtype == B.dtype == C.dtype == "c64":
         return _batched_mul_complex(C, A, B, alpha, beta)
+    if not (A.dtype == B.dtype == C.dtype) or A.dtype not in ("f32", "f16", "bf16", "f64"):
+        # element types that differ, integers, ComplexF64: batched_mul_generic! (src/batched/batchedmul.jl:306-325)
+        return _batched_mul_generic(C, A, B, alpha, beta)
+    if A.dtype == "f64" and not (_is_blas_layout(A) and _is_blas_layout(B) and (C.strides[0] == 1 or C.dims[0] == 1 or C.strides[1] == 1)):
+        return _batched_mul_generic(C, A, B, alpha, beta)
     nb = C.dims[2]
     if A.dims[2] not in (nb, 1):
         raise DimensionMismatch("batch size mismatch: A != C")            # src/gemm.jl:99
@@ -571,8 +576,70 @@ def batched_mul_(C, A, B, alpha=1.0, beta=0.0):
         raise ArgumentError(f"Unsupported array layout for batched mul.\n- Size: {C.dims}\n- Strides: {C.strides}")
     sA = 0 if A.dims[2] == 1 else sA                                     # src/gemm.jl:117-118
     sB = 0 if B.dims[2] == 1 else sB
+    if A.dtype == "f64":     # dgemm_ in the reference (src/gemm.jl:27-32)
+        _lib.check(_lib.load().mi_batched_gemm_f64(tA, tB, m, n, ka, float(alpha), A.ptr, lda, sA, B.ptr, ldb, sB, float(beta),
+                                                   C.ptr, max(C.strides[1], m, 1), C.strides[2], nb, _stream()), DimensionMismatch)
+        return C
     _lib.check(_lib.load().mi_batched_gemm(C.code, tA, tB, m, n, ka, float(alpha), A.ptr, lda, sA, B.ptr, ldb, sB,
                                            float(beta), C.ptr, max(C.strides[1], m, 1), C.strides[2], nb, _stream()),
+               DimensionMismatch)
+    return C
+
+
+def _is_blas_layout(X):
+    """One of the first two strides is 1 (or addresses nothing): 'N' or 'T' for a BLAS call."""
+    return X.strides[0] == 1 or X.strides[1] == 1 or X.dims[0] == 1 or X.dims[1] == 1
+
+
+# Julia's promote_type for the element types batched_mul meets (test/batchedmul.jl:41-73): the result of
+# batched_mul(A, B) has this element type, and batched_mul_generic! computes in it.
+_REAL_RANK = {"i32": 0, "i64": 1, "f16": 2, "bf16": 2, "f32": 3, "f64": 4}
+
+
+def promote_type(a, b):
+    if a == b:
+        return a
+    cplx = a in ("c64", "c128") or b in ("c64", "c128")
+    ra = {"c64": "f32", "c128": "f64"}.get(a, a)
+    rb = {"c64": "f32", "c128": "f64"}.get(b, b)
+    if ra == rb:
+        real = ra
+    elif {ra, rb} == {"f16", "bf16"}:
+        real = "f32"
+    else:
+        hi, lo = (ra, rb) if _REAL_RANK[ra] >= _REAL_RANK[rb] else (rb, ra)
+        real = hi          # an integer joins any float; the wider float wins; Int32 with Int64 gives Int64
+    if cplx:
+        if real in ("i32", "i64"):          # Complex{Int} does not occur here: the complex side fixes the float type
+            real = "f32"
+        return "c128" if real == "f64" else "c64"
+    return real
+
+
+def _batched_mul_generic(C, A, B, alpha, beta):
+    """batched_mul_generic! (src/batched/batchedmul.jl:306-325): any numeric element types and any strides; the
+    arithmetic is that of C's element type, which must be what A's and B's promote to."""
+    if C.conj:
+        raise ArgumentError("batched_mul! cannot write into a batched_adjoint")
+    want = promote_type(A.dtype, B.dtype)
+    if promote_type(want, C.dtype) != C.dtype or C.dtype in ("f16", "bf16"):
+        raise ArgumentError(f"batched_mul!: cannot store the product of {A.dtype} and {B.dtype} arrays into a {C.dtype} array")
+    nb = C.dims[2]
+    if A.dims[2] not in (nb, 1):
+        raise DimensionMismatch("batch size mismatch: A != C")            # src/batched/batchedmul.jl:307-308
+    if B.dims[2] not in (nb, 1):
+        raise DimensionMismatch("batch size mismatch: B != C")
+    m, ka = A.dims[0], A.dims[1]
+    kb, n = B.dims[0], B.dims[1]
+    if ka != kb or m != C.dims[0] or n != C.dims[1]:
+        raise DimensionMismatch(f"A1 has size ({m},{ka}), B1 has size ({kb},{n}), C1 has size {C.dims[:2]}")
+    al, be = complex(alpha), complex(beta)
+    sA = 0 if A.dims[2] == 1 else A.strides[2]
+    sB = 0 if B.dims[2] == 1 else B.strides[2]
+    _lib.check(_lib.load().mi_batched_mul_generic(C.code_any, A.code_any, B.code_any, m, n, ka, al.real, al.imag,
+                                                  A.ptr, A.strides[0], A.strides[1], sA, int(A.conj),
+                                                  B.ptr, B.strides[0], B.strides[1], sB, int(B.conj), be.real, be.imag,
+                                                  C.ptr, C.strides[0], C.strides[1], C.strides[2], nb, _stream()),
                DimensionMismatch)
     return C
 
@@ -630,12 +697,13 @@ def batched_mul(A, B):
         return z.reshape((z.dims[0], z.dims[1]) + tuple(bs))
     if not (A.dims[2] == B.dims[2] or A.dims[2] == 1 or B.dims[2] == 1):
         raise DimensionMismatch("batch size mismatch: A != B")                          # :57-58
-    if A.dtype != B.dtype:
-        raise ArgumentError("batched_mul needs one element type for A and B")
-    C = DeviceArray.empty((A.dims[0], B.dims[1], max(A.dims[2], B.dims[2])), A.dtype)
-    if A.dtype == "c64":
-        return batched_mul_(C, A, B)      # the complex kernel addresses every strided layout itself
-    return batched_mul_(C, _copy_if_faster(A), _copy_if_faster(B))
+    if "bool" in (A.dtype, B.dtype):
+        raise ArgumentError("batched_mul needs numeric arrays")
+    T = promote_type(A.dtype, B.dtype)                         # src/batched/batchedmul.jl:65: promote_type of the eltypes
+    C = DeviceArray.empty((A.dims[0], B.dims[1], max(A.dims[2], B.dims[2])), T)
+    if A.dtype == B.dtype and T in ("f32", "f16", "bf16", "f64"):
+        return batched_mul_(C, _copy_if_faster(A), _copy_if_faster(B))
+    return batched_mul_(C, A, B)          # the complex and generic kernels address every strided layout themselves
 
 
 def batched_vec(A, B):

@@ -159,3 +159,13 @@ def test_host_mirror_shape_errors_without_gpu(L):
         dot_product_attention(fake(6, 3, 1), fake(6, 4, 1), fake(6, 5, 1))
     with pytest.raises(DimensionMismatch, match="batch size mismatch"):      # test/batchedmul.jl:76-78
         batched_mul(fake(2, 2, 2), fake(2, 2, 10))
+
+
+def test_promote_type_table():
+    """Element type of batched_mul(A, B): Julia's promote_type for the pairs test/batchedmul.jl:41-73 exercises."""
+    from nnlib_amd.ops import promote_type as P
+    want = {("f64", "f32"): "f64", ("f64", "f64"): "f64", ("i64", "f64"): "f64", ("i64", "f32"): "f32", ("i64", "i32"): "i64",
+            ("i32", "i32"): "i32", ("c128", "c64"): "c128", ("c128", "f32"): "c128", ("c128", "i64"): "c128", ("c64", "f64"): "c128",
+            ("c64", "f32"): "c64", ("c64", "i64"): "c64", ("f16", "f32"): "f32", ("bf16", "f16"): "f32", ("f32", "f32"): "f32"}
+    for (a, b), t in want.items():
+        assert P(a, b) == t and P(b, a) == t, (a, b)

@@ -266,8 +266,11 @@ def test_complex_adjoints(nn, oracle):
     _close(nn.batched_mul(nn.batched_transpose(dA), dC).to_numpy(), P(cA, cC, transA=True))
     assert nn.batched_adjoint(nn.batched_adjoint(dA)) is dA
     _close(nn.batched_adjoint(dA).to_numpy(), np.conj(np.transpose(cA, (1, 0, 2))))
-    with pytest.raises(nn.ArgumentError):
-        nn.batched_mul(dA, D(np.ones((5, 7, 3), dtype=np.float32)))        # one element type for both
+    # element types that differ promote as in the reference (test/batchedmul.jl:73): ComplexF32 x Float32 -> ComplexF32
+    ones = np.ones((5, 7, 3), dtype=np.float32)
+    mixed = nn.batched_mul(dA, D(ones))
+    assert mixed.dtype == "c64"
+    _close(mixed.to_numpy(), P(cA, ones.astype(np.complex64)))
 
 
 @pytest.mark.parametrize("perm", [(1, 3, 2), (2, 1, 3), (3, 2, 1)])
