@@ -189,9 +189,12 @@ int32_t mi_attention_fwd_static(const mi_attn_desc *desc, mi_stream stream);
  *
  *   fwd      : the forward call (dtype, sizes, q, k, v, bias, mask, causal, flags, and dropout_p /
  *              dropout_seed when the forward call dropped weights: the keep decisions are redrawn
- *              from the same stream, and the pullback of dropout multiplies by them).  fwd.out may
- *              hold the forward RESULT x; the MFMA kernels (f16 / bf16: head dim a multiple of 8 up to 256; f32: of 4 up to 128)
- *              need it and the call falls back to the generic kernels without it.  fwd.weights and fwd.workspace are ignored.
+ *              from the same stream, and the pullback of dropout multiplies by them).  fwd.out holds the
+ *              forward RESULT x, or NULL when the caller did not keep it: the MFMA kernels (f16 / bf16: head dim a
+ *              multiple of 8 up to 256; f32: of 4 up to 128) need it, and where they can take the call the library
+ *              recomputes it with one forward call into the workspace (mi_attention_bwd_plan sizes the workspace for
+ *              that, and it must then be 256-byte aligned); otherwise the generic kernels run.  fwd.weights and
+ *              fwd.workspace are ignored.
  *   dout     : (Ev, Lq, B) cotangent of x, `dtype`.
  *   dweights : NULL, or (Lkv, Lq, H, B) cotangent of the returned weights, `dtype`.
  *   dq, dk, dv : gradients with the shapes of q, k, v, `dtype`; any may be NULL (not computed).

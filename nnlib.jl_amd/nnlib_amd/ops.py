@@ -243,8 +243,8 @@ def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, m
     otherwise (Float32).  The reference gets the same values from AD through src/attention.jl:86-127
     (rrule of batched_mul, src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110; the
     pullback of dropout multiplies by the mask it drew, src/dropout.jl:38-53).
-    ``y`` is the forward result, which the MFMA kernels need; without it (and without ``dalpha``) it is recomputed
-    by one forward call where those kernels can take the gradient."""
+    ``y`` is the forward result, which the MFMA kernels need; without it (and without ``dalpha``) the library
+    recomputes it with one forward call where those kernels can take the gradient."""
     global _last_bwd_kernel
     B, E, Ev, Lq, Lkv, bq = _check_qkv(q, k, v, nheads)
     dy = _contig(dy, "dy")
@@ -276,19 +276,8 @@ def dot_product_attention_grad(dy, q, k, v, bias=None, *, y=None, dalpha=None, m
         dbias = DeviceArray.zeros(bias.dims, "f32")
         d.dbias = dbias.ptr
     kernel, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
-    if y is None and dalpha is None:
-        # Without the forward result only the generic kernels can run (hundreds of times slower on the shapes the
-        # MFMA kernels take): ask the planner what it would pick with a result in place, and if that is an MFMA
-        # family, recompute the result with one forward call.
-        d.fwd.out = dy.ptr                      # a stand-in of the right size and alignment; planning reads no memory
-        _lib.check(lib.mi_attention_bwd_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))
-        d.fwd.out = None
-        if kernel.value != _lib.KERNEL_GENERIC:
-            y, _ = dot_product_attention(q, k, v, bias, fdrop=fdrop, mask=mask, nheads=nheads, return_weights=False,
-                                         save_for_backward=True, _flags=_flags)
-            d.fwd.out = y.ptr
-            if getattr(y, "saved_stats", None) is not None:
-                d.fwd.stats = y.saved_stats.ptr
+    # without the forward result the library recomputes it where its MFMA kernels can take the gradient (the plan's
+    # workspace has room for it)
     _lib.check(lib.mi_attention_bwd_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))
     wbuf, wsize = _get_workspace(ws.value)
     if wbuf is not None:

@@ -300,6 +300,12 @@ def test_forward_result_is_recomputed_when_missing(nn, oracle, dtype, D, expect)
     _run(nn, oracle, dtype, 2 * D, 2 * D, 130, 200, (2,), 2, mask_kind="random", pass_y=False, expect=expect, seed=11, scale=0.5)
     _run(nn, oracle, dtype, 2 * D, 2 * D, 150, 150, (1,), 2, mask_kind="causal", pass_y=False, expect=expect, seed=12, scale=0.5,
          dropout=(0.2, 99))
+    # a single query: the forward call that recomputes the result is the split-kv kernel, which saves no row statistics
+    _run(nn, oracle, dtype, 2 * D, 2 * D, 1, 700, (3,), 2, mask_kind=None, pass_y=False, expect=expect, seed=13, scale=0.5)
+    # key-padding mask (the forward call measures context lengths in its workspace) and a bias with its gradient
+    _run(nn, oracle, dtype, 2 * D, 2 * D, 140, 330, (3,), 2, mask_kind="lengths", pass_y=False, expect=expect, seed=14, scale=0.5)
+    _run(nn, oracle, dtype, 2 * D, 2 * D, 70, 200, (2,), 2, mask_kind=None, bias_shape=(200, 70, 2, 1), pass_y=False, expect=expect,
+         seed=15, scale=0.5)
 
 
 def test_mfma_and_generic_kernels_agree(nn):
