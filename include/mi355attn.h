@@ -270,6 +270,25 @@ int32_t mi_softmax_bwd(int32_t op, int32_t dtype, const void *dy, const void *y,
 int32_t mi_logsumexp_bwd(int32_t dtype, const void *dy, const void *x, const void *lse, void *dx,
                          int64_t inner, int64_t len, int64_t outer, mi_stream stream);
 
+/* The same four operations over ANY set of dimensions of an N-d column-major array (N <= 8), as the reference's
+ * `dims` keyword takes (src/softmax.jl:56, 133, 200; Base's reductions accept any dims).  sizes: the N extents, a HOST
+ * array; dims_mask: bit d set = dimension d + 1 is reduced over (dimensions past N are ignored, having extent 1).  A
+ * set that is a run of adjacent dimensions goes straight to the kernels above; any other set is permuted to the front,
+ * reduced and permuted back inside the library (what permutedims does for the reference), through a caller workspace
+ * of mi_softmax_dims_workspace() bytes (0 for a run), 16-byte aligned.  y of mi_logsumexp_dims and dy / lse of
+ * mi_logsumexp_bwd_dims have the size of x with extent 1 along the reduced dimensions. */
+int32_t mi_softmax_dims_workspace(int32_t dtype, int32_t ndim, const int64_t *sizes, uint32_t dims_mask, size_t *bytes);
+int32_t mi_softmax_dims(int32_t op, int32_t dtype, const void *x, void *y, int32_t ndim, const int64_t *sizes,
+                        uint32_t dims_mask, void *workspace, size_t workspace_bytes, mi_stream stream);
+int32_t mi_logsumexp_dims(int32_t dtype, const void *x, void *y, int32_t ndim, const int64_t *sizes, uint32_t dims_mask,
+                          void *workspace, size_t workspace_bytes, mi_stream stream);
+int32_t mi_softmax_bwd_dims(int32_t op, int32_t dtype, const void *dy, const void *y, void *dx, int32_t ndim,
+                            const int64_t *sizes, uint32_t dims_mask, void *workspace, size_t workspace_bytes,
+                            mi_stream stream);
+int32_t mi_logsumexp_bwd_dims(int32_t dtype, const void *dy, const void *x, const void *lse, void *dx, int32_t ndim,
+                              const int64_t *sizes, uint32_t dims_mask, void *workspace, size_t workspace_bytes,
+                              mi_stream stream);
+
 /* ---- batched GEMM ---------------------------------------------------------------- */
 /* C[:,:,b] = alpha * op(A[:,:,b]) * op(B[:,:,b]) + beta * C[:,:,b],  b in [0, batch).
  * The signature follows the backend hook NNlib._batched_gemm!(transA, transB, alpha,

@@ -78,6 +78,11 @@ SIGNATURES = {
     "mi_softmax": (c_i32, [c_i32, c_i32, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "mi_logsumexp": (c_i32, [c_i32, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "mi_softmax_bwd": (c_i32, [c_i32, c_i32, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, c_vp]),
+    "mi_softmax_dims_workspace": (c_i32, [c_i32, c_i32, ctypes.POINTER(c_i64), ctypes.c_uint32, ctypes.POINTER(c_sz)]),
+    "mi_softmax_dims": (c_i32, [c_i32, c_i32, c_vp, c_vp, c_i32, ctypes.POINTER(c_i64), ctypes.c_uint32, c_vp, c_sz, c_vp]),
+    "mi_logsumexp_dims": (c_i32, [c_i32, c_vp, c_vp, c_i32, ctypes.POINTER(c_i64), ctypes.c_uint32, c_vp, c_sz, c_vp]),
+    "mi_softmax_bwd_dims": (c_i32, [c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, ctypes.POINTER(c_i64), ctypes.c_uint32, c_vp, c_sz, c_vp]),
+    "mi_logsumexp_bwd_dims": (c_i32, [c_i32, c_vp, c_vp, c_vp, c_vp, c_i32, ctypes.POINTER(c_i64), ctypes.c_uint32, c_vp, c_sz, c_vp]),
     "mi_batched_gemm": (c_i32, [c_i32, ctypes.c_char, ctypes.c_char, c_i64, c_i64, c_i64, c_f32, c_vp, c_i64, c_i64,
                                 c_vp, c_i64, c_i64, c_f32, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "mi_dropout_dims": (c_i32, [c_i32, c_vp, c_vp, c_i32, ctypes.POINTER(c_i64), ctypes.c_uint32, c_f32, c_u64, c_vp]),

@@ -352,22 +352,26 @@ def _reduction_geometry(dims_of_x, dims):
     return prod(size[:lo]), prod(size[lo:hi]), prod(size[hi:]), kept
 
 
-def _nonadjacent_plan(dims_of_x, dims):
-    """None when ``dims`` is ``None`` or a run of adjacent dimensions; otherwise ``(perm, inverse, k)``: the 1-based
-    permutation that brings the ``k`` reduced dimensions to the front (Base's reductions take any ``dims``; the
-    kernels take runs, so other sets go through ``permutedims`` there and back)."""
+def _dims_call(x, dims):
+    """Arguments of the `*_dims` entry points for a reduction of ``x`` over ``dims`` (a 1-based dimension, a tuple of
+    dimensions, adjacent or not, or ``None`` for Julia's ``:``): (ndim, sizes, mask, workspace pointer, workspace
+    bytes, size of the reduced result).  The library permutes sets that are not runs of adjacent dimensions."""
+    size = tuple(x.dims)
+    if len(size) > 8:
+        raise ArgumentError("the softmax family takes arrays of up to 8 dimensions")
     if dims is None:
-        return None
-    n = len(dims_of_x)
-    ds = sorted({int(d) for d in (dims if isinstance(dims, (tuple, list)) else (dims,))})
-    if not ds or ds[0] < 1:
-        raise ArgumentError(f"dims must be positive dimension numbers, got {dims}")
-    ds = [d for d in ds if d <= n]
-    if not ds or ds == list(range(ds[0], ds[-1] + 1)):
-        return None
-    perm = ds + [d for d in range(1, n + 1) if d not in ds]
-    inverse = [perm.index(d) + 1 for d in range(1, n + 1)]
-    return tuple(perm), tuple(inverse), len(ds)
+        ds, kept = list(range(1, len(size) + 1)), ()
+    else:
+        ds = sorted({int(d) for d in (dims if isinstance(dims, (tuple, list)) else (dims,))})
+        if not ds or ds[0] < 1:
+            raise ArgumentError(f"dims must be positive dimension numbers, got {dims}")
+        kept = tuple(1 if (i + 1) in ds else d for i, d in enumerate(size))
+    mask = sum(1 << (d - 1) for d in ds if d <= len(size))
+    sizes = (ctypes.c_int64 * max(len(size), 1))(*size)
+    nb = ctypes.c_size_t(0)
+    _lib.check(_lib.load().mi_softmax_dims_workspace(x.code, len(size), sizes, mask, ctypes.byref(nb)))
+    wbuf, wsize = _get_workspace(nb.value)
+    return len(size), sizes, mask, (wbuf.data_ptr() if wbuf is not None else None), wsize, kept
 
 
 def _assign(out, y):
@@ -391,14 +395,8 @@ def _softmax_like(name, op, out, x, dims):
         raise DimensionMismatch(f"output size {out.dims} differs from input size {x.dims}")
     if x.dtype == "bool" or out.dtype != x.dtype:
         raise ArgumentError(f"{name} needs floating-point input and output of one element type")
-    plan = _nonadjacent_plan(x.dims, dims)
-    if plan is not None:
-        perm, inverse, k = plan
-        xp = x.permuted(*perm).copy()
-        yp = _softmax_like(name, op, DeviceArray.empty(xp.dims, xp.dtype), xp, tuple(range(1, k + 1)))
-        return _assign(out, yp.permuted(*inverse).copy())
-    inner, n, outer, _ = _reduction_geometry(x.dims, dims)
-    _lib.check(_lib.load().mi_softmax(op, x.code, x.ptr, out.ptr, inner, n, outer, _stream()))
+    nd, sizes, mask, ws, wsize, _ = _dims_call(x, dims)
+    _lib.check(_lib.load().mi_softmax_dims(op, x.code, x.ptr, out.ptr, nd, sizes, mask, ws, wsize, _stream()))
     return out
 
 
@@ -434,13 +432,9 @@ def logsumexp(x, *, dims=None):
     x = _contig(x, "x")
     if x.dtype == "bool":
         raise ArgumentError("logsumexp needs a floating-point array")
-    plan = _nonadjacent_plan(x.dims, dims)
-    if plan is not None:
-        perm, inverse, k = plan
-        return logsumexp(x.permuted(*perm).copy(), dims=tuple(range(1, k + 1))).permuted(*inverse).copy()
-    inner, n, outer, kept = _reduction_geometry(x.dims, dims)
+    nd, sizes, mask, ws, wsize, kept = _dims_call(x, dims)
     out = DeviceArray.empty(kept, x.dtype)
-    _lib.check(_lib.load().mi_logsumexp(x.code, x.ptr, out.ptr, inner, n, outer, _stream()))
+    _lib.check(_lib.load().mi_logsumexp_dims(x.code, x.ptr, out.ptr, nd, sizes, mask, ws, wsize, _stream()))
     return out
 
 
@@ -450,20 +444,15 @@ def grad_logsumexp(dy, x, *, dims=None, lse=None):
     if not isinstance(x, DeviceArray) or not isinstance(dy, DeviceArray):
         raise _number_error("logsumexp")
     x, dy = _contig(x, "x"), _contig(dy, "dy")
-    plan = _nonadjacent_plan(x.dims, dims)
-    if plan is not None:
-        perm, inverse, k = plan
-        front = tuple(range(1, k + 1))
-        lp = None if lse is None else _contig(lse, "lse").permuted(*perm).copy()
-        return grad_logsumexp(dy.permuted(*perm).copy(), x.permuted(*perm).copy(), dims=front, lse=lp).permuted(*inverse).copy()
-    inner, n, outer, kept = _reduction_geometry(x.dims, dims)
     if lse is None:
         lse = logsumexp(x, dims=dims)
     lse = _contig(lse, "lse")
-    if dy.length != inner * outer or lse.length != inner * outer or not (dy.dtype == lse.dtype == x.dtype):
+    nd, sizes, mask, ws, wsize, kept = _dims_call(x, dims)
+    n_out = int(np.prod(kept, dtype=np.int64)) if kept else 1
+    if dy.length != n_out or lse.length != n_out or not (dy.dtype == lse.dtype == x.dtype):
         raise DimensionMismatch(f"dy and lse must have the size {kept} of logsumexp(x; dims) and the element type of x")
     dx = DeviceArray.empty(x.dims, x.dtype)
-    _lib.check(_lib.load().mi_logsumexp_bwd(x.code, dy.ptr, x.ptr, lse.ptr, dx.ptr, inner, n, outer, _stream()))
+    _lib.check(_lib.load().mi_logsumexp_bwd_dims(x.code, dy.ptr, x.ptr, lse.ptr, dx.ptr, nd, sizes, mask, ws, wsize, _stream()))
     return dx
 
 
@@ -473,14 +462,8 @@ def _softmax_grad(name, op, dx, dy, y, dims):
         raise DimensionMismatch(f"{name}: dx {dx.dims}, dy {dy.dims} and y {y.dims} must have one size")
     if y.dtype == "bool" or not (dy.dtype == y.dtype == dx.dtype):
         raise ArgumentError(f"{name} needs one floating-point element type for dx, dy and y")
-    plan = _nonadjacent_plan(y.dims, dims)
-    if plan is not None:
-        perm, inverse, k = plan
-        yp, dyp = y.permuted(*perm).copy(), dy.permuted(*perm).copy()
-        dxp = _softmax_grad(name, op, DeviceArray.empty(yp.dims, yp.dtype), dyp, yp, tuple(range(1, k + 1)))
-        return _assign(dx, dxp.permuted(*inverse).copy())
-    inner, n, outer, _ = _reduction_geometry(y.dims, dims)
-    _lib.check(_lib.load().mi_softmax_bwd(op, y.code, dy.ptr, y.ptr, dx.ptr, inner, n, outer, _stream()))
+    nd, sizes, mask, ws, wsize, _ = _dims_call(y, dims)
+    _lib.check(_lib.load().mi_softmax_bwd_dims(op, y.code, dy.ptr, y.ptr, dx.ptr, nd, sizes, mask, ws, wsize, _stream()))
     return dx
 
 
