@@ -16,8 +16,12 @@
 #   Dropout(p, seed) as fdrop, dropout(x, p)                       NNlib src/dropout.jl:38-53
 #   ∇dot_product_attention, batched_mul_pullback                   what AD derives from src/attention.jl:86-127
 #
-# All arithmetic happens in the library.  This file has not been executed in the build environment
-# (no Julia toolchain there); the Python mirror in nnlib_amd/ exercises the same entry points.
+# All arithmetic AND all planning (kernel choice, workspace sizes, recomputing a forward result the caller did not
+# keep, permuting for reductions over dimensions that are not neighbours, element type promotion of mixed products)
+# happen in the library: every function below checks sizes the way NNlib does, allocates outputs and workspace, and
+# makes one ccall.  ext/NNlibMI355Ext.jl forwards NNlib's own generics to these methods when NNlib is loaded.
+# This file has not been executed in the build environment (no Julia toolchain there); the Python mirror in
+# nnlib_amd/ exercises the same entry points.
 module MI355Attention
 
 export DeviceArray, CausalMask, CausalAnd, dot_product_attention, dot_product_attention_scores, make_causal_mask,
@@ -25,17 +29,24 @@ export DeviceArray, CausalMask, CausalAnd, dot_product_attention, dot_product_at
        batched_mul, batched_mul!, batched_vec, batched_transpose, batched_adjoint, batched_mul_pullback,
        Dropout, dropout, ∇dot_product_attention
 
-const libmi = get(ENV, "MI355ATTN_LIB", joinpath(@__DIR__, "..", "lib", "libmi355attn.so"))
+const libmi = get(ENV, "MI355ATTN_LIB", joinpath(@__DIR__, "..", "..", "lib", "libmi355attn.so"))
 
 # ---- status codes and element types (include/mi355attn.h) ----------------------------------------
 const MI_OK, MI_EINVAL, MI_EDTYPE, MI_ESHAPE, MI_EHIP, MI_ENOMEM, MI_EWORKSPACE = Int32.(0:6)
-const MI_F32, MI_F16, MI_BF16 = Int32(0), Int32(1), Int32(2)
+const MI_F32, MI_F16, MI_BF16, MI_F64, MI_C64, MI_C128, MI_I32, MI_I64 = Int32.(0:7)
 
 primitive type BFloat16 <: AbstractFloat 16 end     # storage only; use BFloat16s.jl for arithmetic
 const MIFloat = Union{Float32, Float16, BFloat16}
 dtype_code(::Type{Float32}) = MI_F32
 dtype_code(::Type{Float16}) = MI_F16
 dtype_code(::Type{BFloat16}) = MI_BF16
+# element types only batched_mul takes
+dtype_code(::Type{Float64}) = MI_F64
+dtype_code(::Type{ComplexF32}) = MI_C64
+dtype_code(::Type{ComplexF64}) = MI_C128
+dtype_code(::Type{Int32}) = MI_I32
+dtype_code(::Type{Int64}) = MI_I64
+const MINumber = Union{MIFloat, Float64, ComplexF32, ComplexF64, Int32, Int64}
 
 last_error() = unsafe_string(ccall((:mi_last_error_string, libmi), Cstring, ()))
 
@@ -83,7 +94,7 @@ function free!(a::DeviceArray)
     nothing
 end
 
-function DeviceArray(h::Array{T, N}) where {T <: Union{MIFloat, Bool, ComplexF32}, N}
+function DeviceArray(h::Array{T, N}) where {T <: Union{MINumber, Bool}, N}
     d = DeviceArray{T}(undef, size(h)...)
     check(ccall((:mi_memcpy_h2d, libmi), Int32, (Ptr{Cvoid}, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}), d.ptr, h, sizeof(h), C_NULL))
     d
@@ -300,7 +311,7 @@ end
 # NNlib gets these from AD through src/attention.jl:86-127 (rrule of batched_mul,
 # src/batched/batchedmul.jl:96-110; _∇softmax!, src/softmax.jl:107-110; the pullback of dropout
 # multiplies by the mask it drew, src/dropout.jl:38-53).  `y` is the forward result, which the MFMA kernels
-# need; without it (and without dα) one forward call recomputes it where those kernels can take the gradient.
+# need; without it (and without dα) the library recomputes it where those kernels can take the gradient.
 # A ChainRulesCore.rrule for DeviceArray arguments is three lines
 # on top of this function: call the forward, close over (q, k, v, bias, y), return this pullback.
 function ∇dot_product_attention(dy::DeviceArray{T, 3}, q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::DeviceArray{T, 3},
@@ -315,18 +326,8 @@ function ∇dot_product_attention(dy::DeviceArray{T, 3}, q::DeviceArray{T, 3}, k
     p, seed = fdrop isa Dropout ? (fdrop.p, fdrop.seed) : (0f0, UInt64(0))
     fwd_desc(yptr) = AttnDesc(Int32(sizeof(AttnDesc)), dtype_code(T), dtype_code(T), causal, UInt32(0), Int32(0), E, Ev, Lq, Lkv, nheads, B,
                               q.ptr, k.ptr, v.ptr, yptr, C_NULL, bptr, bstr, mptr, mstr, C_NULL, 0, p, UInt32(0), seed, stats === nothing ? C_NULL : stats.ptr)
-    if y === nothing && dα === nothing
-        # Without the forward result only the generic kernels can run (hundreds of times slower on the shapes the
-        # MFMA kernels take): ask the planner what it would pick with a result in place (dy stands in: the right
-        # size and alignment, and planning reads no memory); if that is an MFMA family, recompute the result.
-        kern = Ref{Int32}(0)
-        probe = AttnBwdDesc(Int32(sizeof(AttnBwdDesc)), Int32(0), fwd_desc(dy.ptr), dy.ptr, C_NULL, dq.ptr, dk.ptr, dv.ptr,
-                            dbias === nothing ? C_NULL : dbias.ptr, C_NULL, 0)
-        check(ccall((:mi_attention_bwd_plan, libmi), Int32, (Ref{AttnBwdDesc}, Ptr{Int32}, Ptr{Csize_t}), probe, kern, C_NULL))
-        if kern[] != 0      # MI_ATTN_KERNEL_GENERIC
-            y, _ = dot_product_attention(q, k, v, bias; fdrop, mask, nheads, return_weights = false)
-        end
-    end
+    # y === nothing: the library recomputes the forward result where its MFMA kernels can take the gradient; the
+    # workspace mi_attention_bwd_plan asks for has room for it
     fwd = fwd_desc(y === nothing ? C_NULL : y.ptr)
     mk(ws, wsbytes) = AttnBwdDesc(Int32(sizeof(AttnBwdDesc)), Int32(0), fwd, dy.ptr, dα === nothing ? C_NULL : dα.ptr, dq.ptr, dk.ptr,
                                   dv.ptr, dbias === nothing ? C_NULL : dbias.ptr, ws, wsbytes)
@@ -353,24 +354,28 @@ end
 # ---- softmax family (NNlib src/softmax.jl) ---------------------------------------------------------
 const MI_SOFTMAX, MI_LOGSOFTMAX = Int32(0), Int32(1)
 
-# (inner, len, outer) of a reduction over `dims` (an integer, a tuple of adjacent dimensions, or :)
-function reduction_geometry(sz::Dims, dims)
-    dims isa Colon && return (1, prod(sz), 1)
-    ds = sort!(unique!(collect(Int, dims)))
-    (isempty(ds) || first(ds) < 1) && throw(ArgumentError("dims must be positive dimension numbers, got $dims"))
-    ds == collect(first(ds):last(ds)) ||
-        throw(ArgumentError("dims = $dims: only runs of adjacent dimensions are supported on device arrays"))
-    ext(d) = d <= length(sz) ? sz[d] : 1
-    n = max(length(sz), last(ds))
-    (prod(ext, 1:first(ds)-1; init = 1), prod(ext, ds; init = 1), prod(ext, last(ds)+1:n; init = 1))
+# dims (an integer, a tuple of dimensions, adjacent or not, or :) as the bit mask of the *_dims entry points, the
+# sizes as a host vector, and a workspace of the size the library asks for (0 bytes for a run of adjacent dimensions)
+function dims_call(x::DeviceArray{T, N}, dims) where {T, N}
+    N <= 8 || throw(ArgumentError("the softmax family takes arrays of up to 8 dimensions"))
+    ds = dims isa Colon ? collect(1:N) : collect(Int, dims)
+    (isempty(ds) || minimum(ds) < 1) && throw(ArgumentError("dims must be positive dimension numbers, got $dims"))
+    mask = UInt32(sum(d -> UInt32(1) << (d - 1), filter(d -> d <= N, unique(ds)); init = UInt32(0)))
+    sizes = collect(Int64, size(x))
+    need = Ref{Csize_t}(0)
+    check(ccall((:mi_softmax_dims_workspace, libmi), Int32, (Int32, Int32, Ptr{Int64}, UInt32, Ptr{Csize_t}),
+                dtype_code(T), Int32(N), sizes, mask, need))
+    ws = need[] > 0 ? DeviceArray{UInt8}(undef, Int(need[])) : nothing
+    sizes, mask, ws, need[]
 end
+wsptr(ws) = ws === nothing ? C_NULL : ws.ptr
 
-function softmax_like!(op::Int32, out::DeviceArray{T}, x::DeviceArray{T}, dims) where {T <: MIFloat}
+function softmax_like!(op::Int32, out::DeviceArray{T, N}, x::DeviceArray{T, N}, dims) where {T <: MIFloat, N}
     size(out) == size(x) || throw(DimensionMismatch("output size $(size(out)) differs from input size $(size(x))"))
-    inner, len, outer = reduction_geometry(size(x), dims)
-    GC.@preserve out x check(ccall((:mi_softmax, libmi), Int32,
-                                   (Int32, Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
-                                   op, dtype_code(T), x.ptr, out.ptr, inner, len, outer, C_NULL))
+    sizes, mask, ws, wsb = dims_call(x, dims)
+    GC.@preserve out x sizes ws check(ccall((:mi_softmax_dims, libmi), Int32,
+        (Int32, Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int32, Ptr{Int64}, UInt32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+        op, dtype_code(T), x.ptr, out.ptr, Int32(N), sizes, mask, wsptr(ws), wsb, C_NULL))
     out
 end
 
@@ -385,33 +390,34 @@ logsoftmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloa
 # logsumexp(x; dims = :) returns a scalar for dims = : (one device-to-host copy), else an array that
 # keeps the reduced dimensions with extent 1, as NNlib's does (src/softmax.jl:200-203).
 function logsumexp(x::DeviceArray{T, N}; dims = :) where {T <: MIFloat, N}
-    inner, len, outer = reduction_geometry(size(x), dims)
+    sizes, mask, ws, wsb = dims_call(x, dims)
     kept = dims isa Colon ? () : ntuple(d -> d in dims ? 1 : size(x, d), N)
     out = similar(x, T, kept)
-    GC.@preserve out x check(ccall((:mi_logsumexp, libmi), Int32,
-                                   (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
-                                   dtype_code(T), x.ptr, out.ptr, inner, len, outer, C_NULL))
+    GC.@preserve out x sizes ws check(ccall((:mi_logsumexp_dims, libmi), Int32,
+        (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Int32, Ptr{Int64}, UInt32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+        dtype_code(T), x.ptr, out.ptr, Int32(N), sizes, mask, wsptr(ws), wsb, C_NULL))
     dims isa Colon ? Array(out)[] : out
 end
 
 # Pullback of logsumexp (rrule at src/softmax.jl:205-212): dy and lse are device arrays with the size of the
 # reduced result (for dims = : a 0-dimensional or one-element array holding the cotangent / the result).
-function ∇logsumexp(dy::DeviceArray{T}, x::DeviceArray{T}, lse::DeviceArray{T}; dims = :) where {T <: MIFloat}
-    inner, len, outer = reduction_geometry(size(x), dims)
-    length(dy) == length(lse) == inner * outer || throw(DimensionMismatch("dy and lse must have the size of logsumexp(x; dims)"))
+function ∇logsumexp(dy::DeviceArray{T}, x::DeviceArray{T, N}, lse::DeviceArray{T}; dims = :) where {T <: MIFloat, N}
+    sizes, mask, ws, wsb = dims_call(x, dims)
+    n_out = dims isa Colon ? 1 : prod(d -> d in dims ? 1 : size(x, d), 1:N; init = 1)
+    length(dy) == length(lse) == n_out || throw(DimensionMismatch("dy and lse must have the size of logsumexp(x; dims)"))
     dx = similar(x, T, size(x))
-    GC.@preserve dy x lse dx check(ccall((:mi_logsumexp_bwd, libmi), Int32,
-                                         (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
-                                         dtype_code(T), dy.ptr, x.ptr, lse.ptr, dx.ptr, inner, len, outer, C_NULL))
+    GC.@preserve dy x lse dx sizes ws check(ccall((:mi_logsumexp_bwd_dims, libmi), Int32,
+        (Int32, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Int32, Ptr{Int64}, UInt32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+        dtype_code(T), dy.ptr, x.ptr, lse.ptr, dx.ptr, Int32(N), sizes, mask, wsptr(ws), wsb, C_NULL))
     dx
 end
 
-function softmax_grad!(op::Int32, dx::DeviceArray{T}, dy::DeviceArray{T}, y::DeviceArray{T}, dims) where {T <: MIFloat}
+function softmax_grad!(op::Int32, dx::DeviceArray{T, N}, dy::DeviceArray{T, N}, y::DeviceArray{T, N}, dims) where {T <: MIFloat, N}
     size(dx) == size(dy) == size(y) || throw(DimensionMismatch("dx, dy and y must have one size"))
-    inner, len, outer = reduction_geometry(size(y), dims)
-    GC.@preserve dx dy y check(ccall((:mi_softmax_bwd, libmi), Int32,
-                                     (Int32, Int32, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
-                                     op, dtype_code(T), dy.ptr, y.ptr, dx.ptr, inner, len, outer, C_NULL))
+    sizes, mask, ws, wsb = dims_call(y, dims)
+    GC.@preserve dx dy y sizes ws check(ccall((:mi_softmax_bwd_dims, libmi), Int32,
+        (Int32, Int32, Ptr{Cvoid}, Ptr{Cvoid}, Ptr{Cvoid}, Int32, Ptr{Int64}, UInt32, Ptr{Cvoid}, Csize_t, Ptr{Cvoid}),
+        op, dtype_code(T), dy.ptr, y.ptr, dx.ptr, Int32(N), sizes, mask, wsptr(ws), wsb, C_NULL))
     dx
 end
 ∇softmax!(dx::DeviceArray, dy::DeviceArray, y::DeviceArray; dims = 1) = softmax_grad!(MI_SOFTMAX, dx, dy, y, dims)
@@ -461,6 +467,50 @@ function batched_mul!(C::DeviceArray{T, 3}, A::DeviceArray{T, 3}, B::DeviceArray
     GC.@preserve A B C gemm!(tA, tB, m, n, ka, Float32(α), A.ptr, lda, sA, B.ptr, ldb, sB, Float32(β), C.ptr,
                               max(strides(C)[2], m, 1), strides(C)[3], size(C, 3), T)
     C
+end
+
+# Float64 (dgemm_ in the reference, src/gemm.jl:27-32): the same call on the fp64 matrix cores
+function batched_mul!(C::DeviceArray{Float64, 3}, A::DeviceArray{Float64, 3}, B::DeviceArray{Float64, 3}, α::Number = 1.0, β::Number = 0.0)
+    blasable(X) = strides(X)[1] == 1 || strides(X)[2] == 1 || size(X, 1) == 1 || size(X, 2) == 1
+    (blasable(A) && blasable(B) && strides(C)[1] == 1) || return generic_mul!(C, A, B, α, β)
+    size(A, 3) == size(C, 3) || size(A, 3) == 1 || throw(DimensionMismatch("batch size mismatch: A != C"))
+    size(B, 3) == size(C, 3) || size(B, 3) == 1 || throw(DimensionMismatch("batch size mismatch: B != C"))
+    m, ka = size(A, 1), size(A, 2); kb, n = size(B, 1), size(B, 2)
+    (ka == kb && m == size(C, 1) && n == size(C, 2)) ||
+        throw(DimensionMismatch("A1 has size ($m,$ka), B1 has size ($kb,$n), C1 has size $(size(C)[1:2])"))
+    (tA, lda), (tB, ldb) = blas_layout(A), blas_layout(B)
+    GC.@preserve A B C check(ccall((:mi_batched_gemm_f64, libmi), Int32,
+        (Cchar, Cchar, Int64, Int64, Int64, Float64, Ptr{Cvoid}, Int64, Int64, Ptr{Cvoid}, Int64, Int64, Float64, Ptr{Cvoid}, Int64, Int64, Int64, Ptr{Cvoid}),
+        tA, tB, m, n, ka, Float64(α), A.ptr, lda, size(A, 3) == 1 ? 0 : strides(A)[3], B.ptr, ldb, size(B, 3) == 1 ? 0 : strides(B)[3],
+        Float64(β), C.ptr, max(strides(C)[2], m, 1), strides(C)[3], size(C, 3), C_NULL); shape_error = DimensionMismatch)
+    C
+end
+
+# batched_mul_generic! (src/batched/batchedmul.jl:306-325): element types that differ, integers, ComplexF64, layouts
+# that are neither 'N' nor 'T'.  C's element type is promote_type of A's and B's; the library converts and computes in it.
+const AnyArr = Union{DeviceArray{<:MINumber, 3}, BatchedAdjoint}
+strided_operand(a::DeviceArray{T, 3}) where {T} = (a.ptr, strides(a)[1], strides(a)[2], strides(a)[3], Int32(0), dtype_code(T))
+strided_operand(a::BatchedAdjoint{T}) where {T <: Complex} = (a.parent.ptr, strides(a.parent)[2], strides(a.parent)[1], strides(a.parent)[3], Int32(1), dtype_code(T))
+function generic_mul!(C::DeviceArray{TC, 3}, A::AnyArr, B::AnyArr, α::Number = true, β::Number = false) where {TC <: MINumber}
+    size(A, 3) == size(C, 3) || size(A, 3) == 1 || throw(DimensionMismatch("batch size mismatch: A != C"))
+    size(B, 3) == size(C, 3) || size(B, 3) == 1 || throw(DimensionMismatch("batch size mismatch: B != C"))
+    m, ka = size(A, 1), size(A, 2); kb, n = size(B, 1), size(B, 2)
+    (ka == kb && m == size(C, 1) && n == size(C, 2)) ||
+        throw(DimensionMismatch("A1 has size ($m,$ka), B1 has size ($kb,$n), C1 has size $(size(C)[1:2])"))
+    (pa, ar, ac, ab, ca, da), (pb, br, bc, bb, cb, db) = strided_operand(A), strided_operand(B)
+    al, be = ComplexF64(α), ComplexF64(β)
+    GC.@preserve A B C check(ccall((:mi_batched_mul_generic, libmi), Int32,
+        (Int32, Int32, Int32, Int64, Int64, Int64, Float64, Float64, Ptr{Cvoid}, Int64, Int64, Int64, Int32, Ptr{Cvoid}, Int64, Int64, Int64, Int32,
+         Float64, Float64, Ptr{Cvoid}, Int64, Int64, Int64, Int64, Ptr{Cvoid}),
+        dtype_code(TC), da, db, m, n, ka, real(al), imag(al), pa, ar, ac, size(A, 3) == 1 ? 0 : ab, ca, pb, br, bc, size(B, 3) == 1 ? 0 : bb, cb,
+        real(be), imag(be), C.ptr, strides(C)[1], strides(C)[2], strides(C)[3], size(C, 3), C_NULL); shape_error = DimensionMismatch)
+    C
+end
+batched_mul!(C::DeviceArray{TC, 3}, A::AnyArr, B::AnyArr, α::Number = true, β::Number = false) where {TC <: MINumber} = generic_mul!(C, A, B, α, β)
+function batched_mul(A::AnyArr, B::AnyArr)
+    size(A, 3) == size(B, 3) || size(A, 3) == 1 || size(B, 3) == 1 || throw(DimensionMismatch("batch size mismatch: A != B"))
+    T = promote_type(eltype(A), eltype(B))                     # src/batched/batchedmul.jl:65
+    batched_mul!(DeviceArray{T}(undef, size(A, 1), size(B, 2), max(size(A, 3), size(B, 3))), A, B)
 end
 
 # ComplexF32 (cgemm in the reference, src/gemm.jl:31): one strided kernel takes 'N', 'T', 'C' and every
