@@ -471,3 +471,19 @@ def test_context_length_masks(nn, oracle, dtype, E, H, Lq, Lkv, per_head):
             keep = np.broadcast_to(mask, a.shape)[..., ok]
             assert np.count_nonzero(a[..., ok][~keep]) == 0          # exact zeros past the context length
             assert np.abs(a[..., ok].sum(axis=0) - 1).max() <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,D,H,L,B,causal", [("bf16", 128, 4, 512, 40, True), ("bf16", 128, 4, 512, 40, False),
+                                                  ("f16", 64, 8, 768, 16, True), ("bf16", 128, 2, 1024, 36, True),
+                                                  ("f16", 128, 3, 256, 90, False)])
+def test_prefill_parity_on_grids_larger_than_the_chip(nn, oracle, dtype, D, H, L, B, causal):
+    """More (query tile, head, batch) workgroups than CUs on the software-pipelined kernel (whole 256-row query tiles,
+    L_kv a multiple of 256): several rounds of workgroups per CU.  Every column of every workgroup is checked."""
+    rng = np.random.default_rng(L + B)
+    E = D * H
+    q, k, v = (round_to(rng.standard_normal((E, L, B)), dtype) for _ in range(3))
+    y, _ = _run(nn, q, k, v, dtype, None, None, H, causal, return_weights=False)
+    assert nn.last_attention_kernel() == "flash16"
+    yr, _ = oracle.nnlib_attention_f32(q, k, v, None, oracle.make_causal_mask(L) if causal else None, H, nthreads=8)
+    err = np.abs(y - yr).reshape(E, -1).max(axis=0) / np.abs(yr).max()          # per (query, batch) column
+    assert err.max() <= TOL[dtype], (float(err.max()), int(err.argmax()))
