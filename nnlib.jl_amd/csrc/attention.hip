@@ -91,7 +91,17 @@ static bool fast_kernel_fits(const AttnParams &p) {   // everything but the mask
     if (p.dtype == MI_F16) return flash16_fast_supports_f16(p) || flash16_fast_supports_f16_d64(p);
     return false;
 }
-static bool takes_fast_path(const AttnParams &p) { return !p.mask && fast_kernel_fits(p); }
+static bool takes_fast_path(const AttnParams &p) {
+    if (p.mask || !fast_kernel_fits(p)) return false;
+    // The pipelined kernel never splits the keys and has one workgroup per 256 queries of a (head, batch) pair: with
+    // few queries and many keys (cross-attention, a short chunk of queries against a long context) it would leave most
+    // of the chip idle, where the general kernel cuts the key range into pieces.  f16, head dim 64, 256 queries x 8192
+    // keys, 64 pairs: 0.113 ms on 64 workgroups against 0.061 ms in 512 pieces (bf16, head dim 128: 0.168 against 0.102);
+    // with 512 queries the two are level.
+    const int64_t fast_wgs = ((p.Lq + 255) / 256) * p.H * p.B;
+    if (fast_wgs < 128 && flash_pick_nsplit(p, 128) > 1) return false;
+    return true;
+}
 
 // ---- key-padding masks that are context lengths ------------------------------------------------------------------
 // Batches of sequences padded to one length carry a mask that keeps a prefix of the keys of each (head, batch) pair.

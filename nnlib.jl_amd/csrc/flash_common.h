@@ -352,6 +352,37 @@ __device__ inline void flash_load_key_mask(const FlashArgs &a, int64_t b, int64_
     }
 }
 
+// Mask bytes applied without lane masks (a compare writes a lane mask to scalar registers, which costs the compare, a
+// wait state and the select: three issue slots an element).  flash_mask_bits turns the four bytes of a word into "bit 7
+// of the byte is set iff the byte is non-zero" (no carry crosses a byte: 0x7f + 0x7f < 0x100); flash_mask_apply
+// sign-extends that bit into a word of ones or zeros and picks the score or -Inf with a bit-field insert, which is not
+// arithmetic: a NaN score under a dropped key is dropped like any other, as src/attention.jl:133-138 has it.
+__device__ inline uint32_t flash_mask_bits(uint32_t m4) { return ((m4 & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | m4; }
+// The select is inline assembly (written any other way the compiler turns it back into compare and select), and the
+// compiler does not insert for inline assembly the wait states that a read of a matrix-core result needs.  Callers
+// whose scores come straight from the MFMAs therefore pass `after`, a scalar they obtained with flash_mfma_fence from
+// the same accumulator block: the fence is an instruction the compiler does protect, and the operand orders the
+// select behind it.
+__device__ inline int flash_mfma_fence(const floatx16_t &v) { return __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v[0])); }
+__device__ inline float flash_mask_apply(float s, uint32_t bits, int e, int after) {
+    const int keep = __builtin_amdgcn_sbfe((int)bits, 8 * e + 7, 1);   // 0 or -1
+    float r;
+    asm("v_bfi_b32 %0, %1, %2, %3 ; ordered after %4" : "=v"(r) : "v"(keep), "v"(s), "s"(0xFF800000u), "s"(after));
+    return r;
+}
+// elements 4g .. 4g+3 of a 16-element accumulator block against the four mask bytes of m4
+__device__ inline void flash_mask_apply4(floatx16_t &v, int g, uint32_t m4, int after) {
+    const uint32_t bits = flash_mask_bits(m4);
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[4 * g + e] = flash_mask_apply(v[4 * g + e], bits, e, after);
+}
+
+// The running maximum of the online softmax only has to bound the exponents: it is raised when a tile's maximum
+// exceeds it by more than this many powers of two (and whenever either is infinite), so that the rescaling of the
+// row sum and of the output accumulators is skipped for nearly every tile after the first ones.  Weights relative to
+// it stay below 2^8, which Float32 sums and 16-bit operands hold without loss.
+constexpr float FLASH_LAZY_MAX_LOG2 = 8.0f;
+
 template <typename T, int QB, int NDV, bool CAUSAL, int EXTRAS, int PHASE, typename TW>
 __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB][2], floatx16_t (&o)[QB][NDV],
                                           float (&fm)[QB], float (&fl)[QB], int64_t b, int64_t h, int64_t iw,
@@ -394,10 +425,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                 for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const uint32_t m4 = sg.mask4(stage, row, 4 * kb + g, hh);
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            s[qb][kb][4 * g + e] = (m4 & (0xFFu << (8 * e))) ? s[qb][kb][4 * g + e] : MI_NEG_INF;
+                        flash_mask_apply4(s[qb][kb], g, sg.mask4(stage, row, 4 * kb + g, hh), 0);   // scores already went through the scaling above
                     }
             }
         } else if (EXTRAS == EXTRAS_DIRECT) {
@@ -449,28 +477,22 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
         if (EXTRAS == EXTRAS_MASKTILE) {
             const int row = 32 * qb + r;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < 2; kb++) {
+                const int fence = flash_mfma_fence(s[qb][kb]);
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const uint32_t m4 = sg.mask4(stage, row, 4 * kb + g, hh);
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        s[qb][kb][4 * g + e] = (m4 & (0xFFu << (8 * e))) ? s[qb][kb][4 * g + e] : MI_NEG_INF;
-                }
+                for (int g = 0; g < 4; g++) flash_mask_apply4(s[qb][kb], g, sg.mask4(stage, row, 4 * kb + g, hh), fence);
+            }
         }
         if (EXTRAS == EXTRAS_KEYMASK) {
             // one mask byte per key, shared by every query
             uint32_t own[8];
             if (!key_mask) flash_load_key_mask(a, b, h, j0, hh, own);
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < 2; kb++) {
+                const int fence = flash_mfma_fence(s[qb][kb]);
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const uint32_t m4 = key_mask ? key_mask[4 * kb + g] : own[4 * kb + g];
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        s[qb][kb][4 * g + e] = ((m4 >> (8 * e)) & 0xFFu) ? s[qb][kb][4 * g + e] : MI_NEG_INF;
-                }
+                for (int g = 0; g < 4; g++) flash_mask_apply4(s[qb][kb], g, key_mask ? key_mask[4 * kb + g] : own[4 * kb + g], fence);
+            }
         }
         if (EXTRAS != EXTRAS_DIRECT && edge) {
             // keys past the end of the sequence or, causal, after the query: tile-local limit per lane
@@ -498,19 +520,25 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                 for (int v = 0; v < 16; v++) mx = fmaxf(mx, s[qb][kb][v]);
             mx = fmaxf(mx, mi_swap32(mx));
             const float mold = fm[qb];
-            const float mnew = fmaxf(mold, mx);
-            msafe = mnew == MI_NEG_INF ? 0.0f : mnew;
-            float resc = mi_exp2((mold - msafe) * cs);
-            if (NAT && mold == mnew) resc = 1.0f;  // also covers +Inf == +Inf
-            pinf = mnew == MI_POS_INF;
-            fm[qb] = mnew;
-            fl[qb] *= resc;
-            if (PHASE == PHASE_ONLINE) {
+            // raise the running maximum only when some row of the wavefront outgrows it (see FLASH_LAZY_MAX_LOG2):
+            // -Inf before the first kept key and +Inf logits give an infinite difference; a NaN compares false and
+            // poisons the row through its own exponential
+            if (__builtin_amdgcn_ballot_w64((mx - mold) * cs > FLASH_LAZY_MAX_LOG2) != 0) {
+                const float mnew = fmaxf(mold, mx);
+                const float ms = mnew == MI_NEG_INF ? 0.0f : mnew;
+                float resc = mi_exp2((mold - ms) * cs);
+                if (mold == mnew) resc = 1.0f;  // also covers +Inf == +Inf
+                fm[qb] = mnew;
+                fl[qb] *= resc;
+                if (PHASE == PHASE_ONLINE) {
 #pragma unroll
-                for (int dvb = 0; dvb < NDV; dvb++)
+                    for (int dvb = 0; dvb < NDV; dvb++)
 #pragma unroll
-                    for (int v = 0; v < 16; v++) o[qb][dvb][v] *= resc;
+                        for (int v = 0; v < 16; v++) o[qb][dvb][v] *= resc;
+                }
             }
+            msafe = fm[qb] == MI_NEG_INF ? 0.0f : fm[qb];
+            pinf = fm[qb] == MI_POS_INF;
         } else {
             msafe = fm[qb] == MI_NEG_INF ? 0.0f : fm[qb];
             pinf = fm[qb] == MI_POS_INF;
