@@ -95,11 +95,14 @@ static bool takes_fast_path(const AttnParams &p) {
     if (p.mask || !fast_kernel_fits(p)) return false;
     // The pipelined kernel never splits the keys and has one workgroup per 256 queries of a (head, batch) pair: with
     // few queries and many keys (cross-attention, a short chunk of queries against a long context) it would leave most
-    // of the chip idle, where the general kernel cuts the key range into pieces.  f16, head dim 64, 256 queries x 8192
-    // keys, 64 pairs: 0.113 ms on 64 workgroups against 0.061 ms in 512 pieces (bf16, head dim 128: 0.168 against 0.102);
-    // with 512 queries the two are level.
+    // of the chip idle, where the general kernel cuts the key range into pieces.  Measured, pipelined / general:
+    // f16, head dim 64, 256 queries x 8192 keys, 64 pairs (64 workgroups against 512 pieces): 0.113 / 0.061 ms;
+    // bf16, head dim 128: the same shape 0.168 / 0.102, 128 x 4096 0.086 / 0.043, 256 x 2048 0.048 / 0.038,
+    // 512 x 8192 with 48 pairs (96 workgroups) 0.168 / 0.163.  At 128 workgroups the two are level without a causal
+    // mask (2048 x 2048, 16 pairs: 0.049 / 0.054; 1024 x 4096, 32 pairs: 0.089 / 0.087); with one, the pipelined
+    // kernel's unequal jobs lose (4096 x 4096, 8 pairs: 0.091 / 0.079).  Above that the pipelined kernel wins.
     const int64_t fast_wgs = ((p.Lq + 255) / 256) * p.H * p.B;
-    if (fast_wgs < 128 && flash_pick_nsplit(p, 128) > 1) return false;
+    if ((fast_wgs < 128 || (fast_wgs == 128 && p.causal)) && flash_pick_nsplit(p, 128) > 1) return false;
     return true;
 }
 

@@ -15,10 +15,11 @@ from .array import BatchedTranspose, CausalAnd, CausalMask, DeviceArray, batched
 
 __all__ = ["dot_product_attention", "dot_product_attention_scores", "make_causal_mask", "softmax", "softmax_",
            "logsoftmax", "logsoftmax_", "logsumexp", "grad_softmax", "grad_softmax_", "grad_logsoftmax",
-           "grad_logsoftmax_", "batched_mul", "batched_mul_", "batched_mul_pullback", "last_attention_kernel",
+           "grad_logsoftmax_", "batched_mul", "batched_mul_", "batched_mul_pullback", "last_attention_kernel", "last_attention_workspace",
            "dot_product_attention_grad", "last_attention_bwd_kernel", "Dropout", "dropout", "batched_vec"]
 
 _last_kernel = None
+_last_workspace = 0
 _workspace = None
 
 
@@ -64,6 +65,11 @@ def dropout(x, p, *, seed=0, dims=None):
 def last_attention_kernel():
     """Name of the kernel family the most recent attention call dispatched to."""
     return _lib.KERNEL_NAMES.get(_last_kernel)
+
+
+def last_attention_workspace():
+    """Workspace bytes the library asked for in the most recent attention call (non-zero: a split key range)."""
+    return _last_workspace
 
 
 def _stream():
@@ -133,7 +139,7 @@ def _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags, fdrop=None):
 def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_weights, weights_dtype, flags,
                     fdrop=None, save_stats=False):
     """One mi_attention_fwd call on flattened (F, L, B) operands."""
-    global _last_kernel
+    global _last_kernel, _last_workspace
     lib = _lib.load()
     d = _lib.mi_attn_desc()
     _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags, fdrop)
@@ -158,6 +164,7 @@ def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_we
         d.workspace, d.workspace_bytes = wbuf.data_ptr(), wsize
     _lib.check(lib.mi_attention_fwd(ctypes.byref(d), _stream()))
     _last_kernel = kernel.value
+    _last_workspace = ws.value
     if stats is not None:
         out.saved_stats = stats
     return out, alpha

@@ -487,3 +487,27 @@ def test_prefill_parity_on_grids_larger_than_the_chip(nn, oracle, dtype, D, H, L
     yr, _ = oracle.nnlib_attention_f32(q, k, v, None, oracle.make_causal_mask(L) if causal else None, H, nthreads=8)
     err = np.abs(y - yr).reshape(E, -1).max(axis=0) / np.abs(yr).max()          # per (query, batch) column
     assert err.max() <= TOL[dtype], (float(err.max()), int(err.argmax()))
+
+
+@pytest.mark.parametrize("dtype,D,H,Lq,Lkv,B,causal,split", [
+    ("bf16", 128, 4, 256, 4096, 2, False, True),     # 8 workgroups of 256 queries: the keys are cut into pieces
+    ("f16", 64, 8, 200, 8192, 1, False, True),
+    ("bf16", 128, 2, 130, 2500, 3, False, True),     # ragged lengths on the split path
+    ("bf16", 128, 8, 4096, 4096, 1, True, True),     # 128 unequal causal jobs: split as well
+    ("bf16", 128, 4, 256, 1024, 2, False, False),    # too few keys to cut: stays one piece
+    ("bf16", 128, 32, 1024, 2048, 2, False, False),  # 256 workgroups: the pipelined kernel keeps the call
+])
+def test_few_queries_many_keys_take_the_split_kernel(nn, oracle, dtype, D, H, Lq, Lkv, B, causal, split):
+    """Calls without bias / mask / weights whose (256-query tile, head, batch) count cannot fill the chip leave the
+    software-pipelined kernel, which never splits the keys, for the general kernel with a split key range (seen from
+    outside as a workspace request); parity holds on both sides of the rule."""
+    rng = np.random.default_rng(Lq + Lkv)
+    E = D * H
+    q = round_to(rng.standard_normal((E, Lq, B)), dtype)
+    k, v = (round_to(rng.standard_normal((E, Lkv, B)), dtype) for _ in range(2))
+    y, _ = _run(nn, q, k, v, dtype, None, None, H, causal, return_weights=False)
+    assert nn.last_attention_kernel() == "flash16"
+    assert (nn.last_attention_workspace() > 0) == split
+    yr, _ = oracle.nnlib_attention_f32(q, k, v, None, oracle.make_causal_mask(Lq) if causal else None, H, nthreads=8)
+    err = np.abs(y - yr).reshape(E, -1).max(axis=0) / np.abs(yr).max()
+    assert err.max() <= TOL[dtype], (float(err.max()), int(err.argmax()))
