@@ -484,3 +484,40 @@ def test_dq_split_over_the_keys(nn, oracle, dtype, D, H, Lq, Lkv, B, mask_kind, 
     bias_shape = (Lkv, Lq, H, B) if bias_kind == "full" else None
     _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, mask_kind=mask_kind, bias_shape=bias_shape,
          expect="flash32" if dtype == "f32" else "flash16", saved=True, dropout=dropout, seed=Lq + Lkv, scale=0.4)
+
+
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f16", 64), ("f32", 64)])
+@pytest.mark.parametrize("saved", [False, True])
+def test_gradient_with_logits_that_climb_along_the_keys(nn, oracle, dtype, D, saved):
+    """The forward kernels raise their running maximum lazily (only when a tile outgrows it by 2^8), so the statistics
+    they save need not hold the true row maximum; the gradient kernels must get the same weights out of them.  Logits
+    that climb by about 5 powers of two per 64-key tile (up to 40 at the last key) keep the saved maximum stale for
+    most rows.
+
+    Bounds.  Float32: 1e-4.  16-bit, dk and dv: 1e-2 when the gradient call computes the statistics itself.  With the
+    statistics of the software-pipelined forward kernel the bound is 2e-2: that kernel multiplies q by log2(e)/sqrt(D)
+    and rounds the product to the 16-bit type before QK^T (as the reference rounds q / sqrt(D), src/attention.jl:118),
+    the gradient kernels scale the Float32 product instead, and the two sets of logits differ by up to
+    |logit| * 2^-9 (bf16), which at logits of 40 powers of two is a per cent of a weight.  dq is a sum over keys of
+    terms that cancel (each row of dS sums to zero and k is dominated by the ramp), so 16-bit rounding of dS shows
+    in it: 3e-2."""
+    rng = np.random.default_rng(5)
+    H, L, B = 2, 512, 2
+    E = D * H
+    ramp = 5.0 * np.log(2.0) * np.arange(L) / 64.0
+    q = round_to(rng.uniform(0.5, 1.5, (E, L, B)), dtype)
+    k = round_to((ramp / np.sqrt(D))[None, :, None] + 0.3 * rng.standard_normal((E, L, B)), dtype)
+    v, dy = (round_to(rng.standard_normal((E, L, B)), dtype) for _ in range(2))
+    Dv = nn.DeviceArray.from_numpy
+    dq_, dk_, dv_, ddy = Dv(q, dtype), Dv(k, dtype), Dv(v, dtype), Dv(dy, dtype)
+    y, _ = nn.dot_product_attention(dq_, dk_, dv_, nheads=H, return_weights=False, save_for_backward=saved)
+    assert (getattr(y, "saved_stats", None) is not None) == saved
+    got = nn.dot_product_attention_grad(ddy, dq_, dk_, dv_, y=y, nheads=H)
+    assert nn.last_attention_bwd_kernel() == ("flash32" if dtype == "f32" else "flash16")
+    ref = oracle.attention_bwd_f64(q, k, v, dy, None, None, H)
+    if dtype == "f32":
+        tols = (1e-4, 1e-4, 1e-4)
+    else:
+        tols = (3e-2, 2e-2, 2e-2) if saved else (3e-2, 1e-2, 1e-2)
+    for g, r_, tol in zip(got[:3], ref[:3], tols):
+        assert np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05) <= tol

@@ -511,3 +511,30 @@ def test_few_queries_many_keys_take_the_split_kernel(nn, oracle, dtype, D, H, Lq
     yr, _ = oracle.nnlib_attention_f32(q, k, v, None, oracle.make_causal_mask(Lq) if causal else None, H, nthreads=8)
     err = np.abs(y - yr).reshape(E, -1).max(axis=0) / np.abs(yr).max()
     assert err.max() <= TOL[dtype], (float(err.max()), int(err.argmax()))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("pattern", ["rise5", "rise20", "fall", "zigzag"])
+@pytest.mark.parametrize("weights", [False, True], ids=["noweights", "weights"])
+def test_logits_that_drift_along_the_keys(nn, oracle, dtype, pattern, weights):
+    """The kernels raise their running maximum only when a tile outgrows it by 2^8, so weights relative to a stale
+    maximum reach 2^8 before the next rescale.  Logits that climb by about 5 or 20 powers of two per 64-key tile, fall,
+    or alternate exercise every branch of that rule; results must still match the reference arithmetic."""
+    rng = np.random.default_rng(11)
+    D, H, L, B = 64, 2, 640, 2
+    E = D * H
+    per_tile = {"rise5": 5.0, "rise20": 20.0, "fall": -5.0, "zigzag": 5.0}[pattern] * np.log(2.0)
+    j = np.arange(L, dtype=np.float64)
+    ramp = per_tile * (j / 64.0)
+    if pattern == "zigzag":
+        ramp = per_tile * 2.0 * ((np.floor(j / 64.0) % 2) * 2 - 1)
+    # logits = (k . q) / sqrt(D): q = 1 on every feature, k_j = ramp_j / sqrt(D) on every feature, plus noise
+    q = round_to(np.ones((E, L, B)) + 0.05 * rng.standard_normal((E, L, B)), dtype)
+    k = round_to((ramp / np.sqrt(D))[None, :, None] + 0.05 * rng.standard_normal((E, L, B)), dtype)
+    v = round_to(rng.standard_normal((E, L, B)), dtype)
+    y, a = _run(nn, q, k, v, dtype, None, None, H, False, return_weights=weights, weights_dtype="f32" if weights else None)
+    yr, ar = oracle.nnlib_attention_f32(q, k, v, None, None, H, nthreads=8)
+    assert rel_err(y, yr) <= TOL[dtype], (rel_err(y, yr), nn.last_attention_kernel())
+    if weights:
+        assert float(np.abs(a - ar).max()) <= TOL[dtype]
+        assert float(np.abs(a.sum(axis=0) - 1).max()) <= 1e-5
