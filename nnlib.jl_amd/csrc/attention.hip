@@ -102,7 +102,7 @@ static bool takes_fast_path(const AttnParams &p) {
     // mask (2048 x 2048, 16 pairs: 0.049 / 0.054; 1024 x 4096, 32 pairs: 0.089 / 0.087); with one, the pipelined
     // kernel's unequal jobs lose (4096 x 4096, 8 pairs: 0.091 / 0.079).  Above that the pipelined kernel wins.
     const int64_t fast_wgs = ((p.Lq + 255) / 256) * p.H * p.B;
-    if ((fast_wgs < 128 || (fast_wgs == 128 && p.causal)) && flash_pick_nsplit(p, 128) > 1) return false;
+    if (!p.keep_pipelined && (fast_wgs < 128 || (fast_wgs == 128 && p.causal)) && flash_pick_nsplit(p, 128) > 1) return false;
     return true;
 }
 
@@ -333,7 +333,13 @@ static int32_t attention_forward(const mi_attn_desc *d, mi_stream s, bool static
         return MI_OK;
     }
     size_t ws = 0;
-    const int32_t kernel = choose(d, p, &ws);
+    int32_t kernel = choose(d, p, &ws);
+    if (static_workspace && ws > MI_ATTN_STATIC_WORKSPACE_BYTES && kernel == MI_ATTN_KERNEL_FLASH16) {
+        // few queries against many keys: the key-split plan is the faster one, but the pipelined kernel needs no
+        // workspace at all
+        p.keep_pipelined = true;
+        kernel = choose(d, p, &ws);
+    }
     if (static_workspace) {
         // every kernel writes what it later reads of the workspace, so what an earlier call left there needs no clearing
         if (ws > MI_ATTN_STATIC_WORKSPACE_BYTES)

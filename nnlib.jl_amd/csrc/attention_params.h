@@ -17,6 +17,9 @@ struct AttnParams {
     uint64_t drop_key;
     uint32_t drop_thresh;
     float drop_scale;
+    // plan constraint of the entry point without caller workspace: stay on the software-pipelined kernel (which needs
+    // none) where the key-split plan would ask for more than the built-in workspace holds
+    bool keep_pipelined = false;
 };
 
 #ifdef __HIPCC__

@@ -118,6 +118,39 @@ def test_calls_without_a_workspace(nn):
     _both(nn, "f32", 128, 96, 160, 2, 2, 14, weights=True, expect_kernel="flash32", expect_workspace=False)
 
 
+def test_key_split_plan_too_large_for_the_builtin_workspace_stays_on_the_pipelined_kernel(nn):
+    """512 queries against 2048 keys on 32 heads of 128: mi_attention_fwd cuts the keys into 4 pieces and asks for 34 MB of
+    partial results, more than the built-in array holds; the entry point without caller workspace runs the same call on
+    the software-pipelined kernel, which needs none.  Two different kernels, so the outputs agree to the 16-bit bound,
+    not bit for bit; a smaller call follows."""
+    L = nn._lib
+    lib = L.load()
+    for E, Lq, Lkv, B, H, seed in ((4096, 512, 2048, 1, 32, 21), (4096, 300, 2048, 1, 32, 22)):
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        q, k, v = (torch.randn(E * n * B, device="cuda", generator=g).to(torch.bfloat16) for n in (Lq, Lkv, Lkv))
+        outs = []
+        for static in (False, True):
+            out = torch.full((E * Lq * B,), float("nan"), device="cuda", dtype=torch.bfloat16)
+            d = _desc(L, "bf16", E, Lq, Lkv, B, H, q, k, v, out, None)
+            ws = ctypes.c_size_t(0)
+            L.check(lib.mi_attention_workspace_size(ctypes.byref(d), ctypes.byref(ws)))
+            assert (ws.value > L.MI_ATTN_STATIC_WORKSPACE_BYTES) == (Lq == 512)   # the smaller call's partial results fit
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            if static:
+                torch.cuda.synchronize()
+                before = torch.cuda.memory_allocated()
+                L.check(lib.mi_attention_fwd_static(ctypes.byref(d), stream))
+                assert torch.cuda.memory_allocated() == before
+            else:
+                buf = torch.empty(ws.value, dtype=torch.uint8, device="cuda")
+                d.workspace, d.workspace_bytes = buf.data_ptr(), buf.numel()
+                L.check(lib.mi_attention_fwd(ctypes.byref(d), stream))
+            torch.cuda.synchronize()
+            outs.append(out.float())
+        assert not torch.isnan(outs[0]).any() and not torch.isnan(outs[1]).any()
+        assert float((outs[0] - outs[1]).abs().max() / outs[0].abs().max()) <= 1e-2
+
+
 def test_call_beyond_the_builtin_workspace_is_refused(nn):
     L = nn._lib
     lib = L.load()
