@@ -162,7 +162,10 @@ typedef struct mi_attn_desc {
 } mi_attn_desc;
 
 /* Validates shapes the way src/attention.jl:55-78 does (MI_ESHAPE on failure) and
- * reports the kernel family and workspace need without touching the device. */
+ * reports the kernel family and workspace need without touching the device.  A call that is given less
+ * workspace than planned fails with MI_EWORKSPACE, with one exception: a 16-bit call without bias and mask
+ * whose plan splits the key range (few queries, many keys) is then run unsplit, which needs no workspace
+ * and is slower, not wrong. */
 int32_t mi_attention_plan(const mi_attn_desc *desc, int32_t *kernel, size_t *workspace_bytes);
 int32_t mi_attention_workspace_size(const mi_attn_desc *desc, size_t *bytes);
 int32_t mi_attention_fwd(const mi_attn_desc *desc, mi_stream stream);

@@ -334,9 +334,10 @@ static int32_t attention_forward(const mi_attn_desc *d, mi_stream s, bool static
     }
     size_t ws = 0;
     int32_t kernel = choose(d, p, &ws);
-    if (static_workspace && ws > MI_ATTN_STATIC_WORKSPACE_BYTES && kernel == MI_ATTN_KERNEL_FLASH16) {
+    const size_t have = static_workspace ? (size_t)MI_ATTN_STATIC_WORKSPACE_BYTES : (d->workspace ? d->workspace_bytes : (size_t)0);
+    if (ws > have && kernel == MI_ATTN_KERNEL_FLASH16) {
         // few queries against many keys: the key-split plan is the faster one, but the pipelined kernel needs no
-        // workspace at all
+        // workspace at all, so a caller without (enough of) one is served rather than refused
         p.keep_pipelined = true;
         kernel = choose(d, p, &ws);
     }

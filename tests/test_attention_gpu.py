@@ -538,3 +538,35 @@ def test_logits_that_drift_along_the_keys(nn, oracle, dtype, pattern, weights):
     if weights:
         assert float(np.abs(a - ar).max()) <= TOL[dtype]
         assert float(np.abs(a.sum(axis=0) - 1).max()) <= 1e-5
+
+
+def test_few_queries_without_a_workspace_fall_back_to_the_pipelined_kernel(nn):
+    """mi_attention_fwd with no workspace on a call whose plan is the key-split kernel: served by the software-pipelined
+    kernel (which needs none) instead of MI_EWORKSPACE; same result to the 16-bit bound."""
+    import ctypes
+    import torch
+    L = nn._lib
+    lib = L.load()
+    E, Lq, Lkv, B, H = 512, 256, 4096, 2, 4
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q, k, v = (torch.randn(E * n * B, device="cuda", generator=g).to(torch.bfloat16) for n in (Lq, Lkv, Lkv))
+    outs = []
+    for with_ws in (True, False):
+        out = torch.full((E * Lq * B,), float("nan"), device="cuda", dtype=torch.bfloat16)
+        d = L.mi_attn_desc()
+        d.struct_size = ctypes.sizeof(L.mi_attn_desc)
+        d.dtype = d.weights_dtype = L.MI_BF16
+        d.E = d.Ev = E
+        d.Lq, d.Lkv, d.H, d.B = Lq, Lkv, H, B
+        d.q, d.k, d.v, d.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+        ws = ctypes.c_size_t(0)
+        L.check(lib.mi_attention_workspace_size(ctypes.byref(d), ctypes.byref(ws)))
+        assert ws.value > 0
+        if with_ws:
+            buf = torch.empty(ws.value, dtype=torch.uint8, device="cuda")
+            d.workspace, d.workspace_bytes = buf.data_ptr(), buf.numel()
+        L.check(lib.mi_attention_fwd(ctypes.byref(d), None))
+        torch.cuda.synchronize()
+        outs.append(out.float())
+    assert not torch.isnan(outs[0]).any() and not torch.isnan(outs[1]).any()
+    assert float((outs[0] - outs[1]).abs().max() / outs[0].abs().max()) <= 1e-2
