@@ -90,7 +90,7 @@ enum {
     MI_ATTN_KERNEL_GENERIC = 0,  /* any shape / dtype, scalar FMA                        */
     MI_ATTN_KERNEL_FLASH16 = 1,  /* f16 / bf16 MFMA flash forward, head dims 8..256 (x8) */
     MI_ATTN_KERNEL_FLASH32 = 2,  /* f32 MFMA flash forward, head dims 4..128 (x4)        */
-    MI_ATTN_KERNEL_DECODE = 3    /* split-kv bandwidth-bound path for one query (L_q = 1) */
+    MI_ATTN_KERNEL_DECODE = 3    /* split-kv bandwidth-bound path for one to four queries (L_q <= 4) */
 };
 
 /* flags */

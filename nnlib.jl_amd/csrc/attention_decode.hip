@@ -53,7 +53,10 @@ __device__ inline void unpack8(const u32x4_t &v, float *out, F32) {   // four fe
 }
 
 // workspace layout: [B][nsplit][E] floats of o, then [B][nsplit][H] of m, then [B][nsplit][H] of l
-template <typename T, int D, bool MASKED, bool SCORES>
+// NQ: queries of one batch element that a wavefront carries through the stream (1, 2 or 4).  A handful of queries
+// against a long context (a few speculated tokens, a short chunk) is the same stream over K and V with NQ states: every
+// K / V row is read once for all of them, where the tiled kernel reads head-dim-wide pieces of it per head.
+template <typename T, int D, bool MASKED, bool SCORES, int NQ = 1>
 __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     const AttnParams &p = a.p;
     typedef typename T::type t;
@@ -63,15 +66,20 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     __shared__ float sc_lds[SCORES ? 4 * NH * 64 : 1]; // scores on their way out: [wavefront][head][64 keys]
     const int seg = blockIdx.x * 4 + wave;
     const int split = blockIdx.y;
-    const int64_t b = blockIdx.z;
+    const int64_t ngroups = (p.Lq + NQ - 1) / NQ;      // groups of NQ queries per batch element
+    const int64_t b = blockIdx.z / ngroups, q0 = (blockIdx.z % ngroups) * NQ;
     const int64_t f = (int64_t)seg * SEG + lane * EPL; // first feature of this lane
     const bool lane_ok = f < p.E;                      // E is a multiple of EPL (D is 64 or 128)
     if (seg >= a.nseg) return;
 
     const t *kb = (const t *)p.k + p.E * p.Lkv * b + (lane_ok ? f : 0);
     const t *vb = (const t *)p.v + p.E * p.Lkv * b + (lane_ok ? f : 0);
-    float qf[EPL] = {};
-    if (lane_ok) unpack8(*(const u32x4_t *)((const t *)p.q + p.E * b + f), qf, T());
+    float qf[NQ][EPL] = {};
+#pragma unroll
+    for (int n = 0; n < NQ; n++) {   // queries past Lq: copies of the last one, computed and not stored
+        const int64_t qi = q0 + n < p.Lq ? q0 + n : p.Lq - 1;
+        if (lane_ok) unpack8(*(const u32x4_t *)((const t *)p.q + p.E * (qi + p.Lq * b) + f), qf[n], T());
+    }
 
     // Without the score output the splits take the 8-row blocks of the key range in turn (block t belongs to split
     // t mod nsplit) instead of one contiguous range each: the splits of a batch element run side by side, so at any
@@ -85,8 +93,12 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
     if (j_end > p.Lkv) j_end = p.Lkv;
     const int64_t j_step = interleave ? (int64_t)a.nsplit * ROWS : ROWS;
 
-    float m = MI_NEG_INF, l = 0.0f;
-    float o[EPL] = {};
+    float m[NQ], l[NQ], o[NQ][EPL] = {};
+#pragma unroll
+    for (int n = 0; n < NQ; n++) {
+        m[n] = MI_NEG_INF;
+        l[n] = 0.0f;
+    }
     const u32x4_t zero = {0, 0, 0, 0};
     // mask bytes of this lane's head: element (kv, 0, h, b)
     const uint8_t *mrow = MASKED ? p.mask + (lane_ok ? f / D : 0) * p.mask_strides[2] + b * p.mask_strides[3] : nullptr;
@@ -106,36 +118,47 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
         bool keep[ROWS];
 #pragma unroll
         for (int r = 0; r < ROWS; r++) keep[r] = j + r < j_end && (!MASKED || mrow[(j + r) * p.mask_strides[0]] != 0);
-        float s[ROWS];
-        float mx = MI_NEG_INF;
+        float s[NQ][ROWS];
+        float mx[NQ];
+#pragma unroll
+        for (int n = 0; n < NQ; n++) mx[n] = MI_NEG_INF;
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
             float kf[EPL];
             unpack8(kr[r], kf, T());
-            float d = 0.0f;
 #pragma unroll
-            for (int e = 0; e < EPL; e++) d = fmaf(kf[e], qf[e], d);
+            for (int n = 0; n < NQ; n++) {
+                float d = 0.0f;
 #pragma unroll
-            for (int off = 1; off < LPH; off <<= 1) d += __shfl_xor(d, off, 64);
-            s[r] = keep[r] ? d : MI_NEG_INF;
-            mx = fmaxf(mx, s[r]);
+                for (int e = 0; e < EPL; e++) d = fmaf(kf[e], qf[n][e], d);
+#pragma unroll
+                for (int off = 1; off < LPH; off <<= 1) d += __shfl_xor(d, off, 64);
+                s[n][r] = keep[r] ? d : MI_NEG_INF;
+                mx[n] = fmaxf(mx[n], s[n][r]);
+            }
         }
-        float mnew = fmaxf(m, mx);            // finite without a mask: at least one row of the chunk is valid
-        const float mref = (MASKED && mnew == MI_NEG_INF) ? 0.0f : mnew;   // nothing kept so far: every term below is 0
-        const float resc = mi_exp2((m - mref) * a.c);
-        m = mnew;
-        mnew = mref;
-        l *= resc;
+        float mref[NQ];
 #pragma unroll
-        for (int e = 0; e < EPL; e++) o[e] *= resc;
+        for (int n = 0; n < NQ; n++) {
+            const float mnew = fmaxf(m[n], mx[n]);            // finite without a mask: at least one row of the chunk is valid
+            mref[n] = (MASKED && mnew == MI_NEG_INF) ? 0.0f : mnew;   // nothing kept so far: every term below is 0
+            const float resc = mi_exp2((m[n] - mref[n]) * a.c);
+            m[n] = mnew;
+            l[n] *= resc;
+#pragma unroll
+            for (int e = 0; e < EPL; e++) o[n][e] *= resc;
+        }
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
-            const float pr = mi_exp2((s[r] - mnew) * a.c);
-            l += pr;
             float vf[EPL];
             unpack8(vr[r], vf, T());
 #pragma unroll
-            for (int e = 0; e < EPL; e++) o[e] = fmaf(pr, vf[e], o[e]);
+            for (int n = 0; n < NQ; n++) {
+                const float pr = mi_exp2((s[n][r] - mref[n]) * a.c);
+                l[n] += pr;
+#pragma unroll
+                for (int e = 0; e < EPL; e++) o[n][e] = fmaf(pr, vf[e], o[n][e]);
+            }
         }
         if (SCORES) {
             // Scores leave in runs of 64 keys per head (256 contiguous bytes): written 32 bytes at a time, one piece per
@@ -145,8 +168,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
             const int slot8 = (int)(((j - j_begin) / ROWS) & 7);
             if ((lane & (LPH - 1)) == 0) {
                 float *row = sc_lds + (wave * NH + lane / LPH) * 64 + 8 * slot8;
-                *(floatx4_t *)row = (floatx4_t){s[0], s[1], s[2], s[3]};
-                *(floatx4_t *)(row + 4) = (floatx4_t){s[4], s[5], s[6], s[7]};
+                *(floatx4_t *)row = (floatx4_t){s[0][0], s[0][1], s[0][2], s[0][3]};
+                *(floatx4_t *)(row + 4) = (floatx4_t){s[0][4], s[0][5], s[0][6], s[0][7]};
             }
             if (slot8 == 7 || j + ROWS >= j_end) {
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -166,17 +189,23 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
         }
     }
     if (!lane_ok) return;
+    // partial results: one slot per (batch element, query, split); the merge kernel sees B * Lq batch elements
     float *ws = (float *)p.workspace;
-    const int64_t slot = b * a.nsplit + split;
-    float *wo = ws + slot * p.E + f;
-    *(floatx4_t *)wo = (floatx4_t){o[0], o[1], o[2], o[3]};
-    if constexpr (EPL == 8) *(floatx4_t *)(wo + 4) = (floatx4_t){o[4], o[5], o[6], o[7]};
-    if ((lane & (LPH - 1)) == 0) {
-        const int64_t h = f / D;
-        float *wm = ws + (int64_t)p.B * a.nsplit * p.E;
-        float *wl = wm + (int64_t)p.B * a.nsplit * p.H;
-        wm[slot * p.H + h] = m;
-        wl[slot * p.H + h] = l;
+    const int64_t nbq = p.B * p.Lq;
+#pragma unroll
+    for (int n = 0; n < NQ; n++) {
+        if (q0 + n >= p.Lq) break;
+        const int64_t slot = (b * p.Lq + q0 + n) * a.nsplit + split;
+        float *wo = ws + slot * p.E + f;
+        *(floatx4_t *)wo = (floatx4_t){o[n][0], o[n][1], o[n][2], o[n][3]};
+        if constexpr (EPL == 8) *(floatx4_t *)(wo + 4) = (floatx4_t){o[n][4], o[n][5], o[n][6], o[n][7]};
+        if ((lane & (LPH - 1)) == 0) {
+            const int64_t h = f / D;
+            float *wm = ws + nbq * a.nsplit * p.E;
+            float *wl = wm + nbq * a.nsplit * p.H;
+            wm[slot * p.H + h] = m[n];
+            wl[slot * p.H + h] = l[n];
+        }
     }
 }
 
@@ -250,11 +279,15 @@ __global__ __launch_bounds__(256) void decode_weights_kernel(DecodeArgs a, TW *w
         if (j + e < p.Lkv) dst[j + e] = (TW)(mi_exp2((src[j + e] - m) * a.c) * inv);
 }
 
+// queries per wavefront: 1, 2, or 4 (three queries run as four)
+int decode_nq(const AttnParams &p) { return p.Lq <= 1 ? 1 : p.Lq == 2 ? 2 : 4; }
+
 int pick_nsplit(const AttnParams &p) {
     // enough wavefronts to cover the chip several times over, at least 256 rows per split
     const int64_t SEG = p.dtype == MI_F32 ? seg_width<F32>() : seg_width<BF16>();
     const int64_t nseg = (p.E + SEG - 1) / SEG;
-    int64_t want = 8192 / (nseg * p.B > 0 ? nseg * p.B : 1);   // (C5: 2048, 4096, 16384 ... 65536 wavefronts all measured slower)
+    const int64_t groups = p.B * ((p.Lq + decode_nq(p) - 1) / decode_nq(p));   // (batch element, query group) pairs
+    int64_t want = 8192 / (nseg * groups > 0 ? nseg * groups : 1);   // (C5: 2048, 4096, 16384 ... 65536 wavefronts all measured slower)
     int64_t maxs = (p.Lkv + 255) / 256;
     if (want > maxs) want = maxs;
     if (want < 1) want = 1;
@@ -265,7 +298,9 @@ int pick_nsplit(const AttnParams &p) {
 }  // namespace
 
 bool attention_decode_supports(const AttnParams &p) {
-    if (p.Lq != 1 || p.bias || p.causal || !p.out || p.drop_thresh || p.stats) return false;   // saved statistics: the tiled kernels write them
+    if (p.Lq < 1 || p.Lq > 4 || p.bias || p.causal || !p.out || p.drop_thresh || p.stats) return false;   // saved statistics: the tiled kernels write them
+    // two to four queries: without the weights, and with a mask only when it does not depend on the query
+    if (p.Lq > 1 && (p.weights || (p.mask && p.mask_strides[1] != 0) || p.B * p.Lq > 65535)) return false;
     if (p.weights && p.H * p.B > 65535) return false;
     if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
     if (p.Lkv < 512) return false;   // short contexts: the tiled kernel is fine
@@ -277,7 +312,7 @@ bool attention_decode_supports(const AttnParams &p) {
 size_t attention_decode_workspace(const AttnParams &p) {
     const size_t ns = (size_t)pick_nsplit(p);
     // partial results of the splits, then (weights requested) the raw scores and the final statistics
-    return sizeof(float) * (ns * (size_t)p.B * (size_t)(p.E + 2 * p.H) + (p.weights ? (size_t)(p.Lkv * p.H * p.B + 2 * p.H * p.B) : 0));
+    return sizeof(float) * (ns * (size_t)(p.B * p.Lq) * (size_t)(p.E + 2 * p.H) + (p.weights ? (size_t)(p.Lkv * p.H * p.B + 2 * p.H * p.B) : 0));
 }
 
 int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
@@ -297,30 +332,40 @@ int32_t launch_attention_decode(const AttnParams &p, hipStream_t st) {
         a.scores = (float *)p.workspace + (size_t)pick_nsplit(p) * (size_t)p.B * (size_t)(p.E + 2 * p.H);
         a.final_ml = a.scores + p.Lkv * p.H * p.B;
     }
-    dim3 grid((unsigned)((a.nseg + 3) / 4), (unsigned)a.nsplit, (unsigned)p.B);
-    dim3 mgrid((unsigned)((p.E + 255) / 256), (unsigned)p.B);
+    const int nq = decode_nq(p);
+    dim3 grid((unsigned)((a.nseg + 3) / 4), (unsigned)a.nsplit, (unsigned)(p.B * ((p.Lq + nq - 1) / nq)));
+    dim3 mgrid((unsigned)((p.E + 255) / 256), (unsigned)(p.B * p.Lq));
+    DecodeArgs am = a;      // the merge kernel takes every (batch element, query) pair for a batch element of its own:
+    am.p.B = p.B * p.Lq;    // q and the output are (E, Lq, B) arrays, the partial results [B * Lq][split][...]
+    am.p.Lq = 1;
 #define DECODE_LAUNCH(TT, DD)                                                                                        \
     {                                                                                                                \
         if (p.weights) {                                                                                             \
             if (p.mask) hipLaunchKernelGGL((decode_split_kernel<TT, DD, true, true>), grid, dim3(256), 0, st, a);     \
             else hipLaunchKernelGGL((decode_split_kernel<TT, DD, false, true>), grid, dim3(256), 0, st, a);           \
-        } else {                                                                                                     \
+        } else if (nq == 1) {                                                                                        \
             if (p.mask) hipLaunchKernelGGL((decode_split_kernel<TT, DD, true, false>), grid, dim3(256), 0, st, a);    \
             else hipLaunchKernelGGL((decode_split_kernel<TT, DD, false, false>), grid, dim3(256), 0, st, a);          \
+        } else if (nq == 2) {                                                                                        \
+            if (p.mask) hipLaunchKernelGGL((decode_split_kernel<TT, DD, true, false, 2>), grid, dim3(256), 0, st, a); \
+            else hipLaunchKernelGGL((decode_split_kernel<TT, DD, false, false, 2>), grid, dim3(256), 0, st, a);       \
+        } else {                                                                                                     \
+            if (p.mask) hipLaunchKernelGGL((decode_split_kernel<TT, DD, true, false, 4>), grid, dim3(256), 0, st, a); \
+            else hipLaunchKernelGGL((decode_split_kernel<TT, DD, false, false, 4>), grid, dim3(256), 0, st, a);       \
         }                                                                                                            \
     }
     if (p.dtype == MI_BF16) {
         if (p.D == 128) DECODE_LAUNCH(BF16, 128) else DECODE_LAUNCH(BF16, 64)
         MI_LAUNCH_CHECK();
-        hipLaunchKernelGGL(decode_merge_kernel<BF16>, mgrid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(decode_merge_kernel<BF16>, mgrid, dim3(256), 0, st, am);
     } else if (p.dtype == MI_F32) {
         if (p.D == 128) DECODE_LAUNCH(F32, 128) else DECODE_LAUNCH(F32, 64)
         MI_LAUNCH_CHECK();
-        hipLaunchKernelGGL(decode_merge_kernel<F32>, mgrid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(decode_merge_kernel<F32>, mgrid, dim3(256), 0, st, am);
     } else {
         if (p.D == 128) DECODE_LAUNCH(F16, 128) else DECODE_LAUNCH(F16, 64)
         MI_LAUNCH_CHECK();
-        hipLaunchKernelGGL(decode_merge_kernel<F16>, mgrid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(decode_merge_kernel<F16>, mgrid, dim3(256), 0, st, am);
     }
 #undef DECODE_LAUNCH
     MI_LAUNCH_CHECK();

@@ -570,3 +570,31 @@ def test_few_queries_without_a_workspace_fall_back_to_the_pipelined_kernel(nn):
         outs.append(out.float())
     assert not torch.isnan(outs[0]).any() and not torch.isnan(outs[1]).any()
     assert float((outs[0] - outs[1]).abs().max() / outs[0].abs().max()) <= 1e-2
+
+
+@pytest.mark.parametrize("dtype,E,H,Lkv,B", [("bf16", 512, 4, 1500, 2), ("bf16", 256, 2, 4096, 3), ("f16", 512, 8, 777, 1),
+                                             ("f16", 1024, 8, 2048, 2), ("f32", 512, 4, 1500, 2), ("f32", 64, 1, 777, 1)])
+@pytest.mark.parametrize("Lq", [2, 3, 4])
+@pytest.mark.parametrize("mask", [None, "keys"])
+def test_a_few_queries_stream_like_one(nn, oracle, dtype, E, H, Lkv, B, Lq, mask):
+    """Two to four queries per batch element against a long context (no weights, no bias, a mask only if it does not
+    depend on the query) take the single-query kernels: a wavefront carries 2 or 4 softmax states through one pass over
+    K and V (three queries run as four).  Parity per query against the oracle."""
+    rng = np.random.default_rng(E + Lkv + Lq)
+    q, k, v = (round_to(rng.standard_normal(s), dtype) for s in ((E, Lq, B), (E, Lkv, B), (E, Lkv, B)))
+    m = None
+    if mask == "keys":      # (Lkv, 1, 1, B): the context lengths / scattered keys of a padded batch
+        m = rng.random((Lkv, 1, 1, B)) < 0.8
+        m[0] = True
+    y, _ = _run(nn, q, k, v, dtype, None, m, H, False, return_weights=False)
+    assert nn.last_attention_kernel() == "decode"
+    om = None if m is None else np.broadcast_to(m, (Lkv, Lq, 1, B))
+    yr, _ = oracle.nnlib_attention_f32(q, k, v, None, om, H, nthreads=8)
+    err = np.abs(y - yr).reshape(E, -1).max(axis=0) / np.abs(yr).max()
+    assert err.max() <= TOL[dtype], (float(err.max()), int(err.argmax()))
+
+
+def test_a_few_queries_with_weights_or_a_query_dependent_mask_take_the_tiled_kernel(nn, oracle):
+    rng = np.random.default_rng(9)
+    _check(nn, oracle, rng, "bf16", 256, 3, 1500, 2, 2, expect="flash16", weights=True)
+    _check(nn, oracle, rng, "bf16", 256, 3, 1504, 2, 2, expect="flash16", weights=False, mask_shape=(1504, 3))
