@@ -1,4 +1,6 @@
-// Split-kv attention for a single query per (head, batch) ("decode" shape, Lq = 1), bf16 / f16 / Float32.
+// Split-kv attention for a single query per (head, batch) ("decode" shape, Lq = 1), bf16 / f16 / Float32; calls with
+// two to four queries (no weights, a mask only if it does not depend on the query) run through the same kernels
+// with that many softmax states per wavefront (template parameter NQ).
 //
 // The work is a stream over K and V: every byte is read once and used once, so the kernel is
 // organised around HBM, not around the matrix cores.  A kv row (all heads) is E contiguous elements;
