@@ -183,6 +183,19 @@ struct VecIO {
             for (int e = 0; e < 8; e++) v[e] = T::to_f32(h[e]);
         }
     }
+    __device__ static u32x4_t pack(const float (&v)[VEC]) {
+        if constexpr (VEC == 4) {
+            floatx4_t f;
+#pragma unroll
+            for (int e = 0; e < 4; e++) f[e] = v[e];
+            return __builtin_bit_cast(u32x4_t, f);
+        } else {
+            typename T::vec8 h;
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = T::from_f32(v[e]);
+            return __builtin_bit_cast(u32x4_t, h);
+        }
+    }
     __device__ static void store(t *p, const float (&v)[VEC]) {
         if constexpr (VEC == 4) {
             floatx4_t f;
@@ -229,8 +242,8 @@ __device__ inline int64_t xcd_order(int64_t tile, int64_t n_tiles) {
 }
 
 // lanes with equal (lane & (TI-1)) hold slices of the same positions: butterfly within the wavefront,
-// then the eight wavefronts of a 512-thread workgroup through LDS (red: 8 * 64 * VEC floats)
-template <bool IS_MAX, int VEC>
+// then the NW wavefronts of the workgroup through LDS (red: NW * 64 * VEC floats)
+template <bool IS_MAX, int VEC, int NW>
 __device__ inline void reduce_slices_vec(float (&v)[VEC], int ti_log2, float *red) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, ti = 1 << ti_log2;
     for (int o = 32; o >= ti; o >>= 1) {
@@ -251,7 +264,7 @@ __device__ inline void reduce_slices_vec(float (&v)[VEC], int ti_log2, float *re
     for (int e = 0; e < VEC; e++) {
         float r = red[il * VEC + e];
 #pragma unroll
-        for (int w = 1; w < 8; w++) {
+        for (int w = 1; w < NW; w++) {
             const float u = red[(w * 64 + il) * VEC + e];
             r = IS_MAX ? fmaxf(r, u) : r + u;
         }
@@ -259,34 +272,82 @@ __device__ inline void reduce_slices_vec(float (&v)[VEC], int ti_log2, float *re
     }
 }
 
-// Columns of up to NP * TJ elements (TJ = 512 / TI): the NP 16-byte pieces of a thread stay in registers
+// Keeps a thread's cached pieces in their packed form between the passes: without it the compiler unpacks
+// 16-bit pieces once and carries the Float32 values (twice the registers) from pass to pass, which spills.
+template <int NP>
+__device__ inline void keep_packed(u32x4_t (&raw)[NP]) {
+#pragma unroll
+    for (int u = 0; u < NP; u++) asm volatile("" : "+v"(raw[u]));
+}
+
+// Columns of up to NP * TJ elements (TJ = NT / TI): the NP 16-byte pieces of a thread stay in registers
 // between the reduction and the result, so every element is read once and written once.  All loads are
-// issued before any arithmetic and are unconditional (threads without work read a valid dummy address).
-template <typename T, int OP, int VEC, int NP>
-__global__ __launch_bounds__(512) void softmax_nd_cached_kernel(const typename T::type *x, const typename T::type *x2,
-                                                                 typename T::type *y, Geometry g) {
+// issued before any arithmetic.  One slab (the inner x len elements of one outer index, below 2 GiB) is
+// addressed through a buffer resource: a thread keeps one 32-bit offset, the row of each piece comes from
+// a scalar offset, and pieces past the column's end (or columns past `inner`) get an offset outside the
+// resource, which reads as zeros.  That leaves the registers to the cached pieces.
+template <typename T>
+struct CachedTile {
+    __amdgpu_buffer_rsrc_t rx, rx2, ry;   // the slab of the tile's outer index in x, x2 (gradients) and y
+    int64_t o;                            // outer index
+    int col;                              // first column of the tile
+    int voff, nrows;                      // this thread's byte offset in the slab; pieces it holds
+    bool ok;                              // the thread's columns exist
+};
+
+// FULL: every thread holds NP pieces of a valid column (len = NP * TJ, inner a multiple of TI * VEC), so
+// the passes are straight-line code.  Columns with infinities take the reference's special cases through
+// a branch that is uniform over the wavefront.
+template <typename T, int OP, int VEC, int NP, int NT, bool FULL>
+__global__ __launch_bounds__(NT, (NP * (OP >= OP_GRAD_SOFTMAX ? 2 : 1) <= 16 && OP != OP_LOGSUMEXP ? 2 : 1) * NT / 256) void softmax_nd_cached_kernel(
+        const typename T::type *x, const typename T::type *x2, typename T::type *y, Geometry g) {
     typedef typename T::type t;
     typedef VecIO<T, VEC> IO;
     constexpr bool GRAD = OP >= OP_GRAD_SOFTMAX;
-    __shared__ float red[8 * 64 * VEC];
-    const int ti = 1 << g.ti_log2, tj = 512 >> g.ti_log2;
+    constexpr int NW = NT / 64, OOB = 0x7fffffff, SZ = (int)sizeof(t);
+    __shared__ float red[NW * 64 * VEC];
+    const int ti = 1 << g.ti_log2, tj = NT >> g.ti_log2;
     const int il = threadIdx.x & (ti - 1), js = threadIdx.x >> g.ti_log2;
     const int64_t n_tiles = g.n_itiles * g.outer;
-    const int64_t step = g.inner * tj;   // elements between consecutive rows of one thread
-    for (int64_t tile0 = blockIdx.x; tile0 < n_tiles; tile0 += gridDim.x) {
+    const int inner = (int)g.inner, len = (int)g.len;   // a slab is below 2 GiB (host)
+    const int slab_bytes = inner * len * SZ;
+    const int step_bytes = inner * tj * SZ;   // between consecutive rows of one thread
+    // the thread's offset within a tile whose first column is 0 (threads past the column's end never use it)
+    const int thread_off = js < len ? (il * VEC + inner * js) * SZ : 0;
+    // scalar offset of a thread's u-th piece; 0 for pieces that lie past the column's end for every thread
+    const auto row_off = [&](int u) { return FULL || u * tj < len ? step_bytes * u : 0; };
+    const auto locate = [&](int64_t tile0) {
+        CachedTile<T> c;
         const int64_t tile = xcd_order(tile0, n_tiles);
-        const int64_t o = tile / g.n_itiles, i = ((tile % g.n_itiles) * ti + il) * VEC;
-        const bool ok = i < g.inner;
-        const int nrows = ok && js < g.len ? (int)((g.len - js + tj - 1) / tj) : 0;   // <= NP (host)
-        const int64_t base = nrows ? i + g.inner * g.len * o + g.inner * js : g.inner * g.len * o;
-        const int last = nrows ? nrows - 1 : 0;
-        u32x4_t raw[NP], raw2[GRAD ? NP : 1];
+        c.o = tile / g.n_itiles;
+        c.col = (int)(tile % g.n_itiles) * ti * VEC;
+        c.ok = FULL || c.col + il * VEC < inner;
+        c.nrows = FULL ? NP : (c.ok && js < len ? (len - js + tj - 1) / tj : 0);   // <= NP (host)
+        c.voff = thread_off + c.col * SZ;
+        const int64_t slab = g.inner * g.len * c.o;
+        c.rx = __builtin_amdgcn_make_buffer_rsrc((void *)(x + slab), 0, slab_bytes, 0x00020000);
+        c.rx2 = __builtin_amdgcn_make_buffer_rsrc((void *)((GRAD ? x2 : x) + slab), 0, slab_bytes, 0x00020000);
+        c.ry = __builtin_amdgcn_make_buffer_rsrc((void *)(y + (OP == OP_LOGSUMEXP ? 0 : slab)), 0, slab_bytes, 0x00020000);
+        return c;
+    };
+    u32x4_t raw[NP], raw2[GRAD ? NP : 1];
+    const auto request = [&](const CachedTile<T> &c, int u) {
+        const int vo = FULL || u < c.nrows ? c.voff : OOB;
+        raw[u] = __builtin_amdgcn_raw_buffer_load_b128(c.rx, vo, row_off(u), 0);
+        if constexpr (GRAD) raw2[u] = __builtin_amdgcn_raw_buffer_load_b128(c.rx2, vo, row_off(u), 0);
+    };
+    // Stores carry the row in the vector offset, not in the scalar one: the compiler keeps writes to the
+    // data registers of a 16-byte buffer store away from the store only when its scalar offset is not a
+    // register, and with one the next piece's arithmetic, which reuses those registers at once, now and
+    // then overwrote the first of them before the store had read it (a few elements in ten thousand).
+    const auto put = [&](const CachedTile<T> &c, int u, const u32x4_t &piece) {
+        __builtin_amdgcn_raw_buffer_store_b128(piece, c.ry, c.voff + row_off(u), 0, 0);
+    };
+    for (int64_t tile0 = blockIdx.x; tile0 < n_tiles; tile0 += gridDim.x) {
+        const CachedTile<T> cur = locate(tile0);
 #pragma unroll
-        for (int u = 0; u < NP; u++) {
-            const int64_t at = base + step * (u < last ? u : last);
-            raw[u] = *(const u32x4_t *)(x + at);
-            if (GRAD) raw2[u] = *(const u32x4_t *)(x2 + at);
-        }
+        for (int u = 0; u < NP; u++) request(cur, u);
+        const int nrows = cur.nrows;
         float m[VEC], sum[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
@@ -296,7 +357,7 @@ __global__ __launch_bounds__(512) void softmax_nd_cached_kernel(const typename T
         if constexpr (GRAD) {
 #pragma unroll
             for (int u = 0; u < NP; u++) {
-                if (u < nrows) {
+                if (FULL || u < nrows) {
                     float v[VEC], v2[VEC];
                     IO::unpack(raw[u], v);
                     if (OP == OP_GRAD_SOFTMAX) IO::unpack(raw2[u], v2);
@@ -304,82 +365,106 @@ __global__ __launch_bounds__(512) void softmax_nd_cached_kernel(const typename T
                     for (int e = 0; e < VEC; e++) sum[e] += OP == OP_GRAD_SOFTMAX ? v[e] * v2[e] : v[e];
                 }
             }
-            reduce_slices_vec<false, VEC>(sum, g.ti_log2, red);
+            reduce_slices_vec<false, VEC, NW>(sum, g.ti_log2, red);
+            keep_packed(raw);
+            keep_packed(raw2);
 #pragma unroll
             for (int u = 0; u < NP; u++) {
-                if (u < nrows) {
+                if (FULL || u < nrows) {
                     float v[VEC], v2[VEC], r[VEC];
                     IO::unpack(raw[u], v);
                     IO::unpack(raw2[u], v2);
 #pragma unroll
                     for (int e = 0; e < VEC; e++)
                         r[e] = OP == OP_GRAD_SOFTMAX ? v2[e] * (v[e] - sum[e]) : v[e] - sum[e] * fast_exp(v2[e]);
-                    IO::store(y + base + step * u, r);
+                    put(cur, u, IO::pack(r));
                 }
             }
-            continue;
-        }
-        // forward ops: maximum, sum of exponentials, result, all from the registers
+        } else {
+            // forward ops: maximum, sum of exponentials, result, all from the registers
 #pragma unroll
-        for (int u = 0; u < NP; u++) {
-            if (u < nrows) {
-                float v[VEC];
-                IO::unpack(raw[u], v);
+            for (int u = 0; u < NP; u++) {
+                if (FULL || u < nrows) {
+                    float v[VEC];
+                    IO::unpack(raw[u], v);
 #pragma unroll
-                for (int e = 0; e < VEC; e++) m[e] = fmaxf(m[e], v[e]);
+                    for (int e = 0; e < VEC; e++) m[e] = fmaxf(m[e], v[e]);
+                }
             }
-        }
-        reduce_slices_vec<true, VEC>(m, g.ti_log2, red);
-        bool plain = true;   // finite maxima: no special cases
+            reduce_slices_vec<true, VEC, NW>(m, g.ti_log2, red);
+            bool finite = true;   // finite maxima: no special cases
 #pragma unroll
-        for (int e = 0; e < VEC; e++) plain = plain && m[e] > MI_NEG_INF && m[e] < MI_POS_INF;
-        float c0[VEC];
+            for (int e = 0; e < VEC; e++) finite = finite && m[e] > MI_NEG_INF && m[e] < MI_POS_INF;
+            // the same for the whole wavefront; logsumexp has no special cases (src/softmax.jl:202)
+            const bool plain = OP == OP_LOGSUMEXP || __builtin_amdgcn_ballot_w64(!finite) == 0;
+            keep_packed(raw);
+            if (plain) {
+                float cm[VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; e++) c0[e] = -m[e] * MI_LOG2E;
+                for (int e = 0; e < VEC; e++) cm[e] = -m[e] * MI_LOG2E;
 #pragma unroll
-        for (int u = 0; u < NP; u++) {
-            if (u < nrows) {
-                float v[VEC];
-                IO::unpack(raw[u], v);
+                for (int u = 0; u < NP; u++) {
+                    if (FULL || u < nrows) {
+                        float v[VEC];
+                        IO::unpack(raw[u], v);
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) sum[e] += mi_exp2(fmaf(v[e], MI_LOG2E, cm[e]));
+                    }
+                }
+            } else {
+                // an infinite maximum somewhere in the wavefront (rare): the reference's special cases, one
+                // piece at a time from memory in a rolled loop, so that this path costs the other no registers
+#pragma unroll 1
+                for (int u = 0; u < nrows; u++) {
+                    float v[VEC];
+                    IO::unpack(__builtin_amdgcn_raw_buffer_load_b128(cur.rx, cur.voff + step_bytes * u, 0, 0), v);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++)
+                        sum[e] += OP == OP_SOFTMAX ? softmax_term(v[e], m[e]) : fast_exp(logsoftmax_shift(v[e], m[e]));
+                }
+            }
+            reduce_slices_vec<false, VEC, NW>(sum, g.ti_log2, red);
+            keep_packed(raw);
+            if constexpr (OP == OP_LOGSUMEXP) {
+                if (cur.ok && js == 0) {
+                    float r[VEC];
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) r[e] = m[e] + logf(sum[e]);
+                    IO::store(y + cur.col + il * VEC + g.inner * cur.o, r);
+                }
+            } else if (plain) {
+                // m and sum fold into two constants per position
+                float c0[VEC], c1[VEC];
 #pragma unroll
                 for (int e = 0; e < VEC; e++) {
-                    if (plain) sum[e] += mi_exp2(fmaf(v[e], MI_LOG2E, c0[e]));
-                    else if (OP == OP_SOFTMAX) sum[e] += softmax_term(v[e], m[e]);
-                    else if (OP == OP_LOGSOFTMAX) sum[e] += fast_exp(logsoftmax_shift(v[e], m[e]));
-                    else sum[e] += fast_exp(v[e] - m[e]);   // logsumexp: no special cases (src/softmax.jl:202)
+                    if (OP == OP_SOFTMAX) {
+                        c0[e] = -m[e] * MI_LOG2E;
+                        c1[e] = 1.0f / sum[e];
+                    } else {
+                        c1[e] = -m[e] - logf(sum[e]);
+                    }
                 }
-            }
-        }
-        reduce_slices_vec<false, VEC>(sum, g.ti_log2, red);
-        if constexpr (OP == OP_LOGSUMEXP) {
-            if (ok && js == 0) {
-                float r[VEC];
 #pragma unroll
-                for (int e = 0; e < VEC; e++) r[e] = m[e] + logf(sum[e]);
-                IO::store(y + i + g.inner * o, r);
-            }
-            continue;
-        }
-        float c1[VEC];
+                for (int u = 0; u < NP; u++) {
+                    if (FULL || u < nrows) {
+                        float v[VEC], r[VEC];
+                        IO::unpack(raw[u], v);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-            if (OP == OP_SOFTMAX) c1[e] = 1.0f / sum[e];
-            else {
-                c0[e] = logf(sum[e]);
-                c1[e] = -m[e] - c0[e];
-            }
-        }
+                        for (int e = 0; e < VEC; e++)
+                            r[e] = OP == OP_SOFTMAX ? mi_exp2(fmaf(v[e], MI_LOG2E, c0[e])) * c1[e] : v[e] + c1[e];
+                        put(cur, u, IO::pack(r));
+                    }
+                    }
+            } else {
+#pragma unroll 1
+                for (int u = 0; u < nrows; u++) {
+                    float v[VEC], r[VEC];
+                    IO::unpack(__builtin_amdgcn_raw_buffer_load_b128(cur.rx, cur.voff + step_bytes * u, 0, 0), v);
 #pragma unroll
-        for (int u = 0; u < NP; u++) {
-            if (u < nrows) {
-                float v[VEC], r[VEC];
-                IO::unpack(raw[u], v);
-#pragma unroll
-                for (int e = 0; e < VEC; e++) {
-                    if (OP == OP_SOFTMAX) r[e] = plain ? mi_exp2(fmaf(v[e], MI_LOG2E, c0[e])) * c1[e] : softmax_term(v[e], m[e]) / sum[e];
-                    else r[e] = plain ? v[e] + c1[e] : logsoftmax_shift(v[e], m[e]) - c0[e];
+                    for (int e = 0; e < VEC; e++)
+                        r[e] = OP == OP_SOFTMAX ? softmax_term(v[e], m[e]) / sum[e] : logsoftmax_shift(v[e], m[e]) - logf(sum[e]);
+                    __builtin_amdgcn_raw_buffer_store_b128(IO::pack(r), cur.ry, cur.voff + step_bytes * u, 0, 0);
                 }
-                IO::store(y + base + step * u, r);
             }
         }
     }
@@ -515,18 +600,36 @@ void launch_nd(const void *x, const void *x2, void *y, int64_t inner, int64_t le
     if (inner % VEC == 0 && inner >= 4 * VEC && len > 64 && al(x) && al(y) && (!x2 || al(x2))) {
         // wide rows and columns too long for the register cache of the scalar kernel
         const int64_t chunks = inner / VEC;
+        // register-cached kernel: a thread holds NP pieces (two workgroups per compute unit) or 2 NP (one);
+        // the second is taken when it makes the contiguous pieces of a row wider, which is what the memory
+        // system rewards (256 x 4096 x 128 bf16 over dim 2: 0.185 ms with 32-byte pieces, 0.131 with 64)
         constexpr int NP = OP >= OP_GRAD_SOFTMAX ? 8 : 16;   // the gradients hold two arrays
-        if (len <= 512 * NP) {
-            // register-cached kernel: TI as wide as the column length allows (TJ * NP >= len)
-            g.ti_log2 = 0;
-            while ((1 << g.ti_log2) < 64 && ((int64_t)1 << g.ti_log2) < chunks && (int64_t)(512 >> (g.ti_log2 + 1)) * NP >= len)
-                g.ti_log2++;
-            while (g.ti_log2 > 0 && ((chunks + (1 << g.ti_log2) - 1) >> g.ti_log2) * outer < 1024) g.ti_log2--;
+        if (len <= 512 * 2 * NP && inner * len * (int64_t)sizeof(t) < ((int64_t)1 << 31)) {
+            // TI as wide as the column length allows (TJ * pieces >= len), but at least 1024 tiles
+            const auto widest = [&](int np) {
+                int tl = 0;
+                while ((1 << tl) < 64 && ((int64_t)1 << tl) < chunks && (int64_t)(512 >> (tl + 1)) * np >= len) tl++;
+                while (tl > 0 && ((chunks + (1 << tl) - 1) >> tl) * outer < 1024) tl--;
+                return tl;
+            };
+            const int t1 = len <= 512 * NP ? widest(NP) : -1, t2 = widest(2 * NP);
+            const bool wide = t2 > t1;
+            g.ti_log2 = wide ? t2 : t1;
             g.n_itiles = (chunks + (1 << g.ti_log2) - 1) >> g.ti_log2;
             int64_t blocks = g.n_itiles * outer;
             if (blocks > 262144) blocks = 262144;
-            hipLaunchKernelGGL((softmax_nd_cached_kernel<T, OP, VEC, NP>), dim3((unsigned)blocks), dim3(512), 0, st,
-                               (const t *)x, (const t *)x2, (t *)y, g);
+            const bool full = len == (int64_t)(512 >> g.ti_log2) * (wide ? 2 * NP : NP) && chunks % (1 << g.ti_log2) == 0;
+#define MI_CACHED_LAUNCH(NP_, FULL_)                                                                                 \
+    hipLaunchKernelGGL((softmax_nd_cached_kernel<T, OP, VEC, NP_, 512, FULL_>), dim3((unsigned)blocks), dim3(512), 0, \
+                       st, (const t *)x, (const t *)x2, (t *)y, g)
+            if (wide) {
+                if (full) MI_CACHED_LAUNCH(2 * NP, true);
+                else MI_CACHED_LAUNCH(2 * NP, false);
+            } else {
+                if (full) MI_CACHED_LAUNCH(NP, true);
+                else MI_CACHED_LAUNCH(NP, false);
+            }
+#undef MI_CACHED_LAUNCH
             return;
         }
         g.ti_log2 = 0;

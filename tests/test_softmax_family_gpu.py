@@ -54,7 +54,9 @@ SHAPES = [((2, 2, 2, 2, 2), d) for d in (1, 2, 3, 4, 5)] + [
     ((5, 7), 2), ((3, 4), None), ((33, 65, 3), 2), ((64, 100, 5), 2), ((130, 17, 2), (2, 3)), ((7, 3000, 2), 2),
     ((1, 5000, 3), 2), ((300, 70, 2), 2), ((5000,), 1), ((70000,), None), ((4, 9, 6), (1, 2)), ((128, 40), 1),
     ((9, 5), 3), ((256, 1000, 3), 2), ((96, 129, 2), 2), ((32, 70, 2, 2), (2, 3)), ((1024, 65), 2),
-    ((64, 9000, 2), 2), ((32, 5000, 2), 2), ((8, 8192, 1), 2), ((520, 300, 1), 2)]
+    ((64, 9000, 2), 2), ((32, 5000, 2), 2), ((8, 8192, 1), 2), ((520, 300, 1), 2),
+    # columns that exactly fill the register cache (straight-line kernels): 4096 for the gradients, 8192 and 16384
+    ((32, 4096, 2), 2), ((32, 8192, 2), 2), ((32, 16384, 2), 2), ((64, 12000, 1), 2)]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
@@ -110,11 +112,13 @@ def test_errors(nn):
         nn.grad_softmax_(nn.DeviceArray.zeros((3, 2)), nn.DeviceArray.zeros((2, 3)), nn.DeviceArray.zeros((2, 3)))
 
 
-@pytest.mark.parametrize("length", [200, 9000], ids=["register-cached", "streamed"])
+@pytest.mark.parametrize("length", [200, 8192, 9000, 16384, 20000],
+                         ids=["register-cached", "cache-filled", "register-cached-32-pieces", "cache-filled-32-pieces", "streamed"])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_special_values_on_the_wide_row_kernel(nn, oracle, dtype, length):
-    """Both strided kernels (columns held in registers; longer columns with a one-pass maximum-and-sum)
-    keep the +-Inf / NaN rules of src/softmax.jl:72-75, 140-144 wherever the special entry sits."""
+    """Both strided kernels (columns held in registers, with and without the straight-line variant for columns
+    that fill the cache exactly; longer columns with a one-pass maximum-and-sum) keep the +-Inf / NaN rules of
+    src/softmax.jl:72-75, 140-144 wherever the special entry sits."""
     rng = np.random.default_rng(11)
     x = round_to(rng.standard_normal((64, length, 2)), dtype)
     x[0, :, 0] = -np.inf                      # all -Inf: NaN
@@ -141,7 +145,7 @@ def test_special_values_on_the_wide_row_kernel(nn, oracle, dtype, length):
         assert np.abs(got[fin] - ref[fin]).max() <= tol * 10
 
 
-@pytest.mark.parametrize("length", [200, 9000, 20000], ids=["register-cached", "streamed", "streamed-long"])
+@pytest.mark.parametrize("length", [200, 8192, 9000, 20000], ids=["register-cached", "cache-filled", "register-cached-32-pieces", "streamed"])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_nan_poisons_its_whole_column_wherever_it_sits(nn, oracle, dtype, length):
     """src/softmax.jl:69-70: a NaN becomes the column maximum, so the whole column is NaN.  In the streamed kernel
@@ -243,3 +247,30 @@ def test_dims_that_are_not_neighbours(nn, oracle, shape, dims):
     out = nn.DeviceArray.zeros(shape)
     assert nn.softmax_(out, d, dims=dims) is out
     assert np.abs(out.to_numpy() - sm).max() < 1e-6
+
+
+@pytest.mark.parametrize("outer", [64, 128], ids=["16-pieces", "32-pieces"])
+def test_strided_softmax_at_the_benchmark_shape(nn, oracle, outer):
+    """bench.py's `softmax_dims2` array (256 x 4096 x 128 bf16, dims = 2) and its half: the straight-line
+    register-cached kernels with 32- and 64-byte row pieces.  The oracle is run on three of the outer slices;
+    every column of every slice must sum to one."""
+    rng = np.random.default_rng(outer)
+    x = round_to(rng.standard_normal((256, 4096, outer), dtype=np.float32) * 2, "bf16")
+    d = _dev(nn, x, "bf16")
+    sm = nn.softmax(d, dims=2).to_numpy()
+    ls = nn.logsoftmax(d, dims=2).to_numpy()
+    lse = nn.logsumexp(d, dims=2).to_numpy()
+    assert np.abs(sm.sum(axis=1, dtype=np.float64) - 1.0).max() <= 2.0 ** -8   # every term is rounded to bf16
+    for o in (0, outer // 2 - 1, outer - 1):
+        xs = x[:, :, o:o + 1]
+        assert np.abs(sm[:, :, o:o + 1] - oracle.softmax(xs, 2)).max() <= TOL["bf16"]
+        ref = oracle.logsoftmax(xs, 2)
+        assert np.abs(ls[:, :, o:o + 1] - ref).max() <= TOL["bf16"] * np.abs(ref).max()
+        ref = oracle.logsumexp(xs, 2)
+        assert np.abs(lse[:, :, o:o + 1] - ref).max() <= TOL["bf16"] * np.abs(ref).max()
+    y = round_to(sm, "bf16")
+    dy = round_to(rng.standard_normal(x.shape, dtype=np.float32), "bf16")
+    g = nn.grad_softmax(_dev(nn, dy, "bf16"), _dev(nn, y, "bf16"), dims=2).to_numpy()
+    for o in (0, outer - 1):
+        ref = oracle.grad_softmax(dy[:, :, o:o + 1], y[:, :, o:o + 1], 2)
+        assert np.abs(g[:, :, o:o + 1] - ref).max() <= 4 * TOL["bf16"] * max(1.0, np.abs(ref).max())
