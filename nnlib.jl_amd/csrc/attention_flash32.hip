@@ -9,6 +9,8 @@
 // The contraction index of QK^T is permuted so that a lane fetches K with 16-byte LDS reads:
 // k-step 4c+j of half-wave hh multiplies feature d = 8c + 4hh + j (Q is loaded with the same map).
 #include "flash_common.h"
+#include <cstdlib>
+#include <type_traits>
 
 namespace {
 
@@ -132,8 +134,227 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
     }
 }
 
-template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS>
-// Head dim 64 without bias / mask fits two workgroups per CU (256 registers, 70 KiB of LDS each).
+// ---------------------------------------------------------------------------------------------------
+// Float32 products on the 16-bit matrix cores.  A Float32 value is the exact sum of three bf16 values up
+// to 2^-24 of its size (x = hi + mid + lo, each the bf16 rounding of what the ones before leave), a
+// product of two bf16 values is exact in Float32, and the matrix cores accumulate in Float32; so
+//   a b = a_hi b_hi + (a_hi b_mid + a_mid b_hi) + (a_hi b_lo + a_lo b_hi + a_mid b_mid) + O(2^-24 |a b|)
+// costs six v_mfma_f32_32x32x16_bf16 (6 x 32 cycles for 32x32x16 multiply-adds) where the Float32
+// instruction needs eight v_mfma_f32_32x32x2_f32 of 64 cycles each: 2.7 times less matrix-pipe time at the
+// accuracy of the Float32 instruction (the three dropped terms are below the rounding of the sum).  K and V
+// tiles are split once when they are staged (three bf16 planes per tile in LDS, laid out and read like the
+// tiles of the 16-bit kernel), Q once per workgroup, the softmax weights once per tile in registers.
+typedef bf16x8_t plane8;
+typedef bf16x4_t plane4;
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+// x -> (hi, mid, lo).  An Inf or NaN goes into the lo plane alone: lo only ever multiplies the hi plane of the
+// other operand, which has that operand's sign and is zero only if the operand is (to 2^-133), so the product
+// is the Inf or NaN that the Float32 instruction would give (Inf x Inf excepted, which gives NaN here).
+__device__ inline void split3(float x, __bf16 &hi, __bf16 &mid, __bf16 &lo, bool guard) {
+    hi = (__bf16)x;
+    const float r = x - (float)hi;
+    mid = (__bf16)r;
+    lo = (__bf16)(r - (float)mid);
+    if (guard && !(__builtin_fabsf(x) < MI_POS_INF)) {
+        hi = (__bf16)0.0f;
+        mid = (__bf16)0.0f;
+        lo = (__bf16)x;
+    }
+}
+
+template <int D>
+struct CfgS {
+    static constexpr int ROWB = D * 2;              // bytes per tile row of one plane
+    static constexpr int PLANEB = BN * ROWB;        // one plane of one tile
+    static constexpr int TILEB = 3 * PLANEB;        // K or V tile: hi, mid, lo planes
+    static constexpr int CHUNKS = BN * D / 4 / 256; // float4 pieces per thread, tile and tensor
+    static constexpr size_t SMEM = 2 * TILEB;       // one K and one V tile (the next one waits in registers)
+    // chunk swizzle of the 16-bit kernel (conflict-free 16-byte operand reads and transposing reads)
+    __device__ static inline int swz(int row) {
+        if (D >= 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+        const int x = (row >> 1) & 7;
+        return ((x & 1) << 2) | (x >> 1);
+    }
+};
+
+template <int D, int QB>
+struct Frag32S {
+    plane8 q[QB][3][D / 16];
+    floatx16_t o[QB][D / 32];
+    float m[QB], l[QB];
+};
+
+__device__ inline plane4 lds_tr4s(unsigned addr) {
+    s16x4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t *)(uintptr_t)addr);
+    return __builtin_bit_cast(plane4, r);
+}
+
+__device__ inline floatx16_t mfma_bf16(plane8 a, plane8 b, floatx16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// c += a b with a, b given as planes (small terms first).  Alternating two accumulators between consecutive
+// instructions instead measured 4-8 % slower.
+__device__ inline floatx16_t mfma_split(const plane8 (&a)[3], const plane8 (&b)[3], floatx16_t c) {
+    c = mfma_bf16(a[2], b[0], c);
+    c = mfma_bf16(a[0], b[2], c);
+    c = mfma_bf16(a[1], b[1], c);
+    c = mfma_bf16(a[1], b[0], c);
+    c = mfma_bf16(a[0], b[1], c);
+    return mfma_bf16(a[0], b[0], c);
+}
+
+template <int D, int QB, bool CAUSAL, bool EXTRAS, int PHASE>
+__device__ inline void run_tiles32s(const FlashArgs &a, Frag32S<D, QB> &f, unsigned Ks, unsigned Vs, int64_t kv_len, int64_t b, int64_t h,
+                                    int64_t iw, int n_tiles, unsigned wlds = 0, int jt0 = 0) {
+    typedef CfgS<D> C;
+    constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB, CHUNKS = C::CHUNKS;
+    const AttnParams &p = a.p;
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hh = lane >> 5;
+    constexpr bool NEED_V = PHASE != PHASE_STATS;
+    const bool do_pv = NEED_V && p.out != nullptr;
+    typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+    typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
+
+    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
+    const float *vbase = NEED_V && p.v ? (const float *)p.v + p.Ev * (p.Lkv * b) + p.Dv * h : nullptr;
+    const int dqk = (int)p.D, dv = (int)p.Dv;
+
+    floatx4_t kreg[CHUNKS], vreg[CHUNKS];
+    auto load_tile = [&](int jt) {
+        const int64_t j0 = (int64_t)jt * BN;
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            const bool ok = j0 + row < kv_len;
+            kreg[u] = ldg16f(kbase + p.E * (j0 + row) + col, ok && col < dqk);
+            if (NEED_V) vreg[u] = ldg16f(vbase + p.Ev * (j0 + row) + col, ok && do_pv && col < dv);
+        }
+    };
+    // four consecutive features of one key: 8 bytes in each of the three planes
+    auto store_split = [&](unsigned tile, int row, int col, const floatx4_t &x) {
+        __bf16 pl[3][4];
+        // one test for the four values; a chunk with an Inf or NaN (rare) is split again with the per-value rule
+        const float big = mi_max3(__builtin_fabsf(x[0]), __builtin_fabsf(x[1]), fmaxf(__builtin_fabsf(x[2]), __builtin_fabsf(x[3])));
+        const bool finite = big < MI_POS_INF && x[0] == x[0] && x[1] == x[1] && x[2] == x[2] && x[3] == x[3];
+#pragma unroll
+        for (int e = 0; e < 4; e++) split3(x[e], pl[0][e], pl[1][e], pl[2][e], false);
+        if (!finite) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) split3(x[e], pl[0][e], pl[1][e], pl[2][e], true);
+        }
+        const unsigned at = tile + (unsigned)row * ROWB + (unsigned)((((col >> 3) ^ C::swz(row)) << 4) + (col & 7) * 2);
+#pragma unroll
+        for (int q = 0; q < 3; q++) {
+            const plane4 v4 = {pl[q][0], pl[q][1], pl[q][2], pl[q][3]};
+            *(lds8_t)(uintptr_t)(at + q * PLANEB) = __builtin_bit_cast(u32x2_t, v4);
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            store_split(Ks, row, col, kreg[u]);
+            if (NEED_V) store_split(Vs, row, col, vreg[u]);
+        }
+    };
+
+    if (n_tiles <= jt0) return;
+    load_tile(jt0);
+    __syncthreads();   // a previous phase may still be reading the tile
+    store_tile();
+    __syncthreads();
+
+    for (int jt = jt0; jt < n_tiles; jt++) {
+        const int64_t j0 = (int64_t)jt * BN;
+        const bool more = jt + 1 < n_tiles;
+        if (more) load_tile(jt + 1);
+
+        const bool active = !CAUSAL || j0 <= iw + 32 * QB - 1;
+        if (active) {
+            floatx16_t s[QB][2];
+#pragma unroll
+            for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) s[qb][kb] = (floatx16_t){0};
+            // lane's K operand: row r (+32 per key block), chunk 2t + hh, in each plane
+            const unsigned kt = Ks + (unsigned)r * ROWB;
+            const int ksw = C::swz(r);
+#pragma unroll
+            for (int t = 0; t < D / 16; t++)
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+                    plane8 ka[3];
+#pragma unroll
+                    for (int q = 0; q < 3; q++)
+                        ka[q] = *(lds_plane8_t)(uintptr_t)(kt + q * PLANEB + kb * 32 * ROWB + (((2 * t + hh) ^ ksw) << 4));
+#pragma unroll
+                    for (int qb = 0; qb < QB; qb++) {
+                        const plane8 qq[3] = {f.q[qb][0][t], f.q[qb][1][t], f.q[qb][2][t]};
+                        s[qb][kb] = mfma_split(ka, qq, s[qb][kb]);
+                    }
+                }
+
+            flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0,
+                                                                                                          FlashStaged<QB>(), 0, wlds, nullptr, kv_len);
+
+            if (do_pv) {
+                // P^T operand of k-step u of key block kb: accumulator registers 8u .. 8u+7 (keys 0-3, 8-11 | 4-7, 12-15
+                // of the 16); V^T comes from the row-major planes with the transposing read in that same key order
+                const int vrow = 4 * hh + ((lane & 15) >> 2);
+                const int vchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), vsub = 8 * (lane & 1);
+                const unsigned vt = Vs + (unsigned)vrow * ROWB + vsub;
+                const int vsw_lo = C::swz(vrow), vsw_hi = C::swz(vrow + 8);
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int u = 0; u < 2; u++) {
+                        plane8 pk[QB][3];
+#pragma unroll
+                        for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+                            for (int e = 0; e < 8; e++) {
+                                __bf16 x0, x1, x2;
+                                split3(s[qb][kb][8 * u + e], x0, x1, x2, false);
+                                pk[qb][0][e] = x0;
+                                pk[qb][1][e] = x1;
+                                pk[qb][2][e] = x2;
+                            }
+#pragma unroll
+                        for (int dvb = 0; dvb < D / 32; dvb++) {
+                            const unsigned src = vt + (32 * kb + 16 * u) * ROWB;
+                            plane8 va[3];
+#pragma unroll
+                            for (int q = 0; q < 3; q++) {
+                                const plane4 lo = lds_tr4s(src + q * PLANEB + (((4 * dvb + vchunk) ^ vsw_lo) << 4));
+                                const plane4 hi = lds_tr4s(src + q * PLANEB + 8 * ROWB + (((4 * dvb + vchunk) ^ vsw_hi) << 4));
+                                va[q] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                            }
+#pragma unroll
+                            for (int qb = 0; qb < QB; qb++) f.o[qb][dvb] = mfma_split(va, pk[qb], f.o[qb][dvb]);
+                        }
+                    }
+            }
+        }
+        if (more) {
+            __syncthreads();   // every wavefront is done with the tile in LDS
+            store_tile();
+        }
+        __syncthreads();
+    }
+}
+
+template <int D, int QB, bool SPLIT>
+struct FragSel { typedef Frag32<D, QB> type; };
+template <int D, int QB>
+struct FragSel<D, QB, true> { typedef Frag32S<D, QB> type; };
+
+template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS, bool SPLIT>
+// Head dim 64 without bias / mask fits two workgroups per CU (256 registers, 70 KiB of LDS each; 56 KiB with the
+// bf16 planes, bias / mask or not).
 __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_kernel(FlashArgs a) {
     constexpr int KS = Cfg<D>::KS, VS = Cfg<D>::VS;
     const AttnParams &p = a.p;
@@ -141,6 +362,10 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
     float *Ks = (float *)flash_smem;     // [2][BN][KS]
     float *Vs = Ks + 2 * BN * KS;        // [2][BN][VS]
     (void)VS;
+    // bf16 planes: one K tile, one V tile, as LDS byte addresses
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem;
+    const unsigned Kp = lds0, Vp = lds0 + CfgS<D>::TILEB;
+    constexpr size_t TILES_SMEM = SPLIT ? CfgS<D>::SMEM : Cfg<D>::SMEM;
     constexpr int BM = 128 * QB;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
@@ -161,24 +386,49 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
         if (!EXTRAS) kv_len = len;
     }
 
-    Frag32<D, QB> f;
+    typename FragSel<D, QB, SPLIT>::type f;
     const float *qbase = (const float *)p.q + p.E * (p.Lq * b) + p.D * h;
     const float sq = sqrtf((float)p.D);
 #pragma unroll
     for (int qb = 0; qb < QB; qb++) {
         const int64_t qi = iw + 32 * qb + r;
+        if constexpr (SPLIT) {
+            // lane's features of k-step t: 16t + 8hh .. + 7 (the B-operand layout of the 16-bit instruction)
 #pragma unroll
-        for (int c = 0; c < D / 8; c++) {
-            const floatx4_t q4 = ldg16f(qbase + p.E * qi + 8 * c + 4 * hh, qi < p.Lq && 8 * c + 4 * hh < p.D);
-            // the reference divides q by sqrt(D) before the product (src/attention.jl:118)
+            for (int t = 0; t < D / 16; t++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) f.q[qb][4 * c + j] = q4[j] / sq;
+                for (int half = 0; half < 2; half++) {
+                    const int d0 = 16 * t + 8 * hh + 4 * half;
+                    const floatx4_t q4 = ldg16f(qbase + p.E * qi + d0, qi < p.Lq && d0 < p.D);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        __bf16 x0, x1, x2;
+                        split3(q4[j] / sq, x0, x1, x2, true);   // the reference divides q by sqrt(D) first (src/attention.jl:118)
+                        f.q[qb][0][t][4 * half + j] = x0;
+                        f.q[qb][1][t][4 * half + j] = x1;
+                        f.q[qb][2][t][4 * half + j] = x2;
+                    }
+                }
+        } else {
+#pragma unroll
+            for (int c = 0; c < D / 8; c++) {
+                const floatx4_t q4 = ldg16f(qbase + p.E * qi + 8 * c + 4 * hh, qi < p.Lq && 8 * c + 4 * hh < p.D);
+                // the reference divides q by sqrt(D) before the product (src/attention.jl:118)
+#pragma unroll
+                for (int j = 0; j < 4; j++) f.q[qb][4 * c + j] = q4[j] / sq;
+            }
         }
 #pragma unroll
         for (int dvb = 0; dvb < D / 32; dvb++) f.o[qb][dvb] = (floatx16_t){0};
         f.m[qb] = MI_NEG_INF;
         f.l[qb] = 0.0f;
     }
+    // one entry point for both tile loops
+    auto run = [&](auto phase, int n, unsigned wlds, int jt0) {
+        constexpr int PHASE = decltype(phase)::value;
+        if constexpr (SPLIT) run_tiles32s<D, QB, CAUSAL, EXTRAS, PHASE>(a, f, Kp, Vp, kv_len, b, h, iw, n, wlds, jt0);
+        else run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE>(a, f, Ks, Vs, kv_len, b, h, iw, n, wlds, jt0);
+    };
 
     int64_t kv_end = kv_len;
     if (CAUSAL && i0 + BM < kv_end) kv_end = i0 + BM;
@@ -190,7 +440,7 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
             jt0 = split * a.tiles_per_split;
             if (jt0 + a.tiles_per_split < jt1) jt1 = jt0 + a.tiles_per_split;
         }
-        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_ONLINE>(a, f, Ks, Vs, kv_len, b, h, iw, jt1, 0, jt0);
+        run(std::integral_constant<int, PHASE_ONLINE>(), jt1, 0u, jt0);
         if (a.nsplit > 1) {
             // partial result of this key piece for flash_merge_kernel: unnormalised o, row maximum (log2 units), row sum
             float *wo = (float *)p.workspace + ((int64_t)split * p.B + b) * p.Lq * p.Ev + p.Dv * h;
@@ -218,16 +468,15 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
             return;
         }
     } else {
-        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_STATS>(a, f, Ks, Vs, kv_len, b, h, iw, n_tiles);
+        run(std::integral_constant<int, PHASE_STATS>(), n_tiles, 0u, 0);
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) {
             const float l = f.l[qb] + mi_swap32(f.l[qb]);
             f.l[qb] = 1.0f / l;
         }
         // weight tiles leave through a wavefront-private LDS region behind the K / V buffers
-        const unsigned wlds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem +
-                              (unsigned)Cfg<D>::SMEM + wave * FLASH_WSTAGE_BYTES;
-        run_tiles32<D, QB, CAUSAL, EXTRAS, PHASE_FINAL>(a, f, Ks, Vs, kv_len, b, h, iw, n_tiles, wlds);
+        const unsigned wlds = lds0 + (unsigned)TILES_SMEM + wave * FLASH_WSTAGE_BYTES;
+        run(std::integral_constant<int, PHASE_FINAL>(), n_tiles, wlds, 0);
         if (CAUSAL && p.weights) flash_zero_skipped_weights<QB, float>(a, b, h, iw, n_tiles);
         else if (p.weights && kv_len < p.Lkv) flash_zero_skipped_weights<QB, float>(a, b, h, iw, n_tiles, false);   // keys past the context length
     }
@@ -258,11 +507,11 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
     }
 }
 
-template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS>
+template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS, bool SPLIT>
 int32_t launch_one(const FlashArgs &a, hipStream_t st) {
     const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B * a.nsplit;
-    constexpr size_t smem = Cfg<D>::SMEM + (WEIGHTS ? 4 * FLASH_WSTAGE_BYTES : 0);
-    auto kern = flash32_kernel<D, QB, CAUSAL, EXTRAS, WEIGHTS>;
+    constexpr size_t smem = (SPLIT ? CfgS<D>::SMEM : Cfg<D>::SMEM) + (WEIGHTS ? 4 * FLASH_WSTAGE_BYTES : 0);
+    auto kern = flash32_kernel<D, QB, CAUSAL, EXTRAS, WEIGHTS, SPLIT>;
     static bool attr_set = false;
     if (!attr_set) {
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -273,15 +522,31 @@ int32_t launch_one(const FlashArgs &a, hipStream_t st) {
     return MI_OK;
 }
 
-template <int D, int QB>
-int32_t launch_d(const FlashArgs &a, hipStream_t st, bool extras) {
+template <int D, int QB, bool SPLIT>
+int32_t launch_ds(const FlashArgs &a, hipStream_t st, bool extras) {
     const bool w = a.p.weights != nullptr;
     if (a.p.causal) {
-        if (extras) return w ? launch_one<D, QB, true, true, true>(a, st) : launch_one<D, QB, true, true, false>(a, st);
-        return w ? launch_one<D, QB, true, false, true>(a, st) : launch_one<D, QB, true, false, false>(a, st);
+        if (extras) return w ? launch_one<D, QB, true, true, true, SPLIT>(a, st) : launch_one<D, QB, true, true, false, SPLIT>(a, st);
+        return w ? launch_one<D, QB, true, false, true, SPLIT>(a, st) : launch_one<D, QB, true, false, false, SPLIT>(a, st);
     }
-    if (extras) return w ? launch_one<D, QB, false, true, true>(a, st) : launch_one<D, QB, false, true, false>(a, st);
-    return w ? launch_one<D, QB, false, false, true>(a, st) : launch_one<D, QB, false, false, false>(a, st);
+    if (extras) return w ? launch_one<D, QB, false, true, true, SPLIT>(a, st) : launch_one<D, QB, false, true, false, SPLIT>(a, st);
+    return w ? launch_one<D, QB, false, false, true, SPLIT>(a, st) : launch_one<D, QB, false, false, false, SPLIT>(a, st);
+}
+
+// Products on the 16-bit matrix cores through three bf16 planes (see run_tiles32s) unless the caller's
+// environment asks for the Float32 matrix instruction (MI355ATTN_F32_MFMA=1).
+bool exact_instruction_wanted() {
+    static const bool wanted = [] {
+        const char *e = getenv("MI355ATTN_F32_MFMA");
+        return e && e[0] == '1';
+    }();
+    return wanted;
+}
+
+template <int D, int QB>
+int32_t launch_d(const FlashArgs &a, hipStream_t st, bool extras) {
+    if (exact_instruction_wanted()) return launch_ds<D, QB, false>(a, st, extras);
+    return launch_ds<D, QB, true>(a, st, extras);
 }
 
 }  // namespace

@@ -598,3 +598,83 @@ def test_a_few_queries_with_weights_or_a_query_dependent_mask_take_the_tiled_ker
     rng = np.random.default_rng(9)
     _check(nn, oracle, rng, "bf16", 256, 3, 1500, 2, 2, expect="flash16", weights=True)
     _check(nn, oracle, rng, "bf16", 256, 3, 1504, 2, 2, expect="flash16", weights=False, mask_shape=(1504, 3))
+
+
+def _f64_attention(q, k, v, H, causal=False):
+    """Brute force in float64 on the float32 inputs, with q divided by sqrt(D) in float32 as src/attention.jl:118 does."""
+    E, Lq, B = q.shape
+    Lkv, D = k.shape[1], E // H
+    y = np.zeros((v.shape[0], Lq, B))
+    a = np.zeros((Lkv, Lq, H, B))
+    Dv = v.shape[0] // H
+    for b in range(B):
+        for h in range(H):
+            qs = (q[h * D:(h + 1) * D, :, b] / np.float32(np.sqrt(np.float32(D)))).astype(np.float64)
+            s = k[h * D:(h + 1) * D, :, b].astype(np.float64).T @ qs
+            if causal:
+                s = np.where(np.arange(Lkv)[:, None] <= np.arange(Lq)[None, :], s, -np.inf)
+            w = np.exp(s - s.max(axis=0, keepdims=True))
+            w /= w.sum(axis=0, keepdims=True)
+            a[:, :, h, b] = w
+            y[h * Dv:(h + 1) * Dv, :, b] = v[h * Dv:(h + 1) * Dv, :, b].astype(np.float64) @ w
+    return y, a
+
+
+_F32_SCRIPT = """
+import sys, numpy as np
+sys.path.insert(0, %r)
+import nnlib_amd as nn
+d = np.load(sys.argv[1])
+q, k, v = (nn.DeviceArray.from_numpy(d[n], "f32") for n in "qkv")
+y, a = nn.dot_product_attention(q, k, v, nheads=int(d["H"]), mask=(nn.make_causal_mask(q, dims=2) if int(d["causal"]) else None))
+np.savez(sys.argv[2], y=y.to_numpy(), a=a.to_numpy())
+"""
+
+
+@pytest.mark.parametrize("E,H,L,causal", [(256, 4, 300, False), (256, 4, 257, True), (256, 2, 200, False), (96, 1, 130, True)],
+                         ids=["D64", "D64-causal", "D128", "D96-causal"])
+def test_float32_products_through_bf16_planes_keep_float32_accuracy(nn, oracle, tmp_path, E, H, L, causal):
+    """Float32 calls run their products as six bf16 matrix instructions per Float32 one (three planes per operand).
+    Against float64 on the same inputs the result must be as close as the Float32 matrix instruction's, which a child
+    process computes with MI355ATTN_F32_MFMA=1: values spread over 2^+-12 so that every plane carries weight."""
+    import os, subprocess, sys
+    rng = np.random.default_rng(E + L)
+    spread = lambda shape: (rng.standard_normal(shape) * np.exp2(rng.integers(-12, 1, shape))).astype(np.float32)
+    q, k, v = spread((E, L, 2)), spread((E, L, 2)), spread((E, L, 2))
+    y64, a64 = _f64_attention(q, k, v, H, causal)
+    y, a = _run(nn, q, k, v, "f32", nheads=H, causal=causal, weights_dtype="f32")
+    assert nn.last_attention_kernel() == "flash32"
+    err_y, err_a = np.abs(y - y64).max() / np.abs(y64).max(), np.abs(a - a64).max()
+    assert err_y < 5e-6 and err_a < 5e-6, (err_y, err_a)
+    # the same call on the Float32 matrix instruction, in a process of its own (the choice is made once per process)
+    np.savez(tmp_path / "in.npz", q=q, k=k, v=v, H=H, causal=int(causal))
+    env = dict(os.environ, MI355ATTN_F32_MFMA="1")
+    pkg = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "nnlib.jl_amd")
+    subprocess.run([sys.executable, "-c", _F32_SCRIPT % pkg, str(tmp_path / "in.npz"), str(tmp_path / "out.npz")], env=env, check=True, timeout=300)
+    ref = np.load(tmp_path / "out.npz")
+    err_y2, err_a2 = np.abs(ref["y"] - y64).max() / np.abs(y64).max(), np.abs(ref["a"] - a64).max()
+    assert err_y2 < 5e-6 and err_a2 < 5e-6, (err_y2, err_a2)
+    assert err_y < 4 * err_y2 + 2e-7 and err_a < 4 * err_a2 + 2e-7, (err_y, err_y2, err_a, err_a2)
+
+
+def test_float32_products_with_infinite_inputs(nn, oracle):
+    """An Inf in k whose q entries are all negative makes that key's logits -Inf, as the Float32 instruction would
+    (an Inf goes through the planes with its sign): the key gets no weight and the rest is the call without it.  A NaN
+    in v poisons only the outputs that weight it."""
+    rng = np.random.default_rng(77)
+    E, L = 64, 140
+    q = rng.standard_normal((E, L, 1)).astype(np.float32)
+    k = rng.standard_normal((E, L, 1)).astype(np.float32)
+    v = rng.standard_normal((E, L, 1)).astype(np.float32)
+    q[7] = -np.abs(q[7]) - 0.5
+    k[7, 33, 0] = np.inf
+    y, a = _run(nn, q, k, v, "f32", nheads=1, weights_dtype="f32")
+    assert nn.last_attention_kernel() == "flash32"
+    assert np.all(a[33, :, 0, 0] == 0) and np.isfinite(y).all() and np.isfinite(a).all()
+    keep = np.arange(L) != 33
+    yr, ar = oracle.nnlib_attention_f32(q, k[:, keep], v[:, keep], None, None, 1)
+    assert rel_err(y, yr) < 1e-5 and np.allclose(a[keep], ar, atol=1e-6)
+    v2 = v.copy()
+    v2[5, 90, 0] = np.nan
+    y2, _ = _run(nn, q, k, v2, "f32", nheads=1, weights_dtype="f32")
+    assert np.isnan(y2[5]).all() and np.isfinite(np.delete(y2, 5, axis=0)).all()
