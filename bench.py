@@ -264,6 +264,10 @@ def measure(key, steps, warmup, with_cpu):
         pk = PEAK[w["dtype"]]
         roof = dict(bound="mfma", achieved=tflops, peak=pk, unit="TFLOP/s", frac=tflops / pk, traffic=traffic,
                     traffic_source=source, hbm_frac=gbps / HBM_PEAK)
+        if w["dtype"] == "f32":
+            # Float32 in, out and accumulation; `peak` stays the Float32 matrix instruction's
+            roof["products"] = ("v_mfma_f32_32x32x2_f32" if os.environ.get("MI355ATTN_F32_MFMA", "")[:1] == "1" else
+                                "six v_mfma_f32_32x32x16_bf16 on three bf16 planes per operand (Float32 accuracy)")
     res = dict(workload=w["name"], kernel=r.kernel, preheat_ms=r.preheat_ms, ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, gbps=gbps,
                flops_per_step=flops, bytes_per_step=nbytes, roofline=roof)
     if with_cpu:

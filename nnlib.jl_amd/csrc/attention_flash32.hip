@@ -163,6 +163,33 @@ __device__ inline void split3(float x, __bf16 &hi, __bf16 &mid, __bf16 &lo, bool
     }
 }
 
+// Two values at once, the way the hardware converts (one v_cvt_pk_bf16_f32 per plane and pair): each result word
+// holds the plane's bf16 of x0 in its low half and of x1 in its high half.  Returns true if x0 or x1 is Inf or NaN
+// (their residual x - hi is NaN then); the caller redoes such values with split3's rule.
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t pack_bf16_pair(float a, float b) {
+    const float2_t f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+__device__ inline bool split3_pair(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
+    hi = pack_bf16_pair(x0, x1);
+    const float r0 = x0 - __builtin_bit_cast(float, hi << 16), r1 = x1 - __builtin_bit_cast(float, hi & 0xffff0000u);
+    mid = pack_bf16_pair(r0, r1);
+    lo = pack_bf16_pair(r0 - __builtin_bit_cast(float, mid << 16), r1 - __builtin_bit_cast(float, mid & 0xffff0000u));
+    return __builtin_isunordered(r0, r1);
+}
+// the guarded rule of split3 for a pair
+__device__ inline void split3_pair_guarded(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
+    __bf16 h0, m0, l0, h1, m1, l1;
+    split3(x0, h0, m0, l0, true);
+    split3(x1, h1, m1, l1, true);
+    const bf16x2_t h = {h0, h1}, m = {m0, m1}, l = {l0, l1};
+    hi = __builtin_bit_cast(uint32_t, h);
+    mid = __builtin_bit_cast(uint32_t, m);
+    lo = __builtin_bit_cast(uint32_t, l);
+}
+
 template <int D>
 struct CfgS {
     static constexpr int ROWB = D * 2;              // bytes per tile row of one plane
@@ -235,22 +262,15 @@ __device__ inline void run_tiles32s(const FlashArgs &a, Frag32S<D, QB> &f, unsig
     };
     // four consecutive features of one key: 8 bytes in each of the three planes
     auto store_split = [&](unsigned tile, int row, int col, const floatx4_t &x) {
-        __bf16 pl[3][4];
-        // one test for the four values; a chunk with an Inf or NaN (rare) is split again with the per-value rule
-        const float big = mi_max3(__builtin_fabsf(x[0]), __builtin_fabsf(x[1]), fmaxf(__builtin_fabsf(x[2]), __builtin_fabsf(x[3])));
-        const bool finite = big < MI_POS_INF && x[0] == x[0] && x[1] == x[1] && x[2] == x[2] && x[3] == x[3];
-#pragma unroll
-        for (int e = 0; e < 4; e++) split3(x[e], pl[0][e], pl[1][e], pl[2][e], false);
-        if (!finite) {
-#pragma unroll
-            for (int e = 0; e < 4; e++) split3(x[e], pl[0][e], pl[1][e], pl[2][e], true);
+        uint32_t pl[3][2];
+        const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        if (odd) {   // an Inf or NaN in the chunk (rare)
+            split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+            split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
         }
         const unsigned at = tile + (unsigned)row * ROWB + (unsigned)((((col >> 3) ^ C::swz(row)) << 4) + (col & 7) * 2);
 #pragma unroll
-        for (int q = 0; q < 3; q++) {
-            const plane4 v4 = {pl[q][0], pl[q][1], pl[q][2], pl[q][3]};
-            *(lds8_t)(uintptr_t)(at + q * PLANEB) = __builtin_bit_cast(u32x2_t, v4);
-        }
+        for (int q = 0; q < 3; q++) *(lds8_t)(uintptr_t)(at + q * PLANEB) = (u32x2_t){pl[q][0], pl[q][1]};
     };
     auto store_tile = [&]() {
 #pragma unroll
@@ -314,15 +334,14 @@ __device__ inline void run_tiles32s(const FlashArgs &a, Frag32S<D, QB> &f, unsig
                     for (int u = 0; u < 2; u++) {
                         plane8 pk[QB][3];
 #pragma unroll
-                        for (int qb = 0; qb < QB; qb++)
+                        for (int qb = 0; qb < QB; qb++) {
+                            uint32_t w[3][4];
 #pragma unroll
-                            for (int e = 0; e < 8; e++) {
-                                __bf16 x0, x1, x2;
-                                split3(s[qb][kb][8 * u + e], x0, x1, x2, false);
-                                pk[qb][0][e] = x0;
-                                pk[qb][1][e] = x1;
-                                pk[qb][2][e] = x2;
-                            }
+                            for (int e = 0; e < 4; e++)   // a NaN weight (fully masked column) stays NaN in the hi plane
+                                split3_pair(s[qb][kb][8 * u + 2 * e], s[qb][kb][8 * u + 2 * e + 1], w[0][e], w[1][e], w[2][e]);
+#pragma unroll
+                            for (int q = 0; q < 3; q++) pk[qb][q] = __builtin_bit_cast(plane8, (u32x4_t){w[q][0], w[q][1], w[q][2], w[q][3]});
+                        }
 #pragma unroll
                         for (int dvb = 0; dvb < D / 32; dvb++) {
                             const unsigned src = vt + (32 * kb + 16 * u) * ROWB;
@@ -394,21 +413,27 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
         const int64_t qi = iw + 32 * qb + r;
         if constexpr (SPLIT) {
             // lane's features of k-step t: 16t + 8hh .. + 7 (the B-operand layout of the 16-bit instruction)
+            uint32_t qw[3][D / 16][4];
 #pragma unroll
             for (int t = 0; t < D / 16; t++)
 #pragma unroll
                 for (int half = 0; half < 2; half++) {
                     const int d0 = 16 * t + 8 * hh + 4 * half;
                     const floatx4_t q4 = ldg16f(qbase + p.E * qi + d0, qi < p.Lq && d0 < p.D);
+                    // the reference divides q by sqrt(D) first (src/attention.jl:118)
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        __bf16 x0, x1, x2;
-                        split3(q4[j] / sq, x0, x1, x2, true);   // the reference divides q by sqrt(D) first (src/attention.jl:118)
-                        f.q[qb][0][t][4 * half + j] = x0;
-                        f.q[qb][1][t][4 * half + j] = x1;
-                        f.q[qb][2][t][4 * half + j] = x2;
+                    for (int j = 0; j < 2; j++) {
+                        uint32_t w[3];
+                        const float x0 = q4[2 * j] / sq, x1 = q4[2 * j + 1] / sq;
+                        if (split3_pair(x0, x1, w[0], w[1], w[2])) split3_pair_guarded(x0, x1, w[0], w[1], w[2]);
+#pragma unroll
+                        for (int q = 0; q < 3; q++) qw[q][t][2 * half + j] = w[q];
                     }
                 }
+#pragma unroll
+            for (int q = 0; q < 3; q++)
+#pragma unroll
+                for (int t = 0; t < D / 16; t++) f.q[qb][q][t] = __builtin_bit_cast(plane8, (u32x4_t){qw[q][t][0], qw[q][t][1], qw[q][t][2], qw[q][t][3]});
         } else {
 #pragma unroll
             for (int c = 0; c < D / 8; c++) {
