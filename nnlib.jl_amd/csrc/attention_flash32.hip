@@ -148,48 +148,6 @@ typedef bf16x8_t plane8;
 typedef bf16x4_t plane4;
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
-// x -> (hi, mid, lo).  An Inf or NaN goes into the lo plane alone: lo only ever multiplies the hi plane of the
-// other operand, which has that operand's sign and is zero only if the operand is (to 2^-133), so the product
-// is the Inf or NaN that the Float32 instruction would give (Inf x Inf excepted, which gives NaN here).
-__device__ inline void split3(float x, __bf16 &hi, __bf16 &mid, __bf16 &lo, bool guard) {
-    hi = (__bf16)x;
-    const float r = x - (float)hi;
-    mid = (__bf16)r;
-    lo = (__bf16)(r - (float)mid);
-    if (guard && !(__builtin_fabsf(x) < MI_POS_INF)) {
-        hi = (__bf16)0.0f;
-        mid = (__bf16)0.0f;
-        lo = (__bf16)x;
-    }
-}
-
-// Two values at once, the way the hardware converts (one v_cvt_pk_bf16_f32 per plane and pair): each result word
-// holds the plane's bf16 of x0 in its low half and of x1 in its high half.  Returns true if x0 or x1 is Inf or NaN
-// (their residual x - hi is NaN then); the caller redoes such values with split3's rule.
-typedef float float2_t __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-__device__ inline uint32_t pack_bf16_pair(float a, float b) {
-    const float2_t f = {a, b};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
-}
-__device__ inline bool split3_pair(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
-    hi = pack_bf16_pair(x0, x1);
-    const float r0 = x0 - __builtin_bit_cast(float, hi << 16), r1 = x1 - __builtin_bit_cast(float, hi & 0xffff0000u);
-    mid = pack_bf16_pair(r0, r1);
-    lo = pack_bf16_pair(r0 - __builtin_bit_cast(float, mid << 16), r1 - __builtin_bit_cast(float, mid & 0xffff0000u));
-    return __builtin_isunordered(r0, r1);
-}
-// the guarded rule of split3 for a pair
-__device__ inline void split3_pair_guarded(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
-    __bf16 h0, m0, l0, h1, m1, l1;
-    split3(x0, h0, m0, l0, true);
-    split3(x1, h1, m1, l1, true);
-    const bf16x2_t h = {h0, h1}, m = {m0, m1}, l = {l0, l1};
-    hi = __builtin_bit_cast(uint32_t, h);
-    mid = __builtin_bit_cast(uint32_t, m);
-    lo = __builtin_bit_cast(uint32_t, l);
-}
-
 template <int D>
 struct CfgS {
     static constexpr int ROWB = D * 2;              // bytes per tile row of one plane

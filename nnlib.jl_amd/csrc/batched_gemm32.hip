@@ -9,6 +9,7 @@
 // 4-byte read whatever the memory layout of the matrix.  As in the other GEMM kernels the MFMA runs on
 // the transposed problem so that a half-wave stores 32 consecutive elements of a C column.
 #include "common.h"
+#include <cstdlib>
 
 namespace {
 
@@ -142,6 +143,187 @@ __global__ __launch_bounds__(256, 2) void gemm32_kernel(Gemm32Args g) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The same product on the 16-bit matrix cores: both operands as three bf16 planes (see common.h), six
+// v_mfma_f32_32x32x16_bf16 per 32x32x16 block.  Same workgroup shape and double-buffered 16-k stages; a tile
+// is split when it is stored to LDS and keeps the orientation its memory has, as in the 16-bit kernel:
+//   RMAJ (contiguous along its row index): [16 k][128 rows] per plane, 256-byte k-rows with swizzled
+//        16-byte chunks, MFMA operand through the transposing LDS read;
+//   KMAJ (contiguous along k): [128 rows][16 k] per plane, 32-byte rows whose two 16-byte chunks hold
+//        k {0-3, 8-11} and {4-7, 12-15}, the order in which the transposing read delivers a step to the two
+//        half-waves; the operand is one 16-byte read.
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef bf16x8_t plane8;
+typedef bf16x4_t plane4;
+constexpr int PLANEB = 128 * KC * 2;    // bytes of one plane of one operand tile (4 KiB)
+constexpr int TILE3B = 3 * PLANEB;
+
+__device__ inline int rmaj_swz(int kk) { return ((kk & 3) << 2) | ((kk >> 2) & 3); }
+
+template <bool RM>
+struct OperandS {
+    const float *X;
+    int64_t ld, rows, k, row0;
+    floatx4_t reg[2];
+
+    __device__ void load(int64_t k0) {
+        const int tid = threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int c = tid + 256 * u;
+            const floatx4_t z = {0.f, 0.f, 0.f, 0.f};
+            if (RM) {
+                const int kk = c >> 5, r4 = (c & 31) * 4;     // 32 pieces per k-row
+                reg[u] = (k0 + kk < k && row0 + r4 < rows) ? *(const floatx4_t *)(X + (row0 + r4) + (k0 + kk) * ld) : z;
+            } else {
+                const int r = c >> 2, k4 = (c & 3) * 4;       // 4 pieces per row
+                reg[u] = (row0 + r < rows && k0 + k4 < k) ? *(const floatx4_t *)(X + (k0 + k4) + (row0 + r) * ld) : z;
+            }
+        }
+    }
+    // split into planes; `tile` is the LDS byte address of the hi plane
+    __device__ void store(unsigned tile) const {
+        typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+        const int tid = threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int c = tid + 256 * u;
+            const floatx4_t x = reg[u];
+            uint32_t pl[3][2];
+            const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+            if (odd) {   // an Inf or NaN among the four (rare)
+                split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+                split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+            }
+            unsigned at;
+            if (RM) {
+                const int kk = c >> 5, r4 = (c & 31) * 4;     // rows r4 .. r4+3 of k-row kk
+                at = (unsigned)(kk * 256 + ((((r4 >> 3) ^ rmaj_swz(kk)) << 4) + (r4 & 7) * 2));
+            } else {
+                const int r = c >> 2, k4 = (c & 3) * 4;       // k k4 .. k4+3 of row r: chunk (k4/4)%2, 8-byte slot k4/8
+                at = (unsigned)(r * 32 + (((((k4 >> 2) & 1) ^ ((r >> 3) & 1)) << 4) + 8 * (k4 >> 3)));
+            }
+#pragma unroll
+            for (int q = 0; q < 3; q++) *(lds8_t)(uintptr_t)(tile + at + q * PLANEB) = (u32x2_t){pl[q][0], pl[q][1]};
+        }
+    }
+    // the three planes of the MFMA operand of the 32-row block `blk`
+    __device__ static void fetch(unsigned tile, int blk, int lane, plane8 (&out)[3]) {
+        const int hh = lane >> 5;
+        if (RM) {
+            const int vrow = 4 * hh + ((lane & 15) >> 2);
+            const int vchunk = 4 * blk + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), vsub = 8 * (lane & 1);
+            const unsigned lo_at = tile + (unsigned)(vrow * 256 + vsub + ((vchunk ^ rmaj_swz(vrow)) << 4));
+            const unsigned hi_at = tile + (unsigned)((vrow + 8) * 256 + vsub + ((vchunk ^ rmaj_swz(vrow + 8)) << 4));
+#pragma unroll
+            for (int q = 0; q < 3; q++) {
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t *)(uintptr_t)(lo_at + q * PLANEB));
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t *)(uintptr_t)(hi_at + q * PLANEB));
+                out[q] = __builtin_shufflevector(__builtin_bit_cast(plane4, lo), __builtin_bit_cast(plane4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        } else {
+            const int row = 32 * blk + (lane & 31);
+            const unsigned at = tile + (unsigned)(row * 32 + ((hh ^ ((row >> 3) & 1)) << 4));
+#pragma unroll
+            for (int q = 0; q < 3; q++) out[q] = *(__attribute__((address_space(3))) const plane8 *)(uintptr_t)(at + q * PLANEB);
+        }
+    }
+};
+
+template <bool A_RM, bool B_RM>
+__global__ __launch_bounds__(256, 2) void gemm32s_kernel(Gemm32Args g) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[4 * TILE3B];   // A and B tiles, two buffers each: 48 KiB
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    const int64_t bz = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
+    const int r = lane & 31, hh = lane >> 5;
+
+    OperandS<A_RM> a;
+    OperandS<B_RM> b;
+    a.X = g.A + bz * g.sA;
+    a.ld = g.lda;
+    a.rows = g.m;
+    a.k = g.k;
+    a.row0 = (int64_t)blockIdx.x * TM;
+    b.X = g.B + bz * g.sB;
+    b.ld = g.ldb;
+    b.rows = g.n;
+    b.k = g.k;
+    b.row0 = (int64_t)blockIdx.y * TN;
+
+    floatx16_t acc[2][2];   // [n block][m block]
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = (floatx16_t){0};
+
+    // One stage of loads in flight.  Three (two more register sets) measured 0.25 against 0.19 ms on the
+    // 1024 x 64 x 1024 x 128 product: the registers cost the third workgroup per CU.
+    const int nk = (int)((g.k + KC - 1) / KC);
+    a.load(0);
+    b.load(0);
+    a.store(lds0);
+    b.store(lds0 + 2 * TILE3B);
+    __syncthreads();
+    for (int it = 0; it < nk; it++) {
+        const int buf = it & 1;
+        if (it + 1 < nk) {
+            a.load((int64_t)(it + 1) * KC);
+            b.load((int64_t)(it + 1) * KC);
+        }
+        const unsigned at = lds0 + buf * TILE3B, bt = lds0 + (2 + buf) * TILE3B;
+        plane8 av[2][3], bv[2][3];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            OperandS<A_RM>::fetch(at, 2 * wm + j, lane, av[j]);
+            OperandS<B_RM>::fetch(bt, 2 * wn + j, lane, bv[j]);
+        }
+        // the transposed problem (rows = n, columns = m), small terms first
+        constexpr int ia[6] = {2, 0, 1, 1, 0, 0}, ib[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+        for (int t = 0; t < 6; t++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bv[i][ib[t]], av[j][ia[t]], acc[i][j], 0, 0, 0);
+        if (it + 1 < nk) {
+            a.store(lds0 + (buf ^ 1) * TILE3B);
+            b.store(lds0 + (2 + (buf ^ 1)) * TILE3B);
+        }
+        __syncthreads();
+    }
+
+    // accumulator register v of lane (r, hh) of block (i, j): n = 32i + 8*(v/4) + 4*hh + v%4, m = 32j + r
+    float *C = g.C + bz * g.sC;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int64_t mi = a.row0 + 64 * wm + 32 * j + r;
+        if (mi >= g.m) continue;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int64_t nj = b.row0 + 64 * wn + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
+                if (nj < g.n) {
+                    float *c = C + mi + nj * g.ldc;
+                    float val = g.alpha * acc[i][j][v];
+                    if (g.beta != 0.0f) val += g.beta * *c;
+                    *c = val;
+                }
+            }
+    }
+}
+
+// the Float32 matrix instruction instead of the bf16 planes (MI355ATTN_F32_MFMA=1 in the environment, read once)
+bool exact_instruction_wanted() {
+    static const bool wanted = [] {
+        const char *e = getenv("MI355ATTN_F32_MFMA");
+        return e && e[0] == '1';
+    }();
+    return wanted;
+}
+
 }  // namespace
 
 // true when every 16-byte piece the kernel moves is aligned and wholly inside or outside its matrix
@@ -165,10 +347,17 @@ int32_t launch_batched_gemm32(int transA, int transB, int64_t m, int64_t n, int6
         Gemm32Args g = {(const float *)A + b0 * sA, (const float *)B + b0 * sB, (float *)C + b0 * sC,
                         m, n, k, lda, ldb, ldc, sA, sB, sC, alpha, beta};
         dim3 grid((unsigned)((m + TM - 1) / TM), (unsigned)((n + TN - 1) / TN), (unsigned)nb);
-        if (a_rm && b_rm) hipLaunchKernelGGL((gemm32_kernel<true, true>), grid, dim3(256), 0, st, g);
-        else if (a_rm) hipLaunchKernelGGL((gemm32_kernel<true, false>), grid, dim3(256), 0, st, g);
-        else if (b_rm) hipLaunchKernelGGL((gemm32_kernel<false, true>), grid, dim3(256), 0, st, g);
-        else hipLaunchKernelGGL((gemm32_kernel<false, false>), grid, dim3(256), 0, st, g);
+        if (exact_instruction_wanted()) {
+            if (a_rm && b_rm) hipLaunchKernelGGL((gemm32_kernel<true, true>), grid, dim3(256), 0, st, g);
+            else if (a_rm) hipLaunchKernelGGL((gemm32_kernel<true, false>), grid, dim3(256), 0, st, g);
+            else if (b_rm) hipLaunchKernelGGL((gemm32_kernel<false, true>), grid, dim3(256), 0, st, g);
+            else hipLaunchKernelGGL((gemm32_kernel<false, false>), grid, dim3(256), 0, st, g);
+        } else {
+            if (a_rm && b_rm) hipLaunchKernelGGL((gemm32s_kernel<true, true>), grid, dim3(256), 0, st, g);
+            else if (a_rm) hipLaunchKernelGGL((gemm32s_kernel<true, false>), grid, dim3(256), 0, st, g);
+            else if (b_rm) hipLaunchKernelGGL((gemm32s_kernel<false, true>), grid, dim3(256), 0, st, g);
+            else hipLaunchKernelGGL((gemm32s_kernel<false, false>), grid, dim3(256), 0, st, g);
+        }
         MI_LAUNCH_CHECK();
     }
     return MI_OK;

@@ -112,6 +112,54 @@ __device__ static inline void mi_pair_halves(uint32_t &x, uint32_t &y) {
 
 __device__ static inline float mi_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// ---- Float32 values as three bf16 planes (Float32 products on the 16-bit matrix cores) ----------------
+// x = hi + mid + lo to 2^-24 of |x|, each plane the bf16 rounding of what the ones before leave.  A product of
+// two bf16 values is exact in Float32 and the matrix cores accumulate in Float32, so
+//   a b = a_hi b_hi + (a_hi b_mid + a_mid b_hi) + (a_hi b_lo + a_lo b_hi + a_mid b_mid) + O(2^-24 |a b|):
+// six v_mfma_f32_32x32x16_bf16 give a 32x32x16 block of Float32 products at the accuracy of the Float32
+// instruction in 2.7 times less matrix-pipe time than eight v_mfma_f32_32x32x2_f32.
+// x -> (hi, mid, lo).  An Inf or NaN goes into the lo plane alone: lo only ever multiplies the hi plane of the
+// other operand, which has that operand's sign and is zero only if the operand is (to 2^-133), so the product
+// is the Inf or NaN that the Float32 instruction would give (Inf x Inf excepted, which gives NaN here).
+__device__ static inline void split3(float x, __bf16 &hi, __bf16 &mid, __bf16 &lo, bool guard) {
+    hi = (__bf16)x;
+    const float r = x - (float)hi;
+    mid = (__bf16)r;
+    lo = (__bf16)(r - (float)mid);
+    if (guard && !(__builtin_fabsf(x) < MI_POS_INF)) {
+        hi = (__bf16)0.0f;
+        mid = (__bf16)0.0f;
+        lo = (__bf16)x;
+    }
+}
+
+// Two values at once, the way the hardware converts (one v_cvt_pk_bf16_f32 per plane and pair): each result word
+// holds the plane's bf16 of x0 in its low half and of x1 in its high half.  Returns true if x0 or x1 is Inf or NaN
+// (their residual x - hi is NaN then); the caller redoes such values with split3's rule.
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float mi_float2_t;
+__device__ static inline uint32_t pack_bf16_pair(float a, float b) {
+    const mi_float2_t f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+__device__ static inline bool split3_pair(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
+    hi = pack_bf16_pair(x0, x1);
+    const float r0 = x0 - __builtin_bit_cast(float, hi << 16), r1 = x1 - __builtin_bit_cast(float, hi & 0xffff0000u);
+    mid = pack_bf16_pair(r0, r1);
+    lo = pack_bf16_pair(r0 - __builtin_bit_cast(float, mid << 16), r1 - __builtin_bit_cast(float, mid & 0xffff0000u));
+    return __builtin_isunordered(r0, r1);
+}
+// the guarded rule of split3 for a pair
+__device__ static inline void split3_pair_guarded(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
+    __bf16 h0, m0, l0, h1, m1, l1;
+    split3(x0, h0, m0, l0, true);
+    split3(x1, h1, m1, l1, true);
+    const bf16x2_t h = {h0, h1}, m = {m0, m1}, l = {l0, l1};
+    hi = __builtin_bit_cast(uint32_t, h);
+    mid = __builtin_bit_cast(uint32_t, m);
+    lo = __builtin_bit_cast(uint32_t, l);
+}
+
+
 // max(a, b, c) as one instruction with no quieting of the inputs (fmaxf on MFMA results costs an extra
 // v_max x, x per operand); a NaN operand is ignored like fmaxf does.
 __device__ static inline float mi_max3(float a, float b, float c) {

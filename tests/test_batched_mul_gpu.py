@@ -366,3 +366,34 @@ def test_trivial_dimensions_and_unit_strides(nn, oracle, complex_):
                     _close(C2.to_numpy(), want, 1e-5)
                     ran += 1
     assert ran > 100
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_float32_products_through_bf16_planes_keep_float32_accuracy(nn, ta, tb):
+    """Float32 batched_mul runs its products as six bf16 matrix instructions on three bf16 planes per operand.  Against
+    float64 the error must stay at Float32 rounding level relative to sum |a||b| (2^-24 per product and sum), with
+    operand magnitudes spread over 2^+-12 so that every plane carries weight; an Inf in A gives the Inf the Float32
+    instruction would."""
+    rng = np.random.default_rng(5 + 2 * ta + tb)
+    m, k, n, b = 160, 200, 136, 3
+    spread = lambda shape: (rng.standard_normal(shape) * np.exp2(rng.integers(-12, 13, shape))).astype(np.float32)
+    A, B = spread((k, m, b) if ta else (m, k, b)), spread((n, k, b) if tb else (k, n, b))
+    dA, dB = nn.DeviceArray.from_numpy(A, "f32"), nn.DeviceArray.from_numpy(B, "f32")
+    opA = nn.batched_transpose(dA) if ta else dA
+    opB = nn.batched_transpose(dB) if tb else dB
+    C = nn.batched_mul(opA, opB).to_numpy()
+    A64 = (A.transpose(1, 0, 2) if ta else A).astype(np.float64)
+    B64 = (B.transpose(1, 0, 2) if tb else B).astype(np.float64)
+    ref = np.einsum("mkb,knb->mnb", A64, B64)
+    scale = np.einsum("mkb,knb->mnb", np.abs(A64), np.abs(B64))
+    assert np.abs(C - ref).max() / scale.max() < 1e-6
+    assert (np.abs(C - ref) / scale).max() < 4 * 2.0 ** -24 * np.sqrt(k)
+    A2 = A.copy()
+    if ta:
+        A2[3, 7, 1] = np.inf
+    else:
+        A2[7, 3, 1] = np.inf
+    B2 = np.abs(B) + np.float32(1e-3)
+    d2 = nn.DeviceArray.from_numpy(A2, "f32")
+    C2 = nn.batched_mul(nn.batched_transpose(d2) if ta else d2, nn.batched_transpose(nn.DeviceArray.from_numpy(B2, "f32")) if tb else nn.DeviceArray.from_numpy(B2, "f32")).to_numpy()
+    assert np.all(C2[7, :, 1] == np.inf) and np.isfinite(np.delete(C2[:, :, 1], 7, axis=0)).all() and np.isfinite(C2[:, :, 0]).all()
