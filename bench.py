@@ -393,6 +393,9 @@ def measure_extra(key, steps, warmup, with_cpu):
                     roofline=dict(bound="mfma", achieved=val, peak=peak, unit="TFLOP/s", frac=val / peak, traffic=None),
                     config=dict(workload=EXTRA[key], kernel={"c64": "gemm_c32_kernel", "f64": "gemm64_kernel"}.get(dt_name, "batched_gemm_kernel")),
                     flops_per_step=flops)
+        if dt_name == "f32":   # Float32 in, out and accumulation; `peak` stays the Float32 matrix instruction's
+            line["roofline"]["products"] = ("v_mfma_f32_32x32x2_f32" if os.environ.get("MI355ATTN_F32_MFMA", "")[:1] == "1" else
+                                            "six v_mfma_f32_32x32x16_bf16 on three bf16 planes per operand (Float32 accuracy)")
         if with_cpu and dt_name not in ("c64", "f64"):
             from oracle import oracle as O
             ns = min(nb, 2 if key == "batched_mul" else 32)
