@@ -1,13 +1,17 @@
-// Flash-style attention forward for Float32 inputs on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
+// Flash-style attention forward for Float32 inputs.
 //
 // Same decomposition as the 16-bit kernel: S^T = K Q^T with keys as MFMA rows and queries as
-// columns, online softmax per lane-owned query column, O^T += V^T P^T.  With one fp32 per register
-// no transposition is needed anywhere: the A operand of the second product is a plain 4-byte LDS
-// read of V[key][feature = lane], and the B operand is the softmax accumulator register itself.
-// Products and sums are true fp32 (no down-conversion), which keeps the 1e-4 parity bound.
-//
-// The contraction index of QK^T is permuted so that a lane fetches K with 16-byte LDS reads:
-// k-step 4c+j of half-wave hh multiplies feature d = 8c + 4hh + j (Q is loaded with the same map).
+// columns, online softmax per lane-owned query column, O^T += V^T P^T.  Inputs, outputs, softmax and
+// every sum are Float32; the two products run either
+//   * on the 16-bit matrix cores through three bf16 planes per operand (run_tiles32s: six
+//     v_mfma_f32_32x32x16_bf16 per Float32 product, Float32 accuracy; the default), or
+//   * on the Float32 instruction v_mfma_f32_32x32x2_f32 (run_tiles32; MI355ATTN_F32_MFMA=1 in the
+//     environment).  With one fp32 per register no transposition is needed there: the A operand of the
+//     second product is a plain 4-byte LDS read of V[key][feature = lane], the B operand is the softmax
+//     accumulator register itself, and the contraction index of QK^T is permuted so that a lane fetches K
+//     with 16-byte LDS reads (k-step 4c+j of half-wave hh multiplies feature d = 8c + 4hh + j; Q is loaded
+//     with the same map).
+// Both keep the 1e-4 parity bound with a wide margin (errors of 1e-6 against float64).
 #include "flash_common.h"
 #include <cstdlib>
 #include <type_traits>
@@ -135,15 +139,9 @@ __device__ inline void run_tiles32(const FlashArgs &a, Frag32<D, QB> &f, float *
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Float32 products on the 16-bit matrix cores.  A Float32 value is the exact sum of three bf16 values up
-// to 2^-24 of its size (x = hi + mid + lo, each the bf16 rounding of what the ones before leave), a
-// product of two bf16 values is exact in Float32, and the matrix cores accumulate in Float32; so
-//   a b = a_hi b_hi + (a_hi b_mid + a_mid b_hi) + (a_hi b_lo + a_lo b_hi + a_mid b_mid) + O(2^-24 |a b|)
-// costs six v_mfma_f32_32x32x16_bf16 (6 x 32 cycles for 32x32x16 multiply-adds) where the Float32
-// instruction needs eight v_mfma_f32_32x32x2_f32 of 64 cycles each: 2.7 times less matrix-pipe time at the
-// accuracy of the Float32 instruction (the three dropped terms are below the rounding of the sum).  K and V
-// tiles are split once when they are staged (three bf16 planes per tile in LDS, laid out and read like the
-// tiles of the 16-bit kernel), Q once per workgroup, the softmax weights once per tile in registers.
+// Float32 products on the 16-bit matrix cores (the planes and their arithmetic: common.h).  K and V tiles are
+// split once when they are staged (three bf16 planes per tile in LDS, laid out and read like the tiles of the
+// 16-bit kernel), Q once per workgroup, the softmax weights once per tile in registers.
 typedef bf16x8_t plane8;
 typedef bf16x4_t plane4;
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
