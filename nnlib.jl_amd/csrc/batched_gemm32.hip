@@ -147,33 +147,45 @@ __global__ __launch_bounds__(256, 2) void gemm32_kernel(Gemm32Args g) {
 // The same product on the 16-bit matrix cores: both operands as three bf16 planes (see common.h), six
 // v_mfma_f32_32x32x16_bf16 per 32x32x16 block.  Same workgroup shape and double-buffered 16-k stages; a tile
 // is split when it is stored to LDS and keeps the orientation its memory has, as in the 16-bit kernel:
-//   RMAJ (contiguous along its row index): [16 k][128 rows] per plane, 256-byte k-rows with swizzled
+//   RMAJ (contiguous along its row index): [16 k][rows] per plane, k-rows of 2 bytes per row with swizzled
 //        16-byte chunks, MFMA operand through the transposing LDS read;
-//   KMAJ (contiguous along k): [128 rows][16 k] per plane, 32-byte rows whose two 16-byte chunks hold
+//   KMAJ (contiguous along k): [rows][16 k] per plane, 32-byte rows whose two 16-byte chunks hold
 //        k {0-3, 8-11} and {4-7, 12-15}, the order in which the transposing read delivers a step to the two
 //        half-waves; the operand is one 16-byte read.
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef bf16x8_t plane8;
 typedef bf16x4_t plane4;
-constexpr int PLANEB = 128 * KC * 2;    // bytes of one plane of one operand tile (4 KiB)
-constexpr int TILE3B = 3 * PLANEB;
+// Two shapes, as in the 16-bit kernel: 128 x 128 output tiles on 4 wavefronts (64 x 64 each, two or three
+// workgroups per CU), and 256 x 256 on 8 wavefronts (128 (m) x 64 (n) each, one workgroup per CU), which splits every
+// operand element for twice as many products and reads 3/4 of the LDS operands per matrix instruction.
+template <bool LARGE>
+struct ShapeS {
+    static constexpr int TILE = LARGE ? 256 : 128;       // rows of an operand tile (m of A, n of B)
+    static constexpr int THREADS = LARGE ? 512 : 256;
+    static constexpr int BM = LARGE ? 4 : 2, BNB = 2;     // 32 x 32 blocks per wavefront along m and n
+    static constexpr int RMAJ_ROWB = TILE * 2;            // bytes per k-row of an RMAJ plane
+    static constexpr int PLANEB = TILE * KC * 2;          // bytes of one plane of one operand tile
+    static constexpr int TILE3B = 3 * PLANEB;
+};
 
 __device__ inline int rmaj_swz(int kk) { return ((kk & 3) << 2) | ((kk >> 2) & 3); }
 
-template <bool RM>
+template <bool RM, bool LARGE>
 struct OperandS {
+    typedef ShapeS<LARGE> S;
+    static constexpr int ROWB = S::RMAJ_ROWB, PLANEB = S::PLANEB, CPR = S::TILE / 4;   // float4 pieces per k-row
     const float *X;
     int64_t ld, rows, k, row0;
-    floatx4_t reg[2];
+    floatx4_t reg[2];   // TILE * KC / 4 pieces per tile: 2 per thread in either shape
 
     __device__ void load(int64_t k0) {
         const int tid = threadIdx.x;
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            const int c = tid + 256 * u;
+            const int c = tid + S::THREADS * u;
             const floatx4_t z = {0.f, 0.f, 0.f, 0.f};
             if (RM) {
-                const int kk = c >> 5, r4 = (c & 31) * 4;     // 32 pieces per k-row
+                const int kk = c / CPR, r4 = (c % CPR) * 4;
                 reg[u] = (k0 + kk < k && row0 + r4 < rows) ? *(const floatx4_t *)(X + (row0 + r4) + (k0 + kk) * ld) : z;
             } else {
                 const int r = c >> 2, k4 = (c & 3) * 4;       // 4 pieces per row
@@ -187,18 +199,18 @@ struct OperandS {
         const int tid = threadIdx.x;
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            const int c = tid + 256 * u;
+            const int c = tid + S::THREADS * u;
             const floatx4_t x = reg[u];
             uint32_t pl[3][2];
             const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
-            if (odd) {   // an Inf or NaN among the four (rare)
+            if (odd) {   // an Inf, a NaN or a value beyond the bf16 range among the four (rare)
                 split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
                 split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
             }
             unsigned at;
             if (RM) {
-                const int kk = c >> 5, r4 = (c & 31) * 4;     // rows r4 .. r4+3 of k-row kk
-                at = (unsigned)(kk * 256 + ((((r4 >> 3) ^ rmaj_swz(kk)) << 4) + (r4 & 7) * 2));
+                const int kk = c / CPR, r4 = (c % CPR) * 4;   // rows r4 .. r4+3 of k-row kk
+                at = (unsigned)(kk * ROWB + ((((r4 >> 3) ^ rmaj_swz(kk)) << 4) + (r4 & 7) * 2));
             } else {
                 const int r = c >> 2, k4 = (c & 3) * 4;       // k k4 .. k4+3 of row r: chunk (k4/4)%2, 8-byte slot k4/8
                 at = (unsigned)(r * 32 + (((((k4 >> 2) & 1) ^ ((r >> 3) & 1)) << 4) + 8 * (k4 >> 3)));
@@ -213,8 +225,8 @@ struct OperandS {
         if (RM) {
             const int vrow = 4 * hh + ((lane & 15) >> 2);
             const int vchunk = 4 * blk + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), vsub = 8 * (lane & 1);
-            const unsigned lo_at = tile + (unsigned)(vrow * 256 + vsub + ((vchunk ^ rmaj_swz(vrow)) << 4));
-            const unsigned hi_at = tile + (unsigned)((vrow + 8) * 256 + vsub + ((vchunk ^ rmaj_swz(vrow + 8)) << 4));
+            const unsigned lo_at = tile + (unsigned)(vrow * ROWB + vsub + ((vchunk ^ rmaj_swz(vrow)) << 4));
+            const unsigned hi_at = tile + (unsigned)((vrow + 8) * ROWB + vsub + ((vchunk ^ rmaj_swz(vrow + 8)) << 4));
 #pragma unroll
             for (int q = 0; q < 3; q++) {
                 const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t *)(uintptr_t)(lo_at + q * PLANEB));
@@ -230,35 +242,37 @@ struct OperandS {
     }
 };
 
-template <bool A_RM, bool B_RM>
-__global__ __launch_bounds__(256, 2) void gemm32s_kernel(Gemm32Args g) {
-    __shared__ __attribute__((aligned(16))) unsigned char smem[4 * TILE3B];   // A and B tiles, two buffers each: 48 KiB
-    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+template <bool A_RM, bool B_RM, bool LARGE>
+__global__ __launch_bounds__(ShapeS<LARGE>::THREADS, LARGE ? 1 : 2) void gemm32s_kernel(Gemm32Args g) {
+    typedef ShapeS<LARGE> S;
+    constexpr int TILE3B = S::TILE3B, BM = S::BM, BNB = S::BNB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];   // A and B tiles, two buffers each
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)gemm_smem;
     const int64_t bz = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
     const int r = lane & 31, hh = lane >> 5;
 
-    OperandS<A_RM> a;
-    OperandS<B_RM> b;
+    OperandS<A_RM, LARGE> a;
+    OperandS<B_RM, LARGE> b;
     a.X = g.A + bz * g.sA;
     a.ld = g.lda;
     a.rows = g.m;
     a.k = g.k;
-    a.row0 = (int64_t)blockIdx.x * TM;
+    a.row0 = (int64_t)blockIdx.x * S::TILE;
     b.X = g.B + bz * g.sB;
     b.ld = g.ldb;
     b.rows = g.n;
     b.k = g.k;
-    b.row0 = (int64_t)blockIdx.y * TN;
+    b.row0 = (int64_t)blockIdx.y * S::TILE;
 
-    floatx16_t acc[2][2];   // [n block][m block]
+    floatx16_t acc[BNB][BM];   // [n block][m block]
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < BNB; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = (floatx16_t){0};
+        for (int j = 0; j < BM; j++) acc[i][j] = (floatx16_t){0};
 
     // One stage of loads in flight.  Three (two more register sets) measured 0.25 against 0.19 ms on the
-    // 1024 x 64 x 1024 x 128 product: the registers cost the third workgroup per CU.
+    // 1024 x 64 x 1024 x 128 product with the small shape: the registers cost the third workgroup per CU.
     const int nk = (int)((g.k + KC - 1) / KC);
     a.load(0);
     b.load(0);
@@ -272,20 +286,19 @@ __global__ __launch_bounds__(256, 2) void gemm32s_kernel(Gemm32Args g) {
             b.load((int64_t)(it + 1) * KC);
         }
         const unsigned at = lds0 + buf * TILE3B, bt = lds0 + (2 + buf) * TILE3B;
-        plane8 av[2][3], bv[2][3];
+        plane8 av[BM][3], bv[BNB][3];
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            OperandS<A_RM>::fetch(at, 2 * wm + j, lane, av[j]);
-            OperandS<B_RM>::fetch(bt, 2 * wn + j, lane, bv[j]);
-        }
+        for (int j = 0; j < BM; j++) OperandS<A_RM, LARGE>::fetch(at, BM * wm + j, lane, av[j]);
+#pragma unroll
+        for (int i = 0; i < BNB; i++) OperandS<B_RM, LARGE>::fetch(bt, BNB * wn + i, lane, bv[i]);
         // the transposed problem (rows = n, columns = m), small terms first
         constexpr int ia[6] = {2, 0, 1, 1, 0, 0}, ib[6] = {0, 2, 1, 0, 1, 0};
 #pragma unroll
         for (int t = 0; t < 6; t++)
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < BNB; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < BM; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bv[i][ib[t]], av[j][ia[t]], acc[i][j], 0, 0, 0);
         if (it + 1 < nk) {
             a.store(lds0 + (buf ^ 1) * TILE3B);
@@ -297,14 +310,14 @@ __global__ __launch_bounds__(256, 2) void gemm32s_kernel(Gemm32Args g) {
     // accumulator register v of lane (r, hh) of block (i, j): n = 32i + 8*(v/4) + 4*hh + v%4, m = 32j + r
     float *C = g.C + bz * g.sC;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int64_t mi = a.row0 + 64 * wm + 32 * j + r;
+    for (int j = 0; j < BM; j++) {
+        const int64_t mi = a.row0 + 32 * BM * wm + 32 * j + r;
         if (mi >= g.m) continue;
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < BNB; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int64_t nj = b.row0 + 64 * wn + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
+                const int64_t nj = b.row0 + 32 * BNB * wn + 32 * i + 8 * (v / 4) + 4 * hh + (v % 4);
                 if (nj < g.n) {
                     float *c = C + mi + nj * g.ldc;
                     float val = g.alpha * acc[i][j][v];
@@ -313,6 +326,28 @@ __global__ __launch_bounds__(256, 2) void gemm32s_kernel(Gemm32Args g) {
                 }
             }
     }
+}
+
+template <bool A_RM, bool B_RM, bool LARGE>
+int32_t launch_planes(const Gemm32Args &g, int64_t nb, hipStream_t st) {
+    typedef ShapeS<LARGE> S;
+    auto kern = gemm32s_kernel<A_RM, B_RM, LARGE>;
+    constexpr size_t smem = 4 * S::TILE3B;
+    static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    dim3 grid((unsigned)((g.m + S::TILE - 1) / S::TILE), (unsigned)((g.n + S::TILE - 1) / S::TILE), (unsigned)nb);
+    hipLaunchKernelGGL(kern, grid, dim3(S::THREADS), smem, st, g);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+template <bool LARGE>
+int32_t launch_planes_l(const Gemm32Args &g, bool a_rm, bool b_rm, int64_t nb, hipStream_t st) {
+    if (a_rm) return b_rm ? launch_planes<true, true, LARGE>(g, nb, st) : launch_planes<true, false, LARGE>(g, nb, st);
+    return b_rm ? launch_planes<false, true, LARGE>(g, nb, st) : launch_planes<false, false, LARGE>(g, nb, st);
 }
 
 // the Float32 matrix instruction instead of the bf16 planes (MI355ATTN_F32_MFMA=1 in the environment, read once)
@@ -353,10 +388,11 @@ int32_t launch_batched_gemm32(int transA, int transB, int64_t m, int64_t n, int6
             else if (b_rm) hipLaunchKernelGGL((gemm32_kernel<false, true>), grid, dim3(256), 0, st, g);
             else hipLaunchKernelGGL((gemm32_kernel<false, false>), grid, dim3(256), 0, st, g);
         } else {
-            if (a_rm && b_rm) hipLaunchKernelGGL((gemm32s_kernel<true, true>), grid, dim3(256), 0, st, g);
-            else if (a_rm) hipLaunchKernelGGL((gemm32s_kernel<true, false>), grid, dim3(256), 0, st, g);
-            else if (b_rm) hipLaunchKernelGGL((gemm32s_kernel<false, true>), grid, dim3(256), 0, st, g);
-            else hipLaunchKernelGGL((gemm32s_kernel<false, false>), grid, dim3(256), 0, st, g);
+            // the large tile when it still gives every CU a workgroup and k is long enough to pay for its longer prologue
+            const int64_t big = ((m + 255) / 256) * ((n + 255) / 256) * nb;
+            const bool large = m >= 256 && n >= 256 && big >= 256 && k >= 128;
+            const int32_t rc = large ? launch_planes_l<true>(g, a_rm, b_rm, nb, st) : launch_planes_l<false>(g, a_rm, b_rm, nb, st);
+            if (rc != MI_OK) return rc;
         }
         MI_LAUNCH_CHECK();
     }

@@ -204,11 +204,11 @@ def test_tiled_kernel_all_layouts(nn, dtype, ta, tb, m, n, k, nb):
     assert close(got, bmm(A, B, ta, tb), dtype)
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("dtype", ["bf16", "f16", "f32"])
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
 def test_large_tile_kernel(nn, dtype, ta, tb):
-    """Enough 256 x 256 tiles to fill the chip: the eight-wavefront shape of the 16-bit kernel, ragged in m, n
-    and k, with alpha and beta."""
+    """Enough 256 x 256 tiles to fill the chip: the eight-wavefront shape of the 16-bit kernel and of the Float32
+    kernel on bf16 planes, ragged in m, n and k, with alpha and beta."""
     rng = np.random.default_rng(17)
     m, n, k, nb = 264, 520, 136, 48
     A = round_to(rng.standard_normal((k, m, nb) if ta else (m, k, nb)), dtype)
