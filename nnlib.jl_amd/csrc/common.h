@@ -123,27 +123,19 @@ __device__ static inline float mi_exp2(float x) { return __builtin_amdgcn_exp2f(
 // is the Inf or NaN that the Float32 instruction would give (Inf x Inf excepted, which gives NaN here).
 __device__ static inline void split3(float x, __bf16 &hi, __bf16 &mid, __bf16 &lo, bool guard) {
     hi = (__bf16)x;
-    const float r = x - (float)hi;
+    float r = x - (float)hi;
     mid = (__bf16)r;
     lo = (__bf16)(r - (float)mid);
-    if (guard && !(__builtin_fabsf((float)hi) < MI_POS_INF)) {
-        if (__builtin_fabsf(x) < MI_POS_INF) {
-            // finite, but its bf16 rounding overflowed (|x| > 3.3895e38): truncate the first plane instead
-            const float h = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, x) & 0xffff0000u), r2 = x - h;
-            hi = (__bf16)h;
-            mid = (__bf16)r2;
-            lo = (__bf16)(r2 - (float)mid);
-        } else {
-            hi = (__bf16)0.0f;
-            mid = (__bf16)0.0f;
-            lo = (__bf16)x;
-        }
+    if (guard && !(__builtin_fabsf(x) < MI_POS_INF)) {
+        hi = (__bf16)0.0f;
+        mid = (__bf16)0.0f;
+        lo = (__bf16)x;
     }
 }
 
 // Two values at once, the way the hardware converts (one v_cvt_pk_bf16_f32 per plane and pair): each result word
 // holds the plane's bf16 of x0 in its low half and of x1 in its high half.  Returns true if x0 or x1 is Inf or NaN
-// or rounds to Inf in bf16; the caller redoes such values with split3's rule.
+// (their residual x - hi is NaN then); the caller redoes such values with split3's rule.
 typedef __attribute__((__vector_size__(2 * sizeof(float)))) float mi_float2_t;
 __device__ static inline uint32_t pack_bf16_pair(float a, float b) {
     const mi_float2_t f = {a, b};
@@ -153,10 +145,8 @@ __device__ static inline bool split3_pair(float x0, float x1, uint32_t &hi, uint
     hi = pack_bf16_pair(x0, x1);
     const float r0 = x0 - __builtin_bit_cast(float, hi << 16), r1 = x1 - __builtin_bit_cast(float, hi & 0xffff0000u);
     mid = pack_bf16_pair(r0, r1);
-    const float s0 = r0 - __builtin_bit_cast(float, mid << 16), s1 = r1 - __builtin_bit_cast(float, mid & 0xffff0000u);
-    lo = pack_bf16_pair(s0, s1);
-    // NaN here: x is Inf or NaN, or so large that its bf16 rounding is Inf (then r = -Inf and r - mid = NaN)
-    return __builtin_isunordered(s0, s1);
+    lo = pack_bf16_pair(r0 - __builtin_bit_cast(float, mid << 16), r1 - __builtin_bit_cast(float, mid & 0xffff0000u));
+    return __builtin_isunordered(r0, r1);
 }
 // the guarded rule of split3 for a pair
 __device__ static inline void split3_pair_guarded(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
