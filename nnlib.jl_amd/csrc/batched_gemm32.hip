@@ -21,6 +21,7 @@ struct Gemm32Args {
     float *C;
     int64_t m, n, k, lda, ldb, ldc, sA, sB, sC;
     float alpha, beta;
+    int32_t c_vec;   // C base, leading dimension, slice stride and m allow aligned 16-byte stores
 };
 
 // RM: element (row, kk) at X[row + kk*ld] (contiguous along row); else at X[kk + row*ld]
@@ -309,6 +310,50 @@ __global__ __launch_bounds__(ShapeS<LARGE>::THREADS, LARGE ? 1 : 2) void gemm32s
 
     // accumulator register v of lane (r, hh) of block (i, j): n = 32i + 8*(v/4) + 4*hh + v%4, m = 32j + r
     float *C = g.C + bz * g.sC;
+    if (g.c_vec) {
+        // A lane holds single elements of 16 columns of C: stored directly, every instruction moves 4 bytes per lane.
+        // Instead each wavefront passes [32 n][64 m] blocks through a private LDS region (the operand buffers are
+        // free now) and reads them back as rows of m, so that a store instruction writes four columns of 256
+        // contiguous bytes, 16 bytes per lane (C is 512 MiB of the 1024 x 64 x 1024 x 128 product: 0.195 -> 0.178 ms).
+        typedef __attribute__((address_space(3))) float *ldsf_t;
+        typedef __attribute__((address_space(3))) const floatx4_t *ldsf4_t;
+        constexpr int LDW = 64 + 4;   // floats per LDS row
+        const unsigned region = lds0 + (unsigned)wave * (32 * LDW * 4);
+        const int64_t mw = a.row0 + 32 * BM * wm, nw = b.row0 + 32 * BNB * wn;
+#pragma unroll
+        for (int i = 0; i < BNB; i++)
+#pragma unroll
+            for (int jp = 0; jp < BM / 2; jp++) {
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++)
+                        *(ldsf_t)(uintptr_t)(region + (unsigned)(((8 * (v / 4) + 4 * hh + (v % 4)) * LDW + 32 * jj + r) * 4)) =
+                            g.alpha * acc[i][2 * jp + jj][v];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    const int nl = 4 * q + (lane >> 4), ml = (lane & 15) * 4;
+                    floatx4_t val = *(ldsf4_t)(uintptr_t)(region + (unsigned)((nl * LDW + ml) * 4));
+                    const int64_t nj = nw + 32 * i + nl, mi = mw + 64 * jp + ml;
+                    if (nj < g.n && mi < g.m) {   // m is a multiple of 4 here
+                        floatx4_t *c4 = (floatx4_t *)(C + mi + nj * g.ldc);
+                        if (g.beta != 0.0f) {
+                            const floatx4_t old = *c4;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) val[e] += g.beta * old[e];
+                        }
+                        *c4 = val;
+                    }
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < BM; j++) {
         const int64_t mi = a.row0 + 32 * BM * wm + 32 * j + r;
@@ -380,7 +425,8 @@ int32_t launch_batched_gemm32(int transA, int transB, int64_t m, int64_t n, int6
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {   // gridDim.z is limited to 65535: issue the batch in slabs
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         Gemm32Args g = {(const float *)A + b0 * sA, (const float *)B + b0 * sB, (float *)C + b0 * sC,
-                        m, n, k, lda, ldb, ldc, sA, sB, sC, alpha, beta};
+                        m, n, k, lda, ldb, ldc, sA, sB, sC, alpha, beta,
+                        (int32_t)((((uintptr_t)C) & 15) == 0 && (ldc & 3) == 0 && (sC & 3) == 0 && (m & 3) == 0)};
         dim3 grid((unsigned)((m + TM - 1) / TM), (unsigned)((n + TN - 1) / TN), (unsigned)nb);
         if (exact_instruction_wanted()) {
             if (a_rm && b_rm) hipLaunchKernelGGL((gemm32_kernel<true, true>), grid, dim3(256), 0, st, g);
