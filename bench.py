@@ -354,6 +354,9 @@ def measure_extra(key, steps, warmup, with_cpu):
         line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype=dtn,
                     roofline=dict(bound="mfma", achieved=val, peak=PEAK[dtn], unit="TFLOP/s", frac=val / PEAK[dtn], traffic=None),
                     config=dict(workload=EXTRA[key], kernel=_lib.KERNEL_NAMES[kern.value]), flops_per_step=flops)
+        if dtn == "f32":   # Float32 in, out and accumulation; `peak` stays the Float32 matrix instruction's
+            line["roofline"]["products"] = ("v_mfma_f32_32x32x2_f32" if os.environ.get("MI355ATTN_F32_MFMA", "")[:1] == "1" else
+                                            "six v_mfma_f32_32x32x16_bf16 on three bf16 planes per operand (Float32 accuracy)")
         if with_cpu:
             from oracle import oracle as O
             rng = np.random.default_rng(0)

@@ -14,7 +14,12 @@
 // k-step 4c+j of half-wave hh multiplies feature 8c + 4hh + j), the accumulator registers of P / dS are
 // the B operand of the second products as they stand, and the A operand of those is a plain 4-byte read
 // of tile[row][feature = lane].  Products and sums are true fp32.
+//
+// Calls without bias / mask arrays and without dropout run their products on the 16-bit matrix cores instead, through
+// three bf16 planes per operand (bwd32s_* below: Float32 accuracy at 2.7x less matrix-pipe time), unless
+// MI355ATTN_F32_MFMA=1 in the environment asks for the Float32 instruction, as in the forward kernel.
 #include "flash_common.h"
+#include <cstdlib>
 
 namespace {
 
@@ -465,8 +470,490 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
     }
 }
 
+// ---- the same kernels without bias / mask arrays or dropout, products on the 16-bit matrix cores ----
+// Each Float32 product runs as six v_mfma_f32_32x32x16_bf16 over three bf16 planes per operand (the planes
+// and their arithmetic: common.h; layout and reads of the plane tiles: run_tiles32s in attention_flash32.hip).
+// Streamed tiles are split once when they are staged (one LDS tile per tensor, the next one waits in
+// registers), the stationary rows once per workgroup, P and dS once per block in registers; the A operand of
+// the second products comes from the same row-major planes through the transposing read.
+typedef bf16x8_t plane8;
+typedef bf16x4_t plane4;
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+template <int D>
+struct CfgS {
+    static constexpr int ROWB = D * 2;               // bytes per tile row of one plane
+    static constexpr int PLANEB = BN * ROWB;         // one plane of one tile
+    static constexpr int TILEB = 3 * PLANEB;         // hi, mid, lo
+    static constexpr int CHUNKS = BN * D / 4 / 256;  // float4 pieces per thread, tile and tensor
+    static constexpr size_t SMEM = 2 * TILEB + sizeof(float) * 2 * 3 * BN;   // two tensors + statistics (double buffered)
+    // chunk swizzle of the 16-bit kernels (conflict-free 16-byte operand reads and transposing reads)
+    __device__ static inline int swz(int row) {
+        if (D >= 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+        const int x = (row >> 1) & 7;
+        return ((x & 1) << 2) | (x >> 1);
+    }
+};
+
+__device__ inline floatx16_t mfma_bf16(plane8 a, plane8 b, floatx16_t c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+
+// c += a b with a, b given as planes (small terms first)
+__device__ inline floatx16_t mfma_split(const plane8 (&a)[3], const plane8 (&b)[3], floatx16_t c) {
+    c = mfma_bf16(a[2], b[0], c);
+    c = mfma_bf16(a[0], b[2], c);
+    c = mfma_bf16(a[1], b[1], c);
+    c = mfma_bf16(a[1], b[0], c);
+    c = mfma_bf16(a[0], b[1], c);
+    return mfma_bf16(a[0], b[0], c);
+}
+
+// TileStream32 with the split at the LDS store: one tile per tensor, as LDS byte addresses
+template <int D>
+struct PlaneStream {
+    typedef CfgS<D> C;
+    const float *base1, *base2;   // base2 may be null
+    int64_t stride, nrows;
+    int dh;
+    unsigned s1, s2;
+    floatx4_t r1[C::CHUNKS], r2[C::CHUNKS];
+    __device__ void load(int64_t row0) {
+#pragma unroll
+        for (int u = 0; u < C::CHUNKS; u++) {
+            const int c = threadIdx.x + 256 * u;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            const bool ok = row0 + row < nrows && col < dh;
+            r1[u] = ldg16f(base1 + stride * (row0 + row) + col, ok);
+            if (base2) r2[u] = ldg16f(base2 + stride * (row0 + row) + col, ok);
+        }
+    }
+    // four consecutive features of one row: 8 bytes in each of the three planes
+    __device__ static void put(unsigned tile, int row, int col, const floatx4_t &x) {
+        typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+        uint32_t pl[3][2];
+        const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        if (odd) {   // an Inf or NaN in the chunk (rare)
+            split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+            split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        }
+        const unsigned at = tile + (unsigned)row * C::ROWB + (unsigned)((((col >> 3) ^ C::swz(row)) << 4) + (col & 7) * 2);
+#pragma unroll
+        for (int q = 0; q < 3; q++) *(lds8_t)(uintptr_t)(at + q * C::PLANEB) = (u32x2_t){pl[q][0], pl[q][1]};
+    }
+    __device__ void store() {
+#pragma unroll
+        for (int u = 0; u < C::CHUNKS; u++) {
+            const int c = threadIdx.x + 256 * u;
+            const int row = c / (D / 4), col = (c % (D / 4)) * 4;
+            put(s1, row, col, r1[u]);
+            if (base2) put(s2, row, col, r2[u]);
+        }
+    }
+};
+
+// first_product on plane tiles: the lane's A operand of k-step t is chunk 2t + hh of tile row 32kb + r in each plane
+template <int D>
+__device__ inline floatx16_t first_product_s(unsigned tile, int kb, const plane8 (&x)[3][D / 16], floatx16_t acc, int r, int hh) {
+    typedef CfgS<D> C;
+    typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
+    const unsigned t0 = tile + (unsigned)(32 * kb + r) * C::ROWB;
+    const int sw = C::swz(r);
+#pragma unroll
+    for (int t = 0; t < D / 16; t++) {
+        plane8 ta[3];
+#pragma unroll
+        for (int q = 0; q < 3; q++) ta[q] = *(lds_plane8_t)(uintptr_t)(t0 + q * C::PLANEB + (((2 * t + hh) ^ sw) << 4));
+        const plane8 xb[3] = {x[0][t], x[1][t], x[2][t]};
+        acc = mfma_split(ta, xb, acc);
+    }
+    return acc;
+}
+
+// second_product on plane tiles: the B operand of k-step u is accumulator registers 8u .. 8u+7 of w (tile rows 0-3,
+// 8-11 | 4-7, 12-15 of the 16), split in registers; tile^T comes through the transposing read in that row order
+template <int D>
+__device__ inline void second_product_s(unsigned tile, int kb, const floatx16_t &w, floatx16_t (&out)[D / 32], int lane) {
+    typedef CfgS<D> C;
+    const int hh = lane >> 5;
+    const int vrow = 4 * hh + ((lane & 15) >> 2);
+    const int vchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), vsub = 8 * (lane & 1);
+    const unsigned vt = tile + (unsigned)vrow * C::ROWB + vsub;
+    const int sw_lo = C::swz(vrow), sw_hi = C::swz(vrow + 8);
+    auto tr = [](unsigned addr) {
+        const s16x4_t x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t *)(uintptr_t)addr);
+        return __builtin_bit_cast(plane4, x);
+    };
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        uint32_t ww[3][4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) split3_pair(w[8 * u + 2 * e], w[8 * u + 2 * e + 1], ww[0][e], ww[1][e], ww[2][e]);   // a NaN stays NaN in the hi plane
+        plane8 wb[3];
+#pragma unroll
+        for (int q = 0; q < 3; q++) wb[q] = __builtin_bit_cast(plane8, (u32x4_t){ww[q][0], ww[q][1], ww[q][2], ww[q][3]});
+        const unsigned src = vt + (unsigned)(32 * kb + 16 * u) * C::ROWB;
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++) {
+            plane8 ta[3];
+#pragma unroll
+            for (int q = 0; q < 3; q++) {
+                const plane4 lo = tr(src + q * C::PLANEB + (((4 * dvb + vchunk) ^ sw_lo) << 4));
+                const plane4 hi = tr(src + q * C::PLANEB + 8 * C::ROWB + (((4 * dvb + vchunk) ^ sw_hi) << 4));
+                ta[q] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+            out[dvb] = mfma_split(ta, wb, out[dvb]);
+        }
+    }
+}
+
+// stationary row as planes: the lane's features of k-step t are 16t + 8hh .. + 7 (the B-operand layout of the 16-bit instruction)
+template <int D>
+__device__ inline void load_stationary_s(plane8 (&x)[3][D / 16], const float *row, bool ok, int hh, int dh) {
+#pragma unroll
+    for (int t = 0; t < D / 16; t++) {
+        uint32_t xw[3][4];
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int d0 = 16 * t + 8 * hh + 4 * half;
+            const floatx4_t q4 = ldg16f(row + d0, ok && d0 < dh);
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                uint32_t w[3];
+                if (split3_pair(q4[2 * j], q4[2 * j + 1], w[0], w[1], w[2])) split3_pair_guarded(q4[2 * j], q4[2 * j + 1], w[0], w[1], w[2]);
+#pragma unroll
+                for (int q = 0; q < 3; q++) xw[q][2 * half + j] = w[q];
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 3; q++) x[q][t] = __builtin_bit_cast(plane8, (u32x4_t){xw[q][0], xw[q][1], xw[q][2], xw[q][3]});
+    }
+}
+
+template <int D, bool CAUSAL, bool HAVE_STATS>
+// One workgroup per compute unit: the lane's Q and dO planes, dQ and the two score blocks need some 380 registers.
+// The next tile is fetched during the products where registers are left for it (head dim 64), before the barrier
+// otherwise.
+__global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdParams bp) {
+    typedef CfgS<D> C;
+    constexpr int NDV = D / 32;
+    constexpr bool AHEAD = D == 64;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
+    const unsigned Ks = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)bwd_smem, Vs = Ks + C::TILEB;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * a.nb;
+    const int split = (int)(blockIdx.x % a.nsplit);   // piece of the key range (a.nsplit > 1: calls with saved statistics only)
+    const int64_t bid = blockIdx.x / a.nsplit;
+    const int64_t hb = bid % HB, qt = a.n_qtiles - 1 - bid / HB;
+    const int64_t h = hb % p.H, b = a.b0 + hb / p.H;
+    const int64_t i0 = qt * 128, iw = i0 + 32 * wave, qi = iw + r;
+    const bool qok = qi < p.Lq;
+
+    int64_t kv_len = p.Lkv;
+    if (a.kv_len) {   // context lengths: pairs without one belong to the kernels with mask code
+        kv_len = a.kv_len[b * p.H + h];
+        if (kv_len == 0) return;
+    }
+
+    plane8 qx[3][D / 16], dox[3][D / 16];
+    float delta = 0.0f;
+    {
+        const int64_t off = p.E * (qi + p.Lq * b) + p.D * h;   // E == Ev for these kernels
+        load_stationary_s<D>(qx, (const float *)p.q + off, qok, hh, (int)p.D);
+        load_stationary_s<D>(dox, (const float *)bp.dout + off, qok, hh, (int)p.D);
+#pragma unroll
+        for (int c = 0; c < D / 8; c++) {
+            const bool ok = qok && 8 * c + 4 * hh < p.D;
+            const floatx4_t o4 = ldg16f((const float *)p.out + off + 8 * c + 4 * hh, ok);
+            const floatx4_t d4 = ldg16f((const float *)bp.dout + off + 8 * c + 4 * hh, ok);
+#pragma unroll
+            for (int j = 0; j < 4; j++) delta = fmaf(o4[j], d4[j], delta);
+        }
+        delta += mi_swap32(delta);
+    }
+
+    int64_t kv_end = kv_len;
+    if (CAUSAL && i0 + 128 < kv_end) kv_end = i0 + 128;
+    const int n_tiles = (int)((kv_end + BN - 1) / BN);
+
+    PlaneStream<D> ts;
+    ts.base1 = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
+    ts.dh = (int)p.D;
+    ts.stride = p.E;
+    ts.nrows = kv_len;
+    ts.s1 = Ks;
+    ts.s2 = Vs;
+    floatx16_t unused_o[1][NDV];
+    float fm[1] = {MI_NEG_INF}, fl[1] = {0.0f};
+    const float cs = a.c;
+    const int64_t plane = p.B * p.H * lq_pad(p.Lq), at = (b * p.H + h) * lq_pad(p.Lq) + qi;
+    if (HAVE_STATS) {
+        fm[0] = bp.stats[at] / cs;
+        fl[0] = bp.stats[plane + at];
+        if (hh == 0) bp.stats[2 * plane + at] = qok ? delta : 0.0f;
+    }
+
+    // pass 1: row maximum and row sum (K tiles only)
+    ts.base2 = nullptr;
+    if (!HAVE_STATS) {
+        ts.load(0);
+        ts.store();
+    }
+    __syncthreads();
+    for (int jt = 0; !HAVE_STATS && jt < n_tiles; jt++) {
+        const int64_t j0 = (int64_t)jt * BN;
+        const bool more = jt + 1 < n_tiles;
+        if (more) ts.load(j0 + BN);
+        if (!CAUSAL || j0 <= iw + 31) {
+            floatx16_t s[1][2] = {{(floatx16_t){0}, (floatx16_t){0}}};
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) s[0][kb] = first_product_s<D>(Ks, kb, qx, s[0][kb], r, hh);
+            flash_softmax_tile<T, 1, NDV, CAUSAL, EXTRAS_NONE, PHASE_STATS, float>(a, s, unused_o, fm, fl, b, h, iw, j0, FlashStaged<1>(), 0, 0, nullptr,
+                                                                                   kv_len);
+        }
+        if (more) {
+            __syncthreads();   // every wavefront is done with the tile in LDS
+            ts.store();
+        }
+        __syncthreads();
+    }
+    if (!HAVE_STATS) {
+        fl[0] = 1.0f / (fl[0] + mi_swap32(fl[0]));
+        if (hh == 0) {
+            bp.stats[at] = qok ? fm[0] * cs : 0.0f;
+            bp.stats[plane + at] = qok ? fl[0] : 0.0f;
+            bp.stats[2 * plane + at] = qok ? delta : 0.0f;
+        }
+    }
+    if (!bp.dq) return;
+
+    // pass 2: P, dP = V dO^T, dS = P (dP - delta), dQ^T += K^T dS^T
+    floatx16_t dq[NDV];
+#pragma unroll
+    for (int dvb = 0; dvb < NDV; dvb++) dq[dvb] = (floatx16_t){0};
+    ts.base2 = (const float *)p.v + p.Ev * (p.Lkv * b) + p.D * h;
+    int jt0 = 0, jt1 = n_tiles;
+    if (a.nsplit > 1) {
+        jt0 = split * a.tiles_per_split;
+        if (jt0 + a.tiles_per_split < jt1) jt1 = jt0 + a.tiles_per_split;
+    }
+    ts.load((int64_t)jt0 * BN);
+    __syncthreads();   // pass 1 may still be reading the tile
+    ts.store();
+    __syncthreads();
+    const float m2 = fm[0] * cs, linv = fl[0];
+    for (int jt = jt0; jt < jt1; jt++) {
+        const int64_t j0 = (int64_t)jt * BN;
+        const bool more = jt + 1 < jt1;
+        if (more && AHEAD) ts.load(j0 + BN);
+        if (!CAUSAL || j0 <= iw + 31) {
+            const bool edge = (j0 + BN > kv_len) || (CAUSAL && j0 + BN - 1 > iw);
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                if (CAUSAL && j0 + 32 * kb > iw + 31) break;   // every key of this block is after every query of the wavefront
+                floatx16_t sb = first_product_s<D>(Ks, kb, qx, (floatx16_t){0}, r, hh);
+                const floatx16_t dpb = first_product_s<D>(Vs, kb, dox, (floatx16_t){0}, r, hh);
+                int64_t lim = BN;
+                if (edge) {
+                    lim = kv_len - j0;
+                    if (CAUSAL && qi - j0 + 1 < lim) lim = qi - j0 + 1;
+                }
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int kvl = 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4);
+                    const float pw = (!edge || kvl < lim) ? mi_exp2(fmaf(sb[v], cs, -m2)) * linv : 0.0f;
+                    sb[v] = pw * (dpb[v] - delta);
+                }
+                second_product_s<D>(Ks, kb, sb, dq, lane);
+            }
+        }
+        if (more) {
+            if (!AHEAD) ts.load(j0 + BN);
+            __syncthreads();
+            ts.store();
+        }
+        __syncthreads();
+    }
+    if (qok) {
+        float *dqrow = a.nsplit > 1 ? bp.dq_partial + ((int64_t)split * p.B * p.Lq + qi + p.Lq * b) * p.E + p.D * h
+                                    : (float *)bp.dq + p.E * (qi + p.Lq * b) + p.D * h;
+#pragma unroll
+        for (int dvb = 0; dvb < NDV; dvb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                floatx4_t o4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o4[e] = dq[dvb][4 * g + e] * a.cn;
+                if (32 * dvb + 8 * g + 4 * hh < p.D) *(floatx4_t *)(dqrow + 32 * dvb + 8 * g + 4 * hh) = o4;
+            }
+    }
+}
+
+template <int D, bool CAUSAL, int WHICH>
+// Head dim 64 fits two workgroups per compute unit, each fetching its next tiles only once the products are done (no
+// staging registers live across them): the other workgroup covers the latency.
+__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(FlashArgs a, AttnBwdParams bp) {
+    typedef CfgS<D> C;
+    constexpr int NDV = D / 32;
+    constexpr bool DO_DV = WHICH == BWD_DV, DO_DK = WHICH == BWD_DK;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
+    const unsigned Qs = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)bwd_smem, dOs = Qs + C::TILEB;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t hb = blockIdx.x % HB, kt_idx = blockIdx.x / HB;   // with causal masks the early key tiles are the long ones
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t j0 = kt_idx * 128, jw = j0 + 32 * wave, kv = jw + r;
+    const bool kok = kv < p.Lkv;
+    int64_t kv_len = p.Lkv;
+    if (a.kv_len) {
+        kv_len = a.kv_len[b * p.H + h];
+        if (kv_len == 0) return;
+    }
+    const bool kvalid = kv < kv_len;
+    float *grad = DO_DK ? (float *)bp.dk : (float *)bp.dv;
+    const int64_t off = p.E * (kv + p.Lkv * b) + p.D * h;
+    if (j0 >= kv_len) {   // keys from the pair's length on get zero gradients
+        if (kok) {
+            const floatx4_t z4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int dvb = 0; dvb < NDV; dvb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    if (32 * dvb + 8 * g + 4 * hh < p.D) *(floatx4_t *)(grad + off + 32 * dvb + 8 * g + 4 * hh) = z4;
+        }
+        return;
+    }
+
+    plane8 kx[3][D / 16], vx[DO_DK ? 3 : 1][D / 16];
+    load_stationary_s<D>(kx, (const float *)p.k + off, kvalid, hh, (int)p.D);
+    if constexpr (DO_DK) load_stationary_s<D>(vx, (const float *)p.v + off, kvalid, hh, (int)p.D);
+    floatx16_t acc[NDV];
+#pragma unroll
+    for (int dvb = 0; dvb < NDV; dvb++) acc[dvb] = (floatx16_t){0};
+
+    const int64_t plane = p.B * p.H * lq_pad(p.Lq);
+    // the row statistics of a query tile travel with it through LDS (48 threads x 4 floats)
+    const float *st_src = bp.stats + (b * p.H + h) * lq_pad(p.Lq) + (int64_t)(tid >> 4) * plane + 4 * (tid & 15);
+    float *st_lds = (float *)(bwd_smem + 2 * C::TILEB);
+    floatx4_t st_reg = {0, 0, 0, 0};
+    const float cs = a.c;
+
+    PlaneStream<D> ts;
+    ts.base1 = (const float *)p.q + p.E * (p.Lq * b) + p.D * h;
+    ts.base2 = (const float *)bp.dout + p.E * (p.Lq * b) + p.D * h;
+    ts.dh = (int)p.D;
+    ts.stride = p.E;
+    ts.nrows = p.Lq;
+    ts.s1 = Qs;
+    ts.s2 = dOs;
+    const int n_qt = (int)((p.Lq + BN - 1) / BN);
+    const int it0 = CAUSAL ? (int)(j0 / BN) : 0;   // query tiles before the first key of the workgroup see none of its keys
+    if (it0 < n_qt) {
+        ts.load((int64_t)it0 * BN);
+        ts.store();
+        if (tid < 48) *(floatx4_t *)(st_lds + 4 * tid) = *(const floatx4_t *)(st_src + (int64_t)it0 * BN);
+    }
+    __syncthreads();
+    for (int it = it0; it < n_qt; it++) {
+        const int buf = (it - it0) & 1;
+        const int64_t i0 = (int64_t)it * BN;
+        const bool more = it + 1 < n_qt;
+        if (more && tid < 48) st_reg = *(const floatx4_t *)(st_src + i0 + BN);
+        if (!CAUSAL || i0 + BN - 1 >= jw) {
+            const float *st = st_lds + buf * (3 * BN);
+            const bool diag = CAUSAL && i0 < jw + 32;   // some (query, key) pair of this tile has key > query
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                floatx16_t s = first_product_s<D>(Qs, kb, kx, (floatx16_t){0}, r, hh);
+                floatx16_t dp = (floatx16_t){0};
+                if constexpr (DO_DK) dp = first_product_s<D>(dOs, kb, vx, dp, r, hh);
+                // accumulator register 4g+e of this lane: query i0 + 32kb + 8g + 4hh + e, key kv.  Rows past Lq carry
+                // statistics (0, 0, 0): their weights vanish; keys past the length only feed columns that store zeros
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int sq = 32 * kb + 8 * g + 4 * hh;
+                    const floatx4_t m4 = *(const floatx4_t *)(st + sq);
+                    const floatx4_t linv4 = *(const floatx4_t *)(st + BN + sq);
+                    floatx4_t delta4 = {0.0f, 0.0f, 0.0f, 0.0f};
+                    if (DO_DK) delta4 = *(const floatx4_t *)(st + 2 * BN + sq);
+                    const int dq_ = (int)(jw - (i0 + sq)) + r;   // key index minus query index of element e = 0
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        float pw = mi_exp2(fmaf(s[4 * g + e], cs, -m4[e])) * linv4[e];
+                        if (diag) pw = dq_ - e > 0 ? 0.0f : pw;
+                        if (DO_DK) s[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
+                        else s[4 * g + e] = pw;
+                    }
+                }
+                second_product_s<D>(DO_DK ? Qs : dOs, kb, s, acc, lane);
+            }
+        }
+        if (more) {
+            ts.load(i0 + BN);
+            __syncthreads();   // every wavefront is done with the tiles in LDS
+            ts.store();
+            if (tid < 48) *(floatx4_t *)(st_lds + (buf ^ 1) * (3 * BN) + 4 * tid) = st_reg;
+        }
+        __syncthreads();
+    }
+    if (kok) {
+        const float scale = DO_DK ? a.cn : 1.0f;
+#pragma unroll
+        for (int dvb = 0; dvb < NDV; dvb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                if (32 * dvb + 8 * g + 4 * hh >= p.D) continue;
+                floatx4_t g4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) g4[e] = kvalid ? acc[dvb][4 * g + e] * scale : 0.0f;
+                *(floatx4_t *)(grad + off + 32 * dvb + 8 * g + 4 * hh) = g4;
+            }
+    }
+}
+
+// Products on the 16-bit matrix cores through three bf16 planes unless the caller's environment asks for the
+// Float32 matrix instruction (MI355ATTN_F32_MFMA=1), as in the forward kernel.
+bool exact_instruction_wanted() {
+    static const bool wanted = [] {
+        const char *e = getenv("MI355ATTN_F32_MFMA");
+        return e && e[0] == '1';
+    }();
+    return wanted;
+}
+
+template <int D, bool CAUSAL>
+int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
+    const AttnParams &p = a.p;
+    constexpr size_t SMEM = CfgS<D>::SMEM;
+    auto k1 = bp.have_stats ? bwd32s_dq_kernel<D, CAUSAL, true> : bwd32s_dq_kernel<D, CAUSAL, false>;
+    auto k2 = bwd32s_dkdv_kernel<D, CAUSAL, BWD_DV>;
+    auto k3 = bwd32s_dkdv_kernel<D, CAUSAL, BWD_DK>;
+    static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        attr_set = true;
+    }
+    FlashArgs a1 = a;
+    if (bp.dq_nsplit > 1) {   // the dQ kernel's key range in pieces (the dK / dV kernels keep a.nsplit = 1)
+        a1.nsplit = bp.dq_nsplit;
+        a1.tiles_per_split = (int32_t)(((p.Lkv + BN - 1) / BN + bp.dq_nsplit - 1) / bp.dq_nsplit);
+    }
+    hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B * a1.nsplit)), dim3(256), SMEM, st, a1, bp);
+    MI_LAUNCH_CHECK();
+    const dim3 g2((unsigned)(((p.Lkv + 127) / 128) * p.H * p.B));
+    if (bp.dv) hipLaunchKernelGGL(k2, g2, dim3(256), SMEM, st, a, bp);
+    if (bp.dk) hipLaunchKernelGGL(k3, g2, dim3(256), SMEM, st, a, bp);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
 template <int D, bool CAUSAL, int EXTRAS, bool DROP = false>
 int32_t launch_set(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
+    if constexpr (EXTRAS == EXTRAS_NONE && !DROP)
+        if (!bp.dbias && !exact_instruction_wanted()) return launch_set_planes<D, CAUSAL>(a, bp, st);
     const AttnParams &p = a.p;
     constexpr size_t SMEM = Cfg<D>::SMEM;
     constexpr size_t SMEM_Q = SMEM + (EXTRAS == EXTRAS_NONE ? 0 : 4 * FLASH_WSTAGE_BYTES);   // the dQ kernel's staging for the bias gradient

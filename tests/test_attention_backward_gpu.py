@@ -521,3 +521,51 @@ def test_gradient_with_logits_that_climb_along_the_keys(nn, oracle, dtype, D, sa
         tols = (3e-2, 2e-2, 2e-2) if saved else (3e-2, 1e-2, 1e-2)
     for g, r_, tol in zip(got[:3], ref[:3], tols):
         assert np.abs(g.to_numpy() - r_).max() / max(np.abs(r_).max(), 0.05) <= tol
+
+
+_F32_GRAD_SCRIPT = """
+import sys, numpy as np
+sys.path.insert(0, %r)
+import nnlib_amd as nn
+d = np.load(sys.argv[1])
+q, k, v, dy = (nn.DeviceArray.from_numpy(d[n], "f32") for n in ("q", "k", "v", "dy"))
+mask = nn.make_causal_mask(q, dims=2) if int(d["causal"]) else None
+y, _ = nn.dot_product_attention(q, k, v, nheads=int(d["H"]), mask=mask, return_weights=False, save_for_backward=bool(d["saved"]))
+g = nn.dot_product_attention_grad(dy, q, k, v, y=y, mask=mask, nheads=int(d["H"]))
+assert nn.last_attention_bwd_kernel() == "flash32"
+np.savez(sys.argv[2], dq=g[0].to_numpy(), dk=g[1].to_numpy(), dv=g[2].to_numpy())
+"""
+
+
+@pytest.mark.parametrize("E,H,Lq,Lkv,causal,saved", [(256, 4, 300, 300, False, True), (256, 4, 257, 257, True, False),
+                                                     (256, 2, 200, 330, False, False), (96, 1, 130, 130, True, True)],
+                         ids=["D64-saved", "D64-causal", "D128-cross", "D96-causal-saved"])
+def test_float32_gradient_through_bf16_planes_keeps_float32_accuracy(nn, oracle, tmp_path, E, H, Lq, Lkv, causal, saved):
+    """Float32 gradient calls without bias / mask arrays run their products as six bf16 matrix instructions per Float32
+    one (three planes per operand).  Against float64 on the same inputs every gradient must be as close as the Float32
+    matrix instruction's, which a child process computes with MI355ATTN_F32_MFMA=1: values spread over 2^+-12 so that
+    every plane carries weight."""
+    import os, subprocess, sys
+    rng = np.random.default_rng(E + Lq)
+    spread = lambda shape: (rng.standard_normal(shape) * np.exp2(rng.integers(-12, 1, shape))).astype(np.float32)
+    q, k, v, dy = spread((E, Lq, 2)), spread((E, Lkv, 2)), spread((E, Lkv, 2)), spread((E, Lq, 2))
+    ref = oracle.attention_bwd_f64(q, k, v, dy, None, oracle.make_causal_mask(Lq) if causal else None, H, None)
+    D = nn.DeviceArray.from_numpy
+    dq_, dk_, dv_ = D(q, "f32"), D(k, "f32"), D(v, "f32")
+    mask = nn.make_causal_mask(dq_, dims=2) if causal else None
+    y, _ = nn.dot_product_attention(dq_, dk_, dv_, nheads=H, mask=mask, return_weights=False, save_for_backward=saved)
+    got = nn.dot_product_attention_grad(D(dy, "f32"), dq_, dk_, dv_, y=y, mask=mask, nheads=H)
+    assert nn.last_attention_bwd_kernel() == "flash32"
+    # the same call on the Float32 matrix instruction, in a process of its own (the choice is made once per process)
+    np.savez(tmp_path / "in.npz", q=q, k=k, v=v, dy=dy, H=H, causal=int(causal), saved=int(saved))
+    env = dict(os.environ, MI355ATTN_F32_MFMA="1")
+    pkg = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "nnlib.jl_amd")
+    subprocess.run([sys.executable, "-c", _F32_GRAD_SCRIPT % pkg, str(tmp_path / "in.npz"), str(tmp_path / "out.npz")], env=env, check=True,
+                   timeout=300)
+    exact = np.load(tmp_path / "out.npz")
+    for g, r, name in zip(got, ref, ("dq", "dk", "dv")):
+        scale = np.abs(r).max()
+        err, err_exact = np.abs(g.to_numpy() - r).max() / scale, np.abs(exact[name] - r).max() / scale
+        print(name, err, err_exact)
+        assert err < 5e-6 and err_exact < 5e-6, (name, err, err_exact)
+        assert err < 4 * err_exact + 2e-7, (name, err, err_exact)
