@@ -91,7 +91,9 @@ enum {
     MI_ATTN_KERNEL_FLASH16 = 1,  /* f16 / bf16 MFMA flash forward, head dims 8..256 (x8) */
     MI_ATTN_KERNEL_FLASH32 = 2,  /* f32 MFMA flash forward, head dims 4..128 (x4): Float32 in, out and accumulation;
                                     products as six bf16 matrix instructions on three bf16 planes per operand (Float32
-                                    accuracy), or the Float32 instruction if MI355ATTN_F32_MFMA=1 is in the environment */
+                                    accuracy), or the Float32 instruction if MI355ATTN_F32_MFMA=1 is in the environment
+                                    (the gradient kernels of this family: the same for calls without bias / mask arrays
+                                    and dropout, the Float32 instruction otherwise) */
     MI_ATTN_KERNEL_DECODE = 3    /* split-kv bandwidth-bound path for one to four queries (L_q <= 4) */
 };
 
