@@ -476,6 +476,10 @@ __global__ __launch_bounds__(256, (WHICH != 3 && D == 64 && EXTRAS == EXTRAS_NON
 // Streamed tiles are split once when they are staged (one LDS tile per tensor, the next one waits in
 // registers), the stationary rows once per workgroup, P and dS once per block in registers; the A operand of
 // the second products comes from the same row-major planes through the transposing read.
+// Keeps the compiler from hoisting one product's LDS operand reads across the previous phase of the step (head dim 64:
+// left alone it holds dozens of operand registers in flight and spills the stationary planes; with the fences the
+// 64-wide kernels run 3-13 % faster, the 128-wide ones, which have registers to spare, 5-20 % slower)
+#define SCHED_FENCE() do { if (D == 64) __builtin_amdgcn_sched_barrier(0); } while (0)
 typedef bf16x8_t plane8;
 typedef bf16x4_t plane4;
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
@@ -485,7 +489,6 @@ struct CfgS {
     static constexpr int ROWB = D * 2;               // bytes per tile row of one plane
     static constexpr int PLANEB = BN * ROWB;         // one plane of one tile
     static constexpr int TILEB = 3 * PLANEB;         // hi, mid, lo
-    static constexpr int CHUNKS = BN * D / 4 / 256;  // float4 pieces per thread, tile and tensor
     static constexpr size_t SMEM = 2 * TILEB + sizeof(float) * 2 * 3 * BN;   // two tensors + statistics (double buffered)
     // chunk swizzle of the 16-bit kernels (conflict-free 16-byte operand reads and transposing reads)
     __device__ static inline int swz(int row) {
@@ -508,18 +511,19 @@ __device__ inline floatx16_t mfma_split(const plane8 (&a)[3], const plane8 (&b)[
 }
 
 // TileStream32 with the split at the LDS store: one tile per tensor, as LDS byte addresses
-template <int D>
+template <int D, int NT = 256>
 struct PlaneStream {
     typedef CfgS<D> C;
+    static constexpr int CHUNKS = BN * D / 4 / NT;   // float4 pieces per thread, tile and tensor
     const float *base1, *base2;   // base2 may be null
     int64_t stride, nrows;
     int dh;
     unsigned s1, s2;
-    floatx4_t r1[C::CHUNKS], r2[C::CHUNKS];
+    floatx4_t r1[CHUNKS], r2[CHUNKS];
     __device__ void load(int64_t row0) {
 #pragma unroll
-        for (int u = 0; u < C::CHUNKS; u++) {
-            const int c = threadIdx.x + 256 * u;
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = threadIdx.x + NT * u;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
             const bool ok = row0 + row < nrows && col < dh;
             r1[u] = ldg16f(base1 + stride * (row0 + row) + col, ok);
@@ -541,8 +545,8 @@ struct PlaneStream {
     }
     __device__ void store() {
 #pragma unroll
-        for (int u = 0; u < C::CHUNKS; u++) {
-            const int c = threadIdx.x + 256 * u;
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = threadIdx.x + NT * u;
             const int row = c / (D / 4), col = (c % (D / 4)) * 4;
             put(s1, row, col, r1[u]);
             if (base2) put(s2, row, col, r2[u]);
@@ -563,6 +567,27 @@ __device__ inline floatx16_t first_product_s(unsigned tile, int kb, const plane8
 #pragma unroll
         for (int q = 0; q < 3; q++) ta[q] = *(lds_plane8_t)(uintptr_t)(t0 + q * C::PLANEB + (((2 * t + hh) ^ sw) << 4));
         const plane8 xb[3] = {x[0][t], x[1][t], x[2][t]};
+        acc = mfma_split(ta, xb, acc);
+    }
+    return acc;
+}
+
+// first_product_s with the stationary planes in LDS as well ([3][rows][ROWB], chunks swizzled like a tile's): `xrow` is
+// the byte address of the lane's row in the hi plane, XPLANEB the distance between planes
+template <int D, int XPLANEB>
+__device__ inline floatx16_t first_product_sl(unsigned tile, int kb, unsigned xrow, int xsw, floatx16_t acc, int r, int hh) {
+    typedef CfgS<D> C;
+    typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
+    const unsigned t0 = tile + (unsigned)(32 * kb + r) * C::ROWB;
+    const int sw = C::swz(r);
+#pragma unroll
+    for (int t = 0; t < D / 16; t++) {
+        plane8 ta[3], xb[3];
+#pragma unroll
+        for (int q = 0; q < 3; q++) {
+            ta[q] = *(lds_plane8_t)(uintptr_t)(t0 + q * C::PLANEB + (((2 * t + hh) ^ sw) << 4));
+            xb[q] = *(lds_plane8_t)(uintptr_t)(xrow + q * XPLANEB + (((2 * t + hh) ^ xsw) << 4));
+        }
         acc = mfma_split(ta, xb, acc);
     }
     return acc;
@@ -628,14 +653,18 @@ __device__ inline void load_stationary_s(plane8 (&x)[3][D / 16], const float *ro
     }
 }
 
-template <int D, bool CAUSAL, bool HAVE_STATS>
+template <int D, bool CAUSAL, bool HAVE_STATS, int NW>
 // One workgroup per compute unit: the lane's Q and dO planes, dQ and the two score blocks need some 380 registers.
-// The next tile is fetched during the products where registers are left for it (head dim 64), before the barrier
-// otherwise.
-__global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdParams bp) {
+// NW = 4: everything in registers, one wavefront per SIMD; the next tile is fetched during the products where
+// registers are left for it (head dim 64), before the barrier otherwise.  NW = 8 (head dim 64, 256 queries a
+// workgroup): the dO planes live in LDS behind the tiles (each wavefront reads its own rows back as the B operand of
+// dP), which brings a lane under 256 registers, i.e. two wavefronts per SIMD sharing one pair of tiles.
+__global__ __launch_bounds__(64 * NW, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdParams bp) {
     typedef CfgS<D> C;
-    constexpr int NDV = D / 32;
-    constexpr bool AHEAD = D == 64;
+    constexpr int NDV = D / 32, NT = 64 * NW;
+    constexpr bool X_LDS = NW == 8;
+    constexpr bool AHEAD = D == 64 && !X_LDS;
+    constexpr int XPLANEB = 32 * NW * C::ROWB;
     const AttnParams &p = a.p;
     extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
     const unsigned Ks = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)bwd_smem, Vs = Ks + C::TILEB;
@@ -645,7 +674,7 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdP
     const int64_t bid = blockIdx.x / a.nsplit;
     const int64_t hb = bid % HB, qt = a.n_qtiles - 1 - bid / HB;
     const int64_t h = hb % p.H, b = a.b0 + hb / p.H;
-    const int64_t i0 = qt * 128, iw = i0 + 32 * wave, qi = iw + r;
+    const int64_t i0 = qt * (32 * NW), iw = i0 + 32 * wave, qi = iw + r;
     const bool qok = qi < p.Lq;
 
     int64_t kv_len = p.Lkv;
@@ -654,12 +683,24 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdP
         if (kv_len == 0) return;
     }
 
-    plane8 qx[3][D / 16], dox[3][D / 16];
+    plane8 qx[3][D / 16], dox[X_LDS ? 1 : 3][D / 16];
+    const unsigned xrow = Ks + 2 * C::TILEB + sizeof(float) * 2 * 3 * BN + (unsigned)(32 * wave + r) * C::ROWB;
+    const int xsw = C::swz(r);
     float delta = 0.0f;
     {
         const int64_t off = p.E * (qi + p.Lq * b) + p.D * h;   // E == Ev for these kernels
+        if constexpr (X_LDS) {
+            typedef __attribute__((address_space(3))) plane8 *lds_plane8_t;
+            plane8 tmp[3][D / 16];
+            load_stationary_s<D>(tmp, (const float *)bp.dout + off, qok, hh, (int)p.D);
+#pragma unroll
+            for (int q = 0; q < 3; q++)
+#pragma unroll
+                for (int t = 0; t < D / 16; t++) *(lds_plane8_t)(uintptr_t)(xrow + q * XPLANEB + (((2 * t + hh) ^ xsw) << 4)) = tmp[q][t];
+        } else {
+            load_stationary_s<D>(dox, (const float *)bp.dout + off, qok, hh, (int)p.D);
+        }
         load_stationary_s<D>(qx, (const float *)p.q + off, qok, hh, (int)p.D);
-        load_stationary_s<D>(dox, (const float *)bp.dout + off, qok, hh, (int)p.D);
 #pragma unroll
         for (int c = 0; c < D / 8; c++) {
             const bool ok = qok && 8 * c + 4 * hh < p.D;
@@ -672,10 +713,10 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdP
     }
 
     int64_t kv_end = kv_len;
-    if (CAUSAL && i0 + 128 < kv_end) kv_end = i0 + 128;
+    if (CAUSAL && i0 + 32 * NW < kv_end) kv_end = i0 + 32 * NW;
     const int n_tiles = (int)((kv_end + BN - 1) / BN);
 
-    PlaneStream<D> ts;
+    PlaneStream<D, NT> ts;
     ts.base1 = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
     ts.dh = (int)p.D;
     ts.stride = p.E;
@@ -686,7 +727,8 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdP
     float fm[1] = {MI_NEG_INF}, fl[1] = {0.0f};
     const float cs = a.c;
     const int64_t plane = p.B * p.H * lq_pad(p.Lq), at = (b * p.H + h) * lq_pad(p.Lq) + qi;
-    if (HAVE_STATS) {
+    const bool padded = qi < lq_pad(p.Lq);   // the statistics planes end there; a 256-query workgroup may reach past it
+    if (HAVE_STATS && padded) {
         fm[0] = bp.stats[at] / cs;
         fl[0] = bp.stats[plane + at];
         if (hh == 0) bp.stats[2 * plane + at] = qok ? delta : 0.0f;
@@ -718,7 +760,7 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdP
     }
     if (!HAVE_STATS) {
         fl[0] = 1.0f / (fl[0] + mi_swap32(fl[0]));
-        if (hh == 0) {
+        if (hh == 0 && padded) {
             bp.stats[at] = qok ? fm[0] * cs : 0.0f;
             bp.stats[plane + at] = qok ? fl[0] : 0.0f;
             bp.stats[2 * plane + at] = qok ? delta : 0.0f;
@@ -751,7 +793,11 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdP
             for (int kb = 0; kb < 2; kb++) {
                 if (CAUSAL && j0 + 32 * kb > iw + 31) break;   // every key of this block is after every query of the wavefront
                 floatx16_t sb = first_product_s<D>(Ks, kb, qx, (floatx16_t){0}, r, hh);
-                const floatx16_t dpb = first_product_s<D>(Vs, kb, dox, (floatx16_t){0}, r, hh);
+                SCHED_FENCE();
+                floatx16_t dpb;
+                if constexpr (X_LDS) dpb = first_product_sl<D, XPLANEB>(Vs, kb, xrow, xsw, (floatx16_t){0}, r, hh);
+                else dpb = first_product_s<D>(Vs, kb, dox, (floatx16_t){0}, r, hh);
+                SCHED_FENCE();
                 int64_t lim = BN;
                 if (edge) {
                     lim = kv_len - j0;
@@ -763,7 +809,9 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_kernel(FlashArgs a, AttnBwdP
                     const float pw = (!edge || kvl < lim) ? mi_exp2(fmaf(sb[v], cs, -m2)) * linv : 0.0f;
                     sb[v] = pw * (dpb[v] - delta);
                 }
+                SCHED_FENCE();
                 second_product_s<D>(Ks, kb, sb, dq, lane);
+                SCHED_FENCE();
             }
         }
         if (more) {
@@ -865,8 +913,10 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(Flash
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
                 floatx16_t s = first_product_s<D>(Qs, kb, kx, (floatx16_t){0}, r, hh);
+                SCHED_FENCE();
                 floatx16_t dp = (floatx16_t){0};
                 if constexpr (DO_DK) dp = first_product_s<D>(dOs, kb, vx, dp, r, hh);
+                SCHED_FENCE();
                 // accumulator register 4g+e of this lane: query i0 + 32kb + 8g + 4hh + e, key kv.  Rows past Lq carry
                 // statistics (0, 0, 0): their weights vanish; keys past the length only feed columns that store zeros
 #pragma unroll
@@ -885,7 +935,9 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(Flash
                         else s[4 * g + e] = pw;
                     }
                 }
+                SCHED_FENCE();
                 second_product_s<D>(DO_DK ? Qs : dOs, kb, s, acc, lane);
+                SCHED_FENCE();
             }
         }
         if (more) {
@@ -925,13 +977,23 @@ template <int D, bool CAUSAL>
 int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
     const AttnParams &p = a.p;
     constexpr size_t SMEM = CfgS<D>::SMEM;
-    auto k1 = bp.have_stats ? bwd32s_dq_kernel<D, CAUSAL, true> : bwd32s_dq_kernel<D, CAUSAL, false>;
+    // the dQ kernel on eight wavefronts (256 queries a workgroup) where those workgroups still fill the chip
+    constexpr int NW_WIDE = D == 64 ? 8 : 4;
+    constexpr size_t SMEM_WIDE = SMEM + 3 * 32 * NW_WIDE * CfgS<D>::ROWB;
+    const int64_t wide_tiles = (p.Lq + 32 * NW_WIDE - 1) / (32 * NW_WIDE);
+    const bool wide = NW_WIDE > 4 && bp.dq_nsplit <= 1 && wide_tiles * p.H * p.B >= 256;
+    auto k1 = bp.have_stats ? bwd32s_dq_kernel<D, CAUSAL, true, 4> : bwd32s_dq_kernel<D, CAUSAL, false, 4>;
+    auto k1w = bp.have_stats ? bwd32s_dq_kernel<D, CAUSAL, true, NW_WIDE> : bwd32s_dq_kernel<D, CAUSAL, false, NW_WIDE>;
     auto k2 = bwd32s_dkdv_kernel<D, CAUSAL, BWD_DV>;
     auto k3 = bwd32s_dkdv_kernel<D, CAUSAL, BWD_DK>;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
     if (!attr_set) {
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, true, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, false, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        if (NW_WIDE > 4) {
+            MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, true, NW_WIDE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_WIDE));
+            MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, false, NW_WIDE>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_WIDE));
+        }
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         attr_set = true;
@@ -941,7 +1003,12 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
         a1.nsplit = bp.dq_nsplit;
         a1.tiles_per_split = (int32_t)(((p.Lkv + BN - 1) / BN + bp.dq_nsplit - 1) / bp.dq_nsplit);
     }
-    hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B * a1.nsplit)), dim3(256), SMEM, st, a1, bp);
+    if (wide) {
+        a1.n_qtiles = (int32_t)wide_tiles;
+        hipLaunchKernelGGL(k1w, dim3((unsigned)(wide_tiles * p.H * p.B)), dim3(64 * NW_WIDE), SMEM_WIDE, st, a1, bp);
+    } else {
+        hipLaunchKernelGGL(k1, dim3((unsigned)((int64_t)a.n_qtiles * p.H * p.B * a1.nsplit)), dim3(256), SMEM, st, a1, bp);
+    }
     MI_LAUNCH_CHECK();
     const dim3 g2((unsigned)(((p.Lkv + 127) / 128) * p.H * p.B));
     if (bp.dv) hipLaunchKernelGGL(k2, g2, dim3(256), SMEM, st, a, bp);

@@ -569,3 +569,14 @@ def test_float32_gradient_through_bf16_planes_keeps_float32_accuracy(nn, oracle,
         print(name, err, err_exact)
         assert err < 5e-6 and err_exact < 5e-6, (name, err, err_exact)
         assert err < 4 * err_exact + 2e-7, (name, err, err_exact)
+
+
+@pytest.mark.parametrize("saved", [False, True], ids=["own-stats", "saved-stats"])
+@pytest.mark.parametrize("mask_kind,Lq,Lkv", [(None, 300, 330), ("causal", 300, 300), ("lengths", 257, 300), ("causal", 512, 512)],
+                         ids=["cross", "causal", "lengths", "causal-512"])
+def test_float32_gradient_with_256_query_workgroups(nn, oracle, mask_kind, Lq, Lkv, saved):
+    """With enough (query tile, head, batch) work the Float32 dQ kernel runs 256 queries per workgroup on eight
+    wavefronts (head dim 64 and below, no bias / mask arrays): query counts that end inside the first or the second
+    half of the last workgroup, whose rows reach past the padded statistics planes."""
+    _run(nn, oracle, "f32", 512, 512, Lq, Lkv, (16,), 8, mask_kind=mask_kind, saved=saved, scale=0.5, seed=Lq, expect="flash32")
+    _run(nn, oracle, "f32", 256, 256, Lq, Lkv, (16,), 8, mask_kind=mask_kind, saved=saved, scale=0.5, seed=Lq + 1, expect="flash32")
