@@ -1,12 +1,13 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|bwd|logsoftmax|softmax_dims2] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|bwd|bwd_f32|logsoftmax|softmax|softmax_dims2|batched_mul[_f32|_c32|_f64]] [--no-cpu]
 
 A "step" is one dot_product_attention call on synthetic inputs that are already resident in HBM.
 The default workload is C3 (bf16 causal prefill, head dim 128, L = 4096), the configuration the
 prefill target is quoted on; the other four configurations are measured in the same run and reported under
-"configs" in the same JSON line (C5, the decode target, also under "decode").  Timing is by HIP events on the stream the kernels are launched on.
+"configs" in the same JSON line (C5, the decode target, also under "decode"), and the workloads beyond them (gradient,
+softmax family, batched_mul; GPU leg only) under "next_rows".  Timing is by HIP events on the stream the kernels are launched on.
 """
 import argparse
 import ctypes
@@ -318,7 +319,7 @@ def _event_time(lib, _lib, fn, steps, warmup):
 
 
 def measure_extra(key, steps, warmup, with_cpu):
-    """One JSON line for a workload outside BASELINE.json's five configurations (same fields)."""
+    """The JSON line (as a dict) of a workload outside BASELINE.json's five configurations (same fields)."""
     import numpy as np
     import nnlib_amd as nn
     from nnlib_amd import _lib
@@ -446,7 +447,7 @@ def measure_extra(key, steps, warmup, with_cpu):
                                         sample=f"1/16 of the array, Float32 oracle on one thread as the reference's passes are ({dt:.2f} s)")
     line.update(n_gpus=1, steps=steps, warmup=warmup, ms_per_step=ms, higher_is_better=True, scaling="weak", vs_baseline=None,
                 data="synthetic")
-    print(json.dumps(line))
+    return line
 
 
 def copy_calibration(steps):
@@ -488,7 +489,8 @@ def main():
     if args.workload == "copy":
         return copy_calibration(min(args.steps, 10))
     if args.workload in EXTRA:
-        return measure_extra(args.workload, min(args.steps, 50), min(args.warmup, 10), not args.no_cpu)
+        print(json.dumps(measure_extra(args.workload, min(args.steps, 50), min(args.warmup, 10), not args.no_cpu)))
+        return
     main_res = measure(args.workload, args.steps, args.warmup, not args.no_cpu)
     w = WORKLOADS[args.workload]
     prefill = args.workload not in ("c4", "c5")
@@ -524,6 +526,12 @@ def main():
         dec = dict(line["configs"]["c5"])
         dec["metric"] = "attention GB/s (decode)"
         line["decode"] = dec
+        # the workloads beyond the five configurations (gradient, softmax family, batched_mul), GPU leg only, so that
+        # their figures are measured by whoever runs this script and not only quoted
+        line["next_rows"] = {}
+        for key in EXTRA:
+            res = measure_extra(key, max(5, min(args.steps, 20)), min(args.warmup, 5), False)
+            line["next_rows"][key] = {f: res[f] for f in ("metric", "value", "unit", "ms_per_step", "steps", "dtype", "config", "roofline")}
     print(json.dumps(line))
     sys.stdout.flush()
 
