@@ -530,8 +530,11 @@ def main():
         # their figures are measured by whoever runs this script and not only quoted
         line["next_rows"] = {}
         for key in EXTRA:
-            res = measure_extra(key, max(5, min(args.steps, 20)), min(args.warmup, 5), False)
-            line["next_rows"][key] = {f: res[f] for f in ("metric", "value", "unit", "ms_per_step", "steps", "dtype", "config", "roofline")}
+            try:
+                res = measure_extra(key, max(5, min(args.steps, 20)), min(args.warmup, 5), False)
+                line["next_rows"][key] = {f: res[f] for f in ("metric", "value", "unit", "ms_per_step", "steps", "dtype", "config", "roofline")}
+            except Exception as e:   # a failure here must not cost the headline figures above; it is reported, not hidden
+                line["next_rows"][key] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(line))
     sys.stdout.flush()
 
