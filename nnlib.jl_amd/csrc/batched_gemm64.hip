@@ -9,68 +9,94 @@
 //                            Arithmetic is in the element type of C, as Julia's mul! does after promotion;
 //                            integer products wrap like Julia's (two's complement).
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
 // ---- fp64 MFMA kernel -------------------------------------------------------------------------------------
-// Workgroup = 4 wavefronts, 64 x 64 tile of C; a wavefront owns 32 x 32 of it as 2 x 2 MFMA blocks of 16 x 16.
-// v_mfma_f64_16x16x4_f64: lane l supplies A[row = l % 16][k = l / 16] and B[k = l / 16][col = l % 16]; it receives
-// D[row = l / 16 + 4 * v][col = l % 16] in register pair v = 0..3 (checked on the hardware with structured inputs).
-// Operand tiles sit in LDS k-major: As[k][row], Bs[k][col], rows padded so that the four k groups of a wavefront's
-// read start in different banks.
+// Workgroup = 4 wavefronts, TS x TS tile of C (64 or 128); a wavefront owns a quarter of it as (TS/32)^2 MFMA blocks
+// of 16 x 16.  v_mfma_f64_16x16x4_f64: lane l supplies A[row = l % 16][k = l / 16] and B[k = l / 16][col = l % 16]; it
+// receives D[row = l / 16 + 4 * v][col = l % 16] in register pair v = 0..3 (checked on the hardware with structured
+// inputs).  Operand tiles sit in LDS k-major: As[k][row], Bs[k][col], rows padded so that the four k groups of a
+// wavefront's read start in different banks (64-wide tiles: 8 banks apart; 128-wide: 32 apart, i.e. the two k groups of
+// each half-wave cover all 64 banks exactly).  A 64-wide tile moves 16 KiB per 16 k for 64 matrix instructions, which
+// at full matrix rate is more than L2 delivers (9 TB/s over the chip); the 128-wide tile halves that.
 typedef __attribute__((__vector_size__(4 * sizeof(double)))) double doublex4_t;
-constexpr int TM = 64, TN = 64, TK = 16, PAD = 4;
+constexpr int TK = 16;
 
-template <bool TRANSA, bool TRANSB>
-__global__ __launch_bounds__(256) void gemm64_kernel(int64_t m, int64_t n, int64_t k, double alpha, const double *A, int64_t lda,
+template <int TS>
+struct Tile64 {
+    static constexpr int PAD = TS == 64 ? 4 : 16;
+    static constexpr int LD = TS + PAD;
+    static constexpr int NWV = 4;                       // wavefronts: 2 along m, 2 along n
+    static constexpr int NT = 64 * NWV;
+    static constexpr int PER = TS * TK / NT;            // elements per thread, operand and k step
+    static constexpr int NBI = TS / 32, NBJ = TS / (8 * NWV);   // 16 x 16 blocks per wavefront along m and n
+    static constexpr size_t SMEM = sizeof(double) * 2 * 2 * TK * LD;
+};
+
+template <bool TRANSA, bool TRANSB, int TS>
+// The 128-wide tile is held to 256 registers: two workgroups per CU run 1.4x faster than one with 379 registers, and
+// faster than one workgroup of eight wavefronts with 64 x 32 each.
+__global__ __launch_bounds__(Tile64<TS>::NT, TS == 128 ? 2 : 1) void gemm64_kernel(int64_t m, int64_t n, int64_t k, double alpha, const double *A, int64_t lda,
                                                      int64_t strideA, const double *B, int64_t ldb, int64_t strideB, double beta,
                                                      double *C, int64_t ldc, int64_t strideC, int64_t tiles_m) {
-    __shared__ double As[2][TK][TM + PAD];
-    __shared__ double Bs[2][TK][TN + PAD];
+    typedef Tile64<TS> TC;
+    constexpr int LD = TC::LD, PER = TC::PER, NBI = TC::NBI, NBJ = TC::NBJ, NT = TC::NT;
+    extern __shared__ __attribute__((aligned(16))) unsigned char gemm64_smem[];
+    double (*As)[TK][LD] = (double (*)[TK][LD])gemm64_smem;          // [2][TK][LD]
+    double (*Bs)[TK][LD] = As + 2;                                    // [2][TK][LD]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t tile = blockIdx.x;
-    const int64_t row0 = (tile % tiles_m) * TM, col0 = (tile / tiles_m) * TN;
+    const int64_t row0 = (tile % tiles_m) * TS, col0 = (tile / tiles_m) * TS;
     const int64_t batch = blockIdx.y;
     A += batch * strideA;
     B += batch * strideB;
     C += batch * strideC;
 
-    // each thread moves 4 elements of each operand tile per k step; the fast thread index runs along the
+    // each thread moves PER elements of each operand tile per k step; the fast thread index runs along the
     // direction that is contiguous in memory
-    double ra[4], rb[4];
-    auto fetch = [&](int64_t k0) {
+    double ra[PER], rb[PER];
+    // interior: the tile lies inside C and the k step inside k, so no element needs a bounds test (nor the branch
+    // around its load): the case nearly every step of a large product is
+    const bool inside = row0 + TS <= m && col0 + TS <= n;
+    auto fetch_at = [&](int64_t k0, auto interior) {
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int e = tid + 256 * u;
+        for (int u = 0; u < PER; u++) {
+            const int e = tid + NT * u;
             {
-                const int i = TRANSA ? e / TK : e % TM, kk = TRANSA ? e % TK : e / TM;
+                const int i = TRANSA ? e / TK : e % TS, kk = TRANSA ? e % TK : e / TS;
                 const int64_t gi = row0 + i, gk = k0 + kk;
-                ra[u] = (gi < m && gk < k) ? (TRANSA ? A[gk + gi * lda] : A[gi + gk * lda]) : 0.0;
+                ra[u] = (interior.value || (gi < m && gk < k)) ? (TRANSA ? A[gk + gi * lda] : A[gi + gk * lda]) : 0.0;
             }
             {
-                const int j = TRANSB ? e % TN : e / TK, kk = TRANSB ? e / TN : e % TK;
+                const int j = TRANSB ? e % TS : e / TK, kk = TRANSB ? e / TS : e % TK;
                 const int64_t gj = col0 + j, gk = k0 + kk;
-                rb[u] = (gj < n && gk < k) ? (TRANSB ? B[gj + gk * ldb] : B[gk + gj * ldb]) : 0.0;
+                rb[u] = (interior.value || (gj < n && gk < k)) ? (TRANSB ? B[gj + gk * ldb] : B[gk + gj * ldb]) : 0.0;
             }
         }
     };
+    auto fetch = [&](int64_t k0) {
+        if (inside && k0 + TK <= k) fetch_at(k0, std::true_type());
+        else fetch_at(k0, std::false_type());
+    };
     auto stash = [&](int buf) {
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int e = tid + 256 * u;
-            const int i = TRANSA ? e / TK : e % TM, ka = TRANSA ? e % TK : e / TM;
+        for (int u = 0; u < PER; u++) {
+            const int e = tid + NT * u;
+            const int i = TRANSA ? e / TK : e % TS, ka = TRANSA ? e % TK : e / TS;
             As[buf][ka][i] = ra[u];
-            const int j = TRANSB ? e % TN : e / TK, kb = TRANSB ? e / TN : e % TK;
+            const int j = TRANSB ? e % TS : e / TK, kb = TRANSB ? e / TS : e % TK;
             Bs[buf][kb][j] = rb[u];
         }
     };
 
-    doublex4_t acc[2][2];
+    doublex4_t acc[NBI][NBJ];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < NBI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = (doublex4_t){0.0, 0.0, 0.0, 0.0};
-    const int wr = (wave & 1) * 32, wc = (wave >> 1) * 32;   // this wavefront's corner of the tile
+        for (int j = 0; j < NBJ; j++) acc[i][j] = (doublex4_t){0.0, 0.0, 0.0, 0.0};
+    const int wr = (wave & 1) * (16 * NBI), wc = (wave >> 1) * (16 * NBJ);   // this wavefront's corner of the tile
     const int li = lane & 15, lk = lane >> 4;
 
     const int64_t nk = (k + TK - 1) / TK;
@@ -84,24 +110,27 @@ __global__ __launch_bounds__(256) void gemm64_kernel(int64_t m, int64_t n, int64
         if (kt + 1 < nk) fetch((kt + 1) * TK);
 #pragma unroll
         for (int ks = 0; ks < TK; ks += 4) {
-            double a[2], b[2];
+            // The next tile goes to the other LDS buffer before the last quarter of the matrix instructions, not after
+            // them: the wait for the global loads and the LDS writes then sit behind queued matrix work.  Both
+            // workgroups of a compute unit run in step, so at the end of the loop body they would idle the matrix pipes together.
+            if (ks == TK - 4 && kt + 1 < nk) stash(buf ^ 1);
+            double a[NBI], b[NBJ];
 #pragma unroll
-            for (int i = 0; i < 2; i++) a[i] = As[buf][ks + lk][wr + 16 * i + li];
+            for (int i = 0; i < NBI; i++) a[i] = As[buf][ks + lk][wr + 16 * i + li];
 #pragma unroll
-            for (int j = 0; j < 2; j++) b[j] = Bs[buf][ks + lk][wc + 16 * j + li];
+            for (int j = 0; j < NBJ; j++) b[j] = Bs[buf][ks + lk][wc + 16 * j + li];
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < NBI; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < NBJ; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < nk) stash(buf ^ 1);
         __syncthreads();
     }
     // beta == 0 overwrites C without reading it (BLAS semantics: NaNs in C do not propagate)
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < NBI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NBJ; j++)
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int64_t gr = row0 + wr + 16 * i + lk + 4 * v, gc = col0 + wc + 16 * j + li;
@@ -111,6 +140,24 @@ __global__ __launch_bounds__(256) void gemm64_kernel(int64_t m, int64_t n, int64
                     *c = beta == 0.0 ? x : x + beta * *c;
                 }
             }
+}
+
+template <bool TA, bool TB, int TS>
+int32_t launch_gemm64(int64_t m, int64_t n, int64_t k, double alpha, const double *a, int64_t lda, int64_t strideA, const double *b,
+                      int64_t ldb, int64_t strideB, double beta, double *c, int64_t ldc, int64_t strideC, int64_t batch, hipStream_t st) {
+    const int64_t tm = (m + TS - 1) / TS, tn = (n + TS - 1) / TS;
+    if (tm * tn > 2147483647LL) return mi_set_error(MI_ESHAPE, "mi_batched_gemm_f64: too many tiles");
+    auto kern = gemm64_kernel<TA, TB, TS>;
+    constexpr size_t SMEM = Tile64<TS>::SMEM;
+    static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn), (unsigned)batch), dim3(Tile64<TS>::NT), SMEM, st, m, n, k, alpha, a, lda, strideA, b, ldb, strideB,
+                       beta, c, ldc, strideC, tm);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
 }
 
 // ---- generic strided kernel --------------------------------------------------------------------------------
@@ -344,18 +391,19 @@ MI_API int32_t mi_batched_gemm_f64(char transA, char transB, int64_t m, int64_t 
         return mi_set_error(MI_ESHAPE, "mi_batched_gemm_f64: leading dimension smaller than the matrix it strides");
     if (strideA < 0 || strideB < 0 || strideC < 0) return mi_set_error(MI_ESHAPE, "mi_batched_gemm_f64: negative batch stride");
     if (batch > 65535) return mi_set_error(MI_ESHAPE, "mi_batched_gemm_f64: at most 65535 batch slices per call");
-    const int64_t tm = (m + TM - 1) / TM, tn = (n + TN - 1) / TN;
-    if (tm * tn > 2147483647LL) return mi_set_error(MI_ESHAPE, "mi_batched_gemm_f64: too many tiles");
-    const dim3 grid((unsigned)(tm * tn), (unsigned)batch);
     hipStream_t st = (hipStream_t)s;
     const double *a = (const double *)A, *b = (const double *)B;
     double *c = (double *)C;
-    if (!ta && !tb) hipLaunchKernelGGL((gemm64_kernel<false, false>), grid, dim3(256), 0, st, m, n, k, alpha, a, lda, strideA, b, ldb, strideB, beta, c, ldc, strideC, tm);
-    else if (ta && !tb) hipLaunchKernelGGL((gemm64_kernel<true, false>), grid, dim3(256), 0, st, m, n, k, alpha, a, lda, strideA, b, ldb, strideB, beta, c, ldc, strideC, tm);
-    else if (!ta && tb) hipLaunchKernelGGL((gemm64_kernel<false, true>), grid, dim3(256), 0, st, m, n, k, alpha, a, lda, strideA, b, ldb, strideB, beta, c, ldc, strideC, tm);
-    else hipLaunchKernelGGL((gemm64_kernel<true, true>), grid, dim3(256), 0, st, m, n, k, alpha, a, lda, strideA, b, ldb, strideB, beta, c, ldc, strideC, tm);
-    MI_LAUNCH_CHECK();
-    return MI_OK;
+    // 128 x 128 tiles where those still give every compute unit a workgroup
+    const bool large = m >= 128 && n >= 128 && ((m + 127) / 128) * ((n + 127) / 128) * batch >= 256;
+#define MI_GEMM64(TA_, TB_)                                                                                                              \
+    (large ? launch_gemm64<TA_, TB_, 128>(m, n, k, alpha, a, lda, strideA, b, ldb, strideB, beta, c, ldc, strideC, batch, st)             \
+           : launch_gemm64<TA_, TB_, 64>(m, n, k, alpha, a, lda, strideA, b, ldb, strideB, beta, c, ldc, strideC, batch, st))
+    if (!ta && !tb) return MI_GEMM64(false, false);
+    if (ta && !tb) return MI_GEMM64(true, false);
+    if (!ta && tb) return MI_GEMM64(false, true);
+    return MI_GEMM64(true, true);
+#undef MI_GEMM64
 }
 
 MI_API int32_t mi_batched_mul_generic(int32_t dtype_c, int32_t dtype_a, int32_t dtype_b, int64_t m, int64_t n, int64_t k, double alpha_re,

@@ -202,6 +202,25 @@ def test_large_float64(nn):
         assert close(dC.to_numpy(), 2.5 * ref - 0.5 * C0)
 
 
+def test_large_float64_128_wide_tiles(nn):
+    """Products with at least 256 tiles of 128 x 128 run the wider tile of the fp64 matrix-core kernel: sizes that end
+    inside a tile in both dimensions and inside a k step, a size of whole tiles (no bounds tests on the way), every
+    transpose combination, alpha / beta."""
+    rng = np.random.default_rng(8)
+    T = nn.batched_transpose
+    for (m, k, n, nb) in ((300, 70, 260, 50), (256, 64, 128, 128), (129, 33, 128, 70)):
+        A, B = randn(rng, m, k, nb), randn(rng, k, n, nb)
+        dA, dB = D(nn, A, "f64"), D(nn, B, "f64")
+        dAt, dBt = D(nn, A.transpose(1, 0, 2), "f64"), D(nn, B.transpose(1, 0, 2), "f64")
+        ref = per_slice(A, B)
+        for x, y in ((dA, dB), (T(dAt), dB), (dA, T(dBt)), (T(dAt), T(dBt))):
+            assert close(nn.batched_mul(x, y).to_numpy(), ref)
+        C0 = randn(rng, m, n, nb)
+        dC = D(nn, C0, "f64")
+        nn.batched_mul_(dC, dA, dB, 2.5, -0.5)
+        assert close(dC.to_numpy(), 2.5 * ref - 0.5 * C0)
+
+
 def test_float64_matches_float32_path_semantics(nn):
     """The same call in Float32 and Float64 differs only by rounding: the Float64 kernel is not a widened Float32
     product (entries chosen so that Float32 accumulation is visibly worse)."""
