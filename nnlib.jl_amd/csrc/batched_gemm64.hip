@@ -33,6 +33,11 @@ struct Tile64 {
     static constexpr int PER = TS * TK / NT;            // elements per thread, operand and k step
     static constexpr int NBI = TS / 32, NBJ = TS / (8 * NWV);   // 16 x 16 blocks per wavefront along m and n
     static constexpr size_t SMEM = sizeof(double) * 2 * 2 * TK * LD;
+    // Position of row / column x in the tile's k row (128-wide tiles).  An operand that is contiguous along k in memory
+    // is stored by lanes that run along k first (16 k x 4 columns per instruction): with rows 16 slots apart mod 32
+    // those 64 stores would land on 8 slots; flipping bits 2-3 of the column with k/2 spreads them over all 32 (two
+    // stores per slot, the minimum for 512 bytes).  Reads of 16 consecutive columns of one k row stay a permutation.
+    __device__ static inline int swz(int k, int x) { return TS == 64 ? x : x ^ (((k >> 1) & 3) << 2); }
 };
 
 template <bool TRANSA, bool TRANSB, int TS>
@@ -54,26 +59,29 @@ __global__ __launch_bounds__(Tile64<TS>::NT, TS == 128 ? 2 : 1) void gemm64_kern
     B += batch * strideB;
     C += batch * strideC;
 
-    // each thread moves PER elements of each operand tile per k step; the fast thread index runs along the
-    // direction that is contiguous in memory
+    // Each thread moves PER elements of each operand tile per k step; the fast thread index runs along the direction
+    // that is contiguous in memory.  Element u of a thread is its element 0 moved by a wavefront-uniform step (along k
+    // for an operand stored with its tile rows contiguous, along the rows otherwise), so one per-lane offset serves all
+    // of them and the rest of the address is scalar.
+    constexpr int RSTEP = NT / TK, KSTEP = NT / TS;   // rows / k between consecutive elements of a thread
+    const int ai = TRANSA ? tid / TK : tid % TS, ak = TRANSA ? tid % TK : tid / TS;   // tile row and k of element 0 (A)
+    const int bj = TRANSB ? tid % TS : tid / TK, bk = TRANSB ? tid / TS : tid % TK;   // tile column and k of element 0 (B)
+    const int64_t voffA = TRANSA ? ak + (row0 + ai) * lda : (row0 + ai) + ak * lda;
+    const int64_t voffB = TRANSB ? (col0 + bj) + bk * ldb : bk + (col0 + bj) * ldb;
+    const int64_t kstepA = TRANSA ? 1 : lda, ustepA = TRANSA ? RSTEP * lda : KSTEP * lda;
+    const int64_t kstepB = TRANSB ? ldb : 1, ustepB = TRANSB ? KSTEP * ldb : RSTEP * ldb;
     double ra[PER], rb[PER];
     // interior: the tile lies inside C and the k step inside k, so no element needs a bounds test (nor the branch
     // around its load): the case nearly every step of a large product is
     const bool inside = row0 + TS <= m && col0 + TS <= n;
     auto fetch_at = [&](int64_t k0, auto interior) {
+        const double *pa = A + k0 * kstepA, *pb = B + k0 * kstepB;
 #pragma unroll
         for (int u = 0; u < PER; u++) {
-            const int e = tid + NT * u;
-            {
-                const int i = TRANSA ? e / TK : e % TS, kk = TRANSA ? e % TK : e / TS;
-                const int64_t gi = row0 + i, gk = k0 + kk;
-                ra[u] = (interior.value || (gi < m && gk < k)) ? (TRANSA ? A[gk + gi * lda] : A[gi + gk * lda]) : 0.0;
-            }
-            {
-                const int j = TRANSB ? e % TS : e / TK, kk = TRANSB ? e / TS : e % TK;
-                const int64_t gj = col0 + j, gk = k0 + kk;
-                rb[u] = (interior.value || (gj < n && gk < k)) ? (TRANSB ? B[gj + gk * ldb] : B[gk + gj * ldb]) : 0.0;
-            }
+            const bool oka = interior.value || (row0 + ai + (TRANSA ? RSTEP * u : 0) < m && k0 + ak + (TRANSA ? 0 : KSTEP * u) < k);
+            ra[u] = oka ? (pa + u * ustepA)[voffA] : 0.0;
+            const bool okb = interior.value || (col0 + bj + (TRANSB ? 0 : RSTEP * u) < n && k0 + bk + (TRANSB ? KSTEP * u : 0) < k);
+            rb[u] = okb ? (pb + u * ustepB)[voffB] : 0.0;
         }
     };
     auto fetch = [&](int64_t k0) {
@@ -83,11 +91,10 @@ __global__ __launch_bounds__(Tile64<TS>::NT, TS == 128 ? 2 : 1) void gemm64_kern
     auto stash = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < PER; u++) {
-            const int e = tid + NT * u;
-            const int i = TRANSA ? e / TK : e % TS, ka = TRANSA ? e % TK : e / TS;
-            As[buf][ka][i] = ra[u];
-            const int j = TRANSB ? e % TS : e / TK, kb = TRANSB ? e / TS : e % TK;
-            Bs[buf][kb][j] = rb[u];
+            const int i = ai + (TRANSA ? RSTEP * u : 0), ka = ak + (TRANSA ? 0 : KSTEP * u);
+            As[buf][ka][TC::swz(ka, i)] = ra[u];
+            const int j = bj + (TRANSB ? 0 : RSTEP * u), kb = bk + (TRANSB ? KSTEP * u : 0);
+            Bs[buf][kb][TC::swz(kb, j)] = rb[u];
         }
     };
 
@@ -98,6 +105,8 @@ __global__ __launch_bounds__(Tile64<TS>::NT, TS == 128 ? 2 : 1) void gemm64_kern
         for (int j = 0; j < NBJ; j++) acc[i][j] = (doublex4_t){0.0, 0.0, 0.0, 0.0};
     const int wr = (wave & 1) * (16 * NBI), wc = (wave >> 1) * (16 * NBJ);   // this wavefront's corner of the tile
     const int li = lane & 15, lk = lane >> 4;
+    // swz(ks + lk, x) for the lane's reads: the flipped bits lie inside li, and k steps 0, 8 / 4, 12 share a value
+    const int li_even = TC::swz(lk, li), li_odd = TC::swz(4 + lk, li);
 
     const int64_t nk = (k + TK - 1) / TK;
     if (nk > 0) {
@@ -110,15 +119,15 @@ __global__ __launch_bounds__(Tile64<TS>::NT, TS == 128 ? 2 : 1) void gemm64_kern
         if (kt + 1 < nk) fetch((kt + 1) * TK);
 #pragma unroll
         for (int ks = 0; ks < TK; ks += 4) {
-            // The next tile goes to the other LDS buffer before the last quarter of the matrix instructions, not after
+            // The next tile goes to the other LDS buffer half way through the matrix instructions, not after
             // them: the wait for the global loads and the LDS writes then sit behind queued matrix work.  Both
             // workgroups of a compute unit run in step, so at the end of the loop body they would idle the matrix pipes together.
-            if (ks == TK - 4 && kt + 1 < nk) stash(buf ^ 1);
+            if (ks == TK / 2 && kt + 1 < nk) stash(buf ^ 1);
             double a[NBI], b[NBJ];
 #pragma unroll
-            for (int i = 0; i < NBI; i++) a[i] = As[buf][ks + lk][wr + 16 * i + li];
+            for (int i = 0; i < NBI; i++) a[i] = As[buf][ks + lk][wr + 16 * i + ((ks & 4) ? li_odd : li_even)];
 #pragma unroll
-            for (int j = 0; j < NBJ; j++) b[j] = Bs[buf][ks + lk][wc + 16 * j + li];
+            for (int j = 0; j < NBJ; j++) b[j] = Bs[buf][ks + lk][wc + 16 * j + ((ks & 4) ? li_odd : li_even)];
 #pragma unroll
             for (int i = 0; i < NBI; i++)
 #pragma unroll
