@@ -395,7 +395,7 @@ def measure_extra(key, steps, warmup, with_cpu):
         peak = PEAK["f32"] if dt_name == "c64" else PEAK[dt_name]
         line = dict(metric="batched_mul TFLOP/s", value=val, unit="TFLOP/s", dtype=dt_name,
                     roofline=dict(bound="mfma", achieved=val, peak=peak, unit="TFLOP/s", frac=val / peak, traffic=None),
-                    config=dict(workload=EXTRA[key], kernel={"c64": "gemm_c32_kernel", "f64": "gemm64_kernel"}.get(dt_name, "batched_gemm_kernel")),
+                    config=dict(workload=EXTRA[key]),
                     flops_per_step=flops)
         if dt_name == "f32":   # Float32 in, out and accumulation; `peak` stays the Float32 matrix instruction's
             line["roofline"]["products"] = ("v_mfma_f32_32x32x2_f32" if os.environ.get("MI355ATTN_F32_MFMA", "")[:1] == "1" else
@@ -434,7 +434,7 @@ def measure_extra(key, steps, warmup, with_cpu):
         val = nbytes / (ms * 1e-3) / 1e9
         line = dict(metric=f"{key} GB/s", value=val, unit="GB/s", dtype=dt_name,
                     roofline=dict(bound="hbm", achieved=val, peak=HBM_PEAK, unit="GB/s", frac=val / HBM_PEAK, traffic=None),
-                    config=dict(workload=EXTRA[key], kernel="softmax_dim1_kernel" if key == "softmax" else "softmax_nd_kernel"),
+                    config=dict(workload=EXTRA[key]),
                     bytes_per_step=nbytes)
         if with_cpu:
             from oracle import oracle as O

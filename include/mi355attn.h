@@ -52,7 +52,11 @@ enum {
 /* ---- element types --------------------------------------------------------------- */
 enum {
     MI_F32 = 0, MI_F16 = 1, MI_BF16 = 2,
-    /* taken by mi_batched_gemm_f64 / mi_batched_mul_generic only (every other entry point answers MI_EDTYPE) */
+    /* MI_F64: mi_batched_gemm_f64 / mi_batched_mul_generic, the softmax family (mi_softmax*, mi_logsumexp*), the forward
+     * attention calls (mi_attention_fwd / _plan / _fwd_static; double-precision vector kernels, what the reference computes
+     * for Float64 arrays: src/softmax.jl:56, test/attention.jl:17-34) and mi_convert.  The others: mi_batched_mul_generic
+     * only, and the integers as a source of mi_convert (float(T) of an integer array is Float64).  Every other entry
+     * point answers MI_EDTYPE for them. */
     MI_F64 = 3, MI_C64 = 4 /* ComplexF32 */, MI_C128 = 5 /* ComplexF64 */, MI_I32 = 6, MI_I64 = 7
 };
 
@@ -93,7 +97,10 @@ enum {
                                     products as six bf16 matrix instructions on three bf16 planes per operand (Float32
                                     accuracy), or the Float32 instruction if MI355ATTN_F32_MFMA=1 is in the environment
                                     (the gradient kernels of this family: the same for calls without bias / mask arrays
-                                    and dropout, the Float32 instruction otherwise) */
+                                    and dropout, the Float32 instruction otherwise).  On the planes a finite q, k or v
+                                    entry above the largest bf16 (|x| > 3.3895e38) gives NaN products; calls with a
+                                    128-wide head tile, a bias or mask array and the weights output always use the
+                                    Float32 instruction */
     MI_ATTN_KERNEL_DECODE = 3    /* split-kv bandwidth-bound path for one to four queries (L_q <= 4) */
 };
 
@@ -246,7 +253,7 @@ int32_t mi_dropout_dims(int32_t dtype, const void *x, void *y, int32_t ndim, con
 
 /* ---- softmax over the first dimension -------------------------------------------- */
 /* y[:, c] = softmax(x[:, c]) for a (rows, cols) column-major matrix; y may alias x
- * (softmax!(x), src/softmax.jl:64).  Arithmetic in fp32; +-Inf / NaN rules of
+ * (softmax!(x), src/softmax.jl:64).  Arithmetic in fp32 (Float64 arrays: in double); +-Inf / NaN rules of
  * src/softmax.jl:69-79 (a +Inf maximum turns the column into an indicator of its
  * +Inf entries, normalised; NaN poisons its column; an all -Inf column is NaN). */
 int32_t mi_softmax_dim1(int32_t dtype, const void *x, void *y, int64_t rows, int64_t cols,
@@ -256,7 +263,7 @@ int32_t mi_softmax_dim1(int32_t dtype, const void *x, void *y, int64_t rows, int
 /* The array is viewed as (inner, len, outer): element (i, j, o) at i + inner*(j + len*o), and the
  * reduction runs over j.  `dims = d` of an N-d column-major array gives inner = prod(size[1:d-1]),
  * len = size[d], outer = prod(size[d+1:N]); `dims = :` gives (1, length, 1); a tuple of adjacent
- * dims multiplies their extents into len.  y may alias x.  Arithmetic in fp32. */
+ * dims multiplies their extents into len.  y may alias x.  Arithmetic in fp32 (Float64 arrays: in double). */
 enum { MI_SOFTMAX = 0, MI_LOGSOFTMAX = 1 };
 /* op = MI_SOFTMAX: softmax(x; dims) (src/softmax.jl:56-79).  op = MI_LOGSOFTMAX: logsoftmax(x; dims)
  * (src/softmax.jl:133-147), including its +Inf rule: a column whose maximum is +Inf gives 0 at the
@@ -367,7 +374,8 @@ int32_t mi_randn_fill(void *ptr, int32_t dtype, int64_t n, uint64_t seed, uint64
 /* mask[i] = (u_i < keep_prob) as uint8, same generator. */
 int32_t mi_bernoulli_fill(uint8_t *mask, int64_t n, uint64_t seed, uint64_t stream_id,
                           float keep_prob, mi_stream stream);
-/* dst[i] = dtype_dst(src[i]) with round-to-nearest-even. */
+/* dst[i] = dtype_dst(src[i]) with round-to-nearest-even: between MI_F32, MI_F16 and MI_BF16; to MI_F64 from those and
+ * from MI_I32 / MI_I64; from MI_F64 to the three narrower floating-point types. */
 int32_t mi_convert(void *dst, int32_t dtype_dst, const void *src, int32_t dtype_src, int64_t n,
                    mi_stream stream);
 

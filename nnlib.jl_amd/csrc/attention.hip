@@ -196,7 +196,9 @@ int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_back
     if (d->struct_size != (int32_t)sizeof(mi_attn_desc))
         return mi_set_error(MI_EINVAL, "mi_attention: desc.struct_size is %d, library expects %zu", d->struct_size,
                             sizeof(mi_attn_desc));
-    if (!mi_dtype_ok(d->dtype)) return mi_set_error(MI_EDTYPE, "mi_attention: unknown dtype %d", d->dtype);
+    // Float64 arrays: the forward call only (a double-precision vector kernel, attention_f64.hip)
+    if (!(for_backward ? mi_dtype_ok(d->dtype) : mi_dtype_ok_f64(d->dtype)))
+        return mi_set_error(MI_EDTYPE, "mi_attention: unknown dtype %d", d->dtype);
     if (d->E < 0 || d->Ev < 0 || d->Lq < 0 || d->Lkv < 0 || d->B < 0)
         return mi_set_error(MI_ESHAPE, "mi_attention: negative size");
     if (d->H < 1) return mi_set_error(MI_ESHAPE, "mi_attention: nheads must be at least 1 (got %lld)", (long long)d->H);
@@ -209,8 +211,9 @@ int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_back
         return mi_set_error(MI_ESHAPE, "mi_attention: a causal (len, len) mask needs Lq == Lkv (got %lld, %lld)",
                             (long long)d->Lq, (long long)d->Lkv);
     if (!for_backward && !d->out && !d->weights) return mi_set_error(MI_EINVAL, "mi_attention: both out and weights are NULL");
-    if (d->weights && d->weights_dtype != d->dtype && d->weights_dtype != MI_F32)
-        return mi_set_error(MI_EDTYPE, "mi_attention: weights_dtype must equal dtype or be MI_F32");
+    if (d->weights && d->weights_dtype != d->dtype && (d->weights_dtype != MI_F32 || d->dtype == MI_F64))
+        return mi_set_error(MI_EDTYPE, "mi_attention: weights_dtype must equal dtype or (16-bit inputs) be MI_F32");
+    if (d->dtype == MI_F64 && d->stats) return mi_set_error(MI_EDTYPE, "mi_attention: row statistics are not kept for Float64 calls");
     const bool empty = d->Lq == 0 || d->B == 0 || (d->E == 0 && d->Ev == 0);
     if (!empty) {
         if (d->Lkv > 0 && d->E > 0 && (!d->q || !d->k)) return mi_set_error(MI_EINVAL, "mi_attention: q or k is NULL");
@@ -246,7 +249,7 @@ int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_back
 
 static int32_t choose(const mi_attn_desc *d, const AttnParams &p, size_t *ws) {
     *ws = 0;
-    if (d->flags & MI_ATTN_FORCE_GENERIC) return MI_ATTN_KERNEL_GENERIC;
+    if ((d->flags & MI_ATTN_FORCE_GENERIC) || p.dtype == MI_F64) return MI_ATTN_KERNEL_GENERIC;
     if (attention_decode_supports(p)) {
         *ws = attention_decode_workspace(p);
         return MI_ATTN_KERNEL_DECODE;
@@ -358,6 +361,6 @@ static int32_t attention_forward(const mi_attn_desc *d, mi_stream s, bool static
     case MI_ATTN_KERNEL_DECODE: return launch_attention_decode(p, st);
     case MI_ATTN_KERNEL_FLASH16: return launch_attention_flash16(p, st);
     case MI_ATTN_KERNEL_FLASH32: return launch_attention_flash32(p, st);
-    default: return launch_attention_generic(p, st);
+    default: return p.dtype == MI_F64 ? launch_attention_f64(p, st) : launch_attention_generic(p, st);
     }
 }

@@ -114,6 +114,7 @@ size_t attention_bwd_generic_workspace(const AttnParams &p);
 int32_t attention_validate(const mi_attn_desc *d, AttnParams *out, bool for_backward = false);
 
 int32_t launch_attention_generic(const AttnParams &p, hipStream_t st);
+int32_t launch_attention_f64(const AttnParams &p, hipStream_t st);   // Float64 arrays (attention_f64.hip)
 int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st);
 int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st);
 int32_t launch_attention_decode(const AttnParams &p, hipStream_t st);

@@ -203,10 +203,11 @@ struct OperandS {
             const int c = tid + S::THREADS * u;
             const floatx4_t x = reg[u];
             uint32_t pl[3][2];
-            const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
-            if (odd) {   // an Inf, a NaN or a value beyond the bf16 range among the four (rare)
-                split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
-                split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+            split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+            split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+            if (mi_plane_word_special(pl[0][0]) || mi_plane_word_special(pl[0][1])) {   // an Inf, a NaN or a value beyond the bf16 range among the four (rare)
+                split3_pair_wide(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+                split3_pair_wide(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
             }
             unsigned at;
             if (RM) {

@@ -29,8 +29,14 @@ int32_t mi_set_error(int32_t code, const char *fmt, ...) __attribute__((format(p
                                 hipGetErrorString(_e), __FILE__, __LINE__);                 \
     } while (0)
 
-static inline size_t mi_dtype_size(int32_t dt) { return dt == MI_F32 ? 4 : 2; }
+static inline size_t mi_dtype_size(int32_t dt) { return dt == MI_F64 ? 8 : dt == MI_F32 ? 4 : 2; }
 static inline bool mi_dtype_ok(int32_t dt) { return dt == MI_F32 || dt == MI_F16 || dt == MI_BF16; }
+// entry points that also take Float64 arrays (the softmax family, the attention forward call)
+static inline bool mi_dtype_ok_f64(int32_t dt) { return mi_dtype_ok(dt) || dt == MI_F64; }
+
+// Float64 softmax family (softmax_f64.hip): op 0 softmax, 1 logsoftmax, 2 logsumexp, 3 / 4 the gradients (x = dy, x2 = y)
+int32_t launch_softmax_family_f64(int op, const void *x, const void *x2, void *y, int64_t inner, int64_t len, int64_t outer, hipStream_t st);
+int32_t launch_logsumexp_bwd_f64(const void *dy, const void *x, const void *lse, void *dx, int64_t inner, int64_t len, int64_t outer, hipStream_t st);
 
 // ---- vector types ------------------------------------------------------------------
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
@@ -159,6 +165,36 @@ __device__ static inline void split3_pair_guarded(float x0, float x1, uint32_t &
     lo = __builtin_bit_cast(uint32_t, l);
 }
 
+// The same for callers that also keep finite values whose bf16 rounding overflows (|x| above the largest bf16,
+// 3.3895e38): split3_pair makes (Inf, -Inf, NaN) of those.  mi_plane_word_special tells whether either half of a hi-plane
+// word has an all-ones exponent (Inf, NaN or such an overflow); split3_pair_wide redoes a pair with the first plane
+// truncated instead of rounded where the rounding overflows, and with split3's rule for Inf and NaN.
+__device__ static inline bool mi_plane_word_special(uint32_t hi) {
+    return (hi & 0x7f80u) == 0x7f80u || (hi & 0x7f800000u) == 0x7f800000u;
+}
+__device__ static inline void split3_wide(float x, __bf16 &hi, __bf16 &mid, __bf16 &lo) {
+    if (!(__builtin_fabsf(x) < MI_POS_INF)) {
+        hi = (__bf16)0.0f;
+        mid = (__bf16)0.0f;
+        lo = (__bf16)x;
+        return;
+    }
+    hi = (__bf16)x;
+    if (!(__builtin_fabsf((float)hi) < MI_POS_INF))
+        hi = __builtin_bit_cast(__bf16, (unsigned short)(__builtin_bit_cast(uint32_t, x) >> 16));   // truncated: finite
+    const float r = x - (float)hi;
+    mid = (__bf16)r;
+    lo = (__bf16)(r - (float)mid);
+}
+__device__ static inline void split3_pair_wide(float x0, float x1, uint32_t &hi, uint32_t &mid, uint32_t &lo) {
+    __bf16 h0, m0, l0, h1, m1, l1;
+    split3_wide(x0, h0, m0, l0);
+    split3_wide(x1, h1, m1, l1);
+    const bf16x2_t h = {h0, h1}, m = {m0, m1}, l = {l0, l1};
+    hi = __builtin_bit_cast(uint32_t, h);
+    mid = __builtin_bit_cast(uint32_t, m);
+    lo = __builtin_bit_cast(uint32_t, l);
+}
 
 // max(a, b, c) as one instruction with no quieting of the inputs (fmaxf on MFMA results costs an extra
 // v_max x, x per operand); a NaN operand is ignored like fmaxf does.

@@ -205,7 +205,46 @@ static void launch_convert_from(void *d, const void *src, int32_t ds, int64_t n,
     else hipLaunchKernelGGL((convert_kernel<TD, BF16>), g, b, 0, st, (td *)d, (const __bf16 *)src, n);
 }
 
+// conversions that involve Float64: to it from every real element type (what `float(T)` of an integer array is,
+// src/softmax.jl:56), and from it to the narrower floating-point types
+template <typename TD, typename TS>
+__global__ __launch_bounds__(256) void convert_plain_kernel(TD *dst, const TS *src, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = (TD)src[i];
+}
+template <typename TD>
+static bool launch_convert_plain_from(void *d, const void *src, int32_t ds, int64_t n, hipStream_t st) {
+    dim3 g(grid_for(n)), b(256);
+    switch (ds) {
+    case MI_F64: hipLaunchKernelGGL((convert_plain_kernel<TD, double>), g, b, 0, st, (TD *)d, (const double *)src, n); return true;
+    case MI_F32: hipLaunchKernelGGL((convert_plain_kernel<TD, float>), g, b, 0, st, (TD *)d, (const float *)src, n); return true;
+    case MI_F16: hipLaunchKernelGGL((convert_plain_kernel<TD, _Float16>), g, b, 0, st, (TD *)d, (const _Float16 *)src, n); return true;
+    case MI_BF16: hipLaunchKernelGGL((convert_plain_kernel<TD, __bf16>), g, b, 0, st, (TD *)d, (const __bf16 *)src, n); return true;
+    case MI_I32: hipLaunchKernelGGL((convert_plain_kernel<TD, int32_t>), g, b, 0, st, (TD *)d, (const int32_t *)src, n); return true;
+    case MI_I64: hipLaunchKernelGGL((convert_plain_kernel<TD, int64_t>), g, b, 0, st, (TD *)d, (const int64_t *)src, n); return true;
+    default: return false;
+    }
+}
+
 MI_API int32_t mi_convert(void *dst, int32_t dd, const void *src, int32_t ds, int64_t n, mi_stream s) {
+    if (dd == MI_F64 || ds == MI_F64) {
+        if (n < 0) return mi_set_error(MI_EINVAL, "mi_convert: negative length");
+        if (n == 0) return MI_OK;
+        if (!dst || !src) return mi_set_error(MI_EINVAL, "mi_convert: null pointer");
+        hipStream_t st64 = (hipStream_t)s;
+        bool ok = false;
+        dim3 g64(grid_for(n)), b64(256);
+        const double *s64 = (const double *)src;
+        ok = true;
+        if (dd == MI_F64) ok = launch_convert_plain_from<double>(dst, src, ds, n, st64);
+        else if (dd == MI_F32) hipLaunchKernelGGL((convert_plain_kernel<float, double>), g64, b64, 0, st64, (float *)dst, s64, n);
+        else if (dd == MI_F16) hipLaunchKernelGGL((convert_plain_kernel<_Float16, double>), g64, b64, 0, st64, (_Float16 *)dst, s64, n);
+        else if (dd == MI_BF16) hipLaunchKernelGGL((convert_plain_kernel<__bf16, double>), g64, b64, 0, st64, (__bf16 *)dst, s64, n);
+        else ok = false;
+        if (!ok) return mi_set_error(MI_EDTYPE, "mi_convert: no conversion from dtype %d to dtype %d", ds, dd);
+        MI_LAUNCH_CHECK();
+        return MI_OK;
+    }
     if (!mi_dtype_ok(dd) || !mi_dtype_ok(ds)) return mi_set_error(MI_EDTYPE, "mi_convert: unknown dtype");
     if (n < 0) return mi_set_error(MI_EINVAL, "mi_convert: negative length");
     if (n == 0) return MI_OK;

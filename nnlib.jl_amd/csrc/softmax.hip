@@ -207,11 +207,12 @@ static void launch_softmax(const void *x, void *y, int64_t rows, int64_t cols, h
 }
 
 MI_API int32_t mi_softmax_dim1(int32_t dtype, const void *x, void *y, int64_t rows, int64_t cols, mi_stream s) {
-    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_softmax_dim1: unknown dtype %d", dtype);
+    if (!mi_dtype_ok_f64(dtype)) return mi_set_error(MI_EDTYPE, "mi_softmax_dim1: unknown dtype %d", dtype);
     if (rows < 0 || cols < 0) return mi_set_error(MI_EINVAL, "mi_softmax_dim1: negative size");
     if (rows == 0 || cols == 0) return MI_OK;
     if (!x || !y) return mi_set_error(MI_EINVAL, "mi_softmax_dim1: null pointer");
     hipStream_t st = (hipStream_t)s;
+    if (dtype == MI_F64) return launch_softmax_family_f64(0, x, nullptr, y, 1, rows, cols, st);
     if (dtype == MI_F32) launch_softmax<F32>(x, y, rows, cols, st);
     else if (dtype == MI_F16) launch_softmax<F16>(x, y, rows, cols, st);
     else launch_softmax<BF16>(x, y, rows, cols, st);

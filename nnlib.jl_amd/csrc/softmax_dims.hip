@@ -97,7 +97,7 @@ int32_t back(const Plan &pl, int32_t dtype, const void *src, void *dst, mi_strea
 
 MI_API int32_t mi_softmax_dims_workspace(int32_t dtype, int32_t ndim, const int64_t *sizes, uint32_t dims_mask, size_t *bytes) {
     if (!bytes) return mi_set_error(MI_EINVAL, "mi_softmax_dims_workspace: bytes is NULL");
-    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_softmax_dims_workspace: unknown dtype %d", dtype);
+    if (!mi_dtype_ok_f64(dtype)) return mi_set_error(MI_EDTYPE, "mi_softmax_dims_workspace: unknown dtype %d", dtype);
     Plan pl;
     int32_t rc = make_plan("mi_softmax_dims_workspace", ndim, sizes, dims_mask, &pl);
     if (rc != MI_OK) return rc;
@@ -107,7 +107,7 @@ MI_API int32_t mi_softmax_dims_workspace(int32_t dtype, int32_t ndim, const int6
 
 MI_API int32_t mi_softmax_dims(int32_t op, int32_t dtype, const void *x, void *y, int32_t ndim, const int64_t *sizes, uint32_t dims_mask,
                                void *workspace, size_t workspace_bytes, mi_stream s) {
-    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_softmax_dims: unknown dtype %d", dtype);
+    if (!mi_dtype_ok_f64(dtype)) return mi_set_error(MI_EDTYPE, "mi_softmax_dims: unknown dtype %d", dtype);
     Plan pl;
     int32_t rc = make_plan("mi_softmax_dims", ndim, sizes, dims_mask, &pl);
     if (rc != MI_OK) return rc;
@@ -124,7 +124,7 @@ MI_API int32_t mi_softmax_dims(int32_t op, int32_t dtype, const void *x, void *y
 
 MI_API int32_t mi_logsumexp_dims(int32_t dtype, const void *x, void *y, int32_t ndim, const int64_t *sizes, uint32_t dims_mask,
                                  void *workspace, size_t workspace_bytes, mi_stream s) {
-    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_logsumexp_dims: unknown dtype %d", dtype);
+    if (!mi_dtype_ok_f64(dtype)) return mi_set_error(MI_EDTYPE, "mi_logsumexp_dims: unknown dtype %d", dtype);
     Plan pl;
     int32_t rc = make_plan("mi_logsumexp_dims", ndim, sizes, dims_mask, &pl);
     if (rc != MI_OK) return rc;
@@ -141,7 +141,7 @@ MI_API int32_t mi_logsumexp_dims(int32_t dtype, const void *x, void *y, int32_t 
 
 MI_API int32_t mi_softmax_bwd_dims(int32_t op, int32_t dtype, const void *dy, const void *y, void *dx, int32_t ndim, const int64_t *sizes,
                                    uint32_t dims_mask, void *workspace, size_t workspace_bytes, mi_stream s) {
-    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_softmax_bwd_dims: unknown dtype %d", dtype);
+    if (!mi_dtype_ok_f64(dtype)) return mi_set_error(MI_EDTYPE, "mi_softmax_bwd_dims: unknown dtype %d", dtype);
     Plan pl;
     int32_t rc = make_plan("mi_softmax_bwd_dims", ndim, sizes, dims_mask, &pl);
     if (rc != MI_OK) return rc;
@@ -159,7 +159,7 @@ MI_API int32_t mi_softmax_bwd_dims(int32_t op, int32_t dtype, const void *dy, co
 
 MI_API int32_t mi_logsumexp_bwd_dims(int32_t dtype, const void *dy, const void *x, const void *lse, void *dx, int32_t ndim,
                                      const int64_t *sizes, uint32_t dims_mask, void *workspace, size_t workspace_bytes, mi_stream s) {
-    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_logsumexp_bwd_dims: unknown dtype %d", dtype);
+    if (!mi_dtype_ok_f64(dtype)) return mi_set_error(MI_EDTYPE, "mi_logsumexp_bwd_dims: unknown dtype %d", dtype);
     Plan pl;
     int32_t rc = make_plan("mi_logsumexp_bwd_dims", ndim, sizes, dims_mask, &pl);
     if (rc != MI_OK) return rc;

@@ -655,11 +655,12 @@ void launch_nd(const void *x, const void *x2, void *y, int64_t inner, int64_t le
 template <int OP>
 int32_t dispatch(const char *name, int32_t dtype, const void *x, const void *x2, void *y, int64_t inner, int64_t len,
                  int64_t outer, mi_stream s) {
-    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "%s: unknown dtype %d", name, dtype);
+    if (!mi_dtype_ok_f64(dtype)) return mi_set_error(MI_EDTYPE, "%s: unknown dtype %d", name, dtype);
     if (inner < 0 || len < 0 || outer < 0) return mi_set_error(MI_EINVAL, "%s: negative size", name);
     if (inner == 0 || outer == 0 || (len == 0 && OP != OP_LOGSUMEXP)) return MI_OK;
     if (!x || !y || (OP >= OP_GRAD_SOFTMAX && !x2)) return mi_set_error(MI_EINVAL, "%s: null pointer", name);
     hipStream_t st = (hipStream_t)s;
+    if (dtype == MI_F64) return launch_softmax_family_f64(OP, x, x2, y, inner, len, outer, st);
     if (dtype == MI_F32) launch_nd<F32, OP>(x, x2, y, inner, len, outer, st);
     else if (dtype == MI_F16) launch_nd<F16, OP>(x, x2, y, inner, len, outer, st);
     else launch_nd<BF16, OP>(x, x2, y, inner, len, outer, st);
@@ -698,11 +699,12 @@ void launch_logsumexp_bwd(const void *dy, const void *x, const void *lse, void *
 
 MI_API int32_t mi_logsumexp_bwd(int32_t dtype, const void *dy, const void *x, const void *lse, void *dx, int64_t inner,
                                 int64_t len, int64_t outer, mi_stream s) {
-    if (!mi_dtype_ok(dtype)) return mi_set_error(MI_EDTYPE, "mi_logsumexp_bwd: unknown dtype %d", dtype);
+    if (!mi_dtype_ok_f64(dtype)) return mi_set_error(MI_EDTYPE, "mi_logsumexp_bwd: unknown dtype %d", dtype);
     if (inner < 0 || len < 0 || outer < 0) return mi_set_error(MI_EINVAL, "mi_logsumexp_bwd: negative size");
     if (inner == 0 || len == 0 || outer == 0) return MI_OK;
     if (!dy || !x || !lse || !dx) return mi_set_error(MI_EINVAL, "mi_logsumexp_bwd: null pointer");
     hipStream_t st = (hipStream_t)s;
+    if (dtype == MI_F64) return launch_logsumexp_bwd_f64(dy, x, lse, dx, inner, len, outer, st);
     if (dtype == MI_F32) launch_logsumexp_bwd<F32>(dy, x, lse, dx, inner, len, outer, st);
     else if (dtype == MI_F16) launch_logsumexp_bwd<F16>(dy, x, lse, dx, inner, len, outer, st);
     else launch_logsumexp_bwd<BF16>(dy, x, lse, dx, inner, len, outer, st);

@@ -22,9 +22,11 @@ NNlib.dot_product_attention_scores(q::DA{T, 4}, k::DA{T, 4}, bias = nothing; kws
 NNlib.make_causal_mask(x::DA; dims::Int = 2) = M.make_causal_mask(x; dims)
 
 # ---- batched_mul: the two backend hooks (src/batched/batchedmul.jl:256-298, ext/NNlibAMDGPUExt/batched_mul.jl:11-24)
-# _batched_gemm! receives BLAS-style flags for arrays whose first stride is 1 after un-transposing
+# _batched_gemm! receives BLAS-style flags for arrays whose first stride is 1 after un-transposing: 'N', 'T', or 'C'
+# (what src/batched/batchedmul.jl:268-270 passes for a BatchedAdjoint of a complex array)
+_op(t::Char, X) = t == 'N' ? X : t == 'C' ? M.batched_adjoint(X) : M.batched_transpose(X)
 NNlib._batched_gemm!(::Type{<:DA}, tA::Char, tB::Char, α::Number, A, B, β::Number, C) =
-    M.batched_mul!(C, tA == 'N' ? A : M.batched_transpose(A), tB == 'N' ? B : M.batched_transpose(B), α, β)
+    M.batched_mul!(C, _op(tA, A), _op(tB, B), α, β)
 # element types outside BlasFloat (Float16, BFloat16, integers) and mixed ones never reach _batched_gemm!
 NNlib._batched_mul!(::Type{<:DA}, C, A, B, α::Number, β::Number) = M.batched_mul!(C, A, B, α, β)
 NNlib.batched_mul(A::DA{<:Any, 3}, B::DA{<:Any, 3}) = M.batched_mul(A, B)

@@ -47,6 +47,8 @@ dtype_code(::Type{ComplexF64}) = MI_C128
 dtype_code(::Type{Int32}) = MI_I32
 dtype_code(::Type{Int64}) = MI_I64
 const MINumber = Union{MIFloat, Float64, ComplexF32, ComplexF64, Int32, Int64}
+# the softmax family and the attention forward call also take Float64 (test/softmax.jl:4-29, test/attention.jl:17-34)
+const MIFloat64 = Union{MIFloat, Float64}
 
 last_error() = unsafe_string(ccall((:mi_last_error_string, libmi), Cstring, ()))
 
@@ -242,7 +244,7 @@ end
 # `stats`: nothing, or a Float32 DeviceArray of mi_attention_stats_size bytes that receives the softmax
 # row statistics for ∇dot_product_attention (written by the MFMA flash kernels, with or without bias, mask and dropout)
 function attention_call(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v, bias, mask, H::Int; want_out::Bool,
-                        want_weights::Bool, fdrop::Union{Nothing, Dropout} = nothing, stats = nothing) where {T <: MIFloat}
+                        want_weights::Bool, fdrop::Union{Nothing, Dropout} = nothing, stats = nothing) where {T <: MIFloat64}
     E, Lq, B = size(q); Lkv = size(k, 2); Ev = v === nothing ? E : size(v, 1)
     causal, mptr, mstr, bptr, bstr = mask_and_bias(T, bias, mask, (Lkv, Lq, H, B))
     out = want_out ? DeviceArray{T}(undef, Ev, Lq, B) : nothing
@@ -281,7 +283,7 @@ end
 # `return_weights = false` is this library's one addition: it skips materialising α and returns
 # `nothing` in its place (the reference always returns α).
 function dot_product_attention(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::DeviceArray{T, 3}, bias = nothing;
-                               fdrop = identity, mask = nothing, nheads = 1, return_weights = true, stats = nothing) where {T <: MIFloat}
+                               fdrop = identity, mask = nothing, nheads = 1, return_weights = true, stats = nothing) where {T <: MIFloat64}
     all(size.((q, k, v), 1) .% nheads .== 0) || throw(ArgumentError("First dimension in query, key and value must be divisible by `nheads`.\nInstead:\n- size(q): $(size(q))\n- size(k): $(size(k))\n- size(v): $(size(v))\n- nheads: $nheads"))
     size(q, 3) == size(k, 3) == size(v, 3) || throw(ArgumentError("Batch dimensions have to be the same. Instead:\n- size(q): $(size(q))\n- size(k): $(size(k))\n- size(v): $(size(v))"))
     size(q, 1) == size(k, 1) || throw(ArgumentError("First dimension in query and key has to be the same. Instead:\n- size(q): $(size(q))\n- size(k): $(size(k))"))
@@ -297,7 +299,7 @@ function dot_product_attention(q::DeviceArray{T, 3}, k::DeviceArray{T, 3}, v::De
 end
 
 function dot_product_attention_scores(q::DeviceArray{T, 4}, k::DeviceArray{T, 4}, bias = nothing;
-                                      fdrop = identity, mask = nothing) where {T <: MIFloat}
+                                      fdrop = identity, mask = nothing) where {T <: MIFloat64}
     D, H, Lq, B = size(q)
     (size(k, 1), size(k, 2), size(k, 4)) == (D, H, B) || throw(DimensionMismatch("query $(size(q)) and key $(size(k)) disagree in feature, head or batch size"))
     _, α = attention_call(reshape(q, (D * H, Lq, B)), reshape(k, (D * H, size(k, 3), B)), nothing, bias, mask, H;
@@ -370,7 +372,7 @@ function dims_call(x::DeviceArray{T, N}, dims) where {T, N}
 end
 wsptr(ws) = ws === nothing ? C_NULL : ws.ptr
 
-function softmax_like!(op::Int32, out::DeviceArray{T, N}, x::DeviceArray{T, N}, dims) where {T <: MIFloat, N}
+function softmax_like!(op::Int32, out::DeviceArray{T, N}, x::DeviceArray{T, N}, dims) where {T <: MIFloat64, N}
     size(out) == size(x) || throw(DimensionMismatch("output size $(size(out)) differs from input size $(size(x))"))
     sizes, mask, ws, wsb = dims_call(x, dims)
     GC.@preserve out x sizes ws check(ccall((:mi_softmax_dims, libmi), Int32,
@@ -379,17 +381,27 @@ function softmax_like!(op::Int32, out::DeviceArray{T, N}, x::DeviceArray{T, N}, 
     out
 end
 
-softmax(x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = softmax!(similar(x, T, size(x)), x; dims)
+# float.(x) for an integer array: Float64, what `similar(x, float(T))` is in src/softmax.jl:56
+function to_float64(x::DeviceArray{T, N}) where {T <: Union{Int32, Int64}, N}
+    out = similar(x, Float64, size(x))
+    GC.@preserve out x check(ccall((:mi_convert, libmi), Int32, (Ptr{Cvoid}, Int32, Ptr{Cvoid}, Int32, Int64, Ptr{Cvoid}),
+                                  out.ptr, MI_F64, x.ptr, dtype_code(T), length(x), C_NULL))
+    out
+end
+softmax(x::DeviceArray{<:Union{Int32, Int64}}; dims = 1) = softmax(to_float64(x); dims)
+logsoftmax(x::DeviceArray{<:Union{Int32, Int64}}; dims = 1) = logsoftmax(to_float64(x); dims)
+logsumexp(x::DeviceArray{<:Union{Int32, Int64}}; dims = :) = logsumexp(to_float64(x); dims)
+softmax(x::DeviceArray{T}; dims = 1) where {T <: MIFloat64} = softmax!(similar(x, T, size(x)), x; dims)
 softmax!(x::DeviceArray; dims = 1) = softmax!(x, x; dims)
-softmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = softmax_like!(MI_SOFTMAX, out, x, dims)
+softmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloat64} = softmax_like!(MI_SOFTMAX, out, x, dims)
 
-logsoftmax(x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = logsoftmax!(similar(x, T, size(x)), x; dims)
+logsoftmax(x::DeviceArray{T}; dims = 1) where {T <: MIFloat64} = logsoftmax!(similar(x, T, size(x)), x; dims)
 logsoftmax!(x::DeviceArray; dims = 1) = logsoftmax!(x, x; dims)
-logsoftmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloat} = softmax_like!(MI_LOGSOFTMAX, out, x, dims)
+logsoftmax!(out::DeviceArray{T}, x::DeviceArray{T}; dims = 1) where {T <: MIFloat64} = softmax_like!(MI_LOGSOFTMAX, out, x, dims)
 
 # logsumexp(x; dims = :) returns a scalar for dims = : (one device-to-host copy), else an array that
 # keeps the reduced dimensions with extent 1, as NNlib's does (src/softmax.jl:200-203).
-function logsumexp(x::DeviceArray{T, N}; dims = :) where {T <: MIFloat, N}
+function logsumexp(x::DeviceArray{T, N}; dims = :) where {T <: MIFloat64, N}
     sizes, mask, ws, wsb = dims_call(x, dims)
     kept = dims isa Colon ? () : ntuple(d -> d in dims ? 1 : size(x, d), N)
     out = similar(x, T, kept)
@@ -401,7 +413,7 @@ end
 
 # Pullback of logsumexp (rrule at src/softmax.jl:205-212): dy and lse are device arrays with the size of the
 # reduced result (for dims = : a 0-dimensional or one-element array holding the cotangent / the result).
-function ∇logsumexp(dy::DeviceArray{T}, x::DeviceArray{T, N}, lse::DeviceArray{T}; dims = :) where {T <: MIFloat, N}
+function ∇logsumexp(dy::DeviceArray{T}, x::DeviceArray{T, N}, lse::DeviceArray{T}; dims = :) where {T <: MIFloat64, N}
     sizes, mask, ws, wsb = dims_call(x, dims)
     n_out = dims isa Colon ? 1 : prod(d -> d in dims ? 1 : size(x, d), 1:N; init = 1)
     length(dy) == length(lse) == n_out || throw(DimensionMismatch("dy and lse must have the size of logsumexp(x; dims)"))
@@ -412,7 +424,7 @@ function ∇logsumexp(dy::DeviceArray{T}, x::DeviceArray{T, N}, lse::DeviceArray
     dx
 end
 
-function softmax_grad!(op::Int32, dx::DeviceArray{T, N}, dy::DeviceArray{T, N}, y::DeviceArray{T, N}, dims) where {T <: MIFloat, N}
+function softmax_grad!(op::Int32, dx::DeviceArray{T, N}, dy::DeviceArray{T, N}, y::DeviceArray{T, N}, dims) where {T <: MIFloat64, N}
     size(dx) == size(dy) == size(y) || throw(DimensionMismatch("dx, dy and y must have one size"))
     sizes, mask, ws, wsb = dims_call(y, dims)
     GC.@preserve dx dy y sizes ws check(ccall((:mi_softmax_bwd_dims, libmi), Int32,

@@ -172,6 +172,13 @@ class DeviceArray:
         return _CODE[self.dtype]
 
     @property
+    def code_f64(self):
+        """Element type code for the entry points that also take Float64 (the softmax family, the attention forward)."""
+        if self.dtype == "f64":
+            return _lib.MI_F64
+        return self.code
+
+    @property
     def code_any(self):
         """Element type code for the batched_mul entry points (every numeric element type)."""
         if self.dtype not in _CODE_ANY:

@@ -109,7 +109,7 @@ def _fill_desc(d, q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, flags, fdrop=None):
     d.struct_size = ctypes.sizeof(_lib.mi_attn_desc)
     if fdrop is not None:
         d.dropout_p, d.dropout_seed = fdrop.p, fdrop.seed
-    d.dtype = d.weights_dtype = q.code
+    d.dtype = d.weights_dtype = q.code_f64
     d.flags = flags
     d.E, d.Ev, d.Lq, d.Lkv, d.H, d.B = E, Ev, Lq, Lkv, H, B
     d.q, d.k = q.ptr, k.ptr
@@ -148,7 +148,7 @@ def _attention_call(q, k, v, bias, mask, H, B, E, Ev, Lq, Lkv, want_out, want_we
     alpha = DeviceArray.empty((Lkv, Lq, H, B), wdt) if want_weights else None
     d.out = out.ptr if out is not None else None
     d.weights = alpha.ptr if alpha is not None else None
-    d.weights_dtype = alpha.code if alpha is not None else q.code
+    d.weights_dtype = alpha.code_f64 if alpha is not None else q.code_f64
     kernel, ws = ctypes.c_int32(0), ctypes.c_size_t(0)
     _lib.check(lib.mi_attention_plan(ctypes.byref(d), ctypes.byref(kernel), ctypes.byref(ws)))
     stats = None
@@ -304,6 +304,11 @@ def _weights_times_values(alpha, v, H, B, Ev, Lq, Lkv):
     out = DeviceArray.empty((Ev, Lq, B), v.dtype)
     es = v.itemsize
     for b in range(B):
+        if v.dtype == "f64":
+            _lib.check(lib.mi_batched_gemm_f64(b"N", b"N", Dv, Lq, Lkv, 1.0, v.ptr + es * b * Ev * Lkv, Ev, Dv,
+                                               alpha.ptr + es * b * Lkv * Lq * H, Lkv, Lkv * Lq, 0.0,
+                                               out.ptr + es * b * Ev * Lq, Ev, Dv, H, _stream()), DimensionMismatch)
+            continue
         _lib.check(lib.mi_batched_gemm(v.code, b"N", b"N", Dv, Lq, Lkv, 1.0,
                                        v.ptr + es * b * Ev * Lkv, Ev, Dv,
                                        alpha.ptr + es * b * Lkv * Lq * H, Lkv, Lkv * Lq, 0.0,
@@ -376,7 +381,7 @@ def _dims_call(x, dims):
     mask = sum(1 << (d - 1) for d in ds if d <= len(size))
     sizes = (ctypes.c_int64 * max(len(size), 1))(*size)
     nb = ctypes.c_size_t(0)
-    _lib.check(_lib.load().mi_softmax_dims_workspace(x.code, len(size), sizes, mask, ctypes.byref(nb)))
+    _lib.check(_lib.load().mi_softmax_dims_workspace(x.code_f64, len(size), sizes, mask, ctypes.byref(nb)))
     wbuf, wsize = _get_workspace(nb.value)
     return len(size), sizes, mask, (wbuf.data_ptr() if wbuf is not None else None), wsize, kept
 
@@ -394,24 +399,39 @@ def _number_error(name):
                          "be outside the layer.")
 
 
+def _float(x):
+    """``float.(x)``: integer arrays become Float64 (what ``similar(x, float(T))`` makes of them, src/softmax.jl:56);
+    floating-point arrays are returned as they are."""
+    if x.dtype not in ("i32", "i64"):
+        return x
+    x = _contig(x, "x")
+    out = DeviceArray.empty(x.dims, "f64")
+    _lib.check(_lib.load().mi_convert(out.ptr, _lib.MI_F64, x.ptr, x.code_any, x.length, _stream()))
+    return out
+
+
 def _softmax_like(name, op, out, x, dims):
     if not isinstance(x, DeviceArray) or not isinstance(out, DeviceArray):
         raise _number_error(name)
-    x, out = _contig(x, "x"), _contig(out, "out")
+    x, out = _contig(_float(x), "x"), _contig(out, "out")
     if out.dims != x.dims:
         raise DimensionMismatch(f"output size {out.dims} differs from input size {x.dims}")
     if x.dtype == "bool" or out.dtype != x.dtype:
-        raise ArgumentError(f"{name} needs floating-point input and output of one element type")
+        raise ArgumentError(f"{name} needs floating-point input and output of one element type (integer input: Float64 output)")
     nd, sizes, mask, ws, wsize, _ = _dims_call(x, dims)
-    _lib.check(_lib.load().mi_softmax_dims(op, x.code, x.ptr, out.ptr, nd, sizes, mask, ws, wsize, _stream()))
+    _lib.check(_lib.load().mi_softmax_dims(op, x.code_f64, x.ptr, out.ptr, nd, sizes, mask, ws, wsize, _stream()))
     return out
+
+
+def _float_dtype(x):
+    return "f64" if x.dtype in ("i32", "i64") else x.dtype
 
 
 def softmax(x, *, dims=1):
     """softmax(x; dims=1)  (src/softmax.jl:56).  ``dims=None`` is Julia's ``dims=:``."""
     if not isinstance(x, DeviceArray):
         raise _number_error("softmax")
-    return softmax_(DeviceArray.empty(x.dims, x.dtype), x, dims=dims)
+    return softmax_(DeviceArray.empty(x.dims, _float_dtype(x)), x, dims=dims)
 
 
 def softmax_(out, x=None, *, dims=1):
@@ -423,7 +443,7 @@ def logsoftmax(x, *, dims=1):
     """logsoftmax(x; dims=1)  (src/softmax.jl:133)."""
     if not isinstance(x, DeviceArray):
         raise _number_error("logsoftmax")
-    return logsoftmax_(DeviceArray.empty(x.dims, x.dtype), x, dims=dims)
+    return logsoftmax_(DeviceArray.empty(x.dims, _float_dtype(x)), x, dims=dims)
 
 
 def logsoftmax_(out, x=None, *, dims=1):
@@ -436,12 +456,12 @@ def logsumexp(x, *, dims=None):
     DeviceArray holding the scalar; otherwise the reduced dimensions are kept with extent 1."""
     if not isinstance(x, DeviceArray):
         raise _number_error("logsumexp")
-    x = _contig(x, "x")
+    x = _contig(_float(x), "x")
     if x.dtype == "bool":
         raise ArgumentError("logsumexp needs a floating-point array")
     nd, sizes, mask, ws, wsize, kept = _dims_call(x, dims)
     out = DeviceArray.empty(kept, x.dtype)
-    _lib.check(_lib.load().mi_logsumexp_dims(x.code, x.ptr, out.ptr, nd, sizes, mask, ws, wsize, _stream()))
+    _lib.check(_lib.load().mi_logsumexp_dims(x.code_f64, x.ptr, out.ptr, nd, sizes, mask, ws, wsize, _stream()))
     return out
 
 
@@ -459,7 +479,7 @@ def grad_logsumexp(dy, x, *, dims=None, lse=None):
     if dy.length != n_out or lse.length != n_out or not (dy.dtype == lse.dtype == x.dtype):
         raise DimensionMismatch(f"dy and lse must have the size {kept} of logsumexp(x; dims) and the element type of x")
     dx = DeviceArray.empty(x.dims, x.dtype)
-    _lib.check(_lib.load().mi_logsumexp_bwd_dims(x.code, dy.ptr, x.ptr, lse.ptr, dx.ptr, nd, sizes, mask, ws, wsize, _stream()))
+    _lib.check(_lib.load().mi_logsumexp_bwd_dims(x.code_f64, dy.ptr, x.ptr, lse.ptr, dx.ptr, nd, sizes, mask, ws, wsize, _stream()))
     return dx
 
 
@@ -470,7 +490,7 @@ def _softmax_grad(name, op, dx, dy, y, dims):
     if y.dtype == "bool" or not (dy.dtype == y.dtype == dx.dtype):
         raise ArgumentError(f"{name} needs one floating-point element type for dx, dy and y")
     nd, sizes, mask, ws, wsize, _ = _dims_call(y, dims)
-    _lib.check(_lib.load().mi_softmax_bwd_dims(op, y.code, dy.ptr, y.ptr, dx.ptr, nd, sizes, mask, ws, wsize, _stream()))
+    _lib.check(_lib.load().mi_softmax_bwd_dims(op, y.code_f64, dy.ptr, y.ptr, dx.ptr, nd, sizes, mask, ws, wsize, _stream()))
     return dx
 
 

@@ -397,3 +397,15 @@ def test_float32_products_through_bf16_planes_keep_float32_accuracy(nn, ta, tb):
     d2 = nn.DeviceArray.from_numpy(A2, "f32")
     C2 = nn.batched_mul(nn.batched_transpose(d2) if ta else d2, nn.batched_transpose(nn.DeviceArray.from_numpy(B2, "f32")) if tb else nn.DeviceArray.from_numpy(B2, "f32")).to_numpy()
     assert np.all(C2[7, :, 1] == np.inf) and np.isfinite(np.delete(C2[:, :, 1], 7, axis=0)).all() and np.isfinite(C2[:, :, 0]).all()
+    # a finite value above the largest bf16 (its rounding to bf16 overflows) still multiplies as itself
+    A3 = np.zeros_like(A)
+    big = np.float32(3.4e38)
+    if ta:
+        A3[3, 7, 0] = big
+    else:
+        A3[7, 3, 0] = big
+    B3 = np.full_like(B, np.float32(2.0 ** -20))
+    d3 = nn.DeviceArray.from_numpy(A3, "f32")
+    dB3 = nn.DeviceArray.from_numpy(B3, "f32")
+    C3 = nn.batched_mul(nn.batched_transpose(d3) if ta else d3, nn.batched_transpose(dB3) if tb else dB3).to_numpy()
+    assert np.allclose(C3[7, :, 0], np.float64(big) * 2.0 ** -20, rtol=1e-6) and np.all(np.delete(C3[:, :, 0], 7, axis=0) == 0)
