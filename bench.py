@@ -86,6 +86,19 @@ def algorithmic_work(w):
     return flops, nbytes
 
 
+def f32_products(roof, achieved_tflops, executed_per_counted=1.0):
+    """Float32 workloads keep `peak` = the published Float32 matrix peak, but by default their products are issued as six
+    bf16 matrix instructions on three bf16 planes per operand: the rate the issued instruction allows for Float32 products
+    is the bf16 peak / 6.  `executed_per_counted`: products the kernel executes per product the FLOP count holds."""
+    exact = os.environ.get("MI355ATTN_F32_MFMA", "")[:1] == "1"
+    roof["products"] = ("v_mfma_f32_32x32x2_f32" if exact else
+                        "six v_mfma_f32_32x32x16_bf16 on three bf16 planes per operand (Float32 accuracy)")
+    pk = PEAK["f32"] if exact else PEAK["bf16"] / 6.0
+    roof["products_peak"] = pk
+    roof["products_frac"] = achieved_tflops * executed_per_counted / pk
+    roof["products_executed_per_counted"] = executed_per_counted
+
+
 PREHEAT_S = 1.0     # seconds of the same launches before the counted warm-up (0 = none)
 
 
@@ -256,19 +269,22 @@ def measure(key, steps, warmup, with_cpu):
     flops, nbytes = algorithmic_work(w)
     tflops = flops / (ms * 1e-3) / 1e12
     gbps = nbytes / (ms * 1e-3) / 1e9
-    hbm_bound = key in HBM_BOUND
+    # C2 returns its weights: 512 MiB written put its HBM floor (84 us) above the matrix floor of its products on the
+    # bf16 planes (3 products executed for the 2 counted: 62 us), so HBM is the roofline that binds it
+    hbm_bound = key in HBM_BOUND or (key == "c2" and os.environ.get("MI355ATTN_F32_MFMA", "")[:1] != "1")
     traffic, source = measured_traffic(key)
     if hbm_bound:
         roof = dict(bound="hbm", achieved=gbps, peak=HBM_PEAK, unit="GB/s", frac=gbps / HBM_PEAK, traffic=traffic,
                     traffic_source=source)
+        if w["dtype"] == "f32":
+            roof["mfma"] = dict(achieved=tflops, peak=PEAK["f32"], unit="TFLOP/s", frac=tflops / PEAK["f32"])
+            f32_products(roof["mfma"], tflops, 1.5 if w["weights"] else 1.0)   # weights: QK^T runs in both passes
     else:
         pk = PEAK[w["dtype"]]
         roof = dict(bound="mfma", achieved=tflops, peak=pk, unit="TFLOP/s", frac=tflops / pk, traffic=traffic,
                     traffic_source=source, hbm_frac=gbps / HBM_PEAK)
         if w["dtype"] == "f32":
-            # Float32 in, out and accumulation; `peak` stays the Float32 matrix instruction's
-            roof["products"] = ("v_mfma_f32_32x32x2_f32" if os.environ.get("MI355ATTN_F32_MFMA", "")[:1] == "1" else
-                                "six v_mfma_f32_32x32x16_bf16 on three bf16 planes per operand (Float32 accuracy)")
+            f32_products(roof, tflops, 1.5 if w["weights"] else 1.0)
     res = dict(workload=w["name"], kernel=r.kernel, preheat_ms=r.preheat_ms, ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, gbps=gbps,
                flops_per_step=flops, bytes_per_step=nbytes, roofline=roof)
     if with_cpu:
@@ -355,9 +371,9 @@ def measure_extra(key, steps, warmup, with_cpu):
         line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype=dtn,
                     roofline=dict(bound="mfma", achieved=val, peak=PEAK[dtn], unit="TFLOP/s", frac=val / PEAK[dtn], traffic=None),
                     config=dict(workload=EXTRA[key], kernel=_lib.KERNEL_NAMES[kern.value]), flops_per_step=flops)
-        if dtn == "f32":   # Float32 in, out and accumulation; `peak` stays the Float32 matrix instruction's
-            line["roofline"]["products"] = ("v_mfma_f32_32x32x2_f32" if os.environ.get("MI355ATTN_F32_MFMA", "")[:1] == "1" else
-                                            "six v_mfma_f32_32x32x16_bf16 on three bf16 planes per operand (Float32 accuracy)")
+        line["roofline"]["products_executed_per_counted"] = 8 / 5   # dQ: S, dP, dQ; dV: S, dV; dK: S, dP, dK
+        if dtn == "f32":
+            f32_products(line["roofline"], val, 8 / 5)
         if with_cpu:
             from oracle import oracle as O
             rng = np.random.default_rng(0)
@@ -397,9 +413,10 @@ def measure_extra(key, steps, warmup, with_cpu):
                     roofline=dict(bound="mfma", achieved=val, peak=peak, unit="TFLOP/s", frac=val / peak, traffic=None),
                     config=dict(workload=EXTRA[key]),
                     flops_per_step=flops)
-        if dt_name == "f32":   # Float32 in, out and accumulation; `peak` stays the Float32 matrix instruction's
-            line["roofline"]["products"] = ("v_mfma_f32_32x32x2_f32" if os.environ.get("MI355ATTN_F32_MFMA", "")[:1] == "1" else
-                                            "six v_mfma_f32_32x32x16_bf16 on three bf16 planes per operand (Float32 accuracy)")
+        if dt_name == "f32":
+            f32_products(line["roofline"], val)
+        es_out = {"bf16": 2, "f32": 4, "c64": 8, "f64": 8}[dt_name]
+        line["roofline"]["hbm_frac"] = es_out * (m * kk + kk * n + m * n) * nb / (ms * 1e-3) / 1e9 / HBM_PEAK   # every operand once
         if with_cpu and dt_name not in ("c64", "f64"):
             from oracle import oracle as O
             ns = min(nb, 2 if key == "batched_mul" else 32)
@@ -515,9 +532,10 @@ def main():
         for key in ("c1", "c2", "c4", "c5"):
             ksteps = max(5, min(args.steps, 50))
             res = measure(key, ksteps, min(args.warmup, 10), not args.no_cpu)
-            hbm = key in HBM_BOUND
+            hbm = res["roofline"]["bound"] == "hbm"
             entry = {"metric": "attention GB/s" if hbm else "attention TFLOP/s", "value": res["gbps"] if hbm else res["tflops"],
-                     "unit": "GB/s" if hbm else "TFLOP/s", "ms_per_step": res["ms_per_step"], "steps": ksteps,
+                     "unit": "GB/s" if hbm else "TFLOP/s", "ms_per_step": res["ms_per_step"], "us_per_step": 1e3 * res["ms_per_step"],
+                     "tflops": res["tflops"], "gbps": res["gbps"], "steps": ksteps,
                      "dtype": WORKLOADS[key]["dtype"], "config": {"workload": res["workload"], "kernel": res["kernel"]},
                      "roofline": res["roofline"], "flops_per_step": res["flops_per_step"], "bytes_per_step": res["bytes_per_step"]}
             if "cpu_baseline" in res:
