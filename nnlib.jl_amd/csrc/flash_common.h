@@ -127,18 +127,6 @@ __device__ inline void flash_dma_1k(const i32x4_t &rsrc, unsigned lds_addr, int 
                  : "memory", "m0");
 }
 
-// The same for data that is read exactly once (bias and mask tiles): marked non-temporal, so that it does not push
-// the K / V tiles, which the query tiles of a (head, batch) pair share, out of L2.
-#ifndef FLASH_STREAM_POLICY
-#define FLASH_STREAM_POLICY "nt"
-#endif
-__device__ inline void flash_dma_1k_stream(const i32x4_t &rsrc, unsigned lds_addr, int voffset) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen " FLASH_STREAM_POLICY " lds"
-                 :
-                 : "s"(lds_addr), "v"(voffset), "s"(rsrc)
-                 : "memory", "m0");
-}
-
 __device__ inline i32x4_t flash_make_rsrc(const void *base, uint32_t bytes) {
     const uint64_t addr = (uint64_t)base;
     i32x4_t rs;
@@ -249,11 +237,11 @@ struct FlashStaged {
     __device__ void issue(int stage, int64_t j0) const {
         if (bias) {
 #pragma unroll
-            for (int i = 0; i < 4 * QB; i++) flash_dma_1k_stream(brs, blds + stage * BIAS_STAGE + i * 1024, bvoff[i] + (int)(2 * j0));
+            for (int i = 0; i < 4 * QB; i++) flash_dma_1k(brs, blds + stage * BIAS_STAGE + i * 1024, bvoff[i] + (int)(2 * j0));
         }
         if (mask) {
 #pragma unroll
-            for (int i = 0; i < 2 * QB; i++) flash_dma_1k_stream(mrs, mlds + stage * MASK_STAGE + i * 1024, mvoff[i] + (int)j0);
+            for (int i = 0; i < 2 * QB; i++) flash_dma_1k(mrs, mlds + stage * MASK_STAGE + i * 1024, mvoff[i] + (int)j0);
         }
     }
     // all copies issued so far have landed
