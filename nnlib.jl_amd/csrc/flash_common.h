@@ -363,6 +363,12 @@ __device__ inline uint32_t flash_mask_bits(uint32_t m4) { return ((m4 & 0x7F7F7F
 // whose scores come straight from the MFMAs therefore pass `after`, a scalar they obtained with flash_mfma_fence from
 // the same accumulator block: the fence is an instruction the compiler does protect, and the operand orders the
 // select behind it.
+// Contract: `v` must have been written by a builtin matrix instruction (which the compiler's hazard recogniser knows),
+// not by one issued from inline assembly (T::mfma32_keep_c), and the selects must follow the fence in program order:
+// the recogniser puts the wait states in front of the fence's own read of v[0], by which time the instruction has
+// written all sixteen registers, and the in-order issue keeps the selects behind it.  Every caller (the EXTRAS_MASKTILE
+// and EXTRAS_KEYMASK branches of flash_softmax_tile, reached from flash16_kernel and the gradient kernels) passes the
+// accumulators of T::mfma32 / __builtin_amdgcn_mfma_* calls.
 __device__ inline int flash_mfma_fence(const floatx16_t &v) { return __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v[0])); }
 __device__ inline float flash_mask_apply(float s, uint32_t bits, int e, int after) {
     const int keep = __builtin_amdgcn_sbfe((int)bits, 8 * e + 7, 1);   // 0 or -1

@@ -72,9 +72,12 @@ def _both(nn, dtype, E, Lq, Lkv, B, H, seed, *, weights=False, key_mask=False, b
         if static:
             d.workspace, d.workspace_bytes = None, 0            # ignored by the static entry point
             torch.cuda.synchronize()
-            before = torch.cuda.memory_allocated()
+            before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
             L.check(lib.mi_attention_fwd_static(ctypes.byref(d), stream))
+            torch.cuda.synchronize()
+            # neither through torch's allocator nor behind it: the driver's count of free device memory is unchanged
             assert torch.cuda.memory_allocated() == before
+            assert torch.cuda.mem_get_info()[0] == free_before
         else:
             buf = torch.empty(max(ws.value, 1), dtype=torch.uint8, device="cuda")
             d.workspace, d.workspace_bytes = buf.data_ptr(), buf.numel()
@@ -178,3 +181,37 @@ def test_call_beyond_the_builtin_workspace_is_refused(nn):
     assert "built-in" in L.last_error()
     torch.cuda.synchronize()
     assert bool((out == 7.0).all())               # nothing was launched
+
+
+def test_static_call_inside_a_captured_graph(nn):
+    """Stream capture refuses allocation and synchronisation: the static entry point must record cleanly, and every
+    replay must reproduce the eager result bit for bit (replayed several times with eager work and synchronisations
+    in between).  Split-kv call: partial results go through the built-in workspace and a merge kernel."""
+    L = nn._lib
+    lib = L.load()
+    dtype, E, Lq, Lkv, B, H = "f16", 512, 128, 4096, 2, 8
+    t = TORCH[dtype]
+    g = torch.Generator(device="cuda").manual_seed(21)
+    q = torch.randn(E * Lq * B, device="cuda", generator=g).to(t)
+    k = torch.randn(E * Lkv * B, device="cuda", generator=g).to(t)
+    v = torch.randn(E * Lkv * B, device="cuda", generator=g).to(t)
+    eager = torch.empty(E * Lq * B, device="cuda", dtype=t)
+    d = _desc(L, dtype, E, Lq, Lkv, B, H, q, k, v, eager)
+    kern, ws = ctypes.c_int32(-1), ctypes.c_size_t(0)
+    L.check(lib.mi_attention_plan(ctypes.byref(d), ctypes.byref(kern), ctypes.byref(ws)))
+    assert ws.value > 0                       # the call does use scratch memory
+    L.check(lib.mi_attention_fwd_static(ctypes.byref(d), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    out = torch.zeros_like(eager)
+    dg = _desc(L, dtype, E, Lq, Lkv, B, H, q, k, v, out)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        L.check(lib.mi_attention_fwd_static(ctypes.byref(dg), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    for rep in range(3):
+        out.fill_(float("nan"))
+        other = (q.float() * (rep + 1)).sum()     # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.isfinite(other)
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), rep
