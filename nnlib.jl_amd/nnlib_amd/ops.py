@@ -621,8 +621,20 @@ def _batched_mul_generic(C, A, B, alpha, beta):
     if C.conj:
         raise ArgumentError("batched_mul! cannot write into a batched_adjoint")
     want = promote_type(A.dtype, B.dtype)
-    if promote_type(want, C.dtype) != C.dtype or C.dtype in ("f16", "bf16"):
+    if promote_type(want, C.dtype) != C.dtype:
         raise ArgumentError(f"batched_mul!: cannot store the product of {A.dtype} and {B.dtype} arrays into a {C.dtype} array")
+    if C.dtype in ("f16", "bf16"):
+        # Float16 / BFloat16 times an integer array promotes to the 16-bit type (Julia's promote_type); the generic kernel
+        # has no 16-bit accumulator type, so the product is formed in Float32 and rounded once into C
+        if not C.is_contiguous():
+            raise ArgumentError("batched_mul!: a 16-bit result of mixed element types must be a dense array")
+        lib = _lib.load()
+        tmp = DeviceArray.empty(C.dims, "f32")
+        if beta != 0:
+            _lib.check(lib.mi_convert(tmp.ptr, _lib.MI_F32, C.ptr, C.code, C.length, _stream()))
+        _batched_mul_generic(tmp, A, B, alpha, beta)
+        _lib.check(lib.mi_convert(C.ptr, C.code, tmp.ptr, _lib.MI_F32, C.length, _stream()))
+        return C
     nb = C.dims[2]
     if A.dims[2] not in (nb, 1):
         raise DimensionMismatch("batch size mismatch: A != C")            # src/batched/batchedmul.jl:307-308

@@ -231,3 +231,24 @@ def test_float64_matches_float32_path_semantics(nn):
     r32 = nn.batched_mul(D(nn, A, "f32"), D(nn, B, "f32")).to_numpy()
     e64, e32 = np.abs(r64 - ref).max(), np.abs(r32 - ref).max()
     assert e64 < 1e-11 and e32 > 1e-7 and e64 < 1e-4 * e32
+
+
+@pytest.mark.parametrize("T16", ["f16", "bf16"])
+@pytest.mark.parametrize("TI", ["i32", "i64"])
+def test_sixteen_bit_times_integer(nn, T16, TI):
+    """promote_type(Float16 | BFloat16, Int) is the 16-bit type, and the reference's batched_mul_generic!
+    (src/batched/batchedmul.jl:306-325) returns such an array.  No reference fixture pins the values (parity
+    unpinned); here the product is formed in Float32 and rounded once, checked against the Float64 product of the
+    same (rounded) operands to one unit of the 16-bit type."""
+    from conftest import round_to
+    rng = np.random.default_rng(7)
+    A = round_to(rng.standard_normal((6, 5, 3)), T16)
+    iB = rng.integers(-4, 5, (5, 7, 3))
+    dA = nn.DeviceArray.from_numpy(A.astype(np.float32), T16)
+    r = nn.batched_mul(dA, D(nn, iB, TI))
+    assert r.dtype == T16 and r.dims == (6, 7, 3)
+    ref = per_slice(A, iB)
+    unit = 2.0 ** (-10 if T16 == "f16" else -7)
+    assert np.abs(r.to_numpy() - ref).max() <= unit * np.abs(ref).max()
+    r2 = nn.batched_mul(D(nn, iB.transpose(1, 0, 2), TI), nn.batched_transpose(dA))      # integer on the left
+    assert r2.dtype == T16 and np.abs(r2.to_numpy() - per_slice(iB.transpose(1, 0, 2), A.transpose(1, 0, 2))).max() <= unit * np.abs(ref).max()
