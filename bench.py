@@ -30,22 +30,32 @@ HBM_BOUND = ("c4", "c5")                                # workloads priced again
 MIB = 1 << 20
 TRAFFIC_FILE = os.path.join("profiles", "hbm_traffic_fetch_write_size.md")
 DOMINANT_KERNEL = {"c1": "flash32_kernel", "c2": "flash32_kernel", "c3": "flash16_fast_kernel", "c4": "flash16_kernel",
-                   "c5": "decode_split_kernel"}
+                   "c5": "decode_split_kernel",
+                   # a gradient step is three kernels (dq, dk, dv): every row of the workload whose name contains "bwd"
+                   "bwd": "bwd", "bwd_f32": "bwd", "softmax": "softmax", "logsoftmax": "softmax", "softmax_dims2": "softmax",
+                   "batched_mul": "gemm", "batched_mul_f32": "gemm"}
 
 
 def measured_traffic(key):
-    """(bytes per launch, source) of the workload's dominant kernel from the tracked rocprofv3 summary: the row of
-    its table whose first column is the workload and whose kernel name contains DOMINANT_KERNEL[key]; read MiB +
-    written MiB.  (None, None) when the file has no such row."""
+    """(bytes per step, source) of the workload's kernels from the tracked rocprofv3 summary: the rows of its table
+    whose first column is the workload and whose kernel name contains DOMINANT_KERNEL[key], read MiB + written MiB,
+    summed over those rows (one row for a one-kernel step; the gradient's three).  (None, None) when the file has no
+    such row."""
+    total = None
     try:
         with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
             for line in f:
                 cells = [c.strip() for c in line.strip().strip("|").split("|")]
                 if len(cells) >= 6 and cells[0] == key and DOMINANT_KERNEL.get(key, "\0") in cells[1]:
-                    return (float(cells[4]) + float(cells[5])) * MIB, TRAFFIC_FILE
+                    total = (total or 0.0) + (float(cells[4]) + float(cells[5])) * MIB
     except (OSError, ValueError):
-        pass
-    return None, None
+        return None, None
+    return (total, TRAFFIC_FILE) if total is not None else (None, None)
+
+
+def measured_traffic_fields(key):
+    traffic, source = measured_traffic(key)
+    return dict(traffic=traffic, traffic_source=source)
 
 
 ROTATE_BYTES = 1 << 30                                  # input sets rotated until they cover 4x the last-level cache
@@ -369,7 +379,7 @@ def measure_extra(key, steps, warmup, with_cpu):
         flops = 10 * D * H * B * (L * (L + 1) // 2)
         val = flops / (ms * 1e-3) / 1e12
         line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype=dtn,
-                    roofline=dict(bound="mfma", achieved=val, peak=PEAK[dtn], unit="TFLOP/s", frac=val / PEAK[dtn], traffic=None),
+                    roofline=dict(bound="mfma", achieved=val, peak=PEAK[dtn], unit="TFLOP/s", frac=val / PEAK[dtn], **measured_traffic_fields(key)),
                     config=dict(workload=EXTRA[key], kernel=_lib.KERNEL_NAMES[kern.value]), flops_per_step=flops)
         line["roofline"]["products_executed_per_counted"] = 8 / 5   # dQ: S, dP, dQ; dV: S, dV; dK: S, dP, dK
         if dtn == "f32":
@@ -410,7 +420,7 @@ def measure_extra(key, steps, warmup, with_cpu):
         val = flops / (ms * 1e-3) / 1e12
         peak = PEAK["f32"] if dt_name == "c64" else PEAK[dt_name]
         line = dict(metric="batched_mul TFLOP/s", value=val, unit="TFLOP/s", dtype=dt_name,
-                    roofline=dict(bound="mfma", achieved=val, peak=peak, unit="TFLOP/s", frac=val / peak, traffic=None),
+                    roofline=dict(bound="mfma", achieved=val, peak=peak, unit="TFLOP/s", frac=val / peak, **measured_traffic_fields(key)),
                     config=dict(workload=EXTRA[key]),
                     flops_per_step=flops)
         if dt_name == "f32":
@@ -450,7 +460,7 @@ def measure_extra(key, steps, warmup, with_cpu):
         nbytes = 2 * xs[0].length * xs[0].itemsize       # one read, one write
         val = nbytes / (ms * 1e-3) / 1e9
         line = dict(metric=f"{key} GB/s", value=val, unit="GB/s", dtype=dt_name,
-                    roofline=dict(bound="hbm", achieved=val, peak=HBM_PEAK, unit="GB/s", frac=val / HBM_PEAK, traffic=None),
+                    roofline=dict(bound="hbm", achieved=val, peak=HBM_PEAK, unit="GB/s", frac=val / HBM_PEAK, **measured_traffic_fields(key)),
                     config=dict(workload=EXTRA[key]),
                     bytes_per_step=nbytes)
         if with_cpu:
