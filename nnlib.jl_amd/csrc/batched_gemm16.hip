@@ -150,13 +150,15 @@ __global__ __launch_bounds__(Shape<LARGE>::THREADS, LARGE ? 1 : 2) void gemm16_k
     constexpr int TILEB = S::TILEB, BM = S::BM, BNB = S::BNB;
     extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
     char *As = (char *)gemm_smem, *Bs = As + 2 * TILEB;
-    const int64_t bz = blockIdx.z;
+    // which tile: an order in which the tiles in flight on one die share operands (mi_gemm_tile_order)
+    const MiTile tile = mi_gemm_tile_order(blockIdx.x + (int64_t)gridDim.x * (blockIdx.y + (int64_t)gridDim.y * blockIdx.z), gridDim.x, gridDim.y, gridDim.z);
+    const int64_t bx = tile.m, by = tile.n, bz = tile.batch;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave % S::WM, wn = wave / S::WM;
     const int r = lane & 31, hh = lane >> 5;
 
     Operand<T, A_RM, LARGE> a;
     Operand<T, B_RM, LARGE> b;
-    const int64_t m0 = (int64_t)blockIdx.x * S::TILE, n0 = (int64_t)blockIdx.y * S::TILE;
+    const int64_t m0 = bx * S::TILE, n0 = by * S::TILE;
     a.init((const t *)g.A + bz * g.sA, g.lda, g.m, g.k, m0);
     b.init((const t *)g.B + bz * g.sB, g.ldb, g.n, g.k, n0);
 

@@ -250,7 +250,11 @@ __global__ __launch_bounds__(ShapeS<LARGE>::THREADS, LARGE ? 1 : 2) void gemm32s
     constexpr int TILE3B = S::TILE3B, BM = S::BM, BNB = S::BNB;
     extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];   // A and B tiles, two buffers each
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)gemm_smem;
-    const int64_t bz = blockIdx.z;
+    // which tile: with the large tiles, an order in which the tiles in flight on one die share operands (a few per cent
+    // on k >= 1024; the small tiles' calls are bound by their output and lose 1 % to it)
+    const int64_t id = blockIdx.x + (int64_t)gridDim.x * (blockIdx.y + (int64_t)gridDim.y * blockIdx.z);
+    const MiTile tile = LARGE ? mi_gemm_tile_order(id, gridDim.x, gridDim.y, gridDim.z) : MiTile{blockIdx.x, blockIdx.y, blockIdx.z};
+    const int64_t bz = tile.batch;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave & 1, wn = wave >> 1;
     const int r = lane & 31, hh = lane >> 5;
 
@@ -260,12 +264,12 @@ __global__ __launch_bounds__(ShapeS<LARGE>::THREADS, LARGE ? 1 : 2) void gemm32s
     a.ld = g.lda;
     a.rows = g.m;
     a.k = g.k;
-    a.row0 = (int64_t)blockIdx.x * S::TILE;
+    a.row0 = tile.m * S::TILE;
     b.X = g.B + bz * g.sB;
     b.ld = g.ldb;
     b.rows = g.n;
     b.k = g.k;
-    b.row0 = (int64_t)blockIdx.y * S::TILE;
+    b.row0 = tile.n * S::TILE;
 
     floatx16_t acc[BNB][BM];   // [n block][m block]
 #pragma unroll

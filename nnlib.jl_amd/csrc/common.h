@@ -165,6 +165,33 @@ __device__ static inline void split3_pair_guarded(float x0, float x1, uint32_t &
     lo = __builtin_bit_cast(uint32_t, l);
 }
 
+// Workgroup order for kernels whose neighbouring workgroups share operands.  The hardware hands workgroup `id` of a
+// launch to XCD `id % 8` (eight dies, each with its own L2), so neighbours in launch order never share an L2.
+// mi_xcd_order turns the launch id into the id of the work item to take such that every die works through one
+// contiguous run of the natural order: die c takes items c*ceil(n/8) ... in the order its workgroups start.  A
+// bijection on [0, total) for any total.
+constexpr int MI_XCDS = 8;
+__device__ static inline int64_t mi_xcd_order(int64_t id, int64_t total) {
+    const int64_t chunk = total / MI_XCDS, rem = total % MI_XCDS;
+    const int64_t xcd = id % MI_XCDS, slot = id / MI_XCDS;
+    return xcd * chunk + (xcd < rem ? xcd : rem) + slot;
+}
+
+// Tile of a batched matrix product for workgroup `id` of tiles_m x tiles_n x batches: dies take contiguous runs of
+// (tile, batch) items (mi_xcd_order); within a matrix the tiles run in bands of 8 tile rows, n-major inside a band, so
+// that the 32 or so tiles a die has in flight form a block of about 8 x 4 tiles that share their A row tiles and B
+// column tiles through that die's L2, whatever the matrix's own tile counts.
+struct MiTile { int64_t m, n, batch; };
+__device__ static inline MiTile mi_gemm_tile_order(int64_t id, int64_t tiles_m, int64_t tiles_n, int64_t batches) {
+    constexpr int64_t GROUP_M = 8;
+    const int64_t item = mi_xcd_order(id, tiles_m * tiles_n * batches);
+    const int64_t pid = item % (tiles_m * tiles_n);
+    const int64_t band = pid / (GROUP_M * tiles_n), in_band = pid % (GROUP_M * tiles_n);
+    const int64_t band_rows = tiles_m - band * GROUP_M < GROUP_M ? tiles_m - band * GROUP_M : GROUP_M;
+    return {band * GROUP_M + in_band % band_rows, in_band / band_rows, item / (tiles_m * tiles_n)};
+}
+
+
 // The same for callers that also keep finite values whose bf16 rounding overflows (|x| above the largest bf16,
 // 3.3895e38): split3_pair makes (Inf, -Inf, NaN) of those.  mi_plane_word_special tells whether either half of a hi-plane
 // word has an all-ones exponent (Inf, NaN or such an overflow); split3_pair_wide redoes a pair with the first plane

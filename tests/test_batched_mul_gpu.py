@@ -221,6 +221,20 @@ def test_large_tile_kernel(nn, dtype, ta, tb):
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("m,n,k,nb", [(2310, 600, 136, 5), (1160, 200, 72, 3), (300, 2100, 40, 7)])
+def test_tile_order_covers_every_tile(nn, dtype, m, n, k, nb):
+    """The tiled kernels hand their tiles to the workgroups in a permuted order (runs per die, bands of eight tile
+    rows): tile counts that are not multiples of eight in m, in total, or both, so that a tile the permutation
+    skipped or visited twice shows as a wrong block of the product."""
+    rng = np.random.default_rng(m + n + nb)
+    A = round_to(rng.standard_normal((m, k, nb)), dtype)
+    B = round_to(rng.standard_normal((k, n, nb)), dtype)
+    dC = nn.DeviceArray.from_numpy(np.full((m, n, nb), np.nan), dtype)
+    nn.batched_mul_(dC, nn.DeviceArray.from_numpy(A, dtype), nn.DeviceArray.from_numpy(B, dtype))
+    assert close(dC.to_numpy(), bmm(A, B, False, False), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
 def test_tiled_kernel_alpha_beta_and_shared_operand(nn, dtype):
     """test/ext_amdgpu/batched_mul.jl:15-19 (C .= pi; batched_mul!(C, A, B, 2, 3)) and the batch-1 operand of
     test/batchedmul.jl:104-106 at a size the tiled kernel takes."""
