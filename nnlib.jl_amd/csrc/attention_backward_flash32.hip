@@ -231,14 +231,15 @@ __global__ __launch_bounds__(256, (D == 64 && EXTRAS == EXTRAS_NONE) ? 2 : 1) vo
                     if (CAUSAL && j0 + 32 * kb > iw + 31) break;   // every key of this block is after every query of the wavefront
                     floatx16_t sb = first_product<D>(kt, kb, qx, (floatx16_t){0}, r, hh);
                     const floatx16_t dpb = first_product<D>(vt, kb, dox, (floatx16_t){0}, r, hh);
-                    int64_t lim = BN;
+                    int lim = BN;   // keys of the tile this lane's query keeps, counted from the lane's first key of a group of four
                     if (edge) {
-                        lim = kv_len - j0;
-                        if (CAUSAL && qi - j0 + 1 < lim) lim = qi - j0 + 1;
+                        int64_t lim64 = kv_len - j0;
+                        if (CAUSAL && qi - j0 + 1 < lim64) lim64 = qi - j0 + 1;
+                        lim = (lim64 > BN ? BN : (lim64 < 0 ? 0 : (int)lim64)) - 4 * hh;
                     }
 #pragma unroll
                     for (int v = 0; v < 16; v++) {
-                        const int kvl = 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4);
+                        const int kvl = 32 * kb + 8 * (v / 4) + (v % 4);
                         const float pw = (!edge || kvl < lim) ? mi_exp2(fmaf(sb[v], cs, -m2)) * linv : 0.0f;
                         sb[v] = pw * (dpb[v] - delta);
                     }
@@ -798,14 +799,15 @@ __global__ __launch_bounds__(64 * NW, 1) void bwd32s_dq_kernel(FlashArgs a, Attn
                 if constexpr (X_LDS) dpb = first_product_sl<D, XPLANEB>(Vs, kb, xrow, xsw, (floatx16_t){0}, r, hh);
                 else dpb = first_product_s<D>(Vs, kb, dox, (floatx16_t){0}, r, hh);
                 SCHED_FENCE();
-                int64_t lim = BN;
+                int lim = BN;   // keys of the tile this lane's query keeps, counted from the lane's first key of a group of four
                 if (edge) {
-                    lim = kv_len - j0;
-                    if (CAUSAL && qi - j0 + 1 < lim) lim = qi - j0 + 1;
+                    int64_t lim64 = kv_len - j0;
+                    if (CAUSAL && qi - j0 + 1 < lim64) lim64 = qi - j0 + 1;
+                    lim = (lim64 > BN ? BN : (lim64 < 0 ? 0 : (int)lim64)) - 4 * hh;
                 }
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
-                    const int kvl = 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4);
+                    const int kvl = 32 * kb + 8 * (v / 4) + (v % 4);
                     const float pw = (!edge || kvl < lim) ? mi_exp2(fmaf(sb[v], cs, -m2)) * linv : 0.0f;
                     sb[v] = pw * (dpb[v] - delta);
                 }
