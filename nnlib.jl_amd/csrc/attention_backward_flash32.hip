@@ -36,8 +36,7 @@ struct Cfg {
 };
 
 __device__ inline floatx4_t ldg16f(const float *p, bool ok) {
-    const floatx4_t z = {0.f, 0.f, 0.f, 0.f};
-    return ok ? *(const floatx4_t *)p : z;
+    return mi_load16_or_zero<floatx4_t>(p, ok);
 }
 
 // Streams [BN][D] tiles of up to two row-major arrays through registers into double-buffered LDS tiles;
@@ -100,12 +99,13 @@ __device__ inline void second_product(const float *tile, int kb, const floatx16_
 // stationary row in the permuted feature order of first_product
 template <int D>
 __device__ inline void load_stationary(float (&x)[D / 2], const float *row, bool ok, int hh, int dh) {
+    floatx4_t q4[D / 8];   // every load of the row is issued before the first is used
 #pragma unroll
-    for (int c = 0; c < D / 8; c++) {
-        const floatx4_t q4 = ldg16f(row + 8 * c + 4 * hh, ok && 8 * c + 4 * hh < dh);
+    for (int c = 0; c < D / 8; c++) q4[c] = ldg16f(row + 8 * c + 4 * hh, ok && 8 * c + 4 * hh < dh);
 #pragma unroll
-        for (int j = 0; j < 4; j++) x[4 * c + j] = q4[j];
-    }
+    for (int c = 0; c < D / 8; c++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) x[4 * c + j] = q4[c][j];
 }
 
 __device__ inline int64_t lq_pad(int64_t Lq) { return attention_stats_lq_pad(Lq); }
@@ -634,13 +634,21 @@ __device__ inline void second_product_s(unsigned tile, int kb, const floatx16_t 
 // stationary row as planes: the lane's features of k-step t are 16t + 8hh .. + 7 (the B-operand layout of the 16-bit instruction)
 template <int D>
 __device__ inline void load_stationary_s(plane8 (&x)[3][D / 16], const float *row, bool ok, int hh, int dh) {
+    floatx4_t raw[D / 16][2];   // every load of the row is issued before the first is used: one memory round trip
+#pragma unroll
+    for (int t = 0; t < D / 16; t++)
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int d0 = 16 * t + 8 * hh + 4 * half;
+            raw[t][half] = ldg16f(row + d0, ok && d0 < dh);
+        }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < D / 16; t++) {
         uint32_t xw[3][4];
 #pragma unroll
         for (int half = 0; half < 2; half++) {
-            const int d0 = 16 * t + 8 * hh + 4 * half;
-            const floatx4_t q4 = ldg16f(row + d0, ok && d0 < dh);
+            const floatx4_t q4 = raw[t][half];
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 uint32_t w[3];
@@ -702,14 +710,17 @@ __global__ __launch_bounds__(64 * NW, 1) void bwd32s_dq_kernel(FlashArgs a, Attn
             load_stationary_s<D>(dox, (const float *)bp.dout + off, qok, hh, (int)p.D);
         }
         load_stationary_s<D>(qx, (const float *)p.q + off, qok, hh, (int)p.D);
+        floatx4_t o4[D / 8], d4[D / 8];   // all loads first
 #pragma unroll
         for (int c = 0; c < D / 8; c++) {
             const bool ok = qok && 8 * c + 4 * hh < p.D;
-            const floatx4_t o4 = ldg16f((const float *)p.out + off + 8 * c + 4 * hh, ok);
-            const floatx4_t d4 = ldg16f((const float *)bp.dout + off + 8 * c + 4 * hh, ok);
-#pragma unroll
-            for (int j = 0; j < 4; j++) delta = fmaf(o4[j], d4[j], delta);
+            o4[c] = ldg16f((const float *)p.out + off + 8 * c + 4 * hh, ok);
+            d4[c] = ldg16f((const float *)bp.dout + off + 8 * c + 4 * hh, ok);
         }
+#pragma unroll
+        for (int c = 0; c < D / 8; c++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) delta = fmaf(o4[c][j], d4[c][j], delta);
         delta += mi_swap32(delta);
     }
 

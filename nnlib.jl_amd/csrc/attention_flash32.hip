@@ -37,8 +37,7 @@ struct Cfg {
 };
 
 __device__ inline floatx4_t ldg16f(const float *p, bool ok) {
-    floatx4_t z = {0.f, 0.f, 0.f, 0.f};
-    return ok ? *(const floatx4_t *)p : z;
+    return mi_load16_or_zero<floatx4_t>(p, ok);
 }
 
 template <int D, int QB, bool CAUSAL, bool EXTRAS, int PHASE>
@@ -188,6 +187,78 @@ __device__ inline floatx16_t mfma_split(const plane8 (&a)[3], const plane8 (&b)[
     return mfma_bf16(a[0], b[0], c);
 }
 
+// S^T = K Q^T of one 64-key tile whose planes sit at LDS address Ks: s[query block][key block]
+template <int D, int QB>
+__device__ inline void scores32s(const Frag32S<D, QB> &f, unsigned Ks, floatx16_t (&s)[QB][2]) {
+    typedef CfgS<D> C;
+    constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB;
+    typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
+    const int lane = threadIdx.x & 63, r = lane & 31, hh = lane >> 5;
+#pragma unroll
+    for (int qb = 0; qb < QB; qb++)
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) s[qb][kb] = (floatx16_t){0};
+    // lane's K operand: row r (+32 per key block), chunk 2t + hh, in each plane
+    const unsigned kt = Ks + (unsigned)r * ROWB;
+    const int ksw = C::swz(r);
+#pragma unroll
+    for (int t = 0; t < D / 16; t++)
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            plane8 ka[3];
+#pragma unroll
+            for (int q = 0; q < 3; q++)
+                ka[q] = *(lds_plane8_t)(uintptr_t)(kt + q * PLANEB + kb * 32 * ROWB + (((2 * t + hh) ^ ksw) << 4));
+#pragma unroll
+            for (int qb = 0; qb < QB; qb++) {
+                const plane8 qq[3] = {f.q[qb][0][t], f.q[qb][1][t], f.q[qb][2][t]};
+                s[qb][kb] = mfma_split(ka, qq, s[qb][kb]);
+            }
+        }
+}
+
+// O^T += V^T P^T for one 64-key tile: the weights in s (accumulator layout), V's planes at LDS address Vs
+template <int D, int QB>
+__device__ inline void weights_times_values32s(Frag32S<D, QB> &f, unsigned Vs, const floatx16_t (&s)[QB][2]) {
+    typedef CfgS<D> C;
+    constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB;
+    const int lane = threadIdx.x & 63, hh = lane >> 5;
+    // P^T operand of k-step u of key block kb: accumulator registers 8u .. 8u+7 (keys 0-3, 8-11 | 4-7, 12-15
+    // of the 16); V^T comes from the row-major planes with the transposing read in that same key order
+    const int vrow = 4 * hh + ((lane & 15) >> 2);
+    const int vchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), vsub = 8 * (lane & 1);
+    const unsigned vt = Vs + (unsigned)vrow * ROWB + vsub;
+    const int vsw_lo = C::swz(vrow), vsw_hi = C::swz(vrow + 8);
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            plane8 pk[QB][3];
+#pragma unroll
+            for (int qb = 0; qb < QB; qb++) {
+                uint32_t w[3][4];
+#pragma unroll
+                for (int e = 0; e < 4; e++)   // a NaN weight (fully masked column) stays NaN in the hi plane
+                    split3_pair(s[qb][kb][8 * u + 2 * e], s[qb][kb][8 * u + 2 * e + 1], w[0][e], w[1][e], w[2][e]);
+#pragma unroll
+                for (int q = 0; q < 3; q++) pk[qb][q] = __builtin_bit_cast(plane8, (u32x4_t){w[q][0], w[q][1], w[q][2], w[q][3]});
+            }
+#pragma unroll
+            for (int dvb = 0; dvb < D / 32; dvb++) {
+                const unsigned src = vt + (32 * kb + 16 * u) * ROWB;
+                plane8 va[3];
+#pragma unroll
+                for (int q = 0; q < 3; q++) {
+                    const plane4 lo = lds_tr4s(src + q * PLANEB + (((4 * dvb + vchunk) ^ vsw_lo) << 4));
+                    const plane4 hi = lds_tr4s(src + q * PLANEB + 8 * ROWB + (((4 * dvb + vchunk) ^ vsw_hi) << 4));
+                    va[q] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+#pragma unroll
+                for (int qb = 0; qb < QB; qb++) f.o[qb][dvb] = mfma_split(va, pk[qb], f.o[qb][dvb]);
+            }
+        }
+}
+
 template <int D, int QB, bool CAUSAL, bool EXTRAS, int PHASE>
 __device__ inline void run_tiles32s(const FlashArgs &a, Frag32S<D, QB> &f, unsigned Ks, unsigned Vs, int64_t kv_len, int64_t b, int64_t h,
                                     int64_t iw, int n_tiles, unsigned wlds = 0, int jt0 = 0) {
@@ -252,67 +323,12 @@ __device__ inline void run_tiles32s(const FlashArgs &a, Frag32S<D, QB> &f, unsig
         const bool active = !CAUSAL || j0 <= iw + 32 * QB - 1;
         if (active) {
             floatx16_t s[QB][2];
-#pragma unroll
-            for (int qb = 0; qb < QB; qb++)
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++) s[qb][kb] = (floatx16_t){0};
-            // lane's K operand: row r (+32 per key block), chunk 2t + hh, in each plane
-            const unsigned kt = Ks + (unsigned)r * ROWB;
-            const int ksw = C::swz(r);
-#pragma unroll
-            for (int t = 0; t < D / 16; t++)
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++) {
-                    plane8 ka[3];
-#pragma unroll
-                    for (int q = 0; q < 3; q++)
-                        ka[q] = *(lds_plane8_t)(uintptr_t)(kt + q * PLANEB + kb * 32 * ROWB + (((2 * t + hh) ^ ksw) << 4));
-#pragma unroll
-                    for (int qb = 0; qb < QB; qb++) {
-                        const plane8 qq[3] = {f.q[qb][0][t], f.q[qb][1][t], f.q[qb][2][t]};
-                        s[qb][kb] = mfma_split(ka, qq, s[qb][kb]);
-                    }
-                }
+            scores32s<D, QB>(f, Ks, s);
 
             flash_softmax_tile<T, QB, D / 32, CAUSAL, EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE, PHASE, float>(a, s, f.o, f.m, f.l, b, h, iw, j0,
                                                                                                           FlashStaged<QB>(), 0, wlds, nullptr, kv_len);
 
-            if (do_pv) {
-                // P^T operand of k-step u of key block kb: accumulator registers 8u .. 8u+7 (keys 0-3, 8-11 | 4-7, 12-15
-                // of the 16); V^T comes from the row-major planes with the transposing read in that same key order
-                const int vrow = 4 * hh + ((lane & 15) >> 2);
-                const int vchunk = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), vsub = 8 * (lane & 1);
-                const unsigned vt = Vs + (unsigned)vrow * ROWB + vsub;
-                const int vsw_lo = C::swz(vrow), vsw_hi = C::swz(vrow + 8);
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                    for (int u = 0; u < 2; u++) {
-                        plane8 pk[QB][3];
-#pragma unroll
-                        for (int qb = 0; qb < QB; qb++) {
-                            uint32_t w[3][4];
-#pragma unroll
-                            for (int e = 0; e < 4; e++)   // a NaN weight (fully masked column) stays NaN in the hi plane
-                                split3_pair(s[qb][kb][8 * u + 2 * e], s[qb][kb][8 * u + 2 * e + 1], w[0][e], w[1][e], w[2][e]);
-#pragma unroll
-                            for (int q = 0; q < 3; q++) pk[qb][q] = __builtin_bit_cast(plane8, (u32x4_t){w[q][0], w[q][1], w[q][2], w[q][3]});
-                        }
-#pragma unroll
-                        for (int dvb = 0; dvb < D / 32; dvb++) {
-                            const unsigned src = vt + (32 * kb + 16 * u) * ROWB;
-                            plane8 va[3];
-#pragma unroll
-                            for (int q = 0; q < 3; q++) {
-                                const plane4 lo = lds_tr4s(src + q * PLANEB + (((4 * dvb + vchunk) ^ vsw_lo) << 4));
-                                const plane4 hi = lds_tr4s(src + q * PLANEB + 8 * ROWB + (((4 * dvb + vchunk) ^ vsw_hi) << 4));
-                                va[q] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                            }
-#pragma unroll
-                            for (int qb = 0; qb < QB; qb++) f.o[qb][dvb] = mfma_split(va, pk[qb], f.o[qb][dvb]);
-                        }
-                    }
-            }
+            if (do_pv) weights_times_values32s<D, QB>(f, Vs, s);
         }
         if (more) {
             __syncthreads();   // every wavefront is done with the tile in LDS
@@ -370,12 +386,20 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
         if constexpr (SPLIT) {
             // lane's features of k-step t: 16t + 8hh .. + 7 (the B-operand layout of the 16-bit instruction)
             uint32_t qw[3][D / 16][4];
+            floatx4_t raw[D / 16][2];   // every load of the row is issued before the first is used: one memory round trip
 #pragma unroll
             for (int t = 0; t < D / 16; t++)
 #pragma unroll
                 for (int half = 0; half < 2; half++) {
                     const int d0 = 16 * t + 8 * hh + 4 * half;
-                    const floatx4_t q4 = ldg16f(qbase + p.E * qi + d0, qi < p.Lq && d0 < p.D);
+                    raw[t][half] = ldg16f(qbase + p.E * qi + d0, qi < p.Lq && d0 < p.D);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < D / 16; t++)
+#pragma unroll
+                for (int half = 0; half < 2; half++) {
+                    const floatx4_t q4 = raw[t][half];
                     // the reference divides q by sqrt(D) first (src/attention.jl:118)
 #pragma unroll
                     for (int j = 0; j < 2; j++) {
@@ -488,6 +512,182 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Small problems with the weights returned (the reference's default call, src/attention.jl:83): at most RES_TILES
+// tiles of keys.  flash32_kernel walks such a call as a chain of dependent steps (queries, K tile, statistics, K and
+// V tile again, weights), each waiting for memory or for a barrier.  Here every load of the call is issued at the
+// start, K and V are split into planes once, the scores of all tiles stay in registers between the statistics and the
+// weights, and the workgroup meets at two barriers (K in LDS; V in LDS, split under the score products).
+constexpr int RES_TILES = 2;
+
+template <int D, bool CAUSAL, bool EXTRAS>
+__global__ __launch_bounds__(256, 1) void flash32_resident_kernel(FlashArgs a) {
+    typedef CfgS<D> C;
+    constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB, CHUNKS = C::CHUNKS, TILEB = C::TILEB;
+    constexpr int XT = EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char flash_smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem;
+    const unsigned Kp = lds0, Vp = lds0 + RES_TILES * TILEB;   // K tiles, V tiles, then the weight staging regions
+    typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t hb = blockIdx.x % HB, qt = a.n_qtiles - 1 - blockIdx.x / HB;
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t i0 = qt * 128, iw = i0 + (int64_t)wave * 32, qi = iw + r;
+    int64_t kv_end = p.Lkv;
+    if (CAUSAL && i0 + 128 < kv_end) kv_end = i0 + 128;
+    const int n_tiles = (int)((kv_end + BN - 1) / BN);   // <= RES_TILES: checked by the host
+    const bool do_pv = p.out != nullptr;
+
+    // ---- every load of the call: K, the wavefront's queries, V
+    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
+    const float *vbase = do_pv ? (const float *)p.v + p.Ev * (p.Lkv * b) + p.Dv * h : nullptr;
+    const float *qrow = (const float *)p.q + p.E * (qi + p.Lq * b) + p.D * h;
+    const int dqk = (int)p.D, dv = (int)p.Dv;
+    floatx4_t kreg[RES_TILES][CHUNKS], vreg[RES_TILES][CHUNKS], q4[D / 16][2];
+#pragma unroll
+    for (int t = 0; t < RES_TILES; t++)
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            const int64_t row = (int64_t)t * BN + c / (D / 4);
+            const int col = (c % (D / 4)) * 4;
+            kreg[t][u] = ldg16f(kbase + p.E * row + col, t < n_tiles && row < p.Lkv && col < dqk);
+        }
+#pragma unroll
+    for (int t = 0; t < D / 16; t++)
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int d0 = 16 * t + 8 * hh + 4 * half;   // the B-operand layout of the 16-bit instruction
+            q4[t][half] = ldg16f(qrow + d0, qi < p.Lq && d0 < dqk);
+        }
+#pragma unroll
+    for (int t = 0; t < RES_TILES; t++)
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            const int64_t row = (int64_t)t * BN + c / (D / 4);
+            const int col = (c % (D / 4)) * 4;
+            vreg[t][u] = ldg16f(vbase + p.Ev * row + col, do_pv && t < n_tiles && row < p.Lkv && col < dv);
+        }
+
+    // four consecutive features of one key: 8 bytes in each of the three planes
+    auto store_split = [&](unsigned tile, int row, int col, const floatx4_t &x) {
+        uint32_t pl[3][2];
+        const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        if (odd) {   // an Inf or NaN in the chunk (rare)
+            split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+            split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        }
+        const unsigned at = tile + (unsigned)row * ROWB + (unsigned)((((col >> 3) ^ C::swz(row)) << 4) + (col & 7) * 2);
+#pragma unroll
+        for (int q = 0; q < 3; q++) *(lds8_t)(uintptr_t)(at + q * PLANEB) = (u32x2_t){pl[q][0], pl[q][1]};
+    };
+    auto store_tile = [&](unsigned tile, const floatx4_t (&reg)[CHUNKS]) {
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            store_split(tile, c / (D / 4), (c % (D / 4)) * 4, reg[u]);
+        }
+    };
+
+    // ---- K into planes in LDS, the queries into planes in registers
+#pragma unroll
+    for (int t = 0; t < RES_TILES; t++)
+        if (t < n_tiles) store_tile(Kp + t * TILEB, kreg[t]);
+    Frag32S<D, 1> f;
+    {
+        const float sq = sqrtf((float)p.D);   // the reference divides q by sqrt(D) first (src/attention.jl:118)
+        uint32_t qw[3][D / 16][4];
+#pragma unroll
+        for (int t = 0; t < D / 16; t++)
+#pragma unroll
+            for (int half = 0; half < 2; half++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    uint32_t w[3];
+                    const float x0 = q4[t][half][2 * j] / sq, x1 = q4[t][half][2 * j + 1] / sq;
+                    if (split3_pair(x0, x1, w[0], w[1], w[2])) split3_pair_guarded(x0, x1, w[0], w[1], w[2]);
+#pragma unroll
+                    for (int q = 0; q < 3; q++) qw[q][t][2 * half + j] = w[q];
+                }
+#pragma unroll
+        for (int q = 0; q < 3; q++)
+#pragma unroll
+            for (int t = 0; t < D / 16; t++) f.q[0][q][t] = __builtin_bit_cast(plane8, (u32x4_t){qw[q][t][0], qw[q][t][1], qw[q][t][2], qw[q][t][3]});
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++) f.o[0][dvb] = (floatx16_t){0};
+        f.m[0] = MI_NEG_INF;
+        f.l[0] = 0.0f;
+    }
+    __syncthreads();
+
+    // ---- scores of every tile (kept raw), V into planes under them, statistics
+    floatx16_t keep[RES_TILES][1][2];
+    bool active[RES_TILES];
+#pragma unroll
+    for (int t = 0; t < RES_TILES; t++) {
+        active[t] = t < n_tiles && (!CAUSAL || (int64_t)t * BN <= iw + 31);
+        if (active[t]) scores32s<D, 1>(f, Kp + t * TILEB, keep[t]);
+        if (t < n_tiles && do_pv) store_tile(Vp + t * TILEB, vreg[t]);
+    }
+#pragma unroll
+    for (int t = 0; t < RES_TILES; t++)
+        if (active[t]) {
+            floatx16_t s[1][2] = {{keep[t][0][0], keep[t][0][1]}};
+            flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_STATS, float>(a, s, f.o, f.m, f.l, b, h, iw, (int64_t)t * BN, FlashStaged<1>(), 0, 0u,
+                                                                             nullptr, p.Lkv);
+        }
+    f.l[0] = 1.0f / (f.l[0] + mi_swap32(f.l[0]));
+    __syncthreads();
+
+    // ---- weights and output
+    const unsigned wlds = lds0 + 2u * RES_TILES * TILEB + wave * FLASH_WSTAGE_BYTES;
+#pragma unroll
+    for (int t = 0; t < RES_TILES; t++)
+        if (active[t]) {
+            flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_FINAL, float>(a, keep[t], f.o, f.m, f.l, b, h, iw, (int64_t)t * BN, FlashStaged<1>(), 0, wlds,
+                                                                             nullptr, p.Lkv);
+            if (do_pv) weights_times_values32s<D, 1>(f, Vp + t * TILEB, keep[t]);
+        }
+    if (p.weights) flash_zero_skipped_weights<1, float>(a, b, h, iw, n_tiles, CAUSAL);
+
+    if (p.stats && hh == 0) flash_save_stats(p, b, h, qi, f.m[0] * MI_LOG2E, f.l[0]);
+    if (do_pv && qi < p.Lq) {
+        float *orow = (float *)p.out + p.Ev * (qi + p.Lq * b) + p.Dv * h;
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                floatx4_t o4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o4[e] = f.o[0][dvb][4 * g + e];
+                if (32 * dvb + 8 * g + 4 * hh < p.Dv) *(floatx4_t *)(orow + 32 * dvb + 8 * g + 4 * hh) = o4;
+            }
+    }
+}
+
+template <int D>
+int32_t launch_resident(const FlashArgs &a, hipStream_t st, bool extras) {
+    constexpr size_t smem = 2 * RES_TILES * CfgS<D>::TILEB + 4 * FLASH_WSTAGE_BYTES;
+    static bool attr_set = false;
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    auto kern = a.p.causal ? (extras ? flash32_resident_kernel<D, true, true> : flash32_resident_kernel<D, true, false>)
+                           : (extras ? flash32_resident_kernel<D, false, true> : flash32_resident_kernel<D, false, false>);
+    const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(256), smem, st, a);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
 template <int D, int QB, bool CAUSAL, bool EXTRAS, bool WEIGHTS, bool SPLIT>
 int32_t launch_one(const FlashArgs &a, hipStream_t st) {
     const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B * a.nsplit;
@@ -590,5 +790,7 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
         return narrow ? launch_d<64, 1>(a, st, true) : launch_d<128, 1>(a, st, true);
     }
     const bool extras = p.bias || p.mask;
+    // few keys and the weights returned: everything resident, one pass (flash32_resident_kernel)
+    if (narrow && p.weights && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted()) return launch_resident<64>(a, st, extras);
     return narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
 }

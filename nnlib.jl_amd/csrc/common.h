@@ -165,6 +165,20 @@ __device__ static inline void split3_pair_guarded(float x0, float x1, uint32_t &
     lo = __builtin_bit_cast(uint32_t, l);
 }
 
+// Guarded 16-byte loads without a branch: a lane whose piece of a tile does not exist reads these 16 zero bytes instead.
+// (With `ok ? *p : zero` the compiler put a branch around every load and waited for each one before issuing the next:
+// a tile's or a query row's loads then cost one memory round trip each instead of one in all.)
+__device__ static const uint32_t mi_zero_piece[4] __attribute__((aligned(16))) = {0u, 0u, 0u, 0u};
+template <typename V, typename E>
+__device__ static inline V mi_load16_or_zero(const E *p, bool ok) {
+    static_assert(sizeof(V) == 16, "16-byte pieces");
+    // both addresses as global-memory pointers: a select of generic pointers would make this a flat load, which also
+    // counts against the LDS counter
+    typedef __attribute__((address_space(1))) const V *global_ptr;
+    const global_ptr src = ok ? (global_ptr)(uintptr_t)p : (global_ptr)(uintptr_t)mi_zero_piece;
+    return *src;
+}
+
 // Workgroup order for kernels whose neighbouring workgroups share operands.  The hardware hands workgroup `id` of a
 // launch to XCD `id % 8` (eight dies, each with its own L2), so neighbours in launch order never share an L2.
 // mi_xcd_order turns the launch id into the id of the work item to take such that every die works through one

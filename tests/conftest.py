@@ -48,6 +48,20 @@ def nn():
     return nnlib_amd
 
 
+@pytest.fixture(autouse=True)
+def _stale_device_state(request):
+    """Before every GPU test: NaN-filled device blocks of many sizes, written and freed.  The arrays the test then
+    allocates start out as NaN instead of whatever the box happened to hold, and the SIMDs' register files hold NaN
+    patterns from the fill kernel: a kernel that reads memory or a register it never wrote (one did, through a
+    compiler's partial reload of a spilled operand) then fails every time instead of from run to run."""
+    if "gpu" in request.keywords and _gpu_available():
+        import torch
+        blocks = [torch.full((n,), float("nan"), device="cuda") for n in (1 << 10, 1 << 14, 1 << 18, 1 << 22, 1 << 25) for _ in range(2)]
+        torch.cuda.synchronize()
+        del blocks
+    yield
+
+
 def bf16_round(a):
     """float32 -> nearest-even bfloat16, returned as float32 (pure numpy bit arithmetic)."""
     a = np.ascontiguousarray(a, dtype=np.float32)

@@ -287,6 +287,65 @@ def test_flash32_parity(nn, oracle, case, weights):
     _check(nn, oracle, rng, dtype, E, Lq, Lkv, B, H, expect="flash32", weights=weights, **kw)
 
 
+SMALL_F32_CASES = [
+    # Float32, at most 128 keys, weights returned: every load up front, scores kept in registers between the statistics
+    # and the weights (one pass).  Ragged key counts around the 64-key tile, ragged and multi-tile query counts,
+    # head dims below the 64-wide tile, every combination of causal / bias / mask the two-pass kernel takes.
+    (64, 1, 1, 1, 1, {}),
+    (64, 37, 63, 2, 1, {}),
+    (128, 129, 64, 1, 2, {}),
+    (128, 300, 65, 2, 2, {}),
+    (512, 128, 128, 4, 8, {}),                                           # the smallest benchmark configuration
+    (128, 128, 128, 2, 2, dict(causal=True)),
+    (96, 127, 127, 1, 2, dict(causal=True, scale=0.125)),
+    (40, 65, 65, 3, 2, dict(causal=True)),                               # second key tile: one key, one query
+    (128, 70, 128, 2, 2, dict(bias_shape=(128, 70, 2, 2), mask_shape=(128, 70))),
+    (56, 131, 66, 2, 2, dict(bias_shape=(66, 131), mask_shape=(66, 131, 1, 2))),
+    (128, 96, 96, 1, 2, dict(causal=True, mask_shape=(96, 96))),
+    (48, 33, 90, 2, 2, dict(Ev=96, mask_shape=(90, 1, 2, 2))),           # v wider than q, k; key-padding style mask
+]
+
+
+@pytest.mark.parametrize("case", SMALL_F32_CASES, ids=lambda c: f"E{c[0]}-Lq{c[1]}-Lkv{c[2]}-B{c[3]}-H{c[4]}-" + "-".join(c[5]))
+def test_small_float32_problem_with_weights(nn, oracle, case):
+    E, Lq, Lkv, B, H, kw = case
+    rng = np.random.default_rng(1000 * E + 10 * Lq + Lkv)
+    _check(nn, oracle, rng, "f32", E, Lq, Lkv, B, H, expect="flash32", weights=True, **kw)
+
+
+def test_small_float32_problem_special_values(nn, oracle):
+    """+Inf logits (src/softmax.jl:73-75: the weights become the indicator of the +Inf entries, normalised), a query
+    with nothing kept (NaN) and scores without a value product, at a size the one-pass kernel takes."""
+    rng = np.random.default_rng(77)
+    E, Lq, Lkv, H = 64, 40, 100, 2
+    q, k, v = (rng.standard_normal((E, L, 1)).astype(np.float32) for L in (Lq, Lkv, Lkv))
+    bias = (0.3 * rng.standard_normal((Lkv, Lq))).astype(np.float32)
+    bias[3, 7] = bias[90, 7] = np.inf                 # two +Inf logits in one column, in different key tiles
+    bias[70, 9] = np.inf
+    mask = rng.random((Lkv, Lq)) < 0.8
+    mask[:, 11] = False                               # nothing kept
+    mask[3, 7] = mask[90, 7] = mask[70, 9] = True
+    with np.errstate(invalid="ignore", over="ignore"):
+        yr, ar = oracle.nnlib_attention_f32(q, k, v, bias, mask, H, nthreads=4)
+    y, a = _run(nn, q, k, v, "f32", bias, mask, H, weights_dtype="f32")
+    assert nn.last_attention_kernel() == "flash32"
+    assert np.array_equal(np.isnan(a), np.isnan(ar)) and np.array_equal(np.isnan(y), np.isnan(yr))
+    assert np.isnan(a[:, 11]).all() and np.isnan(y[:, 11]).all()
+    ok = ~np.isnan(ar)
+    assert np.abs(a[ok] - ar[ok]).max() <= 1e-5
+    assert a[3, 7, 0, 0] == 0.5 and a[90, 7, 0, 0] == 0.5 and a[70, 9, 1, 0] == 1.0
+    oky = ~np.isnan(yr)
+    assert np.abs(y[oky] - yr[oky]).max() <= 1e-4 * np.abs(yr[oky]).max()
+    # scores only (no values, no output)
+    D = nn.DeviceArray.from_numpy
+    q4, k4 = (x.reshape(E // H, H, -1, 1, order="F") for x in (q, k))
+    s = nn.dot_product_attention_scores(D(q4), D(k4), D(bias)).to_numpy()
+    assert nn.last_attention_kernel() == "flash32"
+    with np.errstate(invalid="ignore", over="ignore"):
+        sr = oracle.nnlib_attention_f32(q, k, v, bias, None, H, nthreads=4)[1]
+    assert np.abs(s - sr).max() <= 1e-5
+
+
 @pytest.mark.parametrize("dtype,E,H,Lkv,B", [("bf16", 512, 4, 1500, 2), ("bf16", 256, 2, 4096, 3), ("f16", 512, 8, 777, 1),
                                              ("f16", 1024, 8, 2048, 2), ("bf16", 128, 1, 513, 1),
                                              ("f32", 512, 4, 1500, 2), ("f32", 256, 4, 2048, 3), ("f32", 64, 1, 777, 1)])

@@ -38,6 +38,8 @@ CASES = [
     ("f32", 30, 7, 9, 2, 3, False, True, "generic"),
     ("f32", 128, 96, 160, 2, 2, False, True, "flash32"),
     ("f32", 128, 100, 100, 1, 2, True, False, "flash32"),
+    ("f32", 128, 150, 100, 2, 2, False, True, "flash32"),       # at most 128 keys with the weights returned: the resident kernel
+    ("f32", 96, 128, 128, 1, 2, True, True, "flash32"),
     ("bf16", 128, 70, 200, 2, 2, False, False, "flash16"),
     ("bf16", 256, 130, 130, 2, 2, True, True, "flash16"),
     ("f16", 128, 64, 4096, 1, 2, False, False, "flash16"),      # few query tiles, long keys: split-kv + merge
