@@ -669,21 +669,216 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_kernel(FlashArgs a) {
     }
 }
 
+// The same with two wavefronts per 32-query block, one per key tile (128-key problems: C1): eight wavefronts, two per
+// SIMD, each with half of the score products, the softmax arithmetic, the weight stores and the value products of a
+// block, and half of the K / V split per thread.  The two exchange their row statistics (m, l) after the first
+// phase and their partial outputs at the end, through LDS.
+template <int D, bool CAUSAL, bool EXTRAS>
+__global__ __launch_bounds__(512, 1) void flash32_resident_pair_kernel(FlashArgs a) {
+    typedef CfgS<D> C;
+    constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB, TILEB = C::TILEB;
+    constexpr int NT = 512, CHUNKS = BN * D / 4 / NT;
+    constexpr int XT = EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE;
+    static_assert(RES_TILES == 2, "one wavefront of a pair per key tile");
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char flash_smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem;
+    // K tiles (later the partial outputs of the second wavefronts), V tiles, weight staging, exchanged statistics
+    const unsigned Kp = lds0, Vp = lds0 + 2 * TILEB;
+    float *xstat = (float *)(flash_smem + 4 * TILEB + 8 * FLASH_WSTAGE_BYTES);   // [8 wavefronts][32 rows][2]
+    float *xout = (float *)flash_smem;                                           // [4 query blocks][D / 2 registers][64 lanes]
+    typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int qw = wave & 3, tile = wave >> 2;   // query block and key tile of this wavefront
+    const int64_t HB = p.H * p.B;
+    const int64_t hb = blockIdx.x % HB, qt = a.n_qtiles - 1 - blockIdx.x / HB;
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t i0 = qt * 128, iw = i0 + (int64_t)qw * 32, qi = iw + r;
+    int64_t kv_end = p.Lkv;
+    if (CAUSAL && i0 + 128 < kv_end) kv_end = i0 + 128;
+    const int n_tiles = (int)((kv_end + BN - 1) / BN);   // 1 or 2: checked by the host
+    const bool do_pv = p.out != nullptr;
+
+    // ---- every load of the call: K, the wavefront's queries, V
+    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
+    const float *vbase = do_pv ? (const float *)p.v + p.Ev * (p.Lkv * b) + p.Dv * h : nullptr;
+    const float *qrow = (const float *)p.q + p.E * (qi + p.Lq * b) + p.D * h;
+    const int dqk = (int)p.D, dv = (int)p.Dv;
+    floatx4_t kreg[2][CHUNKS], vreg[2][CHUNKS], q4[D / 16][2];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + NT * u;
+            const int64_t row = (int64_t)t * BN + c / (D / 4);
+            const int col = (c % (D / 4)) * 4;
+            kreg[t][u] = ldg16f(kbase + p.E * row + col, t < n_tiles && row < p.Lkv && col < dqk);
+        }
+#pragma unroll
+    for (int t = 0; t < D / 16; t++)
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int d0 = 16 * t + 8 * hh + 4 * half;
+            q4[t][half] = ldg16f(qrow + d0, qi < p.Lq && d0 < dqk);
+        }
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + NT * u;
+            const int64_t row = (int64_t)t * BN + c / (D / 4);
+            const int col = (c % (D / 4)) * 4;
+            vreg[t][u] = ldg16f(vbase + p.Ev * row + col, do_pv && t < n_tiles && row < p.Lkv && col < dv);
+        }
+
+    auto store_split = [&](unsigned at_tile, int row, int col, const floatx4_t &x) {
+        uint32_t pl[3][2];
+        const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        if (odd) {   // an Inf or NaN in the chunk (rare)
+            split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+            split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        }
+        const unsigned at = at_tile + (unsigned)row * ROWB + (unsigned)((((col >> 3) ^ C::swz(row)) << 4) + (col & 7) * 2);
+#pragma unroll
+        for (int q = 0; q < 3; q++) *(lds8_t)(uintptr_t)(at + q * PLANEB) = (u32x2_t){pl[q][0], pl[q][1]};
+    };
+    auto store_tile = [&](unsigned at_tile, const floatx4_t (&reg)[CHUNKS]) {
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + NT * u;
+            store_split(at_tile, c / (D / 4), (c % (D / 4)) * 4, reg[u]);
+        }
+    };
+
+    // ---- K into planes in LDS, the queries into planes in registers
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+        if (t < n_tiles) store_tile(Kp + t * TILEB, kreg[t]);
+    Frag32S<D, 1> f;
+    {
+        const float sq = sqrtf((float)p.D);   // the reference divides q by sqrt(D) first (src/attention.jl:118)
+        uint32_t qw3[3][D / 16][4];
+#pragma unroll
+        for (int t = 0; t < D / 16; t++)
+#pragma unroll
+            for (int half = 0; half < 2; half++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    uint32_t w[3];
+                    const float x0 = q4[t][half][2 * j] / sq, x1 = q4[t][half][2 * j + 1] / sq;
+                    if (split3_pair(x0, x1, w[0], w[1], w[2])) split3_pair_guarded(x0, x1, w[0], w[1], w[2]);
+#pragma unroll
+                    for (int q = 0; q < 3; q++) qw3[q][t][2 * half + j] = w[q];
+                }
+#pragma unroll
+        for (int q = 0; q < 3; q++)
+#pragma unroll
+            for (int t = 0; t < D / 16; t++) f.q[0][q][t] = __builtin_bit_cast(plane8, (u32x4_t){qw3[q][t][0], qw3[q][t][1], qw3[q][t][2], qw3[q][t][3]});
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++) f.o[0][dvb] = (floatx16_t){0};
+        f.m[0] = MI_NEG_INF;
+        f.l[0] = 0.0f;
+    }
+    __syncthreads();
+
+    // ---- scores of the wavefront's tile (kept raw), V into planes, statistics of the tile
+    const int64_t j0 = (int64_t)tile * BN;
+    const bool active = tile < n_tiles && (!CAUSAL || j0 <= iw + 31);
+    floatx16_t keep[1][2];
+    // the two wavefronts of a SIMD (w and w + 4: the two tiles of one query block) take the score products and their
+    // half of the V split in opposite order, so that one's matrix instructions run under the other's vector work
+    auto split_v = [&]() {
+        if (do_pv) {
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+                if (t < n_tiles) store_tile(Vp + t * TILEB, vreg[t]);
+        }
+    };
+    if (tile == 1) split_v();
+    if (active) scores32s<D, 1>(f, Kp + tile * TILEB, keep);
+    if (tile == 0) split_v();
+    if (active) {
+        floatx16_t s[1][2] = {{keep[0][0], keep[0][1]}};
+        flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_STATS, float>(a, s, f.o, f.m, f.l, b, h, iw, j0, FlashStaged<1>(), 0, 0u, nullptr, p.Lkv);
+    }
+    // the pair's statistics: (m, l) of both tiles, combined as the online softmax combines tiles (src/softmax.jl:69-79
+    // over the whole row): m = max, l = sum of l_i 2^((m_i - m) c); equal maxima (two -Inf or two +Inf included) keep
+    // their sums as they are
+    const float lsum = f.l[0] + mi_swap32(f.l[0]);
+    if (hh == 0) {
+        xstat[(wave * 32 + r) * 2] = f.m[0];
+        xstat[(wave * 32 + r) * 2 + 1] = lsum;
+    }
+    __syncthreads();   // statistics exchanged, V in LDS, every wavefront done with the K planes
+    {
+        const float mp = xstat[((wave ^ 4) * 32 + r) * 2], lp = xstat[((wave ^ 4) * 32 + r) * 2 + 1];
+        const float cs = flash_natural_units(XT) ? MI_LOG2E : a.c;
+        const float m = fmaxf(f.m[0], mp);
+        const float fa = f.m[0] == m ? 1.0f : mi_exp2((f.m[0] - m) * cs), fb = mp == m ? 1.0f : mi_exp2((mp - m) * cs);
+        f.m[0] = m;
+        f.l[0] = 1.0f / (lsum * fa + lp * fb);
+    }
+
+    // ---- weights and the wavefront's share of the output
+    const unsigned wlds = lds0 + 4u * TILEB + wave * FLASH_WSTAGE_BYTES;
+    if (active) {
+        flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_FINAL, float>(a, keep, f.o, f.m, f.l, b, h, iw, j0, FlashStaged<1>(), 0, wlds, nullptr, p.Lkv);
+        if (do_pv) weights_times_values32s<D, 1>(f, Vp + tile * TILEB, keep);
+    }
+    if (tile == 0 && p.weights) flash_zero_skipped_weights<1, float>(a, b, h, iw, n_tiles, CAUSAL);
+    if (tile == 0 && p.stats && hh == 0) flash_save_stats(p, b, h, qi, f.m[0] * MI_LOG2E, f.l[0]);
+
+    // the second wavefront's partial output goes through LDS (the K planes' region: nobody reads them any more)
+    if (!do_pv) return;
+    if (tile == 1) {
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) xout[(qw * (D / 2) + 16 * dvb + v) * 64 + lane] = f.o[0][dvb][v];
+    }
+    __syncthreads();
+    if (tile == 0 && qi < p.Lq) {
+        float *orow = (float *)p.out + p.Ev * (qi + p.Lq * b) + p.Dv * h;
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                floatx4_t o4;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o4[e] = f.o[0][dvb][4 * g + e] + xout[(qw * (D / 2) + 16 * dvb + 4 * g + e) * 64 + lane];
+                if (32 * dvb + 8 * g + 4 * hh < p.Dv) *(floatx4_t *)(orow + 32 * dvb + 8 * g + 4 * hh) = o4;
+            }
+    }
+}
+
 template <int D>
 int32_t launch_resident(const FlashArgs &a, hipStream_t st, bool extras) {
     constexpr size_t smem = 2 * RES_TILES * CfgS<D>::TILEB + 4 * FLASH_WSTAGE_BYTES;
+    constexpr size_t smem_pair = 2 * RES_TILES * CfgS<D>::TILEB + 8 * FLASH_WSTAGE_BYTES + 8 * 32 * 2 * sizeof(float);
+    static_assert(4 * 32 * (D / 2) * sizeof(float) <= 2 * CfgS<D>::TILEB, "partial outputs fit the K planes' region");
     static bool attr_set = false;
     if (!attr_set) {
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_pair_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pair));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_pair_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pair));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_pair_kernel<D, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pair));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_pair_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pair));
         attr_set = true;
     }
-    auto kern = a.p.causal ? (extras ? flash32_resident_kernel<D, true, true> : flash32_resident_kernel<D, true, false>)
-                           : (extras ? flash32_resident_kernel<D, false, true> : flash32_resident_kernel<D, false, false>);
     const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B;
-    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(256), smem, st, a);
+    if (a.p.Lkv > BN) {   // two key tiles: a wavefront per tile and query block
+        auto kern = a.p.causal ? (extras ? flash32_resident_pair_kernel<D, true, true> : flash32_resident_pair_kernel<D, true, false>)
+                               : (extras ? flash32_resident_pair_kernel<D, false, true> : flash32_resident_pair_kernel<D, false, false>);
+        hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(512), smem_pair, st, a);
+    } else {
+        auto kern = a.p.causal ? (extras ? flash32_resident_kernel<D, true, true> : flash32_resident_kernel<D, true, false>)
+                               : (extras ? flash32_resident_kernel<D, false, true> : flash32_resident_kernel<D, false, false>);
+        hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(256), smem, st, a);
+    }
     MI_LAUNCH_CHECK();
     return MI_OK;
 }
