@@ -1,13 +1,13 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|bwd|bwd_f32|logsoftmax|softmax|softmax_dims2|batched_mul[_f32|_c32|_f64]] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|dense_mask|bwd|bwd_f32|logsoftmax|softmax|softmax_dims2|batched_mul[_f32|_c32|_f64]] [--no-cpu]
 
 A "step" is one dot_product_attention call on synthetic inputs that are already resident in HBM.
 The default workload is C3 (bf16 causal prefill, head dim 128, L = 4096), the configuration the
 prefill target is quoted on; the other four configurations are measured in the same run and reported under
-"configs" in the same JSON line (C5, the decode target, also under "decode"), and the workloads beyond them (gradient,
-softmax family, batched_mul; GPU leg only) under "next_rows".  Timing is by HIP events on the stream the kernels are launched on.
+"configs" in the same JSON line (C5, the decode target, also under "decode"), and the workloads beyond them (dense mask,
+gradient, softmax family, batched_mul; GPU leg only) under "next_rows".  Timing is by HIP events on the stream the kernels are launched on.
 """
 import argparse
 import ctypes
@@ -313,6 +313,8 @@ def measure(key, steps, warmup, with_cpu):
 
 EXTRA = {
     "bwd": "gradient of C3: causal bf16 (4096,4096,2) H=32 D=128, dq + dk + dv from dy and the forward result",
+    "dense_mask": "forward call of the C3 shape with a dense Bool mask (4096, 4096), 90 % kept, not causal, weights not materialised; "
+                  "the same call without the mask is timed beside it",
     "bwd_f32": "gradient of C2: causal f32 (1024,1024,8) H=16 D=64, dq + dk + dv from dy and the forward result",
     "logsoftmax": "logsoftmax(x; dims=1), x (4096, 65536) f32 (1 GiB in, 1 GiB out)",
     "softmax_dims2": "softmax(x; dims=2), x (256, 4096, 128) bf16 (256 MiB in, 256 MiB out), reduction over the strided dim",
@@ -353,7 +355,28 @@ def measure_extra(key, steps, warmup, with_cpu):
     _lib.check(lib.mi_init(0))
     DA = nn.DeviceArray
     cores = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
-    if key in ("bwd", "bwd_f32"):
+    if key == "dense_mask":
+        # a mask that depends on the query (src/attention.jl:122-124): packed into bits by a pre-pass inside the call and
+        # applied by the software-pipelined kernel; the step timed is the whole call, pre-pass included
+        ms_of = {}
+        for name, extra in (("unmasked", {}), ("masked", dict(mask=True))):
+            WORKLOADS["_dense_mask"] = dict(WORKLOADS["c3"], causal=False, **extra)
+            try:
+                r = Runner("_dense_mask", rotate=False)
+                ms_of[name], _ = r.time(steps, warmup)
+                kernel = r.kernel
+                flops, _ = algorithmic_work(r.w)
+                del r
+            finally:
+                del WORKLOADS["_dense_mask"]
+        ms = ms_of["masked"]
+        val = flops / (ms * 1e-3) / 1e12
+        line = dict(metric="attention forward TFLOP/s (all pairs counted)", value=val, unit="TFLOP/s", dtype="bf16",
+                    roofline=dict(bound="mfma", achieved=val, peak=PEAK["bf16"], unit="TFLOP/s", frac=val / PEAK["bf16"], traffic=None),
+                    config=dict(workload=EXTRA[key], kernel=kernel, unmasked_ms_per_step=ms_of["unmasked"],
+                                rate_against_unmasked=ms_of["unmasked"] / ms),
+                    flops_per_step=flops)
+    elif key in ("bwd", "bwd_f32"):
         w = WORKLOADS["c3" if key == "bwd" else "c2"]
         E, L, B, H = w["E"], w["Lq"], w["B"], w["H"]
         D = E // H
@@ -381,7 +404,8 @@ def measure_extra(key, steps, warmup, with_cpu):
         line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype=dtn,
                     roofline=dict(bound="mfma", achieved=val, peak=PEAK[dtn], unit="TFLOP/s", frac=val / PEAK[dtn], **measured_traffic_fields(key)),
                     config=dict(workload=EXTRA[key], kernel=_lib.KERNEL_NAMES[kern.value]), flops_per_step=flops)
-        line["roofline"]["products_executed_per_counted"] = 8 / 5   # dQ: S, dP, dQ; dV: S, dV; dK: S, dP, dK
+        # 16-bit: dQ kernel S, dP, dQ; fused dK / dV kernel S, dV, dP, dK.  Float32: dQ: S, dP, dQ; dV: S, dV; dK: S, dP, dK
+        line["roofline"]["products_executed_per_counted"] = 8 / 5 if dtn == "f32" else 7 / 5
         if dtn == "f32":
             f32_products(line["roofline"], val, 8 / 5)
         if with_cpu:

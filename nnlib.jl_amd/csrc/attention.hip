@@ -10,12 +10,12 @@ int32_t launch_flash16_f16_d64(const AttnParams &, hipStream_t, const int32_t *k
 int32_t launch_flash16_f16_d128(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
 int32_t launch_flash16_bf16_d256(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
 int32_t launch_flash16_f16_d256(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, bool lengths_variant = false);
-int32_t launch_flash16_fast_bf16(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
-int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_fast_bf16(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, const AttnMaskWords *mw = nullptr);
+int32_t launch_flash16_fast_f16(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, const AttnMaskWords *mw = nullptr);
 bool flash16_fast_supports_bf16(const AttnParams &);
 bool flash16_fast_supports_f16(const AttnParams &);
-int32_t launch_flash16_fast_bf16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
-int32_t launch_flash16_fast_f16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr);
+int32_t launch_flash16_fast_bf16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, const AttnMaskWords *mw = nullptr);
+int32_t launch_flash16_fast_f16_d64(const AttnParams &, hipStream_t, const int32_t *kv_len = nullptr, const AttnMaskWords *mw = nullptr);
 bool flash16_fast_supports_bf16_d64(const AttnParams &);
 bool flash16_fast_supports_f16_d64(const AttnParams &);
 
@@ -166,11 +166,83 @@ static int32_t launch_general16(const AttnParams &p, hipStream_t st, const int32
     return dmax <= 64 ? launch_flash16_f16_d64(p, st, kv_len, lv) : dmax <= 128 ? launch_flash16_f16_d128(p, st, kv_len, lv) : launch_flash16_f16_d256(p, st, kv_len, lv);
 }
 
-static int32_t launch_fast16(const AttnParams &p, hipStream_t st, const int32_t *kv_len) {
-    if (p.dtype == MI_BF16 && flash16_fast_supports_bf16(p)) return launch_flash16_fast_bf16(p, st, kv_len);
-    if (p.dtype == MI_F16 && flash16_fast_supports_f16(p)) return launch_flash16_fast_f16(p, st, kv_len);
-    if (p.dtype == MI_BF16) return launch_flash16_fast_bf16_d64(p, st, kv_len);
-    return launch_flash16_fast_f16_d64(p, st, kv_len);
+static int32_t launch_fast16(const AttnParams &p, hipStream_t st, const int32_t *kv_len, const AttnMaskWords *mw = nullptr) {
+    if (p.dtype == MI_BF16 && flash16_fast_supports_bf16(p)) return launch_flash16_fast_bf16(p, st, kv_len, mw);
+    if (p.dtype == MI_F16 && flash16_fast_supports_f16(p)) return launch_flash16_fast_f16(p, st, kv_len, mw);
+    if (p.dtype == MI_BF16) return launch_flash16_fast_bf16_d64(p, st, kv_len, mw);
+    return launch_flash16_fast_f16_d64(p, st, kv_len, mw);
+}
+
+// ---- dense masks for the software-pipelined kernel ------------------------------------------------------------------
+// A mask that depends on the query (src/attention.jl:122-124 takes any array that broadcasts against the logits) costs
+// the general kernel a byte per score, staged through LDS.  The pipelined kernel takes it as bits instead: a pre-pass
+// packs the mask once per call into one word per query and 32-key block (AttnMaskWords; 1/8 of the mask's bytes, read
+// by every head and batch element that shares the mask), and the kernel turns a word into its 16 scores' worth of
+// -Inf with two instructions per score.  Any strides: the pre-pass reads bytes.
+static AttnMaskWords mask_words_layout(const AttnParams &p) {
+    AttnMaskWords mw;
+    mw.words = p.workspace;
+    mw.lq_pad = (int32_t)((p.Lq + 255) / 256 * 256);
+    mw.groups = (int32_t)((p.Lkv + 127) / 128);
+    const int64_t slice = (int64_t)mw.groups * mw.lq_pad;
+    const bool per_h = p.mask_strides[2] != 0 && p.H > 1, per_b = p.mask_strides[3] != 0 && p.B > 1;
+    mw.stride_h = per_h ? slice : 0;
+    mw.stride_b = per_b ? slice * (per_h ? p.H : 1) : 0;
+    return mw;
+}
+static size_t mask_words_bytes(const AttnParams &p) {
+    const AttnMaskWords mw = mask_words_layout(p);
+    const int64_t slices = (mw.stride_h ? p.H : 1) * (mw.stride_b ? p.B : 1);
+    return (size_t)slices * (size_t)mw.groups * (size_t)mw.lq_pad * 16;
+}
+static bool takes_mask_words_path(const AttnParams &p) {
+    static const bool off = getenv("MI355ATTN_NO_MASK_WORDS") != nullptr;   // A/B switch: masks go to the general kernel
+    if (off) return false;
+    if (!p.mask || p.bias || p.no_mask_words || !fast_kernel_fits(p) || p.Lq > 2147483647LL - 256 || p.Lkv > 2147483647LL - 128) return false;
+    // as for calls without a mask: few workgroups against a key range the general kernel would split
+    const int64_t fast_wgs = ((p.Lq + 255) / 256) * p.H * p.B;
+    if ((fast_wgs < 128 || (fast_wgs == 128 && p.causal)) && flash_pick_nsplit(p, 128) > 1) return false;
+    return true;
+}
+
+// one wavefront per (query, slice, run of 8 groups): a byte per lane and half group, all 16 requested before the first
+// is looked at, two ballots and one 16-byte store per group
+constexpr int PACK_RUN = 8;
+__global__ __launch_bounds__(256) void pack_mask_words_kernel(const uint8_t *mask, int64_t s0, int64_t s1, int64_t s2, int64_t s3, int64_t Lq,
+                                                             int64_t Lkv, int64_t nh, int64_t items, int32_t runs, AttnMaskWords mw) {
+    const int lane = threadIdx.x & 63;
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);   // (run, query, head slice, batch slice), run fastest
+    if (item >= items) return;
+    const int run = (int)(item % runs);
+    const int64_t row = item / runs, q = row % mw.lq_pad, sl = row / mw.lq_pad, h = sl % nh, b = sl / nh;
+    u32x4_t *dst = (u32x4_t *)mw.words + h * mw.stride_h + b * mw.stride_b + q;
+    const uint8_t *src = mask + q * s1 + h * s2 + b * s3;
+    const int g0 = run * PACK_RUN;
+    uint8_t byte[PACK_RUN][2];
+#pragma unroll
+    for (int u = 0; u < PACK_RUN; u++)
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int64_t key = (int64_t)(g0 + u) * 128 + 64 * half + lane;
+            byte[u][half] = q < Lq && key < Lkv ? src[key * s0] : (uint8_t)0;
+        }
+#pragma unroll
+    for (int u = 0; u < PACK_RUN; u++) {
+        const uint64_t lo = __builtin_amdgcn_ballot_w64(byte[u][0] != 0), hi = __builtin_amdgcn_ballot_w64(byte[u][1] != 0);
+        if (lane == 0 && g0 + u < mw.groups)
+            dst[(int64_t)(g0 + u) * mw.lq_pad] = (u32x4_t){(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+    }
+}
+
+static int32_t launch_pack_mask_words(const AttnParams &p, const AttnMaskWords &mw, hipStream_t st) {
+    const int64_t nh = mw.stride_h ? p.H : 1, nb = mw.stride_b ? p.B : 1;
+    const int32_t runs = (mw.groups + PACK_RUN - 1) / PACK_RUN;
+    const int64_t items = (int64_t)mw.lq_pad * nh * nb * runs;
+    if ((items + 3) / 4 > 2147483647LL) return mi_set_error(MI_ESHAPE, "attention: mask too large to pack");
+    hipLaunchKernelGGL(pack_mask_words_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, st, p.mask, p.mask_strides[0],
+                       p.mask_strides[1], p.mask_strides[2], p.mask_strides[3], p.Lq, p.Lkv, nh, items, runs, mw);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
 }
 
 int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
@@ -183,6 +255,12 @@ int32_t launch_attention_flash16(const AttnParams &p, hipStream_t st) {
         rc = fast_kernel_fits(p) ? launch_fast16(p, st, lens) : launch_general16(p, st, lens, true);
         if (rc != MI_OK) return rc;
         return launch_general16(p, st, lens);
+    }
+    if (takes_mask_words_path(p)) {
+        const AttnMaskWords mw = mask_words_layout(p);
+        const int32_t rc = launch_pack_mask_words(p, mw, st);
+        if (rc != MI_OK) return rc;
+        return launch_fast16(p, st, nullptr, &mw);
     }
     if (takes_fast_path(p)) return launch_fast16(p, st, nullptr);
     return launch_general16(p, st, nullptr);
@@ -256,6 +334,7 @@ static int32_t choose(const mi_attn_desc *d, const AttnParams &p, size_t *ws) {
     }
     if (attention_flash16_supports(p)) {
         if (takes_length_path(p)) *ws = length_path_workspace(p);   // one context length per (head, batch) pair
+        else if (takes_mask_words_path(p)) *ws = mask_words_bytes(p);
         else if (!takes_fast_path(p)) *ws = flash_split_workspace(p, flash_pick_nsplit(p, 128));
         return MI_ATTN_KERNEL_FLASH16;
     }
@@ -338,6 +417,11 @@ static int32_t attention_forward(const mi_attn_desc *d, mi_stream s, bool static
     size_t ws = 0;
     int32_t kernel = choose(d, p, &ws);
     const size_t have = static_workspace ? (size_t)MI_ATTN_STATIC_WORKSPACE_BYTES : (d->workspace ? d->workspace_bytes : (size_t)0);
+    if (ws > have && kernel == MI_ATTN_KERNEL_FLASH16 && p.mask) {
+        // a dense mask too large to pack into the workspace at hand: the general kernel reads it as it is
+        p.no_mask_words = true;
+        kernel = choose(d, p, &ws);
+    }
     if (ws > have && kernel == MI_ATTN_KERNEL_FLASH16) {
         // few queries against many keys: the key-split plan is the faster one, but the pipelined kernel needs no
         // workspace at all, so a caller without (enough of) one is served rather than refused

@@ -20,6 +20,19 @@ struct AttnParams {
     // plan constraint of the entry point without caller workspace: stay on the software-pipelined kernel (which needs
     // none) where the key-split plan would ask for more than the built-in workspace holds
     bool keep_pipelined = false;
+    // and the same for the packed dense mask of the pipelined kernel: a caller whose workspace cannot hold it gets the
+    // general kernel, which reads the mask as it is
+    bool no_mask_words = false;
+};
+
+// A dense mask packed for the software-pipelined forward kernel (attention.hip: pack_mask_words_kernel): one 16-byte
+// piece per query and group of 128 keys, word j bit k = mask[128 g + 32 j + k, query] != 0 (0 for keys past Lkv and for
+// queries past Lq); pieces laid out [slice][group][Lq rounded up to 256], slice = h * stride_h + b * stride_b pieces
+// (0 where the mask is shared between heads / batch elements).
+struct AttnMaskWords {
+    const void *words;
+    int64_t stride_h, stride_b;
+    int32_t lq_pad, groups;
 };
 
 #ifdef __HIPCC__

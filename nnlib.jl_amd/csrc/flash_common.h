@@ -30,6 +30,10 @@ struct FlashArgs {
     // leading keys kept when the mask keeps exactly a prefix (the software-pipelined kernel then treats it as that
     // pair's L_kv and the general kernel leaves the pair alone), 0 otherwise (the general kernel applies the mask)
     const int32_t *kv_len = nullptr;
+    // software-pipelined forward kernel with a dense mask: the packed mask (AttnMaskWords), strides in 16-byte pieces
+    const u32x4_t *mask_words = nullptr;
+    int64_t mw_h = 0, mw_b = 0;
+    int32_t mw_lqp = 0, mw_groups = 0;
 };
 
 // Bytes of LDS per wavefront for the weight staging below: 16 query rows x 128 bytes.

@@ -599,6 +599,113 @@ def test_logits_that_drift_along_the_keys(nn, oracle, dtype, pattern, weights):
         assert float(np.abs(a.sum(axis=0) - 1).max()) <= 1e-5
 
 
+def _mask_words_bytes(Lq, Lkv, slices):
+    """Workspace of a call that takes the software-pipelined kernel with a packed dense mask: 16 bytes per query
+    (rounded up to 256) and group of 128 keys, per mask slice."""
+    return slices * ((Lkv + 127) // 128) * ((Lq + 255) // 256 * 256) * 16
+
+
+DENSE_MASK_CASES = [
+    # dtype, E, Lq, Lkv, B, H, causal, mask shape
+    ("bf16", 256, 300, 700, 2, 2, False, (700, 300)),                # head dim 128, one mask for all, ragged sizes
+    ("bf16", 256, 520, 520, 1, 2, True, (520, 520)),                  # causal .& array
+    ("f16", 128, 257, 1100, 2, 2, False, (1100, 257, 2, 1)),          # head dim 64, a mask per head
+    ("f16", 256, 600, 600, 2, 2, True, (600, 600, 1, 2)),             # a mask per batch element, causal
+    ("bf16", 128, 700, 300, 3, 1, False, (300, 700, 1, 3)),
+    ("bf16", 512, 1030, 1290, 1, 4, False, (1290, 1030)),             # more than four tiles: the unrolled steady loop
+    ("f16", 256, 1500, 1500, 1, 4, True, (1500, 1500, 4, 1)),
+]
+
+
+@pytest.mark.parametrize("case", DENSE_MASK_CASES, ids=lambda c: f"{c[0]}-E{c[1]}-Lq{c[2]}-Lkv{c[3]}-B{c[4]}-H{c[5]}-{'causal' if c[6] else 'plain'}-mask{'x'.join(map(str, c[7]))}")
+def test_dense_masks_on_the_pipelined_kernel(nn, oracle, case):
+    """Query-dependent Bool masks without bias, weights and dropout: packed into bits by a pre-pass and applied by the
+    software-pipelined kernel (the plan's workspace is the packed mask).  Besides a random mask the rows hold the
+    special cases of a running maximum that starts without a kept key: a query that keeps nothing (NaN, as the
+    reference's softmax over a column of -Inf gives, src/softmax.jl:73-75), queries whose first kept key comes blocks
+    later, a query that keeps only the last key, and a query whose only kept keys score far below the masked ones
+    of its first block (their weights must not underflow against a maximum taken from nothing)."""
+    dtype, E, Lq, Lkv, B, H, causal, mshape = case
+    rng = np.random.default_rng(hash(case[1:6]) % 2**32)
+    D = E // H
+    q = rng.standard_normal((E, Lq, B))
+    k = rng.standard_normal((E, Lkv, B))
+    v = rng.standard_normal((E, Lkv, B))
+    mask = rng.random(mshape) < 0.85
+    full = mask.reshape(mshape + (1,) * (4 - len(mshape)))
+    full[:, 3] = False                                   # keeps nothing
+    full[:200, 5] = False                                # first kept key in the seventh 32-key block at the earliest
+    full[:, 7] = False
+    full[(7 if causal else Lkv - 1), 7] = True           # one key (the last one the causal pattern allows)
+    full[:, 9] = False
+    full[64:96, 9] = True                                # one block
+    # query 130: scores of +-8 sqrt(D) against keys 0..127; keeps only the strongly negative ones
+    q[:, 130] = 8.0
+    k[:, :64] = 1.0
+    k[:, 64:128] = -1.0
+    full[:, 130] = False
+    full[64:128, 130] = True
+    q, k, v = (round_to(a, dtype) for a in (q, k, v))
+    dq, dk, dv = (nn.DeviceArray.from_numpy(a, dtype) for a in (q, k, v))
+    dm = nn.DeviceArray.from_numpy(mask)
+    y, _ = nn.dot_product_attention(dq, dk, dv, mask=(nn.make_causal_mask(dq, dims=2) & dm) if causal else dm, nheads=H,
+                                    return_weights=False)
+    assert nn.last_attention_kernel() == "flash16"
+    slices = (mshape[2] if len(mshape) > 2 else 1) * (mshape[3] if len(mshape) > 3 else 1)
+    assert nn.ops._last_workspace == _mask_words_bytes(Lq, Lkv, slices)
+    omask = np.broadcast_to(full, (Lkv, Lq, H, B))
+    if causal:
+        omask = omask & oracle.make_causal_mask(Lq).reshape(Lkv, Lq, 1, 1)
+    yr, _ = oracle.nnlib_attention_f32(q, k, v, None, np.ascontiguousarray(omask), H, nthreads=8)
+    y = y.to_numpy()
+    nan_ref = np.isnan(yr)
+    assert nan_ref[:, 3].all() and (nan_ref.sum() == nan_ref[:, 3].size if not causal else True)
+    assert np.array_equal(np.isnan(y), nan_ref)
+    err = rel_err(np.where(nan_ref, 0, y), np.where(nan_ref, 0, yr))
+    assert err <= TOL[dtype], err
+    # the query with the far-away scores averages the values of the keys it keeps
+    assert np.abs(y[:, 130] - v[:, 64:128].mean(axis=1)).max() <= 2e-2
+
+
+def test_dense_mask_with_strides_and_without_room_for_the_packed_copy(nn, oracle):
+    """The pre-pass reads the mask through its strides (here a mask stored query-major, passed as its transpose), and a
+    caller whose workspace cannot hold the packed mask is served by the general kernel with the same result."""
+    import ctypes
+    import torch
+    L = nn._lib
+    lib = L.load()
+    E, Lq, Lkv, B, H = 256, 384, 640, 2, 2
+    rng = np.random.default_rng(11)
+    q, k, v = (round_to(rng.standard_normal((E, n, B)), "bf16") for n in (Lq, Lkv, Lkv))
+    mask_t = rng.random((Lq, Lkv)) < 0.8                      # [query][key] in column-major order: key stride Lq
+    mask_t[:, 0] = True
+    tq, tk, tv = (torch.from_numpy(np.ascontiguousarray(a.transpose(2, 1, 0))).cuda().to(torch.bfloat16) for a in (q, k, v))
+    tm = torch.from_numpy(np.ascontiguousarray(mask_t.T)).cuda().to(torch.uint8)   # memory order: key slowest
+    outs = []
+    for with_ws in (True, False):
+        out = torch.full((B, Lq, E), float("nan"), device="cuda", dtype=torch.bfloat16)
+        d = L.mi_attn_desc()
+        d.struct_size = ctypes.sizeof(L.mi_attn_desc)
+        d.dtype = d.weights_dtype = L.MI_BF16
+        d.E = d.Ev = E
+        d.Lq, d.Lkv, d.H, d.B = Lq, Lkv, H, B
+        d.q, d.k, d.v, d.out = tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), out.data_ptr()
+        d.mask = tm.data_ptr()
+        d.mask_strides = (ctypes.c_int64 * 4)(Lq, 1, 0, 0)
+        ws = ctypes.c_size_t(0)
+        L.check(lib.mi_attention_workspace_size(ctypes.byref(d), ctypes.byref(ws)))
+        assert ws.value == _mask_words_bytes(Lq, Lkv, 1)
+        if with_ws:
+            buf = torch.empty(ws.value, dtype=torch.uint8, device="cuda")
+            d.workspace, d.workspace_bytes = buf.data_ptr(), buf.numel()
+        L.check(lib.mi_attention_fwd(ctypes.byref(d), None))
+        torch.cuda.synchronize()
+        outs.append(out.float().cpu().numpy().transpose(2, 1, 0))
+    yr, _ = oracle.nnlib_attention_f32(q, k, v, None, np.asfortranarray(mask_t.T), H, nthreads=8)
+    for y in outs:
+        assert rel_err(y, yr) <= TOL["bf16"]
+
+
 def test_few_queries_without_a_workspace_fall_back_to_the_pipelined_kernel(nn):
     """mi_attention_fwd with no workspace on a call whose plan is the key-split kernel: served by the software-pipelined
     kernel (which needs none) instead of MI_EWORKSPACE; same result to the 16-bit bound."""
