@@ -198,7 +198,7 @@ static size_t mask_words_bytes(const AttnParams &p) {
 static bool takes_mask_words_path(const AttnParams &p) {
     static const bool off = getenv("MI355ATTN_NO_MASK_WORDS") != nullptr;   // A/B switch: masks go to the general kernel
     if (off) return false;
-    if (!p.mask || p.bias || p.no_mask_words || !fast_kernel_fits(p) || p.Lq > 2147483647LL - 256 || p.Lkv > 2147483647LL - 128) return false;
+    if (!p.mask || p.bias || p.lean_workspace || !fast_kernel_fits(p) || p.Lq > 2147483647LL - 256 || p.Lkv > 2147483647LL - 128) return false;
     // as for calls without a mask: few workgroups against a key range the general kernel would split
     const int64_t fast_wgs = ((p.Lq + 255) / 256) * p.H * p.B;
     if ((fast_wgs < 128 || (fast_wgs == 128 && p.causal)) && flash_pick_nsplit(p, 128) > 1) return false;
@@ -419,7 +419,7 @@ static int32_t attention_forward(const mi_attn_desc *d, mi_stream s, bool static
     const size_t have = static_workspace ? (size_t)MI_ATTN_STATIC_WORKSPACE_BYTES : (d->workspace ? d->workspace_bytes : (size_t)0);
     if (ws > have && kernel == MI_ATTN_KERNEL_FLASH16 && p.mask) {
         // a dense mask too large to pack into the workspace at hand: the general kernel reads it as it is
-        p.no_mask_words = true;
+        p.lean_workspace = true;
         kernel = choose(d, p, &ws);
     }
     if (ws > have && kernel == MI_ATTN_KERNEL_FLASH16) {

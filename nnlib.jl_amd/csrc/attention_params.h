@@ -22,7 +22,7 @@ struct AttnParams {
     bool keep_pipelined = false;
     // and the same for the packed dense mask of the pipelined kernel: a caller whose workspace cannot hold it gets the
     // general kernel, which reads the mask as it is
-    bool no_mask_words = false;
+    bool lean_workspace = false;
 };
 
 // A dense mask packed for the software-pipelined forward kernel (attention.hip: pack_mask_words_kernel): one 16-byte
