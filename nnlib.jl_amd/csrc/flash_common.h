@@ -359,32 +359,20 @@ __device__ inline void flash_load_key_mask(const FlashArgs &a, int64_t b, int64_
 // Mask bytes applied without lane masks (a compare writes a lane mask to scalar registers, which costs the compare, a
 // wait state and the select: three issue slots an element).  flash_mask_bits turns the four bytes of a word into "bit 7
 // of the byte is set iff the byte is non-zero" (no carry crosses a byte: 0x7f + 0x7f < 0x100); flash_mask_apply
-// sign-extends that bit into a word of ones or zeros and picks the score or -Inf with a bit-field insert, which is not
+// sign-extends that bit into a word of ones or zeros and picks the score or -Inf with a bit operation, which is not
 // arithmetic: a NaN score under a dropped key is dropped like any other, as src/attention.jl:133-138 has it.
 __device__ inline uint32_t flash_mask_bits(uint32_t m4) { return ((m4 & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | m4; }
-// The select is inline assembly (written any other way the compiler turns it back into compare and select), and the
-// compiler does not insert for inline assembly the wait states that a read of a matrix-core result needs.  Callers
-// whose scores come straight from the MFMAs therefore pass `after`, a scalar they obtained with flash_mfma_fence from
-// the same accumulator block: the fence is an instruction the compiler does protect, and the operand orders the
-// select behind it.
-// Contract: `v` must have been written by a builtin matrix instruction (which the compiler's hazard recogniser knows),
-// not by one issued from inline assembly (T::mfma32_keep_c), and the selects must follow the fence in program order:
-// the recogniser puts the wait states in front of the fence's own read of v[0], by which time the instruction has
-// written all sixteen registers, and the in-order issue keeps the selects behind it.  Every caller (the EXTRAS_MASKTILE
-// and EXTRAS_KEYMASK branches of flash_softmax_tile, reached from flash16_kernel and the gradient kernels) passes the
-// accumulators of T::mfma32 / __builtin_amdgcn_mfma_* calls.
-__device__ inline int flash_mfma_fence(const floatx16_t &v) { return __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v[0])); }
-__device__ inline float flash_mask_apply(float s, uint32_t bits, int e, int after) {
+// Written on the bit patterns: the compiler keeps it as a bit-field extract and one three-input bit operation (and, being
+// ordinary code, gives a read of a matrix-core result the wait states it needs).
+__device__ inline float flash_mask_apply(float s, uint32_t bits, int e) {
     const int keep = __builtin_amdgcn_sbfe((int)bits, 8 * e + 7, 1);   // 0 or -1
-    float r;
-    asm("v_bfi_b32 %0, %1, %2, %3 ; ordered after %4" : "=v"(r) : "v"(keep), "v"(s), "s"(0xFF800000u), "s"(after));
-    return r;
+    return __builtin_bit_cast(float, (__builtin_bit_cast(int, s) & keep) | ((int)0xFF800000 & ~keep));
 }
 // elements 4g .. 4g+3 of a 16-element accumulator block against the four mask bytes of m4
-__device__ inline void flash_mask_apply4(floatx16_t &v, int g, uint32_t m4, int after) {
+__device__ inline void flash_mask_apply4(floatx16_t &v, int g, uint32_t m4) {
     const uint32_t bits = flash_mask_bits(m4);
 #pragma unroll
-    for (int e = 0; e < 4; e++) v[4 * g + e] = flash_mask_apply(v[4 * g + e], bits, e, after);
+    for (int e = 0; e < 4; e++) v[4 * g + e] = flash_mask_apply(v[4 * g + e], bits, e);
 }
 
 // The running maximum of the online softmax only has to bound the exponents: it is raised when a tile's maximum
@@ -435,7 +423,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                 for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        flash_mask_apply4(s[qb][kb], g, sg.mask4(stage, row, 4 * kb + g, hh), 0);   // scores already went through the scaling above
+                        flash_mask_apply4(s[qb][kb], g, sg.mask4(stage, row, 4 * kb + g, hh));
                     }
             }
         } else if (EXTRAS == EXTRAS_DIRECT) {
@@ -488,9 +476,8 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             const int row = 32 * qb + r;
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
-                const int fence = flash_mfma_fence(s[qb][kb]);
 #pragma unroll
-                for (int g = 0; g < 4; g++) flash_mask_apply4(s[qb][kb], g, sg.mask4(stage, row, 4 * kb + g, hh), fence);
+                for (int g = 0; g < 4; g++) flash_mask_apply4(s[qb][kb], g, sg.mask4(stage, row, 4 * kb + g, hh));
             }
         }
         if (EXTRAS == EXTRAS_KEYMASK) {
@@ -499,9 +486,8 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             if (!key_mask) flash_load_key_mask(a, b, h, j0, hh, own);
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
-                const int fence = flash_mfma_fence(s[qb][kb]);
 #pragma unroll
-                for (int g = 0; g < 4; g++) flash_mask_apply4(s[qb][kb], g, key_mask ? key_mask[4 * kb + g] : own[4 * kb + g], fence);
+                for (int g = 0; g < 4; g++) flash_mask_apply4(s[qb][kb], g, key_mask ? key_mask[4 * kb + g] : own[4 * kb + g]);
             }
         }
         if (EXTRAS != EXTRAS_DIRECT && edge) {
