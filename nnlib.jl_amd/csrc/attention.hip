@@ -205,9 +205,12 @@ static bool takes_mask_words_path(const AttnParams &p) {
     return true;
 }
 
-// one wavefront per (query, slice, run of 8 groups): a byte per lane and half group, all 16 requested before the first
-// is looked at, two ballots and one 16-byte store per group
+// One wavefront per (query, slice, run of 8 groups = 1024 keys); all loads of a run are requested before the first is
+// looked at.  WORDS (unit key stride, rows 4-byte aligned): a lane loads four keys at a time, makes their four bits, and
+// the eight lanes of a 32-key block OR their shifted nibbles together (three exchanges).  Otherwise a byte per lane and
+// half group, through the mask's strides, and two ballots per group.
 constexpr int PACK_RUN = 8;
+template <bool WORDS>
 __global__ __launch_bounds__(256) void pack_mask_words_kernel(const uint8_t *mask, int64_t s0, int64_t s1, int64_t s2, int64_t s3, int64_t Lq,
                                                              int64_t Lkv, int64_t nh, int64_t items, int32_t runs, AttnMaskWords mw) {
     const int lane = threadIdx.x & 63;
@@ -218,19 +221,44 @@ __global__ __launch_bounds__(256) void pack_mask_words_kernel(const uint8_t *mas
     u32x4_t *dst = (u32x4_t *)mw.words + h * mw.stride_h + b * mw.stride_b + q;
     const uint8_t *src = mask + q * s1 + h * s2 + b * s3;
     const int g0 = run * PACK_RUN;
-    uint8_t byte[PACK_RUN][2];
+    if constexpr (WORDS) {
+        uint32_t four[PACK_RUN / 2];   // one load covers 256 keys: two groups
 #pragma unroll
-    for (int u = 0; u < PACK_RUN; u++)
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            const int64_t key = (int64_t)(g0 + u) * 128 + 64 * half + lane;
-            byte[u][half] = q < Lq && key < Lkv ? src[key * s0] : (uint8_t)0;
+        for (int u = 0; u < PACK_RUN / 2; u++) {
+            const int64_t key = (int64_t)(g0 + 2 * u) * 128 + 4 * lane;
+            four[u] = 0;
+            if (q < Lq && key + 3 < Lkv) four[u] = *(const uint32_t *)(src + key);
+            else if (q < Lq)
+                for (int e = 0; e < 4; e++)
+                    if (key + e < Lkv) four[u] |= (uint32_t)src[key + e] << (8 * e);
         }
 #pragma unroll
-    for (int u = 0; u < PACK_RUN; u++) {
-        const uint64_t lo = __builtin_amdgcn_ballot_w64(byte[u][0] != 0), hi = __builtin_amdgcn_ballot_w64(byte[u][1] != 0);
-        if (lane == 0 && g0 + u < mw.groups)
-            dst[(int64_t)(g0 + u) * mw.lq_pad] = (u32x4_t){(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+        for (int u = 0; u < PACK_RUN / 2; u++) {
+            const uint32_t x = four[u];
+            uint32_t v = ((x & 0xFFu) ? 1u : 0u) | ((x & 0xFF00u) ? 2u : 0u) | ((x & 0xFF0000u) ? 4u : 0u) | ((x & 0xFF000000u) ? 8u : 0u);
+            v <<= 4 * (lane & 7);
+            v |= (uint32_t)__shfl_xor((int)v, 1, 64);
+            v |= (uint32_t)__shfl_xor((int)v, 2, 64);
+            v |= (uint32_t)__shfl_xor((int)v, 4, 64);
+            // lane 8j holds the word of block j of the 256 keys: word j % 4 of group g0 + 2u + j / 4
+            const int g = g0 + 2 * u + (lane >> 5);
+            if ((lane & 7) == 0 && g < mw.groups) ((uint32_t *)(dst + (int64_t)g * mw.lq_pad))[(lane >> 3) & 3] = v;
+        }
+    } else {
+        uint8_t byte[PACK_RUN][2];
+#pragma unroll
+        for (int u = 0; u < PACK_RUN; u++)
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                const int64_t key = (int64_t)(g0 + u) * 128 + 64 * half + lane;
+                byte[u][half] = q < Lq && key < Lkv ? src[key * s0] : (uint8_t)0;
+            }
+#pragma unroll
+        for (int u = 0; u < PACK_RUN; u++) {
+            const uint64_t lo = __builtin_amdgcn_ballot_w64(byte[u][0] != 0), hi = __builtin_amdgcn_ballot_w64(byte[u][1] != 0);
+            if (lane == 0 && g0 + u < mw.groups)
+                dst[(int64_t)(g0 + u) * mw.lq_pad] = (u32x4_t){(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+        }
     }
 }
 
@@ -239,8 +267,13 @@ static int32_t launch_pack_mask_words(const AttnParams &p, const AttnMaskWords &
     const int32_t runs = (mw.groups + PACK_RUN - 1) / PACK_RUN;
     const int64_t items = (int64_t)mw.lq_pad * nh * nb * runs;
     if ((items + 3) / 4 > 2147483647LL) return mi_set_error(MI_ESHAPE, "attention: mask too large to pack");
-    hipLaunchKernelGGL(pack_mask_words_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, st, p.mask, p.mask_strides[0],
-                       p.mask_strides[1], p.mask_strides[2], p.mask_strides[3], p.Lq, p.Lkv, nh, items, runs, mw);
+    const bool words = p.mask_strides[0] == 1 && ((((uintptr_t)p.mask) | (uintptr_t)p.mask_strides[1] | (uintptr_t)p.mask_strides[2] | (uintptr_t)p.mask_strides[3]) & 3) == 0;
+    if (words)
+        hipLaunchKernelGGL(pack_mask_words_kernel<true>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, st, p.mask, p.mask_strides[0],
+                           p.mask_strides[1], p.mask_strides[2], p.mask_strides[3], p.Lq, p.Lkv, nh, items, runs, mw);
+    else
+        hipLaunchKernelGGL(pack_mask_words_kernel<false>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, st, p.mask, p.mask_strides[0],
+                           p.mask_strides[1], p.mask_strides[2], p.mask_strides[3], p.Lq, p.Lkv, nh, items, runs, mw);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }
