@@ -33,7 +33,8 @@ DOMINANT_KERNEL = {"c1": "flash32_kernel", "c2": "flash32_kernel", "c3": "flash1
                    "c5": "decode_split_kernel",
                    # a gradient step is three kernels (dq, dk, dv): every row of the workload whose name contains "bwd"
                    "bwd": "bwd", "bwd_f32": "bwd", "softmax": "softmax", "logsoftmax": "softmax", "softmax_dims2": "softmax",
-                   "batched_mul": "gemm", "batched_mul_f32": "gemm"}
+                   "batched_mul": "gemm", "batched_mul_f32": "gemm",
+                   "dense_mask": "flash16_fast_kernel<false, true>"}
 
 
 def measured_traffic(key):
@@ -372,7 +373,7 @@ def measure_extra(key, steps, warmup, with_cpu):
         ms = ms_of["masked"]
         val = flops / (ms * 1e-3) / 1e12
         line = dict(metric="attention forward TFLOP/s (all pairs counted)", value=val, unit="TFLOP/s", dtype="bf16",
-                    roofline=dict(bound="mfma", achieved=val, peak=PEAK["bf16"], unit="TFLOP/s", frac=val / PEAK["bf16"], traffic=None),
+                    roofline=dict(bound="mfma", achieved=val, peak=PEAK["bf16"], unit="TFLOP/s", frac=val / PEAK["bf16"], **measured_traffic_fields(key)),
                     config=dict(workload=EXTRA[key], kernel=kernel, unmasked_ms_per_step=ms_of["unmasked"],
                                 rate_against_unmasked=ms_of["unmasked"] / ms),
                     flops_per_step=flops)
