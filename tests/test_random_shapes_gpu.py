@@ -103,3 +103,46 @@ def test_gradient_head_dims_bias_masks(nn, oracle, seed):
     dropout = (0.2, 17 + seed) if rng.integers(0, 4) == 0 else None
     _run(nn, oracle, dtype, D * H, D * H, Lq, Lkv, (B,), H, bias_shape=bias_shape, mask_kind=mask_kind, seed=seed, scale=0.4,
          dropout=dropout, saved=bool(rng.integers(0, 2)))
+
+
+# ---- third sweep: query-dependent masks on the software-pipelined kernel (16-bit, head dims 64 / 128, no weights) ----
+
+@pytest.mark.parametrize("seed", range(24))
+def test_dense_masks_without_weights(nn, oracle, seed):
+    """Lengths around every edge of the packed mask (32-key words, groups of 128 keys, 256-query padding), masks shared
+    or per head / batch element, sparse enough that whole blocks, whole rows and the
+    first blocks of a row are dropped; with and without the causal pattern on top.  Forward result against the
+    float64 oracle; rows that keep no key are NaN in both."""
+    rng = np.random.default_rng(7000 + seed)
+    dtype = ["bf16", "f16"][seed % 2]
+    D = [64, 128][(seed // 2) % 2]
+    H, B = int(rng.integers(1, 4)), int(rng.integers(1, 3))
+    edges = [1, 31, 33, 64, 127, 128, 129, 255, 256, 257, 300, 513, 700]
+    Lq = int(rng.choice(edges))
+    causal = bool(rng.integers(0, 2))
+    Lkv = Lq if causal else int(rng.choice(edges + [1100, 1290]))
+    E = D * H
+    q = round_to(rng.standard_normal((E, Lq, B)) * 0.7, dtype)
+    k = round_to(rng.standard_normal((E, Lkv, B)) * 0.7, dtype)
+    v = round_to(rng.standard_normal((E, Lkv, B)), dtype)
+    shape = [(Lkv, Lq), (Lkv, Lq, H, 1), (Lkv, Lq, 1, B), (Lkv, Lq, H, B)][int(rng.integers(0, 4))]
+    keep = float(rng.choice([0.9, 0.5, 0.05]))
+    mask = rng.random(shape) < keep
+    full = mask.reshape(shape + (1,) * (4 - len(shape)))
+    if Lq > 2:
+        full[: Lkv // 2, 1] = False      # the first half of the keys dropped for one query
+        full[:, 2] = False               # and everything for another
+    Dv = nn.DeviceArray.from_numpy
+    dq_, dk_, dv_ = Dv(q, dtype), Dv(k, dtype), Dv(v, dtype)
+    dmask = Dv(mask)
+    y, _ = nn.dot_product_attention(dq_, dk_, dv_, mask=(nn.make_causal_mask(dq_) & dmask) if causal else dmask, nheads=H,
+                                    return_weights=False)
+    omask = np.broadcast_to(full, (Lkv, Lq, H, B))
+    if causal:
+        omask = omask & oracle.make_causal_mask(Lq).reshape(Lkv, Lq, 1, 1)
+    y_ref, _ = oracle.attention_f64(q, k, v, None, np.ascontiguousarray(omask), H)
+    y = y.to_numpy()
+    nan_ref = np.isnan(y_ref)
+    assert np.array_equal(np.isnan(y), nan_ref), (dtype, D, H, B, Lq, Lkv, causal, shape, keep)
+    err = rel_err(np.where(nan_ref, 0, y), np.where(nan_ref, 0, y_ref))
+    assert err <= TOL[dtype], (err, dtype, D, H, B, Lq, Lkv, causal, shape, keep, nn.last_attention_kernel())
