@@ -198,7 +198,7 @@ static size_t mask_words_bytes(const AttnParams &p) {
 static bool takes_mask_words_path(const AttnParams &p) {
     static const bool off = getenv("MI355ATTN_NO_MASK_WORDS") != nullptr;   // A/B switch: masks go to the general kernel
     if (off) return false;
-    if (!p.mask || p.bias || p.lean_workspace || !fast_kernel_fits(p) || p.Lq > 2147483647LL - 256 || p.Lkv > 2147483647LL - 128) return false;
+    if (!p.mask || p.bias || p.drop_thresh || p.lean_workspace || !fast_kernel_fits(p) || p.Lq > 2147483647LL - 256 || p.Lkv > 2147483647LL - 128) return false;
     // as for calls without a mask: few workgroups against a key range the general kernel would split
     const int64_t fast_wgs = ((p.Lq + 255) / 256) * p.H * p.B;
     if ((fast_wgs < 128 || (fast_wgs == 128 && p.causal)) && flash_pick_nsplit(p, 128) > 1) return false;

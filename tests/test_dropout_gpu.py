@@ -43,7 +43,10 @@ CASES = [
     ("bf16", 128, 70, 200, 2, 2, False, False, "flash16"),
     ("bf16", 256, 130, 130, 2, 2, True, True, "flash16"),
     ("f16", 128, 64, 4096, 1, 2, False, False, "flash16"),      # few query tiles, long keys: split-kv + merge
-    ("bf16", 256, 300, 300, 1, 2, True, False, "flash16"),      # head dim 128: would take the fast kernel without dropout
+    ("bf16", 256, 300, 300, 1, 2, True, False, "flash16"),      # head dim 128, no weights, runs of four keys: the pipelined kernel
+    ("f16", 256, 520, 1300, 1, 2, False, False, "flash16"),     # its unrolled steady loop (more than four key tiles)
+    ("bf16", 128, 700, 700, 2, 2, True, False, "flash16"),      # head dim 64, causal, steady loop and diagonal steps
+    ("bf16", 256, 100, 301, 1, 2, False, False, "flash16"),     # key count not a multiple of 4: the general kernel
 ]
 
 
