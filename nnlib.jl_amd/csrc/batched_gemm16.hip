@@ -20,6 +20,7 @@
 // Both deliver the 16 k of a step in the order {0-3, 8-11 | 4-7, 12-15} per half-wave, which is what
 // the transposing read produces; A and B only have to agree.
 #include "common.h"
+#include "flash_common.h"   // flash_dma_1k, FLASH_WAIT_VMCNT, flash_make_rsrc
 
 namespace {
 
@@ -143,6 +144,71 @@ struct Operand {
     }
 };
 
+// Writes a workgroup's accumulators: C = alpha * acc + beta * C.  acc[n block][m block] of the wavefront at (wm, wn) of the
+// workgroup's grid; the tile starts at (m0, n0) of slice bz.
+template <typename T, bool LARGE>
+__device__ inline void store_tile(const Gemm16Args &g, const floatx16_t (&acc)[Shape<LARGE>::BNB][Shape<LARGE>::BM], int64_t bz, int64_t m0,
+                                  int64_t n0, int wm, int wn, int lane) {
+    typedef typename T::type t;
+    typedef Shape<LARGE> S;
+    constexpr int BM = S::BM, BNB = S::BNB;
+    const int r = lane & 31, hh = lane >> 5;
+    // accumulator register v of lane (r, hh) of block (i, j): m = 32j + 8*(v/4) + 4*hh + v%4, n = 32i + r
+    t *C = (t *)g.C + bz * g.sC;
+    const bool vec_ok = g.c_vec != 0;   // C columns can be written in aligned 16-byte pieces
+#pragma unroll
+    for (int i = 0; i < BNB; i++) {
+        const int64_t nj = n0 + 32 * BNB * wn + 32 * i + r;
+        t *ccol = C + (nj < g.n ? nj : 0) * g.ldc;
+#pragma unroll
+        for (int j = 0; j < BM; j++)
+#pragma unroll
+            for (int gp = 0; gp < 2; gp++) {
+                // X: m = mb + 4hh .. +3 (v = 8gp ..), Y: m = mb + 8 + 4hh .. +3 (v = 8gp + 4 ..)
+                const int64_t mb = m0 + 32 * BM * wm + 32 * j + 16 * gp;
+                float xv[4], yv[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    xv[e] = g.alpha * acc[i][j][8 * gp + e];
+                    yv[e] = g.alpha * acc[i][j][8 * gp + 4 + e];
+                }
+                if (vec_ok) {
+                    if (g.beta != 0.0f && nj < g.n) {
+                        if (mb + 4 * hh < g.m) {
+                            const typename T::vec4 c4 = *(const typename T::vec4 *)(ccol + mb + 4 * hh);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) xv[e] += g.beta * T::to_f32(c4[e]);
+                        }
+                        if (mb + 8 + 4 * hh < g.m) {
+                            const typename T::vec4 c4 = *(const typename T::vec4 *)(ccol + mb + 8 + 4 * hh);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) yv[e] += g.beta * T::to_f32(c4[e]);
+                        }
+                    }
+                    typename T::vec4 xe, yo;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        xe[e] = T::from_f32(xv[e]);
+                        yo[e] = T::from_f32(yv[e]);
+                    }
+                    const u32x2_t x = __builtin_bit_cast(u32x2_t, xe), y = __builtin_bit_cast(u32x2_t, yo);
+                    uint32_t x0 = x[0], x1 = x[1], y0 = y[0], y1 = y[1];
+                    mi_pair_halves(x0, y0);   // every lane takes part; lanes outside C do not store
+                    mi_pair_halves(x1, y1);
+                    const u32x4_t piece = {x0, x1, y0, y1};
+                    if (nj < g.n && mb + 8 * hh < g.m) *(u32x4_t *)(ccol + mb + 8 * hh) = piece;   // m is a multiple of 8 here
+                } else if (nj < g.n) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int64_t mx = mb + 4 * hh + e, my = mx + 8;
+                        if (mx < g.m) ccol[mx] = T::from_f32(g.beta != 0.0f ? xv[e] + g.beta * T::to_f32(ccol[mx]) : xv[e]);
+                        if (my < g.m) ccol[my] = T::from_f32(g.beta != 0.0f ? yv[e] + g.beta * T::to_f32(ccol[my]) : yv[e]);
+                    }
+                }
+            }
+    }
+}
+
 template <typename T, bool A_RM, bool B_RM, bool LARGE>
 __global__ __launch_bounds__(Shape<LARGE>::THREADS, LARGE ? 1 : 2) void gemm16_kernel(Gemm16Args g) {
     typedef typename T::type t;
@@ -211,60 +277,156 @@ __global__ __launch_bounds__(Shape<LARGE>::THREADS, LARGE ? 1 : 2) void gemm16_k
     }
     if (it < nk) stage(it, 1);
 
-    // accumulator register v of lane (r, hh) of block (i, j): m = 32j + 8*(v/4) + 4*hh + v%4, n = 32i + r
-    t *C = (t *)g.C + bz * g.sC;
-    const bool vec_ok = g.c_vec != 0;   // C columns can be written in aligned 16-byte pieces
+    store_tile<T, LARGE>(g, acc, bz, m0, n0, wm, wn, lane);
+}
+
+// ---- the 256 x 256 tile with the operand tiles copied global -> LDS by the DMA path ---------------------------------
+// Same output tile and wavefront grid as the LARGE shape above; what changes is how the operand tiles arrive: with
+// buffer_load ... lds into a ring of four stages of 32 k each (16 KiB per operand and stage, 128 KiB in all), two stages
+// ahead of their use, one workgroup barrier per two stages.  No staging registers, no LDS stores issued by the
+// wavefronts, and the copies of later stages land while the matrix instructions of the current one run; the
+// register-staged kernel above stores a whole stage to LDS between the last matrix instruction of one stage and the
+// barrier, which every wavefront of the CU then waits behind.
+// Tile layouts (a DMA piece is 16 bytes per lane, 1 KiB per instruction, lane l at byte 16 l of the piece):
+//   RMAJ  [32 k][256 rows]: 512-byte k-rows, 16-byte chunks XOR-swizzled by the k-row; operand through the transposing
+//         read, here with each half-wave taking 8 consecutive k (rows 8 hh .. 8 hh + 7 of the 16-k step);
+//   KMAJ  [256 rows][32 k]: 64-byte rows of four 16-byte chunks (8 consecutive k each), chunk XOR (row / 4) % 4;
+//         operand = one 16-byte read per lane.
+// Both deliver k 8 hh .. 8 hh + 7 to half-wave hh, so any pair of layouts agrees.
+constexpr int RK = 32;                        // k per stage
+constexpr int RING = 4;
+constexpr int RTILEB = 256 * RK * 2;          // bytes per operand and stage
+constexpr size_t RING_SMEM = 2 * RING * RTILEB;
+
+__device__ inline int ring_kswz(int row) { return (row >> 2) & 3; }
+
+template <typename T, bool RM>
+struct RingOperand {
+    typedef typename T::type t;
+    i32x4_t rsrc;
+    int voff[2];     // byte offsets of this lane's two pieces of a stage at k0 = 0 (0x80000000: outside the matrix)
+    int kpiece[2];   // KMAJ: first k of the piece within the stage (to drop pieces past k)
+    int kstep;       // bytes per unit of k0
+    int64_t k;
+    unsigned lds;    // LDS byte address of this wavefront's first piece in stage 0
+    static constexpr int OOB = (int)0x80000000;
+
+    __device__ void init(const t *X, int64_t ld, int64_t rows, int64_t k_, int64_t row0, char *ring, int wave, int lane) {
+        k = k_;
+        const int64_t extent = RM ? (k_ - 1) * ld + rows : (rows - 1) * ld + k_;
+        rsrc = flash_make_rsrc(X, (uint32_t)(extent * 2));
+        kstep = RM ? (int)(ld * 2) : 2;
+        lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)ring + wave * 2048;
 #pragma unroll
-    for (int i = 0; i < BNB; i++) {
-        const int64_t nj = n0 + 32 * BNB * wn + 32 * i + r;
-        t *ccol = C + (nj < g.n ? nj : 0) * g.ldc;
-#pragma unroll
-        for (int j = 0; j < BM; j++)
-#pragma unroll
-            for (int gp = 0; gp < 2; gp++) {
-                // X: m = mb + 4hh .. +3 (v = 8gp ..), Y: m = mb + 8 + 4hh .. +3 (v = 8gp + 4 ..)
-                const int64_t mb = m0 + 32 * BM * wm + 32 * j + 16 * gp;
-                float xv[4], yv[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    xv[e] = g.alpha * acc[i][j][8 * gp + e];
-                    yv[e] = g.alpha * acc[i][j][8 * gp + 4 + e];
-                }
-                if (vec_ok) {
-                    if (g.beta != 0.0f && nj < g.n) {
-                        if (mb + 4 * hh < g.m) {
-                            const typename T::vec4 c4 = *(const typename T::vec4 *)(ccol + mb + 4 * hh);
-#pragma unroll
-                            for (int e = 0; e < 4; e++) xv[e] += g.beta * T::to_f32(c4[e]);
-                        }
-                        if (mb + 8 + 4 * hh < g.m) {
-                            const typename T::vec4 c4 = *(const typename T::vec4 *)(ccol + mb + 8 + 4 * hh);
-#pragma unroll
-                            for (int e = 0; e < 4; e++) yv[e] += g.beta * T::to_f32(c4[e]);
-                        }
-                    }
-                    typename T::vec4 xe, yo;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        xe[e] = T::from_f32(xv[e]);
-                        yo[e] = T::from_f32(yv[e]);
-                    }
-                    const u32x2_t x = __builtin_bit_cast(u32x2_t, xe), y = __builtin_bit_cast(u32x2_t, yo);
-                    uint32_t x0 = x[0], x1 = x[1], y0 = y[0], y1 = y[1];
-                    mi_pair_halves(x0, y0);   // every lane takes part; lanes outside C do not store
-                    mi_pair_halves(x1, y1);
-                    const u32x4_t piece = {x0, x1, y0, y1};
-                    if (nj < g.n && mb + 8 * hh < g.m) *(u32x4_t *)(ccol + mb + 8 * hh) = piece;   // m is a multiple of 8 here
-                } else if (nj < g.n) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int64_t mx = mb + 4 * hh + e, my = mx + 8;
-                        if (mx < g.m) ccol[mx] = T::from_f32(g.beta != 0.0f ? xv[e] + g.beta * T::to_f32(ccol[mx]) : xv[e]);
-                        if (my < g.m) ccol[my] = T::from_f32(g.beta != 0.0f ? yv[e] + g.beta * T::to_f32(ccol[my]) : yv[e]);
-                    }
-                }
+        for (int i = 0; i < 2; i++) {
+            const int piece = 2 * wave + i;   // 16 pieces of 1 KiB per operand and stage
+            if (RM) {
+                const int krow = 2 * piece + (lane >> 5), chunk = (lane & 31) ^ rmaj_swz(krow);
+                kpiece[i] = krow;
+                voff[i] = row0 + 8 * chunk < rows ? (int)(((row0 + 8 * chunk) + krow * ld) * 2) : OOB;   // k-rows past k lie past the extent
+            } else {
+                const int row = 16 * piece + (lane >> 2), chunk = (lane & 3) ^ ring_kswz(row);
+                kpiece[i] = 8 * chunk;
+                voff[i] = row0 + row < rows ? (int)((8 * chunk + (row0 + row) * ld) * 2) : OOB;
             }
+        }
     }
+    // start the copy of the stage whose first k is k0 into ring position `pos`
+    __device__ void issue(int pos, int64_t k0) const {
+        const unsigned dst = __builtin_amdgcn_readfirstlane(lds + pos * RTILEB);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            int o = voff[i] == OOB ? OOB : voff[i] + (int)k0 * kstep;
+            o = k0 + kpiece[i] < k ? o : OOB;   // a piece past k would read the next row (KMAJ) or wrap the 32-bit offset (RMAJ)
+            flash_dma_1k(rsrc, dst + i * 1024, o);
+        }
+    }
+    // MFMA operand of the 32-row block `blk` of the stage at `tile` for k-step ks (0, 1): k 16 ks + 8 hh .. + 7
+    __device__ static typename T::vec8 fetch(const char *tile, int blk, int ks, int lane) {
+        const int hh = lane >> 5;
+        if (RM) {
+            const int vrow = 16 * ks + 8 * hh + ((lane & 15) >> 2);
+            const int vchunk = 4 * blk + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), vsub = 8 * (lane & 1);
+            const char *src = tile + vrow * 512 + vsub;
+            const typename T::vec4 lo = lds_tr4<T>(src + ((vchunk ^ rmaj_swz(vrow)) << 4));
+            const typename T::vec4 hi = lds_tr4<T>(src + 4 * 512 + ((vchunk ^ rmaj_swz(vrow + 4)) << 4));
+            return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        } else {
+            const int row = 32 * blk + (lane & 31);
+            return *(const typename T::vec8 *)(tile + row * 64 + (((2 * ks + hh) ^ ring_kswz(row)) << 4));
+        }
+    }
+};
+
+template <typename T, bool A_RM, bool B_RM>
+__global__ __launch_bounds__(512, 1) void gemm16_ring_kernel(Gemm16Args g) {
+    typedef typename T::type t;
+    typedef Shape<true> S;
+    constexpr int BM = S::BM, BNB = S::BNB;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char gemm_smem[];
+    char *As = (char *)gemm_smem, *Bs = As + RING * RTILEB;
+    const MiTile tile = mi_gemm_tile_order(blockIdx.x + (int64_t)gridDim.x * (blockIdx.y + (int64_t)gridDim.y * blockIdx.z), gridDim.x, gridDim.y, gridDim.z);
+    const int64_t bz = tile.batch, m0 = tile.m * S::TILE, n0 = tile.n * S::TILE;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave % S::WM, wn = wave / S::WM;
+
+    RingOperand<T, A_RM> a;
+    RingOperand<T, B_RM> b;
+    a.init((const t *)g.A + bz * g.sA, g.lda, g.m, g.k, m0, As, wave, lane);
+    b.init((const t *)g.B + bz * g.sB, g.ldb, g.n, g.k, n0, Bs, wave, lane);
+
+    floatx16_t acc[BNB][BM];
+#pragma unroll
+    for (int i = 0; i < BNB; i++)
+#pragma unroll
+        for (int j = 0; j < BM; j++) acc[i][j] = (floatx16_t){0};
+
+    // Stage s lives in ring position s % 4.  An even stage starts with "stages s and s + 1 have landed everywhere and
+    // stages s - 2 and s - 1 are read by nobody any more"; every stage then requests stage s + 2 (past the last stage
+    // the pieces lie outside the matrices and arrive as zeros, which nothing reads).
+    const int ns = (int)((g.k + RK - 1) / RK);
+    a.issue(0, 0);
+    b.issue(0, 0);
+    a.issue(1, RK);
+    b.issue(1, RK);
+    for (int st = 0; st < ns; st++) {
+        if ((st & 1) == 0) {
+            FLASH_WAIT_VMCNT(0);
+            asm volatile("" ::: "memory");
+            __syncthreads();
+        }
+        if (st + 2 < ns) {
+            a.issue((st + 2) & 3, (int64_t)(st + 2) * RK);
+            b.issue((st + 2) & 3, (int64_t)(st + 2) * RK);
+        }
+        const char *at = As + (st & 3) * RTILEB, *bt = Bs + (st & 3) * RTILEB;
+#pragma unroll
+        for (int ks = 0; ks < RK / 16; ks++) {
+            typename T::vec8 av[BM], bv[BNB];
+#pragma unroll
+            for (int j = 0; j < BM; j++) av[j] = RingOperand<T, A_RM>::fetch(at, BM * wm + j, ks, lane);
+#pragma unroll
+            for (int i = 0; i < BNB; i++) bv[i] = RingOperand<T, B_RM>::fetch(bt, BNB * wn + i, ks, lane);
+#pragma unroll
+            for (int i = 0; i < BNB; i++)
+#pragma unroll
+                for (int j = 0; j < BM; j++) acc[i][j] = T::mfma32(av[j], bv[i], acc[i][j]);
+        }
+    }
+    store_tile<T, true>(g, acc, bz, m0, n0, wm, wn, lane);
+}
+
+template <typename T, bool A_RM, bool B_RM>
+int32_t launch_ring(const Gemm16Args &g, int64_t nb, hipStream_t st) {
+    auto kern = gemm16_ring_kernel<T, A_RM, B_RM>;
+    static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RING_SMEM));
+        attr_set = true;
+    }
+    dim3 grid((unsigned)((g.m + 255) / 256), (unsigned)((g.n + 255) / 256), (unsigned)nb);
+    hipLaunchKernelGGL(kern, grid, dim3(512), RING_SMEM, st, g);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
 }
 
 template <typename T, bool A_RM, bool B_RM, bool LARGE>
@@ -294,6 +456,12 @@ template <typename T>
 int32_t launch_t(const Gemm16Args &g, int transA, int transB, int64_t nb, hipStream_t st) {
     // the large tile when it still gives every CU a workgroup; the small one otherwise
     const int64_t big = ((g.m + 255) / 256) * ((g.n + 255) / 256) * nb;
+    static const bool no_ring = getenv("MI355ATTN_GEMM_NO_RING") != nullptr;   // A/B switch: the register-staged 256 x 256 kernel
+    if (g.m >= 256 && g.n >= 256 && big >= 256 && !no_ring) {
+        const bool a_rm = !transA, b_rm = transB != 0;
+        if (a_rm) return b_rm ? launch_ring<T, true, true>(g, nb, st) : launch_ring<T, true, false>(g, nb, st);
+        return b_rm ? launch_ring<T, false, true>(g, nb, st) : launch_ring<T, false, false>(g, nb, st);
+    }
     if (g.m >= 256 && g.n >= 256 && big >= 256) return launch_l<T, true>(g, transA, transB, nb, st);
     return launch_l<T, false>(g, transA, transB, nb, st);
 }
