@@ -295,17 +295,24 @@ __global__ __launch_bounds__(Shape<LARGE>::THREADS, LARGE ? 1 : 2) void gemm16_k
 // Both deliver k 8 hh .. 8 hh + 7 to half-wave hh, so any pair of layouts agrees.
 constexpr int RK = 32;                        // k per stage
 constexpr int RING = 4;
-constexpr int RTILEB = 256 * RK * 2;          // bytes per operand and stage
-constexpr size_t RING_SMEM = 2 * RING * RTILEB;
+template <bool LARGE>
+struct RingShape {
+    static constexpr int TILE = Shape<LARGE>::TILE;
+    static constexpr int TILEB = TILE * RK * 2;                // bytes per operand and stage: 16 KiB (8 KiB for the 128 x 128 shape)
+    static constexpr int ROWB = TILE * 2;                      // bytes per k-row of an RMAJ tile
+    static constexpr size_t SMEM = 2 * RING * TILEB;           // 128 KiB, one workgroup per CU (64 KiB, two)
+};
 
 __device__ inline int ring_kswz(int row) { return (row >> 2) & 3; }
 
-template <typename T, bool RM>
+template <typename T, bool RM, bool LARGE>
 struct RingOperand {
     typedef typename T::type t;
+    static constexpr int TILEB = RingShape<LARGE>::TILEB, ROWB = RingShape<LARGE>::ROWB;
+    static constexpr int CPR = ROWB / 16;   // 16-byte chunks per k-row of an RMAJ tile; a 1 KiB piece holds 64 / CPR k-rows
     i32x4_t rsrc;
     int voff[2];     // byte offsets of this lane's two pieces of a stage at k0 = 0 (0x80000000: outside the matrix)
-    int kpiece[2];   // KMAJ: first k of the piece within the stage (to drop pieces past k)
+    int kpiece[2];   // first k of the piece within the stage (to drop pieces past k)
     int kstep;       // bytes per unit of k0
     int64_t k;
     unsigned lds;    // LDS byte address of this wavefront's first piece in stage 0
@@ -319,11 +326,11 @@ struct RingOperand {
         lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char *)ring + wave * 2048;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            const int piece = 2 * wave + i;   // 16 pieces of 1 KiB per operand and stage
+            const int piece = 2 * wave + i;   // TILEB / 1024 pieces per operand and stage, two per wavefront
             if (RM) {
-                const int krow = 2 * piece + (lane >> 5), chunk = (lane & 31) ^ rmaj_swz(krow);
+                const int krow = (64 / CPR) * piece + lane / CPR, chunk = (lane % CPR) ^ rmaj_swz(krow);
                 kpiece[i] = krow;
-                voff[i] = row0 + 8 * chunk < rows ? (int)(((row0 + 8 * chunk) + krow * ld) * 2) : OOB;   // k-rows past k lie past the extent
+                voff[i] = row0 + 8 * chunk < rows ? (int)(((row0 + 8 * chunk) + krow * ld) * 2) : OOB;
             } else {
                 const int row = 16 * piece + (lane >> 2), chunk = (lane & 3) ^ ring_kswz(row);
                 kpiece[i] = 8 * chunk;
@@ -333,7 +340,7 @@ struct RingOperand {
     }
     // start the copy of the stage whose first k is k0 into ring position `pos`
     __device__ void issue(int pos, int64_t k0) const {
-        const unsigned dst = __builtin_amdgcn_readfirstlane(lds + pos * RTILEB);
+        const unsigned dst = __builtin_amdgcn_readfirstlane(lds + pos * TILEB);
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             int o = voff[i] == OOB ? OOB : voff[i] + (int)k0 * kstep;
@@ -347,9 +354,9 @@ struct RingOperand {
         if (RM) {
             const int vrow = 16 * ks + 8 * hh + ((lane & 15) >> 2);
             const int vchunk = 4 * blk + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), vsub = 8 * (lane & 1);
-            const char *src = tile + vrow * 512 + vsub;
+            const char *src = tile + vrow * ROWB + vsub;
             const typename T::vec4 lo = lds_tr4<T>(src + ((vchunk ^ rmaj_swz(vrow)) << 4));
-            const typename T::vec4 hi = lds_tr4<T>(src + 4 * 512 + ((vchunk ^ rmaj_swz(vrow + 4)) << 4));
+            const typename T::vec4 hi = lds_tr4<T>(src + 4 * ROWB + ((vchunk ^ rmaj_swz(vrow + 4)) << 4));
             return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         } else {
             const int row = 32 * blk + (lane & 31);
@@ -358,19 +365,19 @@ struct RingOperand {
     }
 };
 
-template <typename T, bool A_RM, bool B_RM>
-__global__ __launch_bounds__(512, 1) void gemm16_ring_kernel(Gemm16Args g) {
+template <typename T, bool A_RM, bool B_RM, bool LARGE>
+__global__ __launch_bounds__(Shape<LARGE>::THREADS, LARGE ? 1 : 2) void gemm16_ring_kernel(Gemm16Args g) {
     typedef typename T::type t;
-    typedef Shape<true> S;
-    constexpr int BM = S::BM, BNB = S::BNB;
+    typedef Shape<LARGE> S;
+    constexpr int BM = S::BM, BNB = S::BNB, RTILEB = RingShape<LARGE>::TILEB;
     extern __shared__ __attribute__((aligned(1024))) unsigned char gemm_smem[];
     char *As = (char *)gemm_smem, *Bs = As + RING * RTILEB;
     const MiTile tile = mi_gemm_tile_order(blockIdx.x + (int64_t)gridDim.x * (blockIdx.y + (int64_t)gridDim.y * blockIdx.z), gridDim.x, gridDim.y, gridDim.z);
     const int64_t bz = tile.batch, m0 = tile.m * S::TILE, n0 = tile.n * S::TILE;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave % S::WM, wn = wave / S::WM;
 
-    RingOperand<T, A_RM> a;
-    RingOperand<T, B_RM> b;
+    RingOperand<T, A_RM, LARGE> a;
+    RingOperand<T, B_RM, LARGE> b;
     a.init((const t *)g.A + bz * g.sA, g.lda, g.m, g.k, m0, As, wave, lane);
     b.init((const t *)g.B + bz * g.sB, g.ldb, g.n, g.k, n0, Bs, wave, lane);
 
@@ -381,8 +388,7 @@ __global__ __launch_bounds__(512, 1) void gemm16_ring_kernel(Gemm16Args g) {
         for (int j = 0; j < BM; j++) acc[i][j] = (floatx16_t){0};
 
     // Stage s lives in ring position s % 4.  An even stage starts with "stages s and s + 1 have landed everywhere and
-    // stages s - 2 and s - 1 are read by nobody any more"; every stage then requests stage s + 2 (past the last stage
-    // the pieces lie outside the matrices and arrive as zeros, which nothing reads).
+    // stages s - 2 and s - 1 are read by nobody any more"; every stage then requests stage s + 2.
     const int ns = (int)((g.k + RK - 1) / RK);
     a.issue(0, 0);
     b.issue(0, 0);
@@ -403,30 +409,39 @@ __global__ __launch_bounds__(512, 1) void gemm16_ring_kernel(Gemm16Args g) {
         for (int ks = 0; ks < RK / 16; ks++) {
             typename T::vec8 av[BM], bv[BNB];
 #pragma unroll
-            for (int j = 0; j < BM; j++) av[j] = RingOperand<T, A_RM>::fetch(at, BM * wm + j, ks, lane);
+            for (int j = 0; j < BM; j++) av[j] = RingOperand<T, A_RM, LARGE>::fetch(at, BM * wm + j, ks, lane);
 #pragma unroll
-            for (int i = 0; i < BNB; i++) bv[i] = RingOperand<T, B_RM>::fetch(bt, BNB * wn + i, ks, lane);
+            for (int i = 0; i < BNB; i++) bv[i] = RingOperand<T, B_RM, LARGE>::fetch(bt, BNB * wn + i, ks, lane);
 #pragma unroll
             for (int i = 0; i < BNB; i++)
 #pragma unroll
                 for (int j = 0; j < BM; j++) acc[i][j] = T::mfma32(av[j], bv[i], acc[i][j]);
         }
     }
-    store_tile<T, true>(g, acc, bz, m0, n0, wm, wn, lane);
+    store_tile<T, LARGE>(g, acc, bz, m0, n0, wm, wn, lane);
 }
 
-template <typename T, bool A_RM, bool B_RM>
+template <typename T, bool A_RM, bool B_RM, bool LARGE>
 int32_t launch_ring(const Gemm16Args &g, int64_t nb, hipStream_t st) {
-    auto kern = gemm16_ring_kernel<T, A_RM, B_RM>;
+    typedef Shape<LARGE> S;
+    auto kern = gemm16_ring_kernel<T, A_RM, B_RM, LARGE>;
+    constexpr size_t smem = RingShape<LARGE>::SMEM;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
     if (!attr_set) {
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)RING_SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    dim3 grid((unsigned)((g.m + 255) / 256), (unsigned)((g.n + 255) / 256), (unsigned)nb);
-    hipLaunchKernelGGL(kern, grid, dim3(512), RING_SMEM, st, g);
+    dim3 grid((unsigned)((g.m + S::TILE - 1) / S::TILE), (unsigned)((g.n + S::TILE - 1) / S::TILE), (unsigned)nb);
+    hipLaunchKernelGGL(kern, grid, dim3(S::THREADS), smem, st, g);
     MI_LAUNCH_CHECK();
     return MI_OK;
+}
+
+template <typename T, bool LARGE>
+int32_t launch_ring_l(const Gemm16Args &g, int transA, int transB, int64_t nb, hipStream_t st) {
+    const bool a_rm = !transA, b_rm = transB != 0;
+    if (a_rm) return b_rm ? launch_ring<T, true, true, LARGE>(g, nb, st) : launch_ring<T, true, false, LARGE>(g, nb, st);
+    return b_rm ? launch_ring<T, false, true, LARGE>(g, nb, st) : launch_ring<T, false, false, LARGE>(g, nb, st);
 }
 
 template <typename T, bool A_RM, bool B_RM, bool LARGE>
@@ -456,13 +471,11 @@ template <typename T>
 int32_t launch_t(const Gemm16Args &g, int transA, int transB, int64_t nb, hipStream_t st) {
     // the large tile when it still gives every CU a workgroup; the small one otherwise
     const int64_t big = ((g.m + 255) / 256) * ((g.n + 255) / 256) * nb;
-    static const bool no_ring = getenv("MI355ATTN_GEMM_NO_RING") != nullptr;   // A/B switch: the register-staged 256 x 256 kernel
-    if (g.m >= 256 && g.n >= 256 && big >= 256 && !no_ring) {
-        const bool a_rm = !transA, b_rm = transB != 0;
-        if (a_rm) return b_rm ? launch_ring<T, true, true>(g, nb, st) : launch_ring<T, true, false>(g, nb, st);
-        return b_rm ? launch_ring<T, false, true>(g, nb, st) : launch_ring<T, false, false>(g, nb, st);
-    }
-    if (g.m >= 256 && g.n >= 256 && big >= 256) return launch_l<T, true>(g, transA, transB, nb, st);
+    static const bool no_ring = getenv("MI355ATTN_GEMM_NO_RING") != nullptr;   // A/B switch: the register-staged kernels
+    const bool large = g.m >= 256 && g.n >= 256 && big >= 256;
+    // the ring kernel for the large shape only: at 128 x 128 it was measured level or behind the register-staged kernel
+    // (128 x 4096 x 4096 x 64: 593 against 637 TFLOP/s, 64 x 2048 x 2048 x 64: 252 / 290, 1024^3 x 4: 607 / 573)
+    if (large) return no_ring ? launch_l<T, true>(g, transA, transB, nb, st) : launch_ring_l<T, true>(g, transA, transB, nb, st);
     return launch_l<T, false>(g, transA, transB, nb, st);
 }
 
