@@ -111,3 +111,29 @@ def test_dropout_along_dims(nn, oracle, dtype, shape, dims):
     assert np.abs(got - ref).max() <= (1e-6 if dtype == "f32" else 2e-2) * np.abs(ref).max()
     if len(ds) == len(shape):     # every dimension owns its decisions: the same as dims = :
         assert np.array_equal(got, nn.dropout(nn.DeviceArray.from_numpy(x, dtype), p, seed=seed).to_numpy())
+
+
+@pytest.mark.parametrize("dtype,E,H,Lq,Lkv", [("bf16", 256, 2, 300, 520), ("f16", 128, 2, 140, 332)])
+def test_fused_dropout_with_context_lengths(nn, oracle, dtype, E, H, Lq, Lkv):
+    """A key-padding mask that keeps a prefix of the keys (a context length per batch element) together with dropout:
+    the pairs with a length run the kernels without mask code on that many keys, and the keep decisions are still
+    those of the weight's position in the full (Lkv, Lq, H, B) array."""
+    rng = np.random.default_rng(E + Lq)
+    B, p, seed = 3, 0.2, 77
+    q = round_to(rng.standard_normal((E, Lq, B)) * 0.5, dtype)
+    k = round_to(rng.standard_normal((E, Lkv, B)) * 0.5, dtype)
+    v = round_to(rng.standard_normal((E, Lkv, B)), dtype)
+    lens = [Lkv, Lkv - 37, 64]
+    mask = np.zeros((Lkv, 1, 1, B), dtype=bool)
+    for b, n in enumerate(lens):
+        mask[:n, 0, 0, b] = True
+    D = nn.DeviceArray.from_numpy
+    y, _ = nn.dot_product_attention(D(q, dtype), D(k, dtype), D(v, dtype), mask=D(mask), nheads=H, fdrop=nn.Dropout(p, seed),
+                                    return_weights=False)
+    assert nn.last_attention_kernel() == "flash16"
+    _, a_ref = oracle.attention_f64(q, k, v, None, np.broadcast_to(mask, (Lkv, Lq, H, B)).copy(), H)
+    keep = oracle.dropout_keep_mask(a_ref.shape, p, seed)
+    a_ref = np.where(keep, a_ref / (1.0 - np.float32(p)), 0.0)
+    Dh = E // H
+    y_ref = np.einsum("jihb,dhjb->dhib", a_ref, v.reshape(Dh, H, Lkv, B, order="F")).reshape(E, Lq, B, order="F")
+    assert rel_err(y.to_numpy(), y_ref) <= 1e-2
