@@ -34,7 +34,7 @@ DOMINANT_KERNEL = {"c1": "flash32_kernel", "c2": "flash32_kernel", "c3": "flash1
                    # a gradient step is three kernels (dq, dk, dv): every row of the workload whose name contains "bwd"
                    "bwd": "bwd", "bwd_f32": "bwd", "softmax": "softmax", "logsoftmax": "softmax", "softmax_dims2": "softmax",
                    "batched_mul": "gemm", "batched_mul_f32": "gemm",
-                   "dense_mask": "flash16_fast_kernel<false, true>"}
+                   "dense_mask": "flash16_fast_kernel<false, true"}
 
 
 def measured_traffic(key):
