@@ -150,6 +150,29 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
 #pragma unroll
             for (int e = 0; e < EPL; e++) o[n][e] *= resc;
         }
+        // fused dropout (src/attention.jl:126 with fdrop = dropout; calls without returned weights, Lkv a multiple of 4):
+        // the row sum takes the weight as the softmax gives it, the value product takes it times the keep factor of
+        // weight (key, query, head, batch) in the shared counter stream.  A chunk starts at a multiple of 8 keys, so it
+        // is two hash groups of four; the hashes hide under the K / V stream.
+        float fac[NQ][ROWS];
+#pragma unroll
+        for (int n = 0; n < NQ; n++)
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) fac[n][r] = 1.0f;
+        if (p.drop_thresh != 0) {
+            const int64_t hd = lane_ok ? f / D : 0;
+#pragma unroll
+            for (int n = 0; n < NQ; n++) {
+                const int64_t qi = q0 + n < p.Lq ? q0 + n : p.Lq - 1;
+                const uint64_t i0 = (uint64_t)(j + p.Lkv * (qi + p.Lq * (hd + p.H * b)));
+#pragma unroll
+                for (int g = 0; g < ROWS / 4; g++) {
+                    const uint64_t bits = mi_dropout_group_bits(p.drop_key, (i0 + 4 * g) >> 2);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) fac[n][4 * g + e] = mi_dropout_keep_in(bits, e, p.drop_thresh) ? p.drop_scale : 0.0f;
+                }
+            }
+        }
 #pragma unroll
         for (int r = 0; r < ROWS; r++) {
             float vf[EPL];
@@ -158,8 +181,9 @@ __global__ __launch_bounds__(256) void decode_split_kernel(DecodeArgs a) {
             for (int n = 0; n < NQ; n++) {
                 const float pr = mi_exp2((s[n][r] - mref[n]) * a.c);
                 l[n] += pr;
+                const float pd = pr * fac[n][r];
 #pragma unroll
-                for (int e = 0; e < EPL; e++) o[n][e] = fmaf(pr, vf[e], o[n][e]);
+                for (int e = 0; e < EPL; e++) o[n][e] = fmaf(pd, vf[e], o[n][e]);
             }
         }
         if (SCORES) {
@@ -300,7 +324,8 @@ int pick_nsplit(const AttnParams &p) {
 }  // namespace
 
 bool attention_decode_supports(const AttnParams &p) {
-    if (p.Lq < 1 || p.Lq > 4 || p.bias || p.causal || !p.out || p.drop_thresh || p.stats) return false;   // saved statistics: the tiled kernels write them
+    if (p.Lq < 1 || p.Lq > 4 || p.bias || p.causal || !p.out || p.stats) return false;   // saved statistics: the tiled kernels write them
+    if (p.drop_thresh && (p.weights || (p.Lkv & 3) != 0)) return false;   // fused dropout: in the streaming kernel only, whole hash groups
     // two to four queries: without the weights, and with a mask only when it does not depend on the query
     if (p.Lq > 1 && (p.weights || (p.mask && p.mask_strides[1] != 0) || p.B * p.Lq > 65535)) return false;
     if (p.weights && p.H * p.B > 65535) return false;

@@ -47,6 +47,9 @@ CASES = [
     ("f16", 256, 520, 1300, 1, 2, False, False, "flash16"),     # its unrolled steady loop (more than four key tiles)
     ("bf16", 128, 700, 700, 2, 2, True, False, "flash16"),      # head dim 64, causal, steady loop and diagonal steps
     ("bf16", 256, 100, 301, 1, 2, False, False, "flash16"),     # key count not a multiple of 4: the general kernel
+    ("bf16", 512, 1, 1500, 2, 4, False, False, "decode"),       # one query: the streaming kernels, hashes under the K / V stream
+    ("f16", 256, 3, 2048, 2, 2, False, False, "decode"),        # a few queries carried through one stream
+    ("bf16", 512, 1, 1501, 2, 4, False, False, "flash16"),      # one query, key count not a multiple of 4
 ]
 
 
