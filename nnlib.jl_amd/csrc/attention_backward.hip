@@ -107,7 +107,7 @@ static int32_t resolve_bwd(const mi_attn_bwd_desc *d, mi_attn_bwd_desc *eff, Rec
     return MI_OK;
 }
 
-MI_API int32_t mi_attention_bwd_plan(const mi_attn_bwd_desc *d, int32_t *kernel, size_t *workspace_bytes) {
+static int32_t bwd_plan_impl(const mi_attn_bwd_desc *d, int32_t *kernel, size_t *workspace_bytes) {
     AttnBwdParams bp;
     int32_t rc = validate_bwd(d, &bp);
     if (rc != MI_OK) return rc;
@@ -125,7 +125,7 @@ MI_API int32_t mi_attention_bwd_plan(const mi_attn_bwd_desc *d, int32_t *kernel,
     return MI_OK;
 }
 
-MI_API int32_t mi_attention_bwd(const mi_attn_bwd_desc *d, mi_stream s) {
+static int32_t bwd_impl(const mi_attn_bwd_desc *d, mi_stream s, int64_t scale_D) {
     AttnBwdParams bp;
     int32_t rc = validate_bwd(d, &bp);
     if (rc != MI_OK) return rc;
@@ -135,7 +135,7 @@ MI_API int32_t mi_attention_bwd(const mi_attn_bwd_desc *d, mi_stream s) {
     if (rc != MI_OK) return rc;
     if (re.on) {
         size_t need = 0;
-        rc = mi_attention_bwd_plan(d, nullptr, &need);
+        rc = bwd_plan_impl(d, nullptr, &need);
         if (rc != MI_OK) return rc;
         if (!d->workspace || d->workspace_bytes < need)
             return mi_set_error(MI_EWORKSPACE, "mi_attention_bwd: workspace of %zu bytes required, %zu given", need,
@@ -162,6 +162,7 @@ MI_API int32_t mi_attention_bwd(const mi_attn_bwd_desc *d, mi_stream s) {
     d = &eff;
     rc = validate_bwd(d, &bp);
     if (rc != MI_OK) return rc;
+    bp.p.scale_D = scale_D;
     const AttnParams &p = bp.p;
     hipStream_t st = (hipStream_t)s;
     const size_t es = mi_dtype_size(p.dtype);
@@ -183,4 +184,146 @@ MI_API int32_t mi_attention_bwd(const mi_attn_bwd_desc *d, mi_stream s) {
     bp.stats = (float *)d->workspace;
     bp.have_stats = 0;
     return launch_attention_bwd_generic(bp, st);
+}
+
+// ---- different head dims for q / k and for v -------------------------------------------------------------------------
+// The MFMA gradient kernels take one head dim.  A call whose q / k head dim D differs from v's Dv (src/attention.jl:55-78
+// allows it, and the forward kernels take it) used to drop to the generic kernels, hundreds of times slower.  Instead the
+// narrower side is copied into the workspace with its heads zero-padded to the wider dim: v, dy and the forward result
+// when Dv < D (their padding contributes nothing to dP and delta, and the padded dV columns are dropped on the way back),
+// q and k when D < Dv (zero features add nothing to the scores; the logits keep their scale 1 / sqrt(D) through
+// AttnParams::scale_D; the padded dQ / dK columns are dropped).  Cost: copies of O(L E) next to work of O(L^2 E).
+template <typename T>
+__global__ __launch_bounds__(256) void pad_heads_kernel(const T *src, T *dst, int64_t rows, int64_t H, int64_t d_src, int64_t d_dst) {
+    // 16-byte pieces; dst[row][h][x] = x < d_src ? src[row][h][x] : 0 for x < d_dst (narrowing when d_dst < d_src)
+    constexpr int V = 16 / (int)sizeof(T);
+    const int64_t per_row = H * (d_dst / V), n = rows * per_row;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const int64_t row = i / per_row, c = i % per_row, h = c / (d_dst / V), x = (c % (d_dst / V)) * V;
+        u32x4_t v = {0, 0, 0, 0};
+        if (x < d_src) v = *(const u32x4_t *)(src + (row * H + h) * d_src + x);
+        *(u32x4_t *)(dst + (row * H + h) * d_dst + x) = v;
+    }
+}
+
+static int32_t launch_pad_heads(int32_t dtype, const void *src, void *dst, int64_t rows, int64_t H, int64_t d_src, int64_t d_dst, hipStream_t st) {
+    const int64_t v = 16 / (int64_t)mi_dtype_size(dtype), n = rows * H * (d_dst / v);
+    if (n == 0) return MI_OK;
+    const unsigned grid = (unsigned)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
+    if (mi_dtype_size(dtype) == 2) hipLaunchKernelGGL(pad_heads_kernel<uint16_t>, dim3(grid), dim3(256), 0, st, (const uint16_t *)src, (uint16_t *)dst, rows, H, d_src, d_dst);
+    else hipLaunchKernelGGL(pad_heads_kernel<uint32_t>, dim3(grid), dim3(256), 0, st, (const uint32_t *)src, (uint32_t *)dst, rows, H, d_src, d_dst);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
+struct PadPlan {
+    bool on = false, pad_v = false;   // pad_v: v / dy / x are the narrow side (Dv < D), else q / k
+    int64_t Dmax = 0;
+    size_t in_bytes[3] = {0, 0, 0}, out_bytes[2] = {0, 0};   // padded inputs (v, dy, x | q, k) and outputs (dv | dq, dk)
+    size_t total = 0;
+};
+
+static PadPlan plan_padding(const mi_attn_bwd_desc *d) {
+    PadPlan pp;
+    AttnBwdParams bp;
+    if (!d || !d->fwd.out || d->dweights || (d->fwd.flags & MI_ATTN_FORCE_GENERIC) || validate_bwd(d, &bp) != MI_OK) return pp;
+    const AttnParams &p = bp.p;
+    if (p.D == p.Dv || p.Lq == 0 || p.Lkv == 0 || p.B == 0 || p.E == 0 || p.Ev == 0) return pp;
+    const bool half = p.dtype == MI_F16 || p.dtype == MI_BF16;
+    if (!half && p.dtype != MI_F32) return pp;
+    const int64_t v = half ? 8 : 4, cap = half ? 256 : 128, dmax = p.D > p.Dv ? p.D : p.Dv;
+    if ((p.D % v) || (p.Dv % v) || dmax > cap) return pp;
+    const auto al = [](const void *x) { return (((uintptr_t)x) & 15) == 0; };   // the copies move 16-byte pieces
+    if (!al(p.q) || !al(p.k) || !al(p.v) || !al(p.out) || !al(d->dout) || !al(d->dq) || !al(d->dk) || !al(d->dv)) return pp;
+    const size_t es = mi_dtype_size(p.dtype), eq = (size_t)(dmax * p.H) * es;
+    pp.on = true;
+    pp.pad_v = p.Dv < p.D;
+    pp.Dmax = dmax;
+    if (pp.pad_v) {
+        pp.in_bytes[0] = align256(eq * (size_t)(p.Lkv * p.B));                 // v
+        pp.in_bytes[1] = pp.in_bytes[2] = align256(eq * (size_t)(p.Lq * p.B)); // dy, x
+        pp.out_bytes[0] = bp.dv ? align256(eq * (size_t)(p.Lkv * p.B)) : 0;    // dv
+    } else {
+        pp.in_bytes[0] = align256(eq * (size_t)(p.Lq * p.B));                  // q
+        pp.in_bytes[1] = align256(eq * (size_t)(p.Lkv * p.B));                 // k
+        pp.out_bytes[0] = bp.dq ? align256(eq * (size_t)(p.Lq * p.B)) : 0;     // dq
+        pp.out_bytes[1] = bp.dk ? align256(eq * (size_t)(p.Lkv * p.B)) : 0;    // dk
+    }
+    pp.total = pp.in_bytes[0] + pp.in_bytes[1] + pp.in_bytes[2] + pp.out_bytes[0] + pp.out_bytes[1];
+    return pp;
+}
+
+// the descriptor of the padded call; `base` = start of the padded buffers (null while planning: stand-in pointers)
+static mi_attn_bwd_desc padded_desc(const mi_attn_bwd_desc *d, const PadPlan &pp, char *base) {
+    mi_attn_bwd_desc e = *d;
+    char *at = base ? base : (char *)(uintptr_t)4096;   // planning looks at alignment only
+    char *in0 = at, *in1 = in0 + pp.in_bytes[0], *in2 = in1 + pp.in_bytes[1], *out0 = in2 + pp.in_bytes[2], *out1 = out0 + pp.out_bytes[0];
+    if (pp.pad_v) {
+        e.fwd.Ev = pp.Dmax * d->fwd.H;
+        e.fwd.v = in0;
+        e.dout = in1;
+        e.fwd.out = in2;
+        if (d->dv) e.dv = out0;
+    } else {
+        e.fwd.E = pp.Dmax * d->fwd.H;
+        e.fwd.q = in0;
+        e.fwd.k = in1;
+        if (d->dq) e.dq = out0;
+        if (d->dk) e.dk = out1;
+    }
+    e.workspace = base ? base + pp.total : nullptr;
+    e.workspace_bytes = base && d->workspace_bytes > pp.total ? d->workspace_bytes - pp.total : 0;
+    return e;
+}
+
+MI_API int32_t mi_attention_bwd_plan(const mi_attn_bwd_desc *d, int32_t *kernel, size_t *workspace_bytes) {
+    const PadPlan pp = plan_padding(d);
+    if (!pp.on) return bwd_plan_impl(d, kernel, workspace_bytes);
+    const mi_attn_bwd_desc e = padded_desc(d, pp, nullptr);
+    size_t ws = 0;
+    int32_t k = 0;
+    const int32_t rc = bwd_plan_impl(&e, &k, &ws);
+    if (rc != MI_OK) return rc;
+    if (k == MI_ATTN_KERNEL_GENERIC) return bwd_plan_impl(d, kernel, workspace_bytes);   // padding buys nothing there
+    if (kernel) *kernel = k;
+    if (workspace_bytes) *workspace_bytes = pp.total + ws;
+    return MI_OK;
+}
+
+MI_API int32_t mi_attention_bwd(const mi_attn_bwd_desc *d, mi_stream s) {
+    const PadPlan pp = plan_padding(d);
+    if (pp.on) {
+        size_t need = 0;
+        int32_t k = 0;
+        int32_t rc = mi_attention_bwd_plan(d, &k, &need);
+        if (rc != MI_OK) return rc;
+        if (k != MI_ATTN_KERNEL_GENERIC) {
+            if (!d->workspace || d->workspace_bytes < need)
+                return mi_set_error(MI_EWORKSPACE, "mi_attention_bwd: workspace of %zu bytes required, %zu given", need,
+                                    d->workspace ? d->workspace_bytes : (size_t)0);
+            if ((((uintptr_t)d->workspace) & 255) != 0)
+                return mi_set_error(MI_EWORKSPACE, "mi_attention_bwd: with different head dims for q / k and v the workspace must be 256-byte aligned");
+            const mi_attn_bwd_desc e = padded_desc(d, pp, (char *)d->workspace);
+            hipStream_t st = (hipStream_t)s;
+            const mi_attn_desc &f = d->fwd;
+            const int64_t D = f.E / f.H, Dv = f.Ev / f.H, rq = f.Lq * f.B, rk = f.Lkv * f.B;
+            if (pp.pad_v) {
+                if ((rc = launch_pad_heads(f.dtype, f.v, (void *)e.fwd.v, rk, f.H, Dv, pp.Dmax, st)) != MI_OK) return rc;
+                if ((rc = launch_pad_heads(f.dtype, d->dout, (void *)e.dout, rq, f.H, Dv, pp.Dmax, st)) != MI_OK) return rc;
+                if ((rc = launch_pad_heads(f.dtype, f.out, e.fwd.out, rq, f.H, Dv, pp.Dmax, st)) != MI_OK) return rc;
+            } else {
+                if ((rc = launch_pad_heads(f.dtype, f.q, (void *)e.fwd.q, rq, f.H, D, pp.Dmax, st)) != MI_OK) return rc;
+                if ((rc = launch_pad_heads(f.dtype, f.k, (void *)e.fwd.k, rk, f.H, D, pp.Dmax, st)) != MI_OK) return rc;
+            }
+            if ((rc = bwd_impl(&e, s, D)) != MI_OK) return rc;
+            if (pp.pad_v) {
+                if (d->dv && (rc = launch_pad_heads(f.dtype, e.dv, d->dv, rk, f.H, pp.Dmax, Dv, st)) != MI_OK) return rc;
+            } else {
+                if (d->dq && (rc = launch_pad_heads(f.dtype, e.dq, d->dq, rq, f.H, pp.Dmax, D, st)) != MI_OK) return rc;
+                if (d->dk && (rc = launch_pad_heads(f.dtype, e.dk, d->dk, rk, f.H, pp.Dmax, D, st)) != MI_OK) return rc;
+            }
+            return MI_OK;
+        }
+    }
+    return bwd_impl(d, s, 0);
 }

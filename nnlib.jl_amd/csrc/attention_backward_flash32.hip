@@ -1131,7 +1131,7 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp_in, hipStream_t st)
     a.p.weights = nullptr;
     a.p.workspace = nullptr;
     a.p.stats = nullptr;
-    a.cn = 1.0f / sqrtf((float)bp.p.D);
+    a.cn = 1.0f / sqrtf((float)(bp.p.scale_D ? bp.p.scale_D : bp.p.D));
     a.c = MI_LOG2E * a.cn;
     a.n_qtiles = (int32_t)((bp.p.Lq + 127) / 128);
     a.nsplit = 1;

@@ -23,6 +23,9 @@ struct AttnParams {
     // and the same for the packed dense mask of the pipelined kernel: a caller whose workspace cannot hold it gets the
     // general kernel, which reads the mask as it is
     bool lean_workspace = false;
+    // gradient kernels: the head dim the logits are scaled by (1 / sqrt) when it is not D, i.e. when q and k arrive
+    // zero-padded to the head dim of v (attention_backward.hip pads the narrower of the two); 0: D
+    int64_t scale_D = 0;
 };
 
 // A dense mask packed for the software-pipelined forward kernel (attention.hip: pack_mask_words_kernel): one 16-byte

@@ -580,3 +580,16 @@ def test_float32_gradient_with_256_query_workgroups(nn, oracle, mask_kind, Lq, L
     half of the last workgroup, whose rows reach past the padded statistics planes."""
     _run(nn, oracle, "f32", 512, 512, Lq, Lkv, (16,), 8, mask_kind=mask_kind, saved=saved, scale=0.5, seed=Lq, expect="flash32")
     _run(nn, oracle, "f32", 256, 256, Lq, Lkv, (16,), 8, mask_kind=mask_kind, saved=saved, scale=0.5, seed=Lq + 1, expect="flash32")
+
+
+@pytest.mark.parametrize("dtype,D,Dv", [("bf16", 128, 64), ("bf16", 64, 128), ("f16", 40, 96), ("f16", 256, 64), ("f32", 32, 64), ("f32", 128, 36)])
+@pytest.mark.parametrize("mask_kind,saved", [(None, True), ("causal", False), ("random", True)])
+def test_different_head_dims_for_qk_and_v(nn, oracle, dtype, D, Dv, mask_kind, saved):
+    """q / k and v may have different head dims (src/attention.jl:55-78 only asks for divisibility by nheads and equal
+    q / k dims).  The MFMA gradient kernels take one head dim: the library zero-pads the narrower side in its workspace
+    and drops the padded gradient columns, and the logits keep the scale of the q / k head dim."""
+    H = 2
+    Lq = 150
+    Lkv = Lq if mask_kind == "causal" else 210
+    _run(nn, oracle, dtype, D * H, Dv * H, Lq, Lkv, (2,), H, mask_kind=mask_kind, saved=saved, scale=0.7, seed=D + Dv,
+         expect="flash32" if dtype == "f32" else "flash16")
