@@ -214,7 +214,8 @@ int32_t mi_attention_fwd_static(const mi_attn_desc *desc, mi_stream stream);
  *   dq, dk, dv : gradients with the shapes of q, k, v, `dtype`; any may be NULL (not computed).
  *   dbias    : NULL, or FLOAT32 array addressed with fwd.bias_strides; the gradient is ADDED into
  *              it (dims with stride 0 receive the sum over that dim), so the caller zero-fills it.
- *   workspace: at least mi_attention_bwd_plan()'s size, 16-byte aligned.
+ *   workspace: at least mi_attention_bwd_plan()'s size, 16-byte aligned (256-byte aligned when q / k and v have
+ *              different head dims: the narrower side is zero-padded inside it for the matrix-core kernels).
  * A query whose keys are all dropped has NaN weights in the forward pass and NaN gradients here.
  */
 typedef struct mi_attn_bwd_desc {
