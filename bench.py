@@ -29,7 +29,7 @@ HBM_BOUND = ("c4", "c5")                                # workloads priced again
 # commands and the copy-kernel calibration), and are read from there so that the figure and its source travel together.
 MIB = 1 << 20
 TRAFFIC_FILE = os.path.join("profiles", "hbm_traffic_fetch_write_size.md")
-DOMINANT_KERNEL = {"c1": "flash32_kernel", "c2": "flash32_kernel", "c3": "flash16_fast_kernel", "c4": "flash16_kernel",
+DOMINANT_KERNEL = {"c1": "flash32_resident", "c2": "flash32_kernel", "c3": "flash16_fast_kernel", "c4": "flash16_kernel",
                    "c5": "decode_split_kernel",
                    # a gradient step is three kernels (dq, dk, dv): every row of the workload whose name contains "bwd"
                    "bwd": "bwd", "bwd_f32": "bwd", "softmax": "softmax", "logsoftmax": "softmax", "softmax_dims2": "softmax",

@@ -188,8 +188,9 @@ __device__ inline floatx16_t mfma_split(const plane8 (&a)[3], const plane8 (&b)[
 }
 
 // S^T = K Q^T of one 64-key tile whose planes sit at LDS address Ks: s[query block][key block]
-template <int D, int QB>
-__device__ inline void scores32s(const Frag32S<D, QB> &f, unsigned Ks, floatx16_t (&s)[QB][2]) {
+// (KBLK = 1: of the 32-key block whose first row sits at Ks)
+template <int D, int QB, int KBLK = 2>
+__device__ inline void scores32s(const Frag32S<D, QB> &f, unsigned Ks, floatx16_t (&s)[QB][KBLK]) {
     typedef CfgS<D> C;
     constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB;
     typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
@@ -197,14 +198,14 @@ __device__ inline void scores32s(const Frag32S<D, QB> &f, unsigned Ks, floatx16_
 #pragma unroll
     for (int qb = 0; qb < QB; qb++)
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) s[qb][kb] = (floatx16_t){0};
+        for (int kb = 0; kb < KBLK; kb++) s[qb][kb] = (floatx16_t){0};
     // lane's K operand: row r (+32 per key block), chunk 2t + hh, in each plane
     const unsigned kt = Ks + (unsigned)r * ROWB;
     const int ksw = C::swz(r);
 #pragma unroll
     for (int t = 0; t < D / 16; t++)
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+        for (int kb = 0; kb < KBLK; kb++) {
             plane8 ka[3];
 #pragma unroll
             for (int q = 0; q < 3; q++)
@@ -217,9 +218,10 @@ __device__ inline void scores32s(const Frag32S<D, QB> &f, unsigned Ks, floatx16_
         }
 }
 
-// O^T += V^T P^T for one 64-key tile: the weights in s (accumulator layout), V's planes at LDS address Vs
-template <int D, int QB>
-__device__ inline void weights_times_values32s(Frag32S<D, QB> &f, unsigned Vs, const floatx16_t (&s)[QB][2]) {
+// O^T += V^T P^T for one 64-key tile (KBLK = 1: one 32-key block): the weights in s (accumulator layout), V's planes
+// (the block's first row) at LDS address Vs
+template <int D, int QB, int KBLK = 2>
+__device__ inline void weights_times_values32s(Frag32S<D, QB> &f, unsigned Vs, const floatx16_t (&s)[QB][KBLK]) {
     typedef CfgS<D> C;
     constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB;
     const int lane = threadIdx.x & 63, hh = lane >> 5;
@@ -230,7 +232,7 @@ __device__ inline void weights_times_values32s(Frag32S<D, QB> &f, unsigned Vs, c
     const unsigned vt = Vs + (unsigned)vrow * ROWB + vsub;
     const int vsw_lo = C::swz(vrow), vsw_hi = C::swz(vrow + 8);
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++)
+    for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             plane8 pk[QB][3];
@@ -520,6 +522,27 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
 // weights, and the workgroup meets at two barriers (K in LDS; V in LDS, split under the score products).
 constexpr int RES_TILES = 2;
 
+// The reference divides q by sqrt(D) first (src/attention.jl:118).  When sqrt(D) is a power of two (D = 16, 64, 256)
+// the product with its reciprocal is that quotient bit for bit, at a tenth of the instructions of a division.
+__device__ inline bool sqrt_is_power_of_two(float sq) { return (__builtin_bit_cast(uint32_t, sq) & 0x7fffffu) == 0; }
+template <int D>
+__device__ inline void scale_queries(floatx4_t (&q4)[D / 16][2], float head_dim) {
+    const float sq = sqrtf(head_dim), inv_sq = 1.0f / sq;
+    if (sqrt_is_power_of_two(sq)) {
+#pragma unroll
+        for (int t = 0; t < D / 16; t++)
+#pragma unroll
+            for (int half = 0; half < 2; half++) q4[t][half] *= inv_sq;
+    } else {
+#pragma unroll
+        for (int t = 0; t < D / 16; t++)
+#pragma unroll
+            for (int half = 0; half < 2; half++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) q4[t][half][e] /= sq;
+    }
+}
+
 template <int D, bool CAUSAL, bool EXTRAS>
 __global__ __launch_bounds__(256, 1) void flash32_resident_kernel(FlashArgs a) {
     typedef CfgS<D> C;
@@ -599,7 +622,7 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_kernel(FlashArgs a) {
         if (t < n_tiles) store_tile(Kp + t * TILEB, kreg[t]);
     Frag32S<D, 1> f;
     {
-        const float sq = sqrtf((float)p.D);   // the reference divides q by sqrt(D) first (src/attention.jl:118)
+        scale_queries<D>(q4, (float)p.D);
         uint32_t qw[3][D / 16][4];
 #pragma unroll
         for (int t = 0; t < D / 16; t++)
@@ -608,7 +631,7 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_kernel(FlashArgs a) {
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     uint32_t w[3];
-                    const float x0 = q4[t][half][2 * j] / sq, x1 = q4[t][half][2 * j + 1] / sq;
+                    const float x0 = q4[t][half][2 * j], x1 = q4[t][half][2 * j + 1];
                     if (split3_pair(x0, x1, w[0], w[1], w[2])) split3_pair_guarded(x0, x1, w[0], w[1], w[2]);
 #pragma unroll
                     for (int q = 0; q < 3; q++) qw[q][t][2 * half + j] = w[q];
@@ -757,7 +780,7 @@ __global__ __launch_bounds__(512, 1) void flash32_resident_pair_kernel(FlashArgs
         if (t < n_tiles) store_tile(Kp + t * TILEB, kreg[t]);
     Frag32S<D, 1> f;
     {
-        const float sq = sqrtf((float)p.D);   // the reference divides q by sqrt(D) first (src/attention.jl:118)
+        scale_queries<D>(q4, (float)p.D);
         uint32_t qw3[3][D / 16][4];
 #pragma unroll
         for (int t = 0; t < D / 16; t++)
@@ -766,7 +789,7 @@ __global__ __launch_bounds__(512, 1) void flash32_resident_pair_kernel(FlashArgs
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     uint32_t w[3];
-                    const float x0 = q4[t][half][2 * j] / sq, x1 = q4[t][half][2 * j + 1] / sq;
+                    const float x0 = q4[t][half][2 * j], x1 = q4[t][half][2 * j + 1];
                     if (split3_pair(x0, x1, w[0], w[1], w[2])) split3_pair_guarded(x0, x1, w[0], w[1], w[2]);
 #pragma unroll
                     for (int q = 0; q < 3; q++) qw3[q][t][2 * half + j] = w[q];
@@ -852,10 +875,206 @@ __global__ __launch_bounds__(512, 1) void flash32_resident_pair_kernel(FlashArgs
     }
 }
 
+// The same for calls that leave most of the chip idle (few (head, batch) pairs and queries: C1 has 32 pairs of 128
+// queries): one workgroup per 32-query block, four wavefronts, one per 32-key block.  A wavefront has a quarter of a
+// query block's score products, softmax arithmetic, weight stores and value products; the price is that every
+// workgroup splits K and V of its pair into planes for itself.  The four exchange their row statistics (m, l)
+// after the first phase and add up their partial outputs at the end, through LDS.
+template <int D, bool CAUSAL, bool EXTRAS>
+__global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs a) {
+    typedef CfgS<D> C;
+    constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB, CHUNKS = C::CHUNKS, TILEB = C::TILEB;
+    constexpr int XT = EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE;
+    static_assert(RES_TILES == 2, "four 32-key blocks");
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char flash_smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem;
+    // K tiles (later the partial outputs), V tiles, weight staging, exchanged statistics
+    const unsigned Kp = lds0, Vp = lds0 + 2 * TILEB;
+    float *xstat = (float *)(flash_smem + 4 * TILEB + 4 * FLASH_WSTAGE_BYTES);   // [4 wavefronts][32 rows][2]
+    float *xout = (float *)flash_smem;                                           // [4 wavefronts][D / 2 registers][64 lanes]
+    constexpr int QPLANEB = 32 * ROWB, QCHUNKS = 32 * D / 4 / 256;
+    const unsigned Qp = lds0 + 4 * TILEB + 4 * FLASH_WSTAGE_BYTES + 4 * 32 * 2 * (unsigned)sizeof(float);   // the query block's planes
+    typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
+    typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t n_qblocks = (p.Lq + 31) / 32;
+    const int64_t hb = blockIdx.x % HB, qblk = n_qblocks - 1 - blockIdx.x / HB;
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t iw = qblk * 32, qi = iw + r;
+    int64_t kv_end = p.Lkv;
+    if (CAUSAL && iw + 32 < kv_end) kv_end = iw + 32;
+    const int n_tiles = (int)((kv_end + BN - 1) / BN);   // 1 or 2: checked by the host
+    const bool do_pv = p.out != nullptr;
+
+    // ---- every load of the call: K, the queries, V
+    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
+    const float *vbase = do_pv ? (const float *)p.v + p.Ev * (p.Lkv * b) + p.Dv * h : nullptr;
+    const float *qbase = (const float *)p.q + p.E * (p.Lq * b) + p.D * h;
+    const int dqk = (int)p.D, dv = (int)p.Dv;
+    floatx4_t kreg[2][CHUNKS], vreg[2][CHUNKS], qreg[QCHUNKS];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            const int64_t row = (int64_t)t * BN + c / (D / 4);
+            const int col = (c % (D / 4)) * 4;
+            kreg[t][u] = ldg16f(kbase + p.E * row + col, t < n_tiles && row < p.Lkv && col < dqk);
+        }
+#pragma unroll
+    for (int u = 0; u < QCHUNKS; u++) {   // the four wavefronts share the query block: a quarter each
+        const int c = tid + 256 * u;
+        const int64_t row = iw + c / (D / 4);
+        const int col = (c % (D / 4)) * 4;
+        qreg[u] = ldg16f(qbase + p.E * row + col, row < p.Lq && col < dqk);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            const int64_t row = (int64_t)t * BN + c / (D / 4);
+            const int col = (c % (D / 4)) * 4;
+            vreg[t][u] = ldg16f(vbase + p.Ev * row + col, do_pv && t < n_tiles && row < p.Lkv && col < dv);
+        }
+
+    auto store_split = [&](unsigned at_tile, int row, int col, const floatx4_t &x, int planeb) {
+        uint32_t pl[3][2];
+        const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        if (odd) {   // an Inf or NaN in the chunk (rare)
+            split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+            split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        }
+        const unsigned at = at_tile + (unsigned)row * ROWB + (unsigned)((((col >> 3) ^ C::swz(row)) << 4) + (col & 7) * 2);
+#pragma unroll
+        for (int q = 0; q < 3; q++) *(lds8_t)(uintptr_t)(at + q * planeb) = (u32x2_t){pl[q][0], pl[q][1]};
+    };
+    auto store_tile = [&](unsigned at_tile, const floatx4_t (&reg)[CHUNKS]) {
+#pragma unroll
+        for (int u = 0; u < CHUNKS; u++) {
+            const int c = tid + 256 * u;
+            store_split(at_tile, c / (D / 4), (c % (D / 4)) * 4, reg[u], PLANEB);
+        }
+    };
+
+    // ---- K and the scaled queries into planes in LDS
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+        if (t < n_tiles) store_tile(Kp + t * TILEB, kreg[t]);
+    {
+        // q / sqrt(D) as the reference has it (see scale_queries)
+        const float sq = sqrtf((float)p.D), inv_sq = 1.0f / sq;
+        if (sqrt_is_power_of_two(sq)) {
+#pragma unroll
+            for (int u = 0; u < QCHUNKS; u++) qreg[u] *= inv_sq;
+        } else {
+#pragma unroll
+            for (int u = 0; u < QCHUNKS; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) qreg[u][e] /= sq;
+        }
+#pragma unroll
+        for (int u = 0; u < QCHUNKS; u++) {
+            const int c = tid + 256 * u;
+            store_split(Qp, c / (D / 4), (c % (D / 4)) * 4, qreg[u], QPLANEB);
+        }
+    }
+    Frag32S<D, 1> f;
+#pragma unroll
+    for (int dvb = 0; dvb < D / 32; dvb++) f.o[0][dvb] = (floatx16_t){0};
+    f.m[0] = MI_NEG_INF;
+    f.l[0] = 0.0f;
+    __syncthreads();
+    // the wavefront's B operand: query row r, features 16t + 8hh .. + 7 of step t, in each plane (read like a K row)
+#pragma unroll
+    for (int q = 0; q < 3; q++)
+#pragma unroll
+        for (int t = 0; t < D / 16; t++)
+            f.q[0][q][t] = *(lds_plane8_t)(uintptr_t)(Qp + q * QPLANEB + (unsigned)r * ROWB + (((2 * t + hh) ^ C::swz(r)) << 4));
+
+    // ---- scores of the wavefront's block (kept raw), V into planes, statistics of the block
+    const int tile = wave >> 1;
+    const int64_t j0 = 32 * (int64_t)wave;
+    // every block of a tile that some query of the workgroup reaches takes part (a block past the diagonal yields
+    // the exact zeros its weights are); tiles nobody reaches are zeroed below
+    const bool active = tile < n_tiles;
+    const unsigned blk = (unsigned)tile * TILEB + (unsigned)(wave & 1) * 32u * ROWB;
+    floatx16_t keep[1][1];
+    if (active) scores32s<D, 1, 1>(f, Kp + blk, keep);
+    if (do_pv) {
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+            if (t < n_tiles) store_tile(Vp + t * TILEB, vreg[t]);
+    }
+    if (active) {
+        floatx16_t s[1][1] = {{keep[0][0]}};
+        flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_STATS, float, 1>(a, s, f.o, f.m, f.l, b, h, iw, j0, FlashStaged<1>(), 0, 0u, nullptr, p.Lkv);
+    }
+    // the workgroup's statistics: (m, l) of the four blocks, combined as the online softmax combines tiles
+    // (src/softmax.jl:69-79 over the whole row): m = max, l = sum of l_i 2^((m_i - m) c); a block whose maximum is the
+    // row's keeps its sum as it is (two -Inf or two +Inf included)
+    const float lsum = f.l[0] + mi_swap32(f.l[0]);
+    if (hh == 0) {
+        xstat[(wave * 32 + r) * 2] = f.m[0];
+        xstat[(wave * 32 + r) * 2 + 1] = lsum;
+    }
+    __syncthreads();   // statistics exchanged, V in LDS, every wavefront done with the K planes
+    {
+        const float cs = flash_natural_units(XT) ? MI_LOG2E : a.c;
+        float m = f.m[0];
+#pragma unroll
+        for (int w = 0; w < 4; w++) m = fmaxf(m, xstat[(w * 32 + r) * 2]);
+        float l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float mw = xstat[(w * 32 + r) * 2], lw = xstat[(w * 32 + r) * 2 + 1];
+            l += lw * (mw == m ? 1.0f : mi_exp2((mw - m) * cs));
+        }
+        f.m[0] = m;
+        f.l[0] = 1.0f / l;
+    }
+
+    // ---- weights and the wavefront's share of the output
+    const unsigned wlds = lds0 + 4u * TILEB + wave * FLASH_WSTAGE_BYTES;
+    if (active) {
+        flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_FINAL, float, 1>(a, keep, f.o, f.m, f.l, b, h, iw, j0, FlashStaged<1>(), 0, wlds, nullptr, p.Lkv);
+        if (do_pv) weights_times_values32s<D, 1, 1>(f, Vp + blk, keep);
+    }
+    if (wave == 0 && p.weights) flash_zero_skipped_weights<1, float>(a, b, h, iw, n_tiles, false);
+    if (wave == 0 && p.stats && hh == 0) flash_save_stats(p, b, h, qi, f.m[0] * MI_LOG2E, f.l[0]);
+
+    // the partial outputs go through LDS (the K planes' region: nobody reads them any more); each wavefront adds up
+    // and writes a quarter of the row
+    if (!do_pv) return;
+#pragma unroll
+    for (int dvb = 0; dvb < D / 32; dvb++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) xout[(wave * (D / 2) + 16 * dvb + v) * 64 + lane] = f.o[0][dvb][v];
+    __syncthreads();
+    if (qi < p.Lq) {
+        float *orow = (float *)p.out + p.Ev * (qi + p.Lq * b) + p.Dv * h;
+        constexpr int PER = D / 32;   // a lane's row share is D / 8 16-byte pieces: a quarter per wavefront
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int piece = wave * PER + i, dvb = piece >> 2, g = piece & 3;
+            floatx4_t o4 = (floatx4_t){0};
+#pragma unroll
+            for (int w = 0; w < 4; w++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) o4[e] += xout[(w * (D / 2) + 16 * dvb + 4 * g + e) * 64 + lane];
+            if (32 * dvb + 8 * g + 4 * hh < p.Dv) *(floatx4_t *)(orow + 32 * dvb + 8 * g + 4 * hh) = o4;
+        }
+    }
+}
+
 template <int D>
 int32_t launch_resident(const FlashArgs &a, hipStream_t st, bool extras) {
     constexpr size_t smem = 2 * RES_TILES * CfgS<D>::TILEB + 4 * FLASH_WSTAGE_BYTES;
     constexpr size_t smem_pair = 2 * RES_TILES * CfgS<D>::TILEB + 8 * FLASH_WSTAGE_BYTES + 8 * 32 * 2 * sizeof(float);
+    constexpr size_t smem_quad = 2 * RES_TILES * CfgS<D>::TILEB + 4 * FLASH_WSTAGE_BYTES + 4 * 32 * 2 * sizeof(float) + 3 * 32 * CfgS<D>::ROWB;
     static_assert(4 * 32 * (D / 2) * sizeof(float) <= 2 * CfgS<D>::TILEB, "partial outputs fit the K planes' region");
     static bool attr_set = false;
     if (!attr_set) {
@@ -867,10 +1086,20 @@ int32_t launch_resident(const FlashArgs &a, hipStream_t st, bool extras) {
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_pair_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pair));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_pair_kernel<D, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pair));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_pair_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_pair));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_quad_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_quad));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_quad_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_quad));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_quad_kernel<D, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_quad));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_quad_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_quad));
         attr_set = true;
     }
     const int64_t total = (int64_t)a.n_qtiles * a.p.H * a.p.B;
-    if (a.p.Lkv > BN) {   // two key tiles: a wavefront per tile and query block
+    const int64_t total_quad = (a.p.Lq + 31) / 32 * a.p.H * a.p.B;
+    static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;   // the workgroup of eight, for comparisons
+    if (a.p.Lkv > BN && total_quad <= 256 && !no_quad) {   // one workgroup per compute unit at most: a wavefront per 32-key block
+        auto kern = a.p.causal ? (extras ? flash32_resident_quad_kernel<D, true, true> : flash32_resident_quad_kernel<D, true, false>)
+                               : (extras ? flash32_resident_quad_kernel<D, false, true> : flash32_resident_quad_kernel<D, false, false>);
+        hipLaunchKernelGGL(kern, dim3((unsigned)total_quad), dim3(256), smem_quad, st, a);
+    } else if (a.p.Lkv > BN) {   // two key tiles: a wavefront per tile and query block
         auto kern = a.p.causal ? (extras ? flash32_resident_pair_kernel<D, true, true> : flash32_resident_pair_kernel<D, true, false>)
                                : (extras ? flash32_resident_pair_kernel<D, false, true> : flash32_resident_pair_kernel<D, false, false>);
         hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(512), smem_pair, st, a);

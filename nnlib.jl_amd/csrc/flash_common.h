@@ -381,14 +381,16 @@ __device__ inline void flash_mask_apply4(floatx16_t &v, int g, uint32_t m4) {
 // it stay below 2^8, which Float32 sums and 16-bit operands hold without loss.
 constexpr float FLASH_LAZY_MAX_LOG2 = 8.0f;
 
-template <typename T, int QB, int NDV, bool CAUSAL, int EXTRAS, int PHASE, typename TW>
-__device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB][2], floatx16_t (&o)[QB][NDV],
+// KBLK: 32-key blocks per tile (2: the 64-key tile of the tile loops; 1: a wavefront that owns a single block)
+template <typename T, int QB, int NDV, bool CAUSAL, int EXTRAS, int PHASE, typename TW, int KBLK = 2>
+__device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB][KBLK], floatx16_t (&o)[QB][NDV],
                                           float (&fm)[QB], float (&fl)[QB], int64_t b, int64_t h, int64_t iw,
                                           int64_t j0, const FlashStaged<QB> &sg = FlashStaged<QB>(), int stage = 0,
                                           unsigned wlds = 0, const uint32_t *key_mask = nullptr, int64_t kv_len = -1) {
     const AttnParams &p = a.p;
     typedef typename T::type elem_t;
-    constexpr int BN = FLASH_BN;
+    constexpr int BN = 32 * KBLK;
+    static_assert(KBLK == 2 || ((EXTRAS == EXTRAS_NONE || EXTRAS == EXTRAS_DIRECT) && sizeof(TW) == 4), "single blocks: Float32 kernels without staged tiles");
     const int lane = threadIdx.x & 63, r = lane & 31, hh = lane >> 5;
     // kv_len >= 0: keys from kv_len on do not exist for this (head, batch) pair (a context length shorter than L_kv);
     // the weights of such keys come out as exact zeros
@@ -405,7 +407,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             const int row = 32 * qb + r;
             if (sg.bias) {
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         const typename T::vec4 t4 = sg.template bias4<typename T::vec4>(stage, row, 4 * kb + g, hh);
@@ -414,13 +416,13 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                     }
             } else {
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                     for (int v = 0; v < 16; v++) s[qb][kb][v] *= a.cn;
             }
             if (sg.mask) {
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         flash_mask_apply4(s[qb][kb], g, sg.mask4(stage, row, 4 * kb + g, hh));
@@ -431,7 +433,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             const int64_t boff = qi * p.bias_strides[1] + h * p.bias_strides[2] + b * p.bias_strides[3];
             const int64_t moff = qi * p.mask_strides[1] + h * p.mask_strides[2] + b * p.mask_strides[3];
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     const int64_t kv = j0 + 32 * kb + 8 * g + 4 * hh;
@@ -475,7 +477,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
         if (EXTRAS == EXTRAS_MASKTILE) {
             const int row = 32 * qb + r;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < KBLK; kb++) {
 #pragma unroll
                 for (int g = 0; g < 4; g++) flash_mask_apply4(s[qb][kb], g, sg.mask4(stage, row, 4 * kb + g, hh));
             }
@@ -485,7 +487,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             uint32_t own[8];
             if (!key_mask) flash_load_key_mask(a, b, h, j0, hh, own);
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < KBLK; kb++) {
 #pragma unroll
                 for (int g = 0; g < 4; g++) flash_mask_apply4(s[qb][kb], g, key_mask ? key_mask[4 * kb + g] : own[4 * kb + g]);
             }
@@ -496,7 +498,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             if (CAUSAL && qi - j0 + 1 < lim64) lim64 = qi - j0 + 1;
             const int lim = lim64 > BN ? BN : (lim64 < 0 ? 0 : (int)lim64);
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     const int kvl = 32 * kb + 8 * (v / 4) + 4 * hh + (v % 4);
@@ -511,7 +513,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
         if (PHASE != PHASE_FINAL) {
             float mx = MI_NEG_INF;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) mx = fmaxf(mx, s[qb][kb][v]);
             mx = fmaxf(mx, mi_swap32(mx));
@@ -545,7 +547,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
         if (NAT && __builtin_expect(__builtin_amdgcn_ballot_w64(pinf) != 0, 0)) {
             if (pinf) {
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                     for (int v = 0; v < 16; v++) s[qb][kb][v] = s[qb][kb][v] == MI_POS_INF ? 0.0f : MI_NEG_INF;
                 msafe = 0.0f;
@@ -554,7 +556,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
         const float moff2 = -msafe * cs;
         float lsum = 0.0f;
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+        for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 float x = s[qb][kb][v];
@@ -571,7 +573,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             const uint64_t row0 = (uint64_t)(p.Lkv * (qi + p.Lq * (h + p.H * b)) + j0 + 4 * hh);
             const bool aligned = (p.Lkv & 3) == 0;   // every run of four keys of a lane is one hash group
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     float f[4];
@@ -592,7 +594,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
             typedef __attribute__((address_space(3))) u32x4_t *lds16_t;
             typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
             constexpr int EPC = 16 / (int)sizeof(TW);             // weights per 16-byte chunk
-            constexpr int NKB = sizeof(TW) == 4 ? 2 : 1;          // staging rounds per tile along the keys
+            constexpr int NKB = sizeof(TW) == 4 ? KBLK : 1;       // staging rounds per tile along the keys
             TW *wbase = (TW *)p.weights + p.Lkv * (p.Lq * (h + p.H * b));
 #pragma unroll
             for (int rk = 0; rk < NKB; rk++)
@@ -603,7 +605,7 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                         const int sw = (r >> 1) & 7;
                         if constexpr (sizeof(TW) == 2) {
 #pragma unroll
-                            for (int kb = 0; kb < 2; kb++)
+                            for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                                 for (int g = 0; g < 4; g++) {
                                     typedef TW tw4 __attribute__((ext_vector_type(4)));
@@ -634,14 +636,14 @@ __device__ inline void flash_softmax_tile(const FlashArgs &a, floatx16_t (&s)[QB
                     for (int i = 0; i < 2; i++) {
                         const int rr = (lane >> 3) + 8 * i, c = lane & 7;
                         const u32x4_t piece = pieces[i];
-                        const int64_t qrow = iw + 32 * qb + 16 * half + rr, kv0 = j0 + 32 * rk * (NKB - 1) + (int64_t)c * EPC;
+                        const int64_t qrow = iw + 32 * qb + 16 * half + rr, kv0 = j0 + 32 * rk + (int64_t)c * EPC;
                         if (qrow < p.Lq && kv0 < p.Lkv) *(u32x4_t *)(wbase + p.Lkv * qrow + kv0) = piece;   // Lkv is a multiple of EPC here
                     }
                 }
         } else if (PHASE == PHASE_FINAL && p.weights && qok) {
             TW *w = (TW *)p.weights + p.Lkv * (qi + p.Lq * (h + p.H * b));
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < KBLK; kb++)
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     const int64_t kv = j0 + 32 * kb + 8 * g + 4 * hh;

@@ -303,6 +303,12 @@ SMALL_F32_CASES = [
     (56, 131, 66, 2, 2, dict(bias_shape=(66, 131), mask_shape=(66, 131, 1, 2))),
     (128, 96, 96, 1, 2, dict(causal=True, mask_shape=(96, 96))),
     (48, 33, 90, 2, 2, dict(Ev=96, mask_shape=(90, 1, 2, 2))),           # v wider than q, k; key-padding style mask
+    # more than 256 blocks of 32 queries: the workgroup of eight wavefronts (one per key tile and query block)
+    # instead of one workgroup of four per query block
+    (512, 160, 128, 8, 8, {}),
+    (256, 97, 97, 17, 4, dict(causal=True)),
+    (128, 1100, 100, 4, 2, dict(bias_shape=(100, 1100, 2, 1), mask_shape=(100, 1100))),
+    (256, 128, 128, 17, 4, dict(causal=True, mask_shape=(128, 128, 1, 17))),
 ]
 
 
