@@ -521,6 +521,7 @@ __global__ __launch_bounds__(256, (D == 64 && !EXTRAS) ? 2 : 1) void flash32_ker
 // start, K and V are split into planes once, the scores of all tiles stay in registers between the statistics and the
 // weights, and the workgroup meets at two barriers (K in LDS; V in LDS, split under the score products).
 constexpr int RES_TILES = 2;
+constexpr int64_t RESIDENT_QUAD_MAX_BLOCKS = 256;   // 32-query blocks up to which a call runs one workgroup per block
 
 // The reference divides q by sqrt(D) first (src/attention.jl:118).  When sqrt(D) is a power of two (D = 16, 64, 256)
 // the product with its reciprocal is that quotient bit for bit, at a tenth of the instructions of a division.
@@ -1097,7 +1098,7 @@ int32_t launch_resident(const FlashArgs &a, hipStream_t st, bool extras) {
     static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;   // the workgroup of eight, for comparisons
     // at most one workgroup per compute unit: a wavefront per 32-key block (with two or four workgroups per unit the
     // workgroups below are faster: 16.7 against 15.0 us at 512, 31.8 against 15.4 us at 1024)
-    if (total_quad <= 256 && !no_quad) {
+    if (total_quad <= RESIDENT_QUAD_MAX_BLOCKS && !no_quad) {
         auto kern = a.p.causal ? (extras ? flash32_resident_quad_kernel<D, true, true> : flash32_resident_quad_kernel<D, true, false>)
                                : (extras ? flash32_resident_quad_kernel<D, false, true> : flash32_resident_quad_kernel<D, false, false>);
         hipLaunchKernelGGL(kern, dim3((unsigned)total_quad), dim3(256), smem_quad, st, a);
@@ -1216,7 +1217,9 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
         return narrow ? launch_d<64, 1>(a, st, true) : launch_d<128, 1>(a, st, true);
     }
     const bool extras = p.bias || p.mask;
-    // few keys and the weights returned: everything resident, one pass (flash32_resident_kernel)
-    if (narrow && p.weights && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted()) return launch_resident<64>(a, st, extras);
+    // few keys and the weights returned: everything resident, one pass (flash32_resident_kernel); without the weights
+    // when the call leaves most of the chip idle (the workgroup per 32-query block)
+    const bool few_blocks = (p.Lq + 31) / 32 * p.H * p.B <= RESIDENT_QUAD_MAX_BLOCKS;
+    if (narrow && (p.weights || few_blocks) && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted()) return launch_resident<64>(a, st, extras);
     return narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
 }

@@ -322,6 +322,15 @@ def test_small_float32_problem_with_weights(nn, oracle, case):
     _check(nn, oracle, rng, "f32", E, Lq, Lkv, B, H, expect="flash32", weights=True, **kw)
 
 
+@pytest.mark.parametrize("case", [c for c in SMALL_F32_CASES if (c[1] + 31) // 32 * c[3] * c[4] <= 256],
+                         ids=lambda c: f"E{c[0]}-Lq{c[1]}-Lkv{c[2]}-B{c[3]}-H{c[4]}-" + "-".join(c[5]))
+def test_small_float32_problem_without_weights(nn, oracle, case):
+    """Calls of at most 256 blocks of 32 queries take the one-pass kernel without the weights output too."""
+    E, Lq, Lkv, B, H, kw = case
+    rng = np.random.default_rng(1000 * E + 10 * Lq + Lkv + 1)
+    _check(nn, oracle, rng, "f32", E, Lq, Lkv, B, H, expect="flash32", weights=False, **kw)
+
+
 def test_small_float32_problem_special_values(nn, oracle):
     """+Inf logits (src/softmax.jl:73-75: the weights become the indicator of the +Inf entries, normalised), a query
     with nothing kept (NaN) and scores without a value product, at a size the one-pass kernel takes."""
