@@ -1046,6 +1046,7 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs
     }
     if (wave == 0 && p.weights) flash_zero_skipped_weights<1, float>(a, b, h, iw, n_tiles, false);
     if (wave == 0 && p.stats && hh == 0) flash_save_stats(p, b, h, qi, f.m[0] * MI_LOG2E, f.l[0]);
+    if (wave == 1 && p.stats && qblk == n_qblocks - 1) flash_zero_stats_padding(p, b, h, iw + 32);   // rows no query block covers
 
     // the partial outputs go through LDS (the K planes' region: nobody reads them any more); each wavefront adds up
     // and writes a quarter of the row
@@ -1071,12 +1072,237 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs
     }
 }
 
+// The workgroup per 32-query block for up to RES_CHUNKS * 128 keys: the keys in chunks of 128 (four 32-key blocks, one per
+// wavefront), the raw scores of every chunk kept in registers between the statistics and the weights, so the score
+// product still runs once.  First phase: K chunks through two LDS buffers (the next chunk's loads in flight, one
+// barrier per chunk); second phase: V chunks through the same two buffers.
+constexpr int RES_CHUNKS = 4;
+
+template <int D, bool CAUSAL, bool EXTRAS>
+__global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashArgs a) {
+    typedef CfgS<D> C;
+    constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB, CHUNKS = C::CHUNKS, TILEB = C::TILEB;
+    constexpr int XT = EXTRAS ? EXTRAS_DIRECT : EXTRAS_NONE;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char flash_smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem;
+    // two chunk buffers of two tiles each, weight staging, exchanged statistics, the query block's planes, partial outputs
+    constexpr int QPLANEB = 32 * ROWB, QCHUNKS = 32 * D / 4 / 256;
+    constexpr unsigned OFF_STAGE = 4 * TILEB, OFF_STAT = OFF_STAGE + 4 * FLASH_WSTAGE_BYTES, OFF_Q = OFF_STAT + 4 * 32 * 2 * sizeof(float),
+                       OFF_OUT = OFF_Q + 3 * QPLANEB;
+    float *xstat = (float *)(flash_smem + OFF_STAT);   // [4 wavefronts][32 rows][2]
+    float *xout = (float *)(flash_smem + OFF_OUT);     // [4 wavefronts][D / 2 registers][64 lanes]
+    const unsigned Qp = lds0 + OFF_Q;
+    typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+    typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t n_qblocks = (p.Lq + 31) / 32;
+    const int64_t hb = blockIdx.x % HB, qblk = n_qblocks - 1 - blockIdx.x / HB;
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t iw = qblk * 32, qi = iw + r;
+    int64_t kv_end = p.Lkv;
+    if (CAUSAL && iw + 32 < kv_end) kv_end = iw + 32;
+    const int n_chunks = (int)((kv_end + 127) / 128);   // <= RES_CHUNKS: checked by the host
+    const bool do_pv = p.out != nullptr;
+
+    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
+    const float *vbase = do_pv ? (const float *)p.v + p.Ev * (p.Lkv * b) + p.Dv * h : nullptr;
+    const float *qbase = (const float *)p.q + p.E * (p.Lq * b) + p.D * h;
+    const int dqk = (int)p.D, dv = (int)p.Dv;
+    auto load_chunk = [&](floatx4_t (&reg)[2][CHUNKS], const float *base, int64_t ld, int dlim, int c, bool on) {
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int u = 0; u < CHUNKS; u++) {
+                const int i = tid + 256 * u;
+                const int64_t row = 128 * (int64_t)c + 64 * t + i / (D / 4);
+                const int col = (i % (D / 4)) * 4;
+                reg[t][u] = ldg16f(base + ld * row + col, on && row < p.Lkv && col < dlim);
+            }
+    };
+    auto store_split = [&](unsigned at_tile, int row, int col, const floatx4_t &x, int planeb) {
+        uint32_t pl[3][2];
+        const bool odd = split3_pair(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        if (odd) {   // an Inf or NaN in the chunk (rare)
+            split3_pair_guarded(x[0], x[1], pl[0][0], pl[1][0], pl[2][0]);
+            split3_pair_guarded(x[2], x[3], pl[0][1], pl[1][1], pl[2][1]);
+        }
+        const unsigned at = at_tile + (unsigned)row * ROWB + (unsigned)((((col >> 3) ^ C::swz(row)) << 4) + (col & 7) * 2);
+#pragma unroll
+        for (int q = 0; q < 3; q++) *(lds8_t)(uintptr_t)(at + q * planeb) = (u32x2_t){pl[q][0], pl[q][1]};
+    };
+    auto store_chunk = [&](unsigned buf, const floatx4_t (&reg)[2][CHUNKS]) {
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int u = 0; u < CHUNKS; u++) {
+                const int i = tid + 256 * u;
+                store_split(buf + t * TILEB, i / (D / 4), (i % (D / 4)) * 4, reg[t][u], PLANEB);
+            }
+    };
+
+    // ---- the first K chunk and the queries
+    floatx4_t reg[2][CHUNKS], nxt[2][CHUNKS], qreg[QCHUNKS];
+    load_chunk(reg, kbase, p.E, dqk, 0, true);
+#pragma unroll
+    for (int u = 0; u < QCHUNKS; u++) {   // the four wavefronts share the query block: a quarter each
+        const int i = tid + 256 * u;
+        const int64_t row = iw + i / (D / 4);
+        const int col = (i % (D / 4)) * 4;
+        qreg[u] = ldg16f(qbase + p.E * row + col, row < p.Lq && col < dqk);
+    }
+    {
+        // q / sqrt(D) as the reference has it (see scale_queries)
+        const float sq = sqrtf((float)p.D), inv_sq = 1.0f / sq;
+        if (sqrt_is_power_of_two(sq)) {
+#pragma unroll
+            for (int u = 0; u < QCHUNKS; u++) qreg[u] *= inv_sq;
+        } else {
+#pragma unroll
+            for (int u = 0; u < QCHUNKS; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) qreg[u][e] /= sq;
+        }
+#pragma unroll
+        for (int u = 0; u < QCHUNKS; u++) {
+            const int i = tid + 256 * u;
+            store_split(Qp, i / (D / 4), (i % (D / 4)) * 4, qreg[u], QPLANEB);
+        }
+    }
+    Frag32S<D, 1> f;
+#pragma unroll
+    for (int dvb = 0; dvb < D / 32; dvb++) f.o[0][dvb] = (floatx16_t){0};
+    f.m[0] = MI_NEG_INF;
+    f.l[0] = 0.0f;
+
+    // ---- first phase: scores of the wavefront's block of every chunk (kept raw), running statistics
+    const unsigned blk = (unsigned)(wave >> 1) * TILEB + (unsigned)(wave & 1) * 32u * ROWB;
+    floatx16_t keep[RES_CHUNKS][1][1];
+#pragma unroll
+    for (int c = 0; c < RES_CHUNKS; c++) {
+        if (c < n_chunks) {
+            if (c + 1 < n_chunks) load_chunk(nxt, kbase, p.E, dqk, c + 1, true);
+            else load_chunk(nxt, vbase, p.Ev, dv, 0, do_pv);   // the first V chunk
+            const unsigned buf = lds0 + (unsigned)(c & 1) * 2u * TILEB;
+            store_chunk(buf, reg);
+            __syncthreads();   // chunk c (and the queries) in LDS; every wavefront is done with chunk c - 1
+            if (c == 0) {
+                // the wavefront's B operand: query row r, features 16t + 8hh .. + 7 of step t, in each plane
+#pragma unroll
+                for (int q = 0; q < 3; q++)
+#pragma unroll
+                    for (int t = 0; t < D / 16; t++)
+                        f.q[0][q][t] = *(lds_plane8_t)(uintptr_t)(Qp + q * QPLANEB + (unsigned)r * ROWB + (((2 * t + hh) ^ C::swz(r)) << 4));
+            }
+            scores32s<D, 1, 1>(f, buf + blk, keep[c]);
+            floatx16_t s[1][1] = {{keep[c][0][0]}};
+            flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_STATS, float, 1>(a, s, f.o, f.m, f.l, b, h, iw, 128 * (int64_t)c + 32 * wave, FlashStaged<1>(), 0,
+                                                                                 0u, nullptr, p.Lkv);
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int u = 0; u < CHUNKS; u++) reg[t][u] = nxt[t][u];
+        }
+    }
+    // the workgroup's statistics, combined as the online softmax combines tiles (see flash32_resident_quad_kernel)
+    const float lsum = f.l[0] + mi_swap32(f.l[0]);
+    if (hh == 0) {
+        xstat[(wave * 32 + r) * 2] = f.m[0];
+        xstat[(wave * 32 + r) * 2 + 1] = lsum;
+    }
+    __syncthreads();   // statistics exchanged, every wavefront done with the K chunks
+    {
+        const float cs = flash_natural_units(XT) ? MI_LOG2E : a.c;
+        float m = f.m[0];
+#pragma unroll
+        for (int w = 0; w < 4; w++) m = fmaxf(m, xstat[(w * 32 + r) * 2]);
+        float l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float mw = xstat[(w * 32 + r) * 2], lw = xstat[(w * 32 + r) * 2 + 1];
+            l += lw * (mw == m ? 1.0f : mi_exp2((mw - m) * cs));
+        }
+        f.m[0] = m;
+        f.l[0] = 1.0f / l;
+    }
+
+    // ---- second phase: weights and the wavefront's share of the output, V chunks through the same buffers
+    const unsigned wlds = lds0 + OFF_STAGE + wave * FLASH_WSTAGE_BYTES;
+#pragma unroll
+    for (int c = 0; c < RES_CHUNKS; c++) {
+        if (c < n_chunks) {
+            const unsigned buf = lds0 + (unsigned)(c & 1) * 2u * TILEB;
+            if (do_pv) {
+                if (c + 1 < n_chunks) load_chunk(nxt, vbase, p.Ev, dv, c + 1, true);
+                store_chunk(buf, reg);
+                __syncthreads();   // V chunk c in LDS; every wavefront is done with chunk c - 1
+            }
+            flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_FINAL, float, 1>(a, keep[c], f.o, f.m, f.l, b, h, iw, 128 * (int64_t)c + 32 * wave, FlashStaged<1>(),
+                                                                                 0, wlds, nullptr, p.Lkv);
+            if (do_pv) {
+                weights_times_values32s<D, 1, 1>(f, buf + blk, keep[c]);
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int u = 0; u < CHUNKS; u++) reg[t][u] = nxt[t][u];
+            }
+        }
+    }
+    if (wave == 0 && p.weights) flash_zero_skipped_weights<1, float>(a, b, h, iw, 2 * n_chunks, false);
+    if (wave == 0 && p.stats && hh == 0) flash_save_stats(p, b, h, qi, f.m[0] * MI_LOG2E, f.l[0]);
+    if (wave == 1 && p.stats && qblk == n_qblocks - 1) flash_zero_stats_padding(p, b, h, iw + 32);   // rows no query block covers
+
+    // the partial outputs go through LDS; each wavefront adds up and writes a quarter of the row
+    if (!do_pv) return;
+#pragma unroll
+    for (int dvb = 0; dvb < D / 32; dvb++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) xout[(wave * (D / 2) + 16 * dvb + v) * 64 + lane] = f.o[0][dvb][v];
+    __syncthreads();
+    if (qi < p.Lq) {
+        float *orow = (float *)p.out + p.Ev * (qi + p.Lq * b) + p.Dv * h;
+        constexpr int PER = D / 32;   // a lane's row share is D / 8 16-byte pieces: a quarter per wavefront
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            const int piece = wave * PER + i, dvb = piece >> 2, g = piece & 3;
+            floatx4_t o4 = (floatx4_t){0};
+#pragma unroll
+            for (int w = 0; w < 4; w++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) o4[e] += xout[(w * (D / 2) + 16 * dvb + 4 * g + e) * 64 + lane];
+            if (32 * dvb + 8 * g + 4 * hh < p.Dv) *(floatx4_t *)(orow + 32 * dvb + 8 * g + 4 * hh) = o4;
+        }
+    }
+}
+
+template <int D>
+int32_t launch_resident_chunks(const FlashArgs &a, hipStream_t st, bool extras) {
+    constexpr size_t smem = 4 * CfgS<D>::TILEB + 4 * FLASH_WSTAGE_BYTES + 4 * 32 * 2 * sizeof(float) + 3 * 32 * CfgS<D>::ROWB + 4 * 64 * (D / 2) * sizeof(float);
+    static_assert(smem <= 160 * 1024, "fits a compute unit's LDS");
+    static bool attr_set = false;
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_set = true;
+    }
+    const int64_t total = (a.p.Lq + 31) / 32 * a.p.H * a.p.B;
+    auto kern = a.p.causal ? (extras ? flash32_resident_chunks_kernel<D, true, true> : flash32_resident_chunks_kernel<D, true, false>)
+                           : (extras ? flash32_resident_chunks_kernel<D, false, true> : flash32_resident_chunks_kernel<D, false, false>);
+    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(256), smem, st, a);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+
 template <int D>
 int32_t launch_resident(const FlashArgs &a, hipStream_t st, bool extras) {
     constexpr size_t smem = 2 * RES_TILES * CfgS<D>::TILEB + 4 * FLASH_WSTAGE_BYTES;
     constexpr size_t smem_pair = 2 * RES_TILES * CfgS<D>::TILEB + 8 * FLASH_WSTAGE_BYTES + 8 * 32 * 2 * sizeof(float);
     constexpr size_t smem_quad = 2 * RES_TILES * CfgS<D>::TILEB + 4 * FLASH_WSTAGE_BYTES + 4 * 32 * 2 * sizeof(float) + 3 * 32 * CfgS<D>::ROWB;
-    static_assert(4 * 32 * (D / 2) * sizeof(float) <= 2 * CfgS<D>::TILEB, "partial outputs fit the K planes' region");
+    static_assert(4 * 64 * (D / 2) * sizeof(float) <= 2 * CfgS<D>::TILEB, "partial outputs (D / 2 registers of 64 lanes per wavefront) fit the K planes' region");
     static bool attr_set = false;
     if (!attr_set) {
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -1221,5 +1447,7 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     // when the call leaves most of the chip idle (the workgroup per 32-query block)
     const bool few_blocks = (p.Lq + 31) / 32 * p.H * p.B <= RESIDENT_QUAD_MAX_BLOCKS;
     if (narrow && (p.weights || few_blocks) && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted()) return launch_resident<64>(a, st, extras);
+    static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;
+    if (narrow && few_blocks && p.Lkv <= RES_CHUNKS * 128 && !exact_instruction_wanted() && !no_quad) return launch_resident_chunks<64>(a, st, extras);
     return narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
 }

@@ -50,6 +50,17 @@ __device__ inline void flash_save_stats(const AttnParams &p, int64_t b, int64_t 
     p.stats[p.B * p.H * pad + at] = qi < p.Lq ? linv : 0.0f;
 }
 
+// The zeros of the padding rows from `from` on, written by one wavefront: for kernels whose workgroups do not cover
+// the padding themselves.
+__device__ inline void flash_zero_stats_padding(const AttnParams &p, int64_t b, int64_t h, int64_t from) {
+    const int64_t pad = attention_stats_lq_pad(p.Lq);
+    for (int64_t qi = from + (threadIdx.x & 63); qi < pad; qi += 64) {
+        const int64_t at = (b * p.H + h) * pad + qi;
+        p.stats[at] = 0.0f;
+        p.stats[p.B * p.H * pad + at] = 0.0f;
+    }
+}
+
 // Split-kv bookkeeping shared by the planner (workspace size) and the launchers.
 // Partials live in the caller's workspace: o as [split][B][Lq][Ev] floats, then (m, l) as
 // [split][B][H][Lq][2] floats, m in log2 units.

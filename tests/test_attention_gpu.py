@@ -331,6 +331,32 @@ def test_small_float32_problem_without_weights(nn, oracle, case):
     _check(nn, oracle, rng, "f32", E, Lq, Lkv, B, H, expect="flash32", weights=False, **kw)
 
 
+MID_F32_CASES = [
+    # Float32, 129 to 512 keys, at most 256 blocks of 32 queries: a workgroup per query block that keeps the scores of
+    # every 128-key chunk in registers (one to four chunks, ragged last chunk and last block, causal diagonal inside a
+    # chunk, bias / mask, v wider than q and k)
+    (128, 129, 129, 1, 2, {}),
+    (512, 256, 256, 4, 8, {}),
+    (256, 100, 512, 2, 4, {}),
+    (128, 77, 385, 3, 2, {}),
+    (64, 300, 300, 1, 1, dict(causal=True)),
+    (512, 256, 256, 4, 8, dict(causal=True)),
+    (128, 511, 511, 1, 2, dict(causal=True, scale=0.125)),
+    (128, 70, 200, 2, 2, dict(bias_shape=(200, 70, 2, 2), mask_shape=(200, 70))),
+    (56, 131, 450, 2, 2, dict(bias_shape=(450, 131), mask_shape=(450, 131, 1, 2))),
+    (128, 260, 260, 1, 2, dict(causal=True, mask_shape=(260, 260))),
+    (48, 33, 290, 2, 2, dict(Ev=96, bias_shape=(290, 33, 2, 1))),
+]
+
+
+@pytest.mark.parametrize("weights", [True, False], ids=["weights", "no-weights"])
+@pytest.mark.parametrize("case", MID_F32_CASES, ids=lambda c: f"E{c[0]}-Lq{c[1]}-Lkv{c[2]}-B{c[3]}-H{c[4]}-" + "-".join(c[5]))
+def test_mid_float32_problem_on_few_workgroups(nn, oracle, case, weights):
+    E, Lq, Lkv, B, H, kw = case
+    rng = np.random.default_rng(1000 * E + 10 * Lq + Lkv + 7)
+    _check(nn, oracle, rng, "f32", E, Lq, Lkv, B, H, expect="flash32", weights=weights, **kw)
+
+
 def test_small_float32_problem_special_values(nn, oracle):
     """+Inf logits (src/softmax.jl:73-75: the weights become the indicator of the +Inf entries, normalised), a query
     with nothing kept (NaN) and scores without a value product, at a size the one-pass kernel takes."""
