@@ -1075,7 +1075,8 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs
 // The workgroup per 32-query block for up to RES_CHUNKS * 128 keys: the keys in chunks of 128 (four 32-key blocks, one per
 // wavefront), the raw scores of every chunk kept in registers between the statistics and the weights, so the score
 // product still runs once.  First phase: K chunks through two LDS buffers (the next chunk's loads in flight, one
-// barrier per chunk); second phase: V chunks through the same two buffers.
+// barrier per chunk); second phase: V chunks through the same two buffers.  128-wide tiles have room for one buffer
+// (96 KiB): a second barrier per chunk before it is overwritten, and the partial outputs share it at the end.
 constexpr int RES_CHUNKS = 4;
 
 template <int D, bool CAUSAL, bool EXTRAS>
@@ -1086,12 +1087,13 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
     const AttnParams &p = a.p;
     extern __shared__ __attribute__((aligned(16))) unsigned char flash_smem[];
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem;
-    // two chunk buffers of two tiles each, weight staging, exchanged statistics, the query block's planes, partial outputs
+    // chunk buffers of two tiles each, weight staging, exchanged statistics, the query block's planes, partial outputs
+    constexpr bool TWO_BUFFERS = D <= 64;
     constexpr int QPLANEB = 32 * ROWB, QCHUNKS = 32 * D / 4 / 256;
-    constexpr unsigned OFF_STAGE = 4 * TILEB, OFF_STAT = OFF_STAGE + 4 * FLASH_WSTAGE_BYTES, OFF_Q = OFF_STAT + 4 * 32 * 2 * sizeof(float),
+    constexpr unsigned OFF_STAGE = (TWO_BUFFERS ? 4 : 2) * TILEB, OFF_STAT = OFF_STAGE + 4 * FLASH_WSTAGE_BYTES, OFF_Q = OFF_STAT + 4 * 32 * 2 * sizeof(float),
                        OFF_OUT = OFF_Q + 3 * QPLANEB;
     float *xstat = (float *)(flash_smem + OFF_STAT);   // [4 wavefronts][32 rows][2]
-    float *xout = (float *)(flash_smem + OFF_OUT);     // [4 wavefronts][D / 2 registers][64 lanes]
+    float *xout = (float *)(flash_smem + (TWO_BUFFERS ? OFF_OUT : 0));   // [4 wavefronts][D / 2 registers][64 lanes]
     const unsigned Qp = lds0 + OFF_Q;
     typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
     typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
@@ -1185,9 +1187,10 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
         if (c < n_chunks) {
             if (c + 1 < n_chunks) load_chunk(nxt, kbase, p.E, dqk, c + 1, true);
             else load_chunk(nxt, vbase, p.Ev, dv, 0, do_pv);   // the first V chunk
-            const unsigned buf = lds0 + (unsigned)(c & 1) * 2u * TILEB;
+            const unsigned buf = lds0 + (TWO_BUFFERS ? (unsigned)(c & 1) * 2u * TILEB : 0u);
+            if (!TWO_BUFFERS && c > 0) __syncthreads();   // every wavefront is done with chunk c - 1
             store_chunk(buf, reg);
-            __syncthreads();   // chunk c (and the queries) in LDS; every wavefront is done with chunk c - 1
+            __syncthreads();   // chunk c (and the queries) in LDS; with two buffers: every wavefront is done with chunk c - 1
             if (c == 0) {
                 // the wavefront's B operand: query row r, features 16t + 8hh .. + 7 of step t, in each plane
 #pragma unroll
@@ -1233,11 +1236,12 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
 #pragma unroll
     for (int c = 0; c < RES_CHUNKS; c++) {
         if (c < n_chunks) {
-            const unsigned buf = lds0 + (unsigned)(c & 1) * 2u * TILEB;
+            const unsigned buf = lds0 + (TWO_BUFFERS ? (unsigned)(c & 1) * 2u * TILEB : 0u);
             if (do_pv) {
                 if (c + 1 < n_chunks) load_chunk(nxt, vbase, p.Ev, dv, c + 1, true);
+                if (!TWO_BUFFERS && c > 0) __syncthreads();   // every wavefront is done with chunk c - 1
                 store_chunk(buf, reg);
-                __syncthreads();   // V chunk c in LDS; every wavefront is done with chunk c - 1
+                __syncthreads();   // V chunk c in LDS; with two buffers: every wavefront is done with chunk c - 1
             }
             flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_FINAL, float, 1>(a, keep[c], f.o, f.m, f.l, b, h, iw, 128 * (int64_t)c + 32 * wave, FlashStaged<1>(),
                                                                                  0, wlds, nullptr, p.Lkv);
@@ -1256,6 +1260,7 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
 
     // the partial outputs go through LDS; each wavefront adds up and writes a quarter of the row
     if (!do_pv) return;
+    if (!TWO_BUFFERS) __syncthreads();   // the partial outputs share the chunk buffer: every wavefront is done with the last V chunk
 #pragma unroll
     for (int dvb = 0; dvb < D / 32; dvb++)
 #pragma unroll
@@ -1279,8 +1284,10 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
 
 template <int D>
 int32_t launch_resident_chunks(const FlashArgs &a, hipStream_t st, bool extras) {
-    constexpr size_t smem = 4 * CfgS<D>::TILEB + 4 * FLASH_WSTAGE_BYTES + 4 * 32 * 2 * sizeof(float) + 3 * 32 * CfgS<D>::ROWB + 4 * 64 * (D / 2) * sizeof(float);
+    constexpr size_t smem = (D <= 64 ? 4 * CfgS<D>::TILEB + 4 * 64 * (D / 2) * sizeof(float) : 2 * CfgS<D>::TILEB) + 4 * FLASH_WSTAGE_BYTES +
+                            4 * 32 * 2 * sizeof(float) + 3 * 32 * CfgS<D>::ROWB;
     static_assert(smem <= 160 * 1024, "fits a compute unit's LDS");
+    static_assert(4 * 64 * (D / 2) * sizeof(float) <= 2 * CfgS<D>::TILEB, "the partial outputs fit a chunk buffer");
     static bool attr_set = false;
     if (!attr_set) {
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -1448,6 +1455,7 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     const bool few_blocks = (p.Lq + 31) / 32 * p.H * p.B <= RESIDENT_QUAD_MAX_BLOCKS;
     if (narrow && (p.weights || few_blocks) && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted()) return launch_resident<64>(a, st, extras);
     static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;
-    if (narrow && few_blocks && p.Lkv <= RES_CHUNKS * 128 && !exact_instruction_wanted() && !no_quad) return launch_resident_chunks<64>(a, st, extras);
+    if (few_blocks && p.Lkv <= RES_CHUNKS * 128 && !exact_instruction_wanted() && !no_quad)
+        return narrow ? launch_resident_chunks<64>(a, st, extras) : launch_resident_chunks<128>(a, st, extras);
     return narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
 }

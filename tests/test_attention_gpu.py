@@ -346,6 +346,14 @@ MID_F32_CASES = [
     (56, 131, 450, 2, 2, dict(bias_shape=(450, 131), mask_shape=(450, 131, 1, 2))),
     (128, 260, 260, 1, 2, dict(causal=True, mask_shape=(260, 260))),
     (48, 33, 290, 2, 2, dict(Ev=96, bias_shape=(290, 33, 2, 1))),
+    # head dims above 64 (128-wide tiles: one chunk buffer)
+    (1024, 128, 128, 4, 8, {}),
+    (256, 100, 100, 2, 2, dict(causal=True)),
+    (192, 77, 385, 3, 2, {}),
+    (144, 260, 260, 1, 2, dict(causal=True, mask_shape=(260, 260))),
+    (256, 70, 200, 2, 2, dict(bias_shape=(200, 70, 2, 2), mask_shape=(200, 70))),
+    (128, 40, 512, 2, 1, dict(Ev=96, bias_shape=(512, 40))),
+    (80, 1, 130, 2, 1, {}),
 ]
 
 
