@@ -976,6 +976,284 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(Flash
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Gradient calls that leave most of the chip idle (few (head, batch) pairs, short sequences).  The kernels above give a
+// workgroup 128 queries or 128 keys; these give it 32, with four wavefronts that each take one 32-row block of every
+// 128-row chunk of the other sequence and add up their partial gradients through LDS at the end: four times the
+// workgroups, a quarter of the products, the softmax arithmetic and the operand splits per wavefront.  The stationary
+// rows (Q and dO, or K and V) are split once per workgroup, a quarter per wavefront, and read back from LDS as the B
+// operand.  They need the forward call's statistics; dK and dV come from one kernel that computes S and dP once
+// (seven products for the gradient instead of eight).
+template <int D>
+struct SmallBwd {
+    typedef CfgS<D> C;
+    static constexpr int XPLANEB = 32 * C::ROWB;            // one plane of a stationary 32-row block
+    static constexpr int XB = 3 * XPLANEB;                  // a stationary block
+    static constexpr unsigned OFF_X = 4 * C::TILEB;         // behind the two chunks (two tiles each)
+    static constexpr unsigned OFF_ST = OFF_X + 2 * XB;      // statistics of a query chunk: [3][128] floats
+    static constexpr size_t SMEM = OFF_ST + 3 * 128 * sizeof(float);
+    static constexpr int XCHUNKS = 32 * D / 4 / 256, CHUNKS = BN * D / 4 / 256;
+    static_assert(2 * 4 * 64 * (D / 2) * sizeof(float) <= 4 * C::TILEB, "the partial gradients of four wavefronts fit the chunk buffers");
+
+    // a quarter of a stationary 32-row block per wavefront: loaded, split, stored as planes at `x`
+    __device__ static void split_block(unsigned x, const float *base, int64_t stride, int64_t row0, int64_t nrows, int dh, float scale) {
+        typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
+        floatx4_t reg[XCHUNKS];
+#pragma unroll
+        for (int u = 0; u < XCHUNKS; u++) {
+            const int i = threadIdx.x + 256 * u;
+            const int64_t row = row0 + i / (D / 4);
+            const int col = (i % (D / 4)) * 4;
+            reg[u] = ldg16f(base + stride * row + col, row < nrows && col < dh);
+        }
+#pragma unroll
+        for (int u = 0; u < XCHUNKS; u++) {
+            const int i = threadIdx.x + 256 * u;
+            const int row = i / (D / 4), col = (i % (D / 4)) * 4;
+            const floatx4_t v = reg[u] * scale;
+            uint32_t pl[3][2];
+            const bool odd = split3_pair(v[0], v[1], pl[0][0], pl[1][0], pl[2][0]) | split3_pair(v[2], v[3], pl[0][1], pl[1][1], pl[2][1]);
+            if (odd) {   // an Inf or NaN in the chunk (rare)
+                split3_pair_guarded(v[0], v[1], pl[0][0], pl[1][0], pl[2][0]);
+                split3_pair_guarded(v[2], v[3], pl[0][1], pl[1][1], pl[2][1]);
+            }
+            const unsigned at = x + (unsigned)row * C::ROWB + (unsigned)((((col >> 3) ^ C::swz(row)) << 4) + (col & 7) * 2);
+#pragma unroll
+            for (int q = 0; q < 3; q++) *(lds8_t)(uintptr_t)(at + q * XPLANEB) = (u32x2_t){pl[q][0], pl[q][1]};
+        }
+    }
+
+    // a 128-row chunk of two tensors: loaded into registers, later split into the two-tile buffers at s1 and s2
+    struct Chunk {
+        floatx4_t r1[2][CHUNKS], r2[2][CHUNKS];
+        __device__ void load(const float *b1, const float *b2, int64_t stride, int64_t row0, int64_t nrows, int dh) {
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int u = 0; u < CHUNKS; u++) {
+                    const int i = threadIdx.x + 256 * u;
+                    const int64_t row = row0 + 64 * t + i / (D / 4);
+                    const int col = (i % (D / 4)) * 4;
+                    const bool ok = row < nrows && col < dh;
+                    r1[t][u] = ldg16f(b1 + stride * row + col, ok);
+                    r2[t][u] = ldg16f(b2 + stride * row + col, ok);
+                }
+        }
+        __device__ void store(unsigned s1, unsigned s2) const {
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int u = 0; u < CHUNKS; u++) {
+                    const int i = threadIdx.x + 256 * u;
+                    const int row = i / (D / 4), col = (i % (D / 4)) * 4;
+                    PlaneStream<D>::put(s1 + t * C::TILEB, row, col, r1[t][u]);
+                    PlaneStream<D>::put(s2 + t * C::TILEB, row, col, r2[t][u]);
+                }
+        }
+    };
+
+    // the partial gradients of the four wavefronts added up: each wavefront sums and stores a quarter of the lane's row
+    __device__ static void reduce_store(float *xout, const floatx16_t (&acc)[D / 32], float *grad_row, bool ok, int dh, float scale, bool zero) {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, hh = lane >> 5;
+#pragma unroll
+        for (int dvb = 0; dvb < D / 32; dvb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) xout[(wave * (D / 2) + 16 * dvb + v) * 64 + lane] = acc[dvb][v];
+        __syncthreads();
+        if (ok) {
+            constexpr int PER = D / 32;
+#pragma unroll
+            for (int i = 0; i < PER; i++) {
+                const int piece = wave * PER + i, dvb = piece >> 2, g = piece & 3;
+                floatx4_t o4 = (floatx4_t){0};
+#pragma unroll
+                for (int w = 0; w < 4; w++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o4[e] += xout[(w * (D / 2) + 16 * dvb + 4 * g + e) * 64 + lane];
+                if (zero) o4 = (floatx4_t){0};
+                if (32 * dvb + 8 * g + 4 * hh < dh) *(floatx4_t *)(grad_row + 32 * dvb + 8 * g + 4 * hh) = o4 * scale;
+            }
+        }
+    }
+};
+
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(256, 1) void bwd32s_dq_small_kernel(FlashArgs a, AttnBwdParams bp) {
+    typedef CfgS<D> C;
+    typedef SmallBwd<D> SB;
+    constexpr int NDV = D / 32;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)bwd_smem;
+    const unsigned Ks = lds0, Vs = lds0 + 2 * C::TILEB, Xq = lds0 + SB::OFF_X, Xdo = Xq + SB::XB;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t n_qblocks = (p.Lq + 31) / 32;
+    const int64_t hb = blockIdx.x % HB, qblk = n_qblocks - 1 - blockIdx.x / HB;
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t iw = qblk * 32, qi = iw + r;
+    const bool qok = qi < p.Lq;
+
+    const int64_t head = p.E * (p.Lq * b) + p.D * h;   // E == Ev for these kernels
+    SB::split_block(Xq, (const float *)p.q + head, p.E, iw, p.Lq, (int)p.D, 1.0f);
+    SB::split_block(Xdo, (const float *)bp.dout + head, p.E, iw, p.Lq, (int)p.D, 1.0f);
+    typename SB::Chunk ch;
+    const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h, *vbase = (const float *)p.v + p.E * (p.Lkv * b) + p.D * h;
+    int64_t kv_end = p.Lkv;
+    if (CAUSAL && iw + 32 < kv_end) kv_end = iw + 32;
+    const int n_chunks = (int)((kv_end + 127) / 128);
+    if (bp.dq && n_chunks > 0) ch.load(kbase, vbase, p.E, 0, p.Lkv, (int)p.D);
+
+    // delta = rowsum(O * dO) of the lane's query, saved for the dK / dV kernel
+    float delta = 0.0f;
+    {
+        const int64_t off = head + p.E * qi;
+        floatx4_t o4[D / 8], d4[D / 8];
+#pragma unroll
+        for (int c = 0; c < D / 8; c++) {
+            const bool ok = qok && 8 * c + 4 * hh < p.D;
+            o4[c] = ldg16f((const float *)p.out + off + 8 * c + 4 * hh, ok);
+            d4[c] = ldg16f((const float *)bp.dout + off + 8 * c + 4 * hh, ok);
+        }
+#pragma unroll
+        for (int c = 0; c < D / 8; c++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) delta = fmaf(o4[c][j], d4[c][j], delta);
+        delta += mi_swap32(delta);
+    }
+    const int64_t pad = lq_pad(p.Lq), plane = p.B * p.H * pad, at = (b * p.H + h) * pad + qi;
+    const float m2 = bp.stats[at], linv = bp.stats[plane + at];
+    if (wave == 0 && hh == 0) bp.stats[2 * plane + at] = qok ? delta : 0.0f;
+    if (wave == 1 && qblk == n_qblocks - 1)   // rows no query block covers: a finite delta, their weights are zeros
+        for (int64_t q2 = iw + 32 + lane; q2 < pad; q2 += 64) bp.stats[2 * plane + (b * p.H + h) * pad + q2] = 0.0f;
+    if (!bp.dq) return;
+
+    floatx16_t dq[NDV];
+#pragma unroll
+    for (int dvb = 0; dvb < NDV; dvb++) dq[dvb] = (floatx16_t){0};
+    const float cs = a.c;
+    const unsigned xq_row = Xq + (unsigned)r * C::ROWB, xdo_row = Xdo + (unsigned)r * C::ROWB;
+    const int xsw = C::swz(r);
+    const unsigned blk_tile = (unsigned)(wave >> 1) * C::TILEB;
+    const int kb = wave & 1;
+    for (int c = 0; c < n_chunks; c++) {
+        if (c > 0) __syncthreads();   // every wavefront is done with chunk c - 1
+        ch.store(Ks, Vs);
+        __syncthreads();              // chunk c (and the stationary planes) in LDS
+        if (c + 1 < n_chunks) ch.load(kbase, vbase, p.E, 128 * (int64_t)(c + 1), p.Lkv, (int)p.D);
+        const int64_t j0 = 128 * (int64_t)c + 32 * wave;   // the wavefront's key block
+        if (j0 < p.Lkv && (!CAUSAL || j0 <= iw + 31)) {
+            floatx16_t sb = first_product_sl<D, SB::XPLANEB>(Ks + blk_tile, kb, xq_row, xsw, (floatx16_t){0}, r, hh);
+            SCHED_FENCE();
+            const floatx16_t dpb = first_product_sl<D, SB::XPLANEB>(Vs + blk_tile, kb, xdo_row, xsw, (floatx16_t){0}, r, hh);
+            SCHED_FENCE();
+            // keys of the block this lane's query keeps, counted from the lane's first key of a group of four
+            int64_t lim64 = p.Lkv - j0;
+            if (CAUSAL && qi - j0 + 1 < lim64) lim64 = qi - j0 + 1;
+            const int lim = (lim64 > 32 ? 32 : (lim64 < 0 ? 0 : (int)lim64)) - 4 * hh;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int kvl = 8 * (v / 4) + (v % 4);
+                const float pw = kvl < lim ? mi_exp2(fmaf(sb[v], cs, -m2)) * linv : 0.0f;
+                sb[v] = pw * (dpb[v] - delta);
+            }
+            SCHED_FENCE();
+            second_product_s<D>(Ks + blk_tile, kb, sb, dq, lane);
+            SCHED_FENCE();
+        }
+    }
+    __syncthreads();   // the partial gradients share the chunk buffers
+    SB::reduce_store((float *)bwd_smem, dq, (float *)bp.dq + head + p.E * qi, qok, (int)p.D, a.cn, false);
+}
+
+template <int D, bool CAUSAL>
+__global__ __launch_bounds__(256, 1) void bwd32s_dkdv_small_kernel(FlashArgs a, AttnBwdParams bp) {
+    typedef CfgS<D> C;
+    typedef SmallBwd<D> SB;
+    constexpr int NDV = D / 32;
+    const AttnParams &p = a.p;
+    extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)bwd_smem;
+    const unsigned Qs = lds0, dOs = lds0 + 2 * C::TILEB, Xk = lds0 + SB::OFF_X, Xv = Xk + SB::XB;
+    float *st_lds = (float *)(bwd_smem + SB::OFF_ST);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hh = lane >> 5;
+    const int64_t HB = p.H * p.B;
+    const int64_t hb = blockIdx.x % HB, kblk = blockIdx.x / HB;   // with causal masks the early key blocks are the long ones
+    const int64_t h = hb % p.H, b = hb / p.H;
+    const int64_t jw = kblk * 32, kv = jw + r;
+    const bool kok = kv < p.Lkv;
+
+    const int64_t khead = p.E * (p.Lkv * b) + p.D * h, qhead = p.E * (p.Lq * b) + p.D * h;
+    SB::split_block(Xk, (const float *)p.k + khead, p.E, jw, p.Lkv, (int)p.D, 1.0f);
+    SB::split_block(Xv, (const float *)p.v + khead, p.E, jw, p.Lkv, (int)p.D, 1.0f);
+    const float *qbase = (const float *)p.q + qhead, *dobase = (const float *)bp.dout + qhead;
+    const int64_t pad = lq_pad(p.Lq), plane = p.B * p.H * pad;
+    // the statistics of a query chunk travel with it through LDS: 96 threads x 4 floats (maximum, 1 / row sum, delta)
+    const float *st_src = bp.stats + (b * p.H + h) * pad + (int64_t)(tid >> 5) * plane + 4 * (tid & 31);
+    const int n_qchunks = (int)((p.Lq + 127) / 128);
+    const int c0 = CAUSAL ? (int)(jw / 128) : 0;   // query chunks before the first key of the workgroup see none of its keys
+    typename SB::Chunk ch;
+    floatx4_t st_reg = {0, 0, 0, 0};
+    if (c0 < n_qchunks) {
+        ch.load(qbase, dobase, p.E, 128 * (int64_t)c0, p.Lq, (int)p.D);
+        if (tid < 96) st_reg = *(const floatx4_t *)(st_src + 128 * (int64_t)c0);
+    }
+    floatx16_t acck[NDV], accv[NDV];
+#pragma unroll
+    for (int dvb = 0; dvb < NDV; dvb++) acck[dvb] = accv[dvb] = (floatx16_t){0};
+    const float cs = a.c;
+    const unsigned xk_row = Xk + (unsigned)r * C::ROWB, xv_row = Xv + (unsigned)r * C::ROWB;
+    const int xsw = C::swz(r);
+    const unsigned blk_tile = (unsigned)(wave >> 1) * C::TILEB;
+    const int kb = wave & 1;
+    for (int c = c0; c < n_qchunks; c++) {
+        if (c > c0) __syncthreads();   // every wavefront is done with chunk c - 1
+        ch.store(Qs, dOs);
+        if (tid < 96) *(floatx4_t *)(st_lds + 4 * tid) = st_reg;
+        __syncthreads();               // chunk c (and the stationary planes) in LDS
+        if (c + 1 < n_qchunks) {
+            ch.load(qbase, dobase, p.E, 128 * (int64_t)(c + 1), p.Lq, (int)p.D);
+            if (tid < 96) st_reg = *(const floatx4_t *)(st_src + 128 * (int64_t)(c + 1));
+        }
+        const int64_t i0 = 128 * (int64_t)c + 32 * wave;   // the wavefront's query block
+        if (i0 < p.Lq && (!CAUSAL || i0 + 31 >= jw)) {
+            floatx16_t s = first_product_sl<D, SB::XPLANEB>(Qs + blk_tile, kb, xk_row, xsw, (floatx16_t){0}, r, hh);
+            SCHED_FENCE();
+            floatx16_t dp = first_product_sl<D, SB::XPLANEB>(dOs + blk_tile, kb, xv_row, xsw, (floatx16_t){0}, r, hh);
+            SCHED_FENCE();
+            // accumulator register 4g+e of this lane: query i0 + 8g + 4hh + e, key kv.  Rows past Lq carry statistics
+            // (0, 0, 0): their weights vanish; keys past the length only feed columns that store zeros
+            const bool diag = CAUSAL && i0 < jw + 32;   // some (query, key) pair of this block has key > query
+            const float *st = st_lds + 32 * wave;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int sq = 8 * g + 4 * hh;
+                const floatx4_t m4 = *(const floatx4_t *)(st + sq);
+                const floatx4_t linv4 = *(const floatx4_t *)(st + 128 + sq);
+                const floatx4_t delta4 = *(const floatx4_t *)(st + 256 + sq);
+                const int dq_ = (int)(jw - (i0 + sq)) + r;   // key index minus query index of element e = 0
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float pw = mi_exp2(fmaf(s[4 * g + e], cs, -m4[e])) * linv4[e];
+                    if (diag) pw = dq_ - e > 0 ? 0.0f : pw;
+                    s[4 * g + e] = pw;
+                    dp[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
+                }
+            }
+            SCHED_FENCE();
+            if (bp.dv) second_product_s<D>(dOs + blk_tile, kb, s, accv, lane);
+            SCHED_FENCE();
+            if (bp.dk) second_product_s<D>(Qs + blk_tile, kb, dp, acck, lane);
+            SCHED_FENCE();
+        }
+    }
+    __syncthreads();   // the partial gradients share the chunk buffers
+    float *xout = (float *)bwd_smem;
+    const int64_t off = khead + p.E * kv;
+    if (bp.dv) SB::reduce_store(xout, accv, (float *)bp.dv + off, kok, (int)p.D, 1.0f, false);
+    if (bp.dk) SB::reduce_store(xout + 4 * 64 * (D / 2), acck, (float *)bp.dk + off, kok, (int)p.D, a.cn, false);
+}
+
 // Products on the 16-bit matrix cores through three bf16 planes unless the caller's environment asks for the
 // Float32 matrix instruction (MI355ATTN_F32_MFMA=1), as in the forward kernel.
 bool exact_instruction_wanted() {
@@ -1011,12 +1289,33 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         attr_set = true;
     }
+    // few 32-row blocks (at most two workgroups per compute unit) and the forward call's statistics: the workgroups per
+    // 32 queries / 32 keys
+    static const bool no_small = getenv("MI355ATTN_NO_QUAD") != nullptr;
+    const int64_t q_blocks = (p.Lq + 31) / 32 * p.H * p.B, k_blocks = (p.Lkv + 31) / 32 * p.H * p.B;
+    bool small_q = false, small_k = false;
+    if constexpr (D == 64) {
+        const bool can = bp.have_stats && !a.kv_len && bp.dq_nsplit <= 1 && !no_small;
+        // measured at 32 pairs: 512 blocks 91 against 144 us (causal 65 against 134), 1024 blocks 73 against 66
+        small_q = can && q_blocks <= 512;
+        small_k = can && k_blocks <= 512;
+        if (small_q || small_k) {
+            static bool small_attr_set = false;
+            if (!small_attr_set) {
+                MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_small_kernel<D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
+                MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dkdv_small_kernel<D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
+                small_attr_set = true;
+            }
+        }
+    }
     FlashArgs a1 = a;
     if (bp.dq_nsplit > 1) {   // the dQ kernel's key range in pieces (the dK / dV kernels keep a.nsplit = 1)
         a1.nsplit = bp.dq_nsplit;
         a1.tiles_per_split = (int32_t)(((p.Lkv + BN - 1) / BN + bp.dq_nsplit - 1) / bp.dq_nsplit);
     }
-    if (wide) {
+    if (small_q) {
+        if constexpr (D == 64) hipLaunchKernelGGL((bwd32s_dq_small_kernel<D, CAUSAL>), dim3((unsigned)q_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+    } else if (wide) {
         a1.n_qtiles = (int32_t)wide_tiles;
         hipLaunchKernelGGL(k1w, dim3((unsigned)(wide_tiles * p.H * p.B)), dim3(64 * NW_WIDE), SMEM_WIDE, st, a1, bp);
     } else {
@@ -1024,8 +1323,13 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
     }
     MI_LAUNCH_CHECK();
     const dim3 g2((unsigned)(((p.Lkv + 127) / 128) * p.H * p.B));
-    if (bp.dv) hipLaunchKernelGGL(k2, g2, dim3(256), SMEM, st, a, bp);
-    if (bp.dk) hipLaunchKernelGGL(k3, g2, dim3(256), SMEM, st, a, bp);
+    if (small_k) {
+        if constexpr (D == 64)
+            if (bp.dv || bp.dk) hipLaunchKernelGGL((bwd32s_dkdv_small_kernel<D, CAUSAL>), dim3((unsigned)k_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+    } else {
+        if (bp.dv) hipLaunchKernelGGL(k2, g2, dim3(256), SMEM, st, a, bp);
+        if (bp.dk) hipLaunchKernelGGL(k3, g2, dim3(256), SMEM, st, a, bp);
+    }
     MI_LAUNCH_CHECK();
     return MI_OK;
 }

@@ -180,6 +180,16 @@ F32_CASES = [
     (64, 2, 40, 100, (2,), None, True),
     (64, 1, 70, 70, (1,), "causal", True),
     (32, 2, 33, 300, (1,), None, True),
+    # ... and the gradient kernels that run a workgroup per 32 queries / 32 keys (at most 512 such blocks, saved
+    # statistics, head dim <= 64): several 128-row chunks, ragged ends, the causal diagonal inside a chunk
+    (64, 2, 300, 300, (1,), "causal", True),
+    (48, 2, 129, 257, (2,), None, True),
+    (64, 8, 128, 128, (4,), None, True),
+    (64, 1, 1, 200, (3,), None, True),
+    (64, 1, 500, 31, (1,), None, True),
+    # more blocks than that: the workgroups of 128 queries / keys with saved statistics
+    (64, 4, 128, 128, (40,), None, True),
+    (64, 4, 100, 100, (40,), "causal", True),
 ]
 
 
