@@ -1295,9 +1295,11 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
     const int64_t q_blocks = (p.Lq + 31) / 32 * p.H * p.B, k_blocks = (p.Lkv + 31) / 32 * p.H * p.B;
     bool small_q = false, small_k = false;
     if constexpr (D == 64) {
-        const bool can = bp.have_stats && !a.kv_len && bp.dq_nsplit <= 1 && !no_small;
-        // measured at 32 pairs: 512 blocks 91 against 144 us (causal 65 against 134), 1024 blocks 73 against 66
-        small_q = can && q_blocks <= 512;
+        // measured at 32 pairs: 512 blocks 91 against 144 us (causal 65 against 134), 1024 blocks 73 against 66.  The dQ
+        // kernel reads the statistics it is given; the dK / dV kernel reads what the dQ kernel before it left in
+        // bp.stats, whichever that was
+        const bool can = !a.kv_len && !no_small;
+        small_q = can && bp.have_stats && bp.dq_nsplit <= 1 && q_blocks <= 512;
         small_k = can && k_blocks <= 512;
         if (small_q || small_k) {
             static bool small_attr_set = false;
