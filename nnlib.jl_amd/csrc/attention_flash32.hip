@@ -1455,7 +1455,11 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     const bool few_blocks = (p.Lq + 31) / 32 * p.H * p.B <= RESIDENT_QUAD_MAX_BLOCKS;
     if (narrow && (p.weights || few_blocks) && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted()) return launch_resident<64>(a, st, extras);
     static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;
-    if (few_blocks && p.Lkv <= RES_CHUNKS * 128 && !exact_instruction_wanted() && !no_quad)
+    // against the two-pass kernel the workgroup per query block still wins at two workgroups per compute unit when the
+    // weights are written or the mask is causal (512 blocks of 512 keys: 43 against 58 us with weights, causal 36 against
+    // 62; without weights 40 against 36, causal 28 against 41); beyond that it loses
+    const int64_t chunk_max = (p.weights || p.causal) ? 2 * RESIDENT_QUAD_MAX_BLOCKS : RESIDENT_QUAD_MAX_BLOCKS;
+    if ((p.Lq + 31) / 32 * p.H * p.B <= chunk_max && (!narrow || p.Lkv > RES_TILES * BN) && p.Lkv <= RES_CHUNKS * 128 && !exact_instruction_wanted() && !no_quad)
         return narrow ? launch_resident_chunks<64>(a, st, extras) : launch_resident_chunks<128>(a, st, extras);
     return narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
 }

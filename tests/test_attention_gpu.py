@@ -354,6 +354,9 @@ MID_F32_CASES = [
     (256, 70, 200, 2, 2, dict(bias_shape=(200, 70, 2, 2), mask_shape=(200, 70))),
     (128, 40, 512, 2, 1, dict(Ev=96, bias_shape=(512, 40))),
     (80, 1, 130, 2, 1, {}),
+    # 257 to 512 blocks: with the weights or the causal mask this kernel, otherwise the two-pass kernel
+    (256, 256, 256, 12, 4, {}),
+    (256, 200, 200, 16, 4, dict(causal=True)),
 ]
 
 
