@@ -146,3 +146,31 @@ def test_dense_masks_without_weights(nn, oracle, seed):
     assert np.array_equal(np.isnan(y), nan_ref), (dtype, D, H, B, Lq, Lkv, causal, shape, keep)
     err = rel_err(np.where(nan_ref, 0, y), np.where(nan_ref, 0, y_ref))
     assert err <= TOL[dtype], (err, dtype, D, H, B, Lq, Lkv, causal, shape, keep, nn.last_attention_kernel())
+
+
+# ---- fourth sweep: Float32 calls on few workgroups (a workgroup per 32 queries / 32 keys, forward and gradient) ----
+
+N_SMALL = int(os.environ.get("MI355ATTN_SMALL_SEEDS", "40"))
+
+
+@pytest.mark.parametrize("seed", range(N_SMALL))
+def test_float32_calls_on_few_workgroups(nn, oracle, seed):
+    """Lengths around the 32-row blocks and 128-row chunks those kernels cut the sequences into, head dims on both tile
+    widths, with and without the weights, the causal mask and bias / mask arrays in the forward call, saved statistics
+    or not in the gradient call (which takes no bias / mask arrays on those kernels)."""
+    from test_attention_gpu import _check
+    from test_attention_backward_gpu import _run
+    rng = np.random.default_rng(9000 + seed)
+    D = int(rng.choice([16, 32, 48, 64, 64, 64, 96, 128]))
+    H, B = int(rng.integers(1, 5)), int(rng.integers(1, 4))
+    edges = [1, 5, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 160, 255, 256, 257, 300, 383, 385, 500, 512]
+    Lq = int(rng.choice(edges))
+    causal = bool(rng.integers(0, 2))
+    Lkv = Lq if causal else int(rng.choice(edges))
+    extras = int(rng.integers(0, 3)) == 0
+    bias_shape = (Lkv, Lq, H, 1) if extras else None
+    mask_shape = (Lkv, Lq) if extras and not causal else None
+    _check(nn, oracle, rng, "f32", D * H, Lq, Lkv, B, H, causal=causal, bias_shape=bias_shape, mask_shape=mask_shape,
+           scale=0.5, expect="flash32", weights=bool(seed % 2))
+    _run(nn, oracle, "f32", D * H, D * H, Lq, Lkv, (B,), H, mask_kind="causal" if causal else None, seed=seed, scale=0.4,
+         saved=bool((seed // 2) % 2))
