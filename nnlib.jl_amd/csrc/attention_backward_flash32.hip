@@ -1301,6 +1301,18 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
         const bool can = !a.kv_len && !no_small;
         small_q = can && bp.have_stats && bp.dq_nsplit <= 1 && q_blocks <= 512;
         small_k = can && k_blocks <= 512;
+        // no statistics from the caller: where the forward kernels of this shape of call apply (a workgroup per 32
+        // queries, at most 512 keys), their statistics-only run (no values, no output) fills bp.stats first
+        if (can && !bp.have_stats && bp.dq_nsplit <= 1 && q_blocks <= 256 && p.Lkv <= 512 && p.scale_D == 0 && !exact_instruction_wanted()) {
+            AttnParams pf = p;
+            pf.out = nullptr;
+            pf.weights = nullptr;
+            pf.workspace = nullptr;
+            pf.stats = bp.stats;
+            const int32_t rc = launch_attention_flash32(pf, st);
+            if (rc != MI_OK) return rc;
+            small_q = true;
+        }
         if (small_q || small_k) {
             static bool small_attr_set = false;
             if (!small_attr_set) {
