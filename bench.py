@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|dense_mask|bwd|bwd_f32|logsoftmax|softmax|softmax_dims2|batched_mul[_f32|_c32|_f64]] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1|c2|c3|c4|c5|dense_mask|bwd|bwd_f32|bwd_c1|logsoftmax|softmax|softmax_dims2|batched_mul[_f32|_c32|_f64]] [--no-cpu]
 
 A "step" is one dot_product_attention call on synthetic inputs that are already resident in HBM.
 The default workload is C3 (bf16 causal prefill, head dim 128, L = 4096), the configuration the
@@ -32,7 +32,7 @@ TRAFFIC_FILE = os.path.join("profiles", "hbm_traffic_fetch_write_size.md")
 DOMINANT_KERNEL = {"c1": "flash32_resident", "c2": "flash32_kernel", "c3": "flash16_fast_kernel", "c4": "flash16_kernel",
                    "c5": "decode_split_kernel",
                    # a gradient step is three kernels (dq, dk, dv): every row of the workload whose name contains "bwd"
-                   "bwd": "bwd", "bwd_f32": "bwd", "softmax": "softmax", "logsoftmax": "softmax", "softmax_dims2": "softmax",
+                   "bwd": "bwd", "bwd_f32": "bwd", "bwd_c1": "bwd", "softmax": "softmax", "logsoftmax": "softmax", "softmax_dims2": "softmax",
                    "batched_mul": "gemm", "batched_mul_f32": "gemm",
                    "dense_mask": "flash16_fast_kernel<false, true"}
 
@@ -317,6 +317,7 @@ EXTRA = {
     "dense_mask": "forward call of the C3 shape with a dense Bool mask (4096, 4096), 90 % kept, not causal, weights not materialised; "
                   "the same call without the mask is timed beside it",
     "bwd_f32": "gradient of C2: causal f32 (1024,1024,8) H=16 D=64, dq + dk + dv from dy and the forward result",
+    "bwd_c1": "gradient of C1: f32 (512,128,4) H=8 D=64, not causal, dq + dk + dv from dy and the forward result (a call on few workgroups: report us)",
     "logsoftmax": "logsoftmax(x; dims=1), x (4096, 65536) f32 (1 GiB in, 1 GiB out)",
     "softmax_dims2": "softmax(x; dims=2), x (256, 4096, 128) bf16 (256 MiB in, 256 MiB out), reduction over the strided dim",
     "softmax": "softmax(x; dims=1), x (1024, 131072) f32: the logits of C2 (512 MiB in, 512 MiB out)",
@@ -377,8 +378,8 @@ def measure_extra(key, steps, warmup, with_cpu):
                     config=dict(workload=EXTRA[key], kernel=kernel, unmasked_ms_per_step=ms_of["unmasked"],
                                 rate_against_unmasked=ms_of["unmasked"] / ms),
                     flops_per_step=flops)
-    elif key in ("bwd", "bwd_f32"):
-        w = WORKLOADS["c3" if key == "bwd" else "c2"]
+    elif key in ("bwd", "bwd_f32", "bwd_c1"):
+        w = WORKLOADS[{"bwd": "c3", "bwd_f32": "c2", "bwd_c1": "c1"}[key]]
         E, L, B, H = w["E"], w["Lq"], w["B"], w["H"]
         D = E // H
         dtn = w["dtype"]
@@ -386,11 +387,12 @@ def measure_extra(key, steps, warmup, with_cpu):
         for sid, a in enumerate(arrs):
             _lib.check(lib.mi_randn_fill(a.ptr, a.code, a.length, w["seed"], sid, w["scale"] if sid < 2 else 1.0, None))
         q, k, v, dy = arrs
-        y, _ = nn.dot_product_attention(q, k, v, mask=nn.make_causal_mask(q), nheads=H, return_weights=False,
+        cmask = nn.make_causal_mask(q) if w["causal"] else None
+        y, _ = nn.dot_product_attention(q, k, v, mask=cmask, nheads=H, return_weights=False,
                                         save_for_backward=True)   # as an AD rule would: the pullback reuses the row statistics
         d = _lib.mi_attn_bwd_desc()
         d.struct_size = ctypes.sizeof(_lib.mi_attn_bwd_desc)
-        nn.ops._fill_desc(d.fwd, q, k, v, None, nn.make_causal_mask(q), H, B, E, E, L, L, 0)
+        nn.ops._fill_desc(d.fwd, q, k, v, None, cmask, H, B, E, E, L, L, 0)
         d.fwd.out, d.dout, d.fwd.stats = y.ptr, dy.ptr, y.saved_stats.ptr
         grads = [DA.empty((E, L, B), dtn) for _ in range(3)]
         d.dq, d.dk, d.dv = (g.ptr for g in grads)
@@ -400,22 +402,24 @@ def measure_extra(key, steps, warmup, with_cpu):
         d.workspace, d.workspace_bytes = wsbuf.ptr, ws.value
         ms = _event_time(lib, _lib, lambda: _lib.check(lib.mi_attention_bwd(ctypes.byref(d), None)), steps, warmup)
         # five products (S, dP, dV, dK, dQ) of 2*D FLOP per unmasked (query, key) pair
-        flops = 10 * D * H * B * (L * (L + 1) // 2)
+        flops = 10 * D * H * B * (L * (L + 1) // 2 if w["causal"] else L * L)
         val = flops / (ms * 1e-3) / 1e12
         line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype=dtn,
                     roofline=dict(bound="mfma", achieved=val, peak=PEAK[dtn], unit="TFLOP/s", frac=val / PEAK[dtn], **measured_traffic_fields(key)),
                     config=dict(workload=EXTRA[key], kernel=_lib.KERNEL_NAMES[kern.value]), flops_per_step=flops)
         # 16-bit: dQ kernel S, dP, dQ; fused dK / dV kernel S, dV, dP, dK.  Float32: dQ: S, dP, dQ; dV: S, dV; dK: S, dP, dK
-        line["roofline"]["products_executed_per_counted"] = 8 / 5 if dtn == "f32" else 7 / 5
+        # (the Float32 kernels of calls on few workgroups: dQ: S, dP, dQ; dK / dV: S, dP, dV, dK)
+        per_counted = 7 / 5 if dtn != "f32" or key == "bwd_c1" else 8 / 5
+        line["roofline"]["products_executed_per_counted"] = per_counted
         if dtn == "f32":
-            f32_products(line["roofline"], val, 8 / 5)
+            f32_products(line["roofline"], val, per_counted)
         if with_cpu:
             from oracle import oracle as O
             rng = np.random.default_rng(0)
             nh, nb = (4, 1) if key == "bwd" else (H, 2)          # a bounded sample of whole (head, batch) slices
             a1 = [np.asfortranarray(rng.standard_normal((nh * D, L, nb))) for _ in range(4)]
             t0 = time.perf_counter()
-            O.attention_bwd_f64(a1[0], a1[1], a1[2], a1[3], None, O.make_causal_mask(L), nh)
+            O.attention_bwd_f64(a1[0], a1[1], a1[2], a1[3], None, O.make_causal_mask(L) if w["causal"] else None, nh)
             dt = time.perf_counter() - t0
             line["cpu_baseline"] = dict(value=flops * nh * nb / (dt * H * B) / 1e12, unit="TFLOP/s", cores=1, kind="port",
                                         sample=f"{nh * nb} of {H * B} (head, batch) slices, forward + gradient oracle in Float64 on one "
