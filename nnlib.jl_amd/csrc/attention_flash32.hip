@@ -1439,7 +1439,20 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
         if (rc != MI_OK) return rc;
         return launch_flash_merge(p, a.nsplit, st);
     }
-    if (attention_flash32_lengths_bytes(p) != 0) {
+    const bool extras = p.bias || p.mask;
+    // few keys and the weights returned: everything resident, one pass (flash32_resident_kernel); without the weights
+    // when the call leaves most of the chip idle (the workgroup per 32-query block)
+    const bool few_blocks = (p.Lq + 31) / 32 * p.H * p.B <= RESIDENT_QUAD_MAX_BLOCKS;
+    const bool resident = narrow && (p.weights || few_blocks) && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted();
+    static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;
+    // against the two-pass kernel the workgroup per query block still wins at two workgroups per compute unit when the
+    // weights are written or the mask is causal (512 blocks of 512 keys: 43 against 58 us with weights, causal 36 against
+    // 62; without weights 40 against 36, causal 28 against 41); beyond that it loses
+    const int64_t chunk_max = (p.weights || p.causal) ? 2 * RESIDENT_QUAD_MAX_BLOCKS : RESIDENT_QUAD_MAX_BLOCKS;
+    const bool chunks = (p.Lq + 31) / 32 * p.H * p.B <= chunk_max && (!narrow || p.Lkv > RES_TILES * BN) && p.Lkv <= RES_CHUNKS * 128 &&
+                        !exact_instruction_wanted() && !no_quad;
+    // (calls on few workgroups take a key-padding mask like any other mask: one launch instead of three)
+    if (attention_flash32_lengths_bytes(p) != 0 && !((resident && few_blocks && !no_quad) || chunks)) {
         // key-padding mask: classify the (head, batch) pairs on the device, then launch both variants
         int32_t *lens = (int32_t *)p.workspace;
         int32_t rc = launch_key_mask_lengths(p, lens, st);
@@ -1449,17 +1462,7 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
         if (rc != MI_OK) return rc;
         return narrow ? launch_d<64, 1>(a, st, true) : launch_d<128, 1>(a, st, true);
     }
-    const bool extras = p.bias || p.mask;
-    // few keys and the weights returned: everything resident, one pass (flash32_resident_kernel); without the weights
-    // when the call leaves most of the chip idle (the workgroup per 32-query block)
-    const bool few_blocks = (p.Lq + 31) / 32 * p.H * p.B <= RESIDENT_QUAD_MAX_BLOCKS;
-    if (narrow && (p.weights || few_blocks) && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted()) return launch_resident<64>(a, st, extras);
-    static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;
-    // against the two-pass kernel the workgroup per query block still wins at two workgroups per compute unit when the
-    // weights are written or the mask is causal (512 blocks of 512 keys: 43 against 58 us with weights, causal 36 against
-    // 62; without weights 40 against 36, causal 28 against 41); beyond that it loses
-    const int64_t chunk_max = (p.weights || p.causal) ? 2 * RESIDENT_QUAD_MAX_BLOCKS : RESIDENT_QUAD_MAX_BLOCKS;
-    if ((p.Lq + 31) / 32 * p.H * p.B <= chunk_max && (!narrow || p.Lkv > RES_TILES * BN) && p.Lkv <= RES_CHUNKS * 128 && !exact_instruction_wanted() && !no_quad)
-        return narrow ? launch_resident_chunks<64>(a, st, extras) : launch_resident_chunks<128>(a, st, extras);
+    if (resident) return launch_resident<64>(a, st, extras);
+    if (chunks) return narrow ? launch_resident_chunks<64>(a, st, extras) : launch_resident_chunks<128>(a, st, extras);
     return narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
 }
