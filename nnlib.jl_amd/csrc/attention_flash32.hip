@@ -1072,14 +1072,14 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs
     }
 }
 
-// The workgroup per 32-query block for up to RES_CHUNKS * 128 keys: the keys in chunks of 128 (four 32-key blocks, one per
+// The workgroup per 32-query block for up to NCH * 128 keys (NCH = 4, or 8 at head dims up to 64): the keys in chunks of 128 (four 32-key blocks, one per
 // wavefront), the raw scores of every chunk kept in registers between the statistics and the weights, so the score
 // product still runs once.  First phase: K chunks through two LDS buffers (the next chunk's loads in flight, one
 // barrier per chunk); second phase: V chunks through the same two buffers.  128-wide tiles have room for one buffer
 // (96 KiB): a second barrier per chunk before it is overwritten, and the partial outputs share it at the end.
-constexpr int RES_CHUNKS = 4;
+constexpr int RES_CHUNKS = 4, RES_CHUNKS_NARROW = 8;
 
-template <int D, bool CAUSAL, bool EXTRAS>
+template <int D, bool CAUSAL, bool EXTRAS, int NCH>
 __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashArgs a) {
     typedef CfgS<D> C;
     constexpr int ROWB = C::ROWB, PLANEB = C::PLANEB, CHUNKS = C::CHUNKS, TILEB = C::TILEB;
@@ -1106,7 +1106,7 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
     const int64_t iw = qblk * 32, qi = iw + r;
     int64_t kv_end = p.Lkv;
     if (CAUSAL && iw + 32 < kv_end) kv_end = iw + 32;
-    const int n_chunks = (int)((kv_end + 127) / 128);   // <= RES_CHUNKS: checked by the host
+    const int n_chunks = (int)((kv_end + 127) / 128);   // <= NCH: checked by the host
     const bool do_pv = p.out != nullptr;
 
     const float *kbase = (const float *)p.k + p.E * (p.Lkv * b) + p.D * h;
@@ -1181,9 +1181,9 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
 
     // ---- first phase: scores of the wavefront's block of every chunk (kept raw), running statistics
     const unsigned blk = (unsigned)(wave >> 1) * TILEB + (unsigned)(wave & 1) * 32u * ROWB;
-    floatx16_t keep[RES_CHUNKS][1][1];
+    floatx16_t keep[NCH][1][1];
 #pragma unroll
-    for (int c = 0; c < RES_CHUNKS; c++) {
+    for (int c = 0; c < NCH; c++) {
         if (c < n_chunks) {
             if (c + 1 < n_chunks) load_chunk(nxt, kbase, p.E, dqk, c + 1, true);
             else load_chunk(nxt, vbase, p.Ev, dv, 0, do_pv);   // the first V chunk
@@ -1234,7 +1234,7 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
     // ---- second phase: weights and the wavefront's share of the output, V chunks through the same buffers
     const unsigned wlds = lds0 + OFF_STAGE + wave * FLASH_WSTAGE_BYTES;
 #pragma unroll
-    for (int c = 0; c < RES_CHUNKS; c++) {
+    for (int c = 0; c < NCH; c++) {
         if (c < n_chunks) {
             const unsigned buf = lds0 + (TWO_BUFFERS ? (unsigned)(c & 1) * 2u * TILEB : 0u);
             if (do_pv) {
@@ -1282,7 +1282,7 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_chunks_kernel(FlashAr
     }
 }
 
-template <int D>
+template <int D, int NCH>
 int32_t launch_resident_chunks(const FlashArgs &a, hipStream_t st, bool extras) {
     constexpr size_t smem = (D <= 64 ? 4 * CfgS<D>::TILEB + 4 * 64 * (D / 2) * sizeof(float) : 2 * CfgS<D>::TILEB) + 4 * FLASH_WSTAGE_BYTES +
                             4 * 32 * 2 * sizeof(float) + 3 * 32 * CfgS<D>::ROWB;
@@ -1290,15 +1290,15 @@ int32_t launch_resident_chunks(const FlashArgs &a, hipStream_t st, bool extras) 
     static_assert(4 * 64 * (D / 2) * sizeof(float) <= 2 * CfgS<D>::TILEB, "the partial outputs fit a chunk buffer");
     static bool attr_set = false;
     if (!attr_set) {
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, false, false, NCH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, false, true, NCH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, true, false, NCH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)flash32_resident_chunks_kernel<D, true, true, NCH>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
     const int64_t total = (a.p.Lq + 31) / 32 * a.p.H * a.p.B;
-    auto kern = a.p.causal ? (extras ? flash32_resident_chunks_kernel<D, true, true> : flash32_resident_chunks_kernel<D, true, false>)
-                           : (extras ? flash32_resident_chunks_kernel<D, false, true> : flash32_resident_chunks_kernel<D, false, false>);
+    auto kern = a.p.causal ? (extras ? flash32_resident_chunks_kernel<D, true, true, NCH> : flash32_resident_chunks_kernel<D, true, false, NCH>)
+                           : (extras ? flash32_resident_chunks_kernel<D, false, true, NCH> : flash32_resident_chunks_kernel<D, false, false, NCH>);
     hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(256), smem, st, a);
     MI_LAUNCH_CHECK();
     return MI_OK;
@@ -1449,7 +1449,7 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     // weights are written or the mask is causal (512 blocks of 512 keys: 43 against 58 us with weights, causal 36 against
     // 62; without weights 40 against 36, causal 28 against 41); beyond that it loses
     const int64_t chunk_max = (p.weights || p.causal) ? 2 * RESIDENT_QUAD_MAX_BLOCKS : RESIDENT_QUAD_MAX_BLOCKS;
-    const bool chunks = (p.Lq + 31) / 32 * p.H * p.B <= chunk_max && (!narrow || p.Lkv > RES_TILES * BN) && p.Lkv <= RES_CHUNKS * 128 &&
+    const bool chunks = (p.Lq + 31) / 32 * p.H * p.B <= chunk_max && (!narrow || p.Lkv > RES_TILES * BN) && p.Lkv <= (narrow ? RES_CHUNKS_NARROW : RES_CHUNKS) * 128 &&
                         !exact_instruction_wanted() && !no_quad;
     // (calls on few workgroups take a key-padding mask like any other mask: one launch instead of three)
     if (attention_flash32_lengths_bytes(p) != 0 && !((resident && few_blocks && !no_quad) || chunks)) {
@@ -1463,6 +1463,9 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
         return narrow ? launch_d<64, 1>(a, st, true) : launch_d<128, 1>(a, st, true);
     }
     if (resident) return launch_resident<64>(a, st, extras);
-    if (chunks) return narrow ? launch_resident_chunks<64>(a, st, extras) : launch_resident_chunks<128>(a, st, extras);
+    if (chunks) {
+        if (!narrow) return launch_resident_chunks<128, RES_CHUNKS>(a, st, extras);
+        return p.Lkv <= RES_CHUNKS * 128 ? launch_resident_chunks<64, RES_CHUNKS>(a, st, extras) : launch_resident_chunks<64, RES_CHUNKS_NARROW>(a, st, extras);
+    }
     return narrow ? launch_d<64, 1>(a, st, extras) : launch_d<128, 1>(a, st, extras);
 }

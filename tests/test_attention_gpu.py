@@ -332,7 +332,7 @@ def test_small_float32_problem_without_weights(nn, oracle, case):
 
 
 MID_F32_CASES = [
-    # Float32, 129 to 512 keys, at most 256 blocks of 32 queries: a workgroup per query block that keeps the scores of
+    # Float32, 129 to 512 keys (1024 at head dims up to 64), few blocks of 32 queries: a workgroup per query block that keeps the scores of
     # every 128-key chunk in registers (one to four chunks, ragged last chunk and last block, causal diagonal inside a
     # chunk, bias / mask, v wider than q and k)
     (128, 129, 129, 1, 2, {}),
@@ -354,6 +354,11 @@ MID_F32_CASES = [
     (256, 70, 200, 2, 2, dict(bias_shape=(200, 70, 2, 2), mask_shape=(200, 70))),
     (128, 40, 512, 2, 1, dict(Ev=96, bias_shape=(512, 40))),
     (80, 1, 130, 2, 1, {}),
+    # 513 to 1024 keys at head dims up to 64: eight chunks
+    (128, 100, 1024, 1, 2, {}),
+    (64, 700, 700, 1, 1, dict(causal=True)),
+    (128, 40, 770, 2, 2, dict(bias_shape=(770, 40, 2, 1), mask_shape=(770, 40))),
+    (96, 513, 513, 1, 3, dict(causal=True, mask_shape=(513, 513))),
     # 257 to 512 blocks: with the weights or the causal mask this kernel, otherwise the two-pass kernel
     (256, 256, 256, 12, 4, {}),
     (256, 200, 200, 16, 4, dict(causal=True)),

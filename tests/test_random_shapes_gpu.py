@@ -164,9 +164,9 @@ def test_float32_calls_on_few_workgroups(nn, oracle, seed):
     D = int(rng.choice([16, 32, 48, 64, 64, 64, 96, 128]))
     H, B = int(rng.integers(1, 5)), int(rng.integers(1, 4))
     edges = [1, 5, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 160, 255, 256, 257, 300, 383, 385, 500, 512]
-    Lq = int(rng.choice(edges))
+    Lq = int(rng.choice(edges + [640, 1000]))
     causal = bool(rng.integers(0, 2))
-    Lkv = Lq if causal else int(rng.choice(edges))
+    Lkv = Lq if causal else int(rng.choice(edges + [513, 769, 897, 1024]))
     extras = int(rng.integers(0, 3)) == 0
     bias_shape = (Lkv, Lq, H, 1) if extras else None
     mask_shape = (Lkv, Lq) if extras and not causal else None
