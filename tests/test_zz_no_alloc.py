@@ -113,7 +113,7 @@ def test_split_kv_calls_then_a_smaller_one(nn):
 def test_context_length_masks_then_a_smaller_one(nn):
     """Key-padding masks: one measured context length per (head, batch) pair goes through the workspace."""
     _both(nn, "bf16", 256, 300, 1100, 6, 2, 11, key_mask=True, expect_kernel="flash16")
-    _both(nn, "bf16", 128, 140, 332, 3, 1, 12, key_mask=True, weights=True, expect_kernel="flash16")
+    _both(nn, "bf16", 128, 140, 716, 3, 1, 12, key_mask=True, weights=True, expect_kernel="flash16")
 
 
 def test_calls_without_a_workspace(nn):
