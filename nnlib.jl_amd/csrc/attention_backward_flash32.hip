@@ -1077,7 +1077,9 @@ struct SmallBwd {
     }
 };
 
-template <int D, bool CAUSAL>
+// MASKED: a Bool mask array of any strides (no bias): one byte per (key, query) pair of the lane, requested before the
+// products
+template <int D, bool CAUSAL, bool MASKED>
 __global__ __launch_bounds__(256, 1) void bwd32s_dq_small_kernel(FlashArgs a, AttnBwdParams bp) {
     typedef CfgS<D> C;
     typedef SmallBwd<D> SB;
@@ -1143,6 +1145,15 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_small_kernel(FlashArgs a, At
         if (c + 1 < n_chunks) ch.load(kbase, vbase, p.E, 128 * (int64_t)(c + 1), p.Lkv, (int)p.D);
         const int64_t j0 = 128 * (int64_t)c + 32 * wave;   // the wavefront's key block
         if (j0 < p.Lkv && (!CAUSAL || j0 <= iw + 31)) {
+            uint8_t mk[16];
+            if constexpr (MASKED) {
+                const uint8_t *mrow = p.mask + (qok ? qi : 0) * p.mask_strides[1] + h * p.mask_strides[2] + b * p.mask_strides[3];
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int64_t key = j0 + 8 * (v / 4) + 4 * hh + (v % 4);
+                    mk[v] = mrow[(key < p.Lkv ? key : 0) * p.mask_strides[0]];
+                }
+            }
             floatx16_t sb = first_product_sl<D, SB::XPLANEB>(Ks + blk_tile, kb, xq_row, xsw, (floatx16_t){0}, r, hh);
             SCHED_FENCE();
             const floatx16_t dpb = first_product_sl<D, SB::XPLANEB>(Vs + blk_tile, kb, xdo_row, xsw, (floatx16_t){0}, r, hh);
@@ -1154,7 +1165,9 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_small_kernel(FlashArgs a, At
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int kvl = 8 * (v / 4) + (v % 4);
-                const float pw = kvl < lim ? mi_exp2(fmaf(sb[v], cs, -m2)) * linv : 0.0f;
+                bool keep = kvl < lim;
+                if constexpr (MASKED) keep = keep && mk[v] != 0;
+                const float pw = keep ? mi_exp2(fmaf(sb[v], cs, -m2)) * linv : 0.0f;
                 sb[v] = pw * (dpb[v] - delta);
             }
             SCHED_FENCE();
@@ -1166,7 +1179,7 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_small_kernel(FlashArgs a, At
     SB::reduce_store((float *)bwd_smem, dq, (float *)bp.dq + head + p.E * qi, qok, (int)p.D, a.cn, false);
 }
 
-template <int D, bool CAUSAL>
+template <int D, bool CAUSAL, bool MASKED>
 __global__ __launch_bounds__(256, 1) void bwd32s_dkdv_small_kernel(FlashArgs a, AttnBwdParams bp) {
     typedef CfgS<D> C;
     typedef SmallBwd<D> SB;
@@ -1217,6 +1230,15 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dkdv_small_kernel(FlashArgs a, 
         }
         const int64_t i0 = 128 * (int64_t)c + 32 * wave;   // the wavefront's query block
         if (i0 < p.Lq && (!CAUSAL || i0 + 31 >= jw)) {
+            uint8_t mk[16];
+            if constexpr (MASKED) {
+                const uint8_t *mcol = p.mask + (kok ? kv : 0) * p.mask_strides[0] + h * p.mask_strides[2] + b * p.mask_strides[3];
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int64_t qq = i0 + 8 * (v / 4) + 4 * hh + (v % 4);
+                    mk[v] = mcol[(qq < p.Lq ? qq : 0) * p.mask_strides[1]];
+                }
+            }
             floatx16_t s = first_product_sl<D, SB::XPLANEB>(Qs + blk_tile, kb, xk_row, xsw, (floatx16_t){0}, r, hh);
             SCHED_FENCE();
             floatx16_t dp = first_product_sl<D, SB::XPLANEB>(dOs + blk_tile, kb, xv_row, xsw, (floatx16_t){0}, r, hh);
@@ -1236,6 +1258,7 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dkdv_small_kernel(FlashArgs a, 
                 for (int e = 0; e < 4; e++) {
                     float pw = mi_exp2(fmaf(s[4 * g + e], cs, -m4[e])) * linv4[e];
                     if (diag) pw = dq_ - e > 0 ? 0.0f : pw;
+                    if constexpr (MASKED) pw = mk[4 * g + e] != 0 ? pw : 0.0f;
                     s[4 * g + e] = pw;
                     dp[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
                 }
@@ -1316,8 +1339,8 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
         if (small_q || small_k) {
             static bool small_attr_set = false;
             if (!small_attr_set) {
-                MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_small_kernel<D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
-                MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dkdv_small_kernel<D, CAUSAL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
+                MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_small_kernel<D, CAUSAL, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
+                MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dkdv_small_kernel<D, CAUSAL, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
                 small_attr_set = true;
             }
         }
@@ -1328,7 +1351,7 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
         a1.tiles_per_split = (int32_t)(((p.Lkv + BN - 1) / BN + bp.dq_nsplit - 1) / bp.dq_nsplit);
     }
     if (small_q) {
-        if constexpr (D == 64) hipLaunchKernelGGL((bwd32s_dq_small_kernel<D, CAUSAL>), dim3((unsigned)q_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+        if constexpr (D == 64) hipLaunchKernelGGL((bwd32s_dq_small_kernel<D, CAUSAL, false>), dim3((unsigned)q_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
     } else if (wide) {
         a1.n_qtiles = (int32_t)wide_tiles;
         hipLaunchKernelGGL(k1w, dim3((unsigned)(wide_tiles * p.H * p.B)), dim3(64 * NW_WIDE), SMEM_WIDE, st, a1, bp);
@@ -1339,7 +1362,7 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
     const dim3 g2((unsigned)(((p.Lkv + 127) / 128) * p.H * p.B));
     if (small_k) {
         if constexpr (D == 64)
-            if (bp.dv || bp.dk) hipLaunchKernelGGL((bwd32s_dkdv_small_kernel<D, CAUSAL>), dim3((unsigned)k_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+            if (bp.dv || bp.dk) hipLaunchKernelGGL((bwd32s_dkdv_small_kernel<D, CAUSAL, false>), dim3((unsigned)k_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
     } else {
         if (bp.dv) hipLaunchKernelGGL(k2, g2, dim3(256), SMEM, st, a, bp);
         if (bp.dk) hipLaunchKernelGGL(k3, g2, dim3(256), SMEM, st, a, bp);
@@ -1438,6 +1461,46 @@ bool attention_bwd_flash32_supports(const AttnBwdParams &bp) {
     return tiles * p.H * p.B <= 2147483647LL;
 }
 
+namespace {
+// Small calls with a Bool mask array and no bias: the workgroups per 32 queries / 32 keys read the mask bytes of their
+// pairs themselves (any strides; a key-padding mask needs no classification of context lengths)
+bool small_masked_call(const AttnBwdParams &bp) {
+    static const bool no_small = getenv("MI355ATTN_NO_QUAD") != nullptr;
+    const AttnParams &p = bp.p;
+    if (no_small || !p.mask || p.bias || bp.dbias || p.drop_thresh || p.D > 64 || exact_instruction_wanted() || bp.dq_nsplit > 1) return false;
+    const int64_t q_blocks = (p.Lq + 31) / 32 * p.H * p.B, k_blocks = (p.Lkv + 31) / 32 * p.H * p.B;
+    if (q_blocks > 512 || k_blocks > 512) return false;
+    // without the caller's statistics the forward kernels' statistics-only run has to apply (see launch_set_planes)
+    return bp.have_stats || (q_blocks <= 256 && p.Lkv <= 512 && p.scale_D == 0);
+}
+
+template <bool CAUSAL>
+int32_t launch_small_masked(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
+    constexpr int D = 64;
+    const AttnParams &p = a.p;
+    static bool attr_set = false;
+    if (!attr_set) {
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_small_kernel<D, CAUSAL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dkdv_small_kernel<D, CAUSAL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
+        attr_set = true;
+    }
+    if (!bp.have_stats) {
+        AttnParams pf = p;
+        pf.out = nullptr;
+        pf.weights = nullptr;
+        pf.workspace = nullptr;
+        pf.stats = bp.stats;
+        const int32_t rc = launch_attention_flash32(pf, st);
+        if (rc != MI_OK) return rc;
+    }
+    const int64_t q_blocks = (p.Lq + 31) / 32 * p.H * p.B, k_blocks = (p.Lkv + 31) / 32 * p.H * p.B;
+    hipLaunchKernelGGL((bwd32s_dq_small_kernel<D, CAUSAL, true>), dim3((unsigned)q_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+    if (bp.dv || bp.dk) hipLaunchKernelGGL((bwd32s_dkdv_small_kernel<D, CAUSAL, true>), dim3((unsigned)k_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+    MI_LAUNCH_CHECK();
+    return MI_OK;
+}
+}  // namespace
+
 int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp_in, hipStream_t st) {
     AttnBwdParams bp = bp_in;
     // few queries, many keys, saved statistics: the dQ kernel's key range in pieces (the 16-bit kernels' rule); the
@@ -1460,6 +1523,7 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp_in, hipStream_t st)
     flash_fill_vec_flags(a);
     a.bias_lds = a.mask_lds = 0;
     a.p.drop_thresh = 0;   // the shared softmax step yields the weights before dropout; the kernels apply bp.p's dropout themselves
+    if (small_masked_call(bp)) return bp.p.causal ? launch_small_masked<true>(a, bp, st) : launch_small_masked<false>(a, bp, st);
     if (attention_bwd_flash32_lengths_bytes(bp) != 0) {
         // the lengths follow the statistics planes when those live in the workspace too
         int32_t *lens = (int32_t *)((char *)bp.workspace + (bp.have_stats ? 0 : attention_stats_bytes(bp.p)));

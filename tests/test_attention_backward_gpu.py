@@ -187,6 +187,10 @@ F32_CASES = [
     (64, 8, 128, 128, (4,), None, True),
     (64, 1, 1, 200, (3,), None, True),
     (64, 1, 500, 31, (1,), None, True),
+    # the same kernels reading a Bool mask array (no bias), with and without saved statistics
+    (64, 2, 100, 200, (2,), "random", True),
+    (32, 4, 257, 129, (1,), "random", True),
+    (64, 2, 130, 600, (1,), "random", False),
     # more blocks than that: the workgroups of 128 queries / keys with saved statistics
     (64, 4, 128, 128, (40,), None, True),
     (64, 4, 100, 100, (40,), "causal", True),
