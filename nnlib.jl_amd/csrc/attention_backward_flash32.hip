@@ -1156,8 +1156,17 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dq_small_kernel(FlashArgs a, At
             }
             floatx16_t sb = first_product_sl<D, SB::XPLANEB>(Ks + blk_tile, kb, xq_row, xsw, (floatx16_t){0}, r, hh);
             SCHED_FENCE();
-            const floatx16_t dpb = first_product_sl<D, SB::XPLANEB>(Vs + blk_tile, kb, xdo_row, xsw, (floatx16_t){0}, r, hh);
+            floatx16_t dpb = first_product_sl<D, SB::XPLANEB>(Vs + blk_tile, kb, xdo_row, xsw, (floatx16_t){0}, r, hh);
             SCHED_FENCE();
+            if (bp.p.drop_thresh != 0) {   // fused dropout: the forward multiplied the weight by g (0 or 1 / (1 - p)), its pullback multiplies dP
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    float gf[4];
+                    attention_drop_factors_run4<false>(bp.p, (uint64_t)(p.Lkv * (qi + p.Lq * (h + p.H * b)) + 4 * hh + j0), g, gf);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) dpb[4 * g + e] *= gf[e];
+                }
+            }
             // keys of the block this lane's query keeps, counted from the lane's first key of a group of four
             int64_t lim64 = p.Lkv - j0;
             if (CAUSAL && qi - j0 + 1 < lim64) lim64 = qi - j0 + 1;
@@ -1246,6 +1255,7 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dkdv_small_kernel(FlashArgs a, 
             // accumulator register 4g+e of this lane: query i0 + 8g + 4hh + e, key kv.  Rows past Lq carry statistics
             // (0, 0, 0): their weights vanish; keys past the length only feed columns that store zeros
             const bool diag = CAUSAL && i0 < jw + 32;   // some (query, key) pair of this block has key > query
+            const bool drop = bp.p.drop_thresh != 0;
             const float *st = st_lds + 32 * wave;
 #pragma unroll
             for (int g = 0; g < 4; g++) {
@@ -1259,8 +1269,10 @@ __global__ __launch_bounds__(256, 1) void bwd32s_dkdv_small_kernel(FlashArgs a, 
                     float pw = mi_exp2(fmaf(s[4 * g + e], cs, -m4[e])) * linv4[e];
                     if (diag) pw = dq_ - e > 0 ? 0.0f : pw;
                     if constexpr (MASKED) pw = mk[4 * g + e] != 0 ? pw : 0.0f;
-                    s[4 * g + e] = pw;
-                    dp[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
+                    // fused dropout: the value product saw pw * gd, and the pullback multiplies dP by gd
+                    const float gd = drop ? attention_drop_factor(bp.p, kv, i0 + sq + e, h, b) : 1.0f;
+                    s[4 * g + e] = pw * gd;
+                    dp[4 * g + e] = pw * (gd * dp[4 * g + e] - delta4[e]);
                 }
             }
             SCHED_FENCE();
@@ -1462,40 +1474,42 @@ bool attention_bwd_flash32_supports(const AttnBwdParams &bp) {
 }
 
 namespace {
-// Small calls with a Bool mask array and no bias: the workgroups per 32 queries / 32 keys read the mask bytes of their
-// pairs themselves (any strides; a key-padding mask needs no classification of context lengths)
-bool small_masked_call(const AttnBwdParams &bp) {
+// Small calls with a Bool mask array and / or fused dropout, no bias: the workgroups per 32 queries / 32 keys read the
+// mask bytes of their pairs themselves (any strides; a key-padding mask needs no classification of context lengths)
+// and redraw the keep decisions
+bool small_extras_call(const AttnBwdParams &bp) {
     static const bool no_small = getenv("MI355ATTN_NO_QUAD") != nullptr;
     const AttnParams &p = bp.p;
-    if (no_small || !p.mask || p.bias || bp.dbias || p.drop_thresh || p.D > 64 || exact_instruction_wanted() || bp.dq_nsplit > 1) return false;
+    if (no_small || (!p.mask && !p.drop_thresh) || p.bias || bp.dbias || p.D > 64 || exact_instruction_wanted() || bp.dq_nsplit > 1) return false;
     const int64_t q_blocks = (p.Lq + 31) / 32 * p.H * p.B, k_blocks = (p.Lkv + 31) / 32 * p.H * p.B;
     if (q_blocks > 512 || k_blocks > 512) return false;
     // without the caller's statistics the forward kernels' statistics-only run has to apply (see launch_set_planes)
     return bp.have_stats || (q_blocks <= 256 && p.Lkv <= 512 && p.scale_D == 0);
 }
 
-template <bool CAUSAL>
-int32_t launch_small_masked(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
+template <bool CAUSAL, bool MASKED>
+int32_t launch_small_extras(const FlashArgs &a, const AttnBwdParams &bp, hipStream_t st) {
     constexpr int D = 64;
     const AttnParams &p = a.p;
     static bool attr_set = false;
     if (!attr_set) {
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_small_kernel<D, CAUSAL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
-        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dkdv_small_kernel<D, CAUSAL, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_small_kernel<D, CAUSAL, MASKED>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dkdv_small_kernel<D, CAUSAL, MASKED>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SmallBwd<D>::SMEM));
         attr_set = true;
     }
-    if (!bp.have_stats) {
+    if (!bp.have_stats) {   // the statistics are those of the weights before dropout
         AttnParams pf = p;
         pf.out = nullptr;
         pf.weights = nullptr;
         pf.workspace = nullptr;
         pf.stats = bp.stats;
+        pf.drop_thresh = 0;
         const int32_t rc = launch_attention_flash32(pf, st);
         if (rc != MI_OK) return rc;
     }
     const int64_t q_blocks = (p.Lq + 31) / 32 * p.H * p.B, k_blocks = (p.Lkv + 31) / 32 * p.H * p.B;
-    hipLaunchKernelGGL((bwd32s_dq_small_kernel<D, CAUSAL, true>), dim3((unsigned)q_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
-    if (bp.dv || bp.dk) hipLaunchKernelGGL((bwd32s_dkdv_small_kernel<D, CAUSAL, true>), dim3((unsigned)k_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+    hipLaunchKernelGGL((bwd32s_dq_small_kernel<D, CAUSAL, MASKED>), dim3((unsigned)q_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+    if (bp.dv || bp.dk) hipLaunchKernelGGL((bwd32s_dkdv_small_kernel<D, CAUSAL, MASKED>), dim3((unsigned)k_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
     MI_LAUNCH_CHECK();
     return MI_OK;
 }
@@ -1523,7 +1537,10 @@ int32_t launch_attention_bwd_flash32(const AttnBwdParams &bp_in, hipStream_t st)
     flash_fill_vec_flags(a);
     a.bias_lds = a.mask_lds = 0;
     a.p.drop_thresh = 0;   // the shared softmax step yields the weights before dropout; the kernels apply bp.p's dropout themselves
-    if (small_masked_call(bp)) return bp.p.causal ? launch_small_masked<true>(a, bp, st) : launch_small_masked<false>(a, bp, st);
+    if (small_extras_call(bp)) {
+        if (bp.p.mask) return bp.p.causal ? launch_small_extras<true, true>(a, bp, st) : launch_small_extras<false, true>(a, bp, st);
+        return bp.p.causal ? launch_small_extras<true, false>(a, bp, st) : launch_small_extras<false, false>(a, bp, st);
+    }
     if (attention_bwd_flash32_lengths_bytes(bp) != 0) {
         // the lengths follow the statistics planes when those live in the workspace too
         int32_t *lens = (int32_t *)((char *)bp.workspace + (bp.have_stats ? 0 : attention_stats_bytes(bp.p)));

@@ -368,6 +368,7 @@ def test_fully_masked_query_gives_nan_gradients(nn):
     ("f32", 128, 2, 150, 200, (2,), None, None, False, True, "flash32"),         # D = 64
     ("f32", 256, 2, 192, 192, (1,), "causal", None, False, False, "flash32"),    # D = 128
     ("f32", 128, 2, 70, 300, (1,), "random", None, False, False, "flash32"),
+    ("f32", 128, 2, 150, 200, (60,), None, None, False, True, "flash32"),        # more than 512 blocks of 32 queries: the per-element kernels
 ])
 def test_gradient_through_fused_dropout(nn, oracle, dtype, E, H, Lq, Lkv, batch, mask_kind, bias_shape, with_dalpha, saved,
                                         expect):
