@@ -157,7 +157,7 @@ N_SMALL = int(os.environ.get("MI355ATTN_SMALL_SEEDS", "40"))
 def test_float32_calls_on_few_workgroups(nn, oracle, seed):
     """Lengths around the 32-row blocks and 128-row chunks those kernels cut the sequences into, head dims on both tile
     widths, with and without the weights, the causal mask and bias / mask arrays in the forward call, saved statistics
-    or not in the gradient call (which takes no bias / mask arrays on those kernels)."""
+    or not, Bool mask arrays of every layout and fused dropout in the gradient call."""
     from test_attention_gpu import _check
     from test_attention_backward_gpu import _run
     rng = np.random.default_rng(9000 + seed)
@@ -172,5 +172,9 @@ def test_float32_calls_on_few_workgroups(nn, oracle, seed):
     mask_shape = (Lkv, Lq) if extras and not causal else None
     _check(nn, oracle, rng, "f32", D * H, Lq, Lkv, B, H, causal=causal, bias_shape=bias_shape, mask_shape=mask_shape,
            scale=0.5, expect="flash32", weights=bool(seed % 2))
-    _run(nn, oracle, "f32", D * H, D * H, Lq, Lkv, (B,), H, mask_kind="causal" if causal else None, seed=seed, scale=0.4,
-         saved=bool((seed // 2) % 2))
+    gmask = "causal" if causal else [None, "random", "keys", "random_hb"][int(rng.integers(0, 4))]
+    if gmask == "keys" and Lkv < 100:   # the key-padding pattern of the gradient helper drops the first 70 keys of one batch element
+        gmask = "random"
+    dropout = (0.2, 31 + seed) if rng.integers(0, 4) == 0 else None
+    _run(nn, oracle, "f32", D * H, D * H, Lq, Lkv, (B,), H, mask_kind=gmask, seed=seed, scale=0.4,
+         saved=bool((seed // 2) % 2), dropout=dropout)
