@@ -407,9 +407,8 @@ def measure_extra(key, steps, warmup, with_cpu):
         line = dict(metric="attention gradient TFLOP/s", value=val, unit="TFLOP/s", dtype=dtn,
                     roofline=dict(bound="mfma", achieved=val, peak=PEAK[dtn], unit="TFLOP/s", frac=val / PEAK[dtn], **measured_traffic_fields(key)),
                     config=dict(workload=EXTRA[key], kernel=_lib.KERNEL_NAMES[kern.value]), flops_per_step=flops)
-        # 16-bit: dQ kernel S, dP, dQ; fused dK / dV kernel S, dV, dP, dK.  Float32: dQ: S, dP, dQ; dV: S, dV; dK: S, dP, dK
-        # (the Float32 kernels of calls on few workgroups: dQ: S, dP, dQ; dK / dV: S, dP, dV, dK)
-        per_counted = 7 / 5 if dtn != "f32" or key == "bwd_c1" else 8 / 5
+        # dQ kernel S, dP, dQ; fused dK / dV kernel S, dP, dV, dK (16-bit and Float32 alike)
+        per_counted = 7 / 5
         line["roofline"]["products_executed_per_counted"] = per_counted
         if dtn == "f32":
             f32_products(line["roofline"], val, per_counted)

@@ -851,11 +851,12 @@ __global__ __launch_bounds__(64 * NW, 1) void bwd32s_dq_kernel(FlashArgs a, Attn
 
 template <int D, bool CAUSAL, int WHICH>
 // Head dim 64 fits two workgroups per compute unit, each fetching its next tiles only once the products are done (no
-// staging registers live across them): the other workgroup covers the latency.
-__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(FlashArgs a, AttnBwdParams bp) {
+// staging registers live across them): the other workgroup covers the latency.  WHICH = BWD_DV | BWD_DK: both
+// gradients from one S and dP, one workgroup per compute unit (see launch_set_planes).
+__global__ __launch_bounds__(256, D == 64 && WHICH != 3 ? 2 : 1) void bwd32s_dkdv_kernel(FlashArgs a, AttnBwdParams bp) {
     typedef CfgS<D> C;
     constexpr int NDV = D / 32;
-    constexpr bool DO_DV = WHICH == BWD_DV, DO_DK = WHICH == BWD_DK;
+    constexpr bool DO_DV = (WHICH & BWD_DV) != 0, DO_DK = (WHICH & BWD_DK) != 0;   // 3: both from one S and dP
     const AttnParams &p = a.p;
     extern __shared__ __attribute__((aligned(16))) unsigned char bwd_smem[];
     const unsigned Qs = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)bwd_smem, dOs = Qs + C::TILEB;
@@ -871,7 +872,6 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(Flash
         if (kv_len == 0) return;
     }
     const bool kvalid = kv < kv_len;
-    float *grad = DO_DK ? (float *)bp.dk : (float *)bp.dv;
     const int64_t off = p.E * (kv + p.Lkv * b) + p.D * h;
     if (j0 >= kv_len) {   // keys from the pair's length on get zero gradients
         if (kok) {
@@ -880,7 +880,10 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(Flash
             for (int dvb = 0; dvb < NDV; dvb++)
 #pragma unroll
                 for (int g = 0; g < 4; g++)
-                    if (32 * dvb + 8 * g + 4 * hh < p.D) *(floatx4_t *)(grad + off + 32 * dvb + 8 * g + 4 * hh) = z4;
+                    if (32 * dvb + 8 * g + 4 * hh < p.D) {
+                        if (DO_DV && bp.dv) *(floatx4_t *)((float *)bp.dv + off + 32 * dvb + 8 * g + 4 * hh) = z4;
+                        if (DO_DK && bp.dk) *(floatx4_t *)((float *)bp.dk + off + 32 * dvb + 8 * g + 4 * hh) = z4;
+                    }
         }
         return;
     }
@@ -888,9 +891,11 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(Flash
     plane8 kx[3][D / 16], vx[DO_DK ? 3 : 1][D / 16];
     load_stationary_s<D>(kx, (const float *)p.k + off, kvalid, hh, (int)p.D);
     if constexpr (DO_DK) load_stationary_s<D>(vx, (const float *)p.v + off, kvalid, hh, (int)p.D);
-    floatx16_t acc[NDV];
+    floatx16_t accv[DO_DV ? NDV : 1], acck[DO_DK ? NDV : 1];
 #pragma unroll
-    for (int dvb = 0; dvb < NDV; dvb++) acc[dvb] = (floatx16_t){0};
+    for (int dvb = 0; dvb < (DO_DV ? NDV : 1); dvb++) accv[dvb] = (floatx16_t){0};
+#pragma unroll
+    for (int dvb = 0; dvb < (DO_DK ? NDV : 1); dvb++) acck[dvb] = (floatx16_t){0};
 
     const int64_t plane = p.B * p.H * lq_pad(p.Lq);
     // the row statistics of a query tile travel with it through LDS (48 threads x 4 floats)
@@ -944,13 +949,19 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(Flash
                     for (int e = 0; e < 4; e++) {
                         float pw = mi_exp2(fmaf(s[4 * g + e], cs, -m4[e])) * linv4[e];
                         if (diag) pw = dq_ - e > 0 ? 0.0f : pw;
-                        if (DO_DK) s[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
-                        else s[4 * g + e] = pw;
+                        if (DO_DK) dp[4 * g + e] = pw * (dp[4 * g + e] - delta4[e]);
+                        s[4 * g + e] = pw;
                     }
                 }
                 SCHED_FENCE();
-                second_product_s<D>(DO_DK ? Qs : dOs, kb, s, acc, lane);
-                SCHED_FENCE();
+                if constexpr (DO_DV) {
+                    second_product_s<D>(dOs, kb, s, accv, lane);
+                    SCHED_FENCE();
+                }
+                if constexpr (DO_DK) {
+                    second_product_s<D>(Qs, kb, dp, acck, lane);
+                    SCHED_FENCE();
+                }
             }
         }
         if (more) {
@@ -962,16 +973,23 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd32s_dkdv_kernel(Flash
         __syncthreads();
     }
     if (kok) {
-        const float scale = DO_DK ? a.cn : 1.0f;
 #pragma unroll
         for (int dvb = 0; dvb < NDV; dvb++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 if (32 * dvb + 8 * g + 4 * hh >= p.D) continue;
-                floatx4_t g4;
+                if constexpr (DO_DV) {
+                    floatx4_t g4;
 #pragma unroll
-                for (int e = 0; e < 4; e++) g4[e] = kvalid ? acc[dvb][4 * g + e] * scale : 0.0f;
-                *(floatx4_t *)(grad + off + 32 * dvb + 8 * g + 4 * hh) = g4;
+                    for (int e = 0; e < 4; e++) g4[e] = kvalid ? accv[dvb][4 * g + e] : 0.0f;
+                    if (bp.dv) *(floatx4_t *)((float *)bp.dv + off + 32 * dvb + 8 * g + 4 * hh) = g4;
+                }
+                if constexpr (DO_DK) {
+                    floatx4_t g4;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) g4[e] = kvalid ? acck[dvb][4 * g + e] * a.cn : 0.0f;
+                    if (bp.dk) *(floatx4_t *)((float *)bp.dk + off + 32 * dvb + 8 * g + 4 * hh) = g4;
+                }
             }
     }
 }
@@ -1312,6 +1330,13 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
     auto k1w = bp.have_stats ? bwd32s_dq_kernel<D, CAUSAL, true, NW_WIDE> : bwd32s_dq_kernel<D, CAUSAL, false, NW_WIDE>;
     auto k2 = bwd32s_dkdv_kernel<D, CAUSAL, BWD_DV>;
     auto k3 = bwd32s_dkdv_kernel<D, CAUSAL, BWD_DK>;
+    // Both from one S and dP (seven products for the gradient instead of eight) at one workgroup per compute unit: the
+    // two stationary rows and two accumulators of a lane do not fit 256 registers (428-512 bytes of scratch at two
+    // workgroups per unit).  Measured against the pair: C2-shaped gradient 0.437 -> 0.425 ms, the same without the causal
+    // mask 0.823 -> 0.712, 2048 x 2048 with 32 pairs 0.538 -> 0.440 (causal) and 0.777 -> 0.661, 4096 x 4096 with 8 pairs
+    // 0.94 -> 0.75.  128-wide tiles keep the pair (512 registers either way, 688-1108 bytes of scratch fused).
+    auto k23 = bwd32s_dkdv_kernel<D, CAUSAL, BWD_DV | BWD_DK>;
+    static const bool fused_dkdv = D == 64 && getenv("MI355ATTN_F32_DKDV_PAIR") == nullptr;   // the switch: for comparisons
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, so a race is harmless
     if (!attr_set) {
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)bwd32s_dq_kernel<D, CAUSAL, true, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
@@ -1322,6 +1347,7 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
         }
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k2, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         MI_HIP_CHECK(hipFuncSetAttribute((const void *)k3, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
+        MI_HIP_CHECK(hipFuncSetAttribute((const void *)k23, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM));
         attr_set = true;
     }
     // few 32-row blocks (at most two workgroups per compute unit) and the forward call's statistics: the workgroups per
@@ -1375,6 +1401,8 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
     if (small_k) {
         if constexpr (D == 64)
             if (bp.dv || bp.dk) hipLaunchKernelGGL((bwd32s_dkdv_small_kernel<D, CAUSAL, false>), dim3((unsigned)k_blocks), dim3(256), SmallBwd<D>::SMEM, st, a, bp);
+    } else if (bp.dv && bp.dk && fused_dkdv) {
+        hipLaunchKernelGGL(k23, g2, dim3(256), SMEM, st, a, bp);
     } else {
         if (bp.dv) hipLaunchKernelGGL(k2, g2, dim3(256), SMEM, st, a, bp);
         if (bp.dk) hipLaunchKernelGGL(k3, g2, dim3(256), SMEM, st, a, bp);
