@@ -1325,7 +1325,8 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
     constexpr int NW_WIDE = D == 64 ? 8 : 4;
     constexpr size_t SMEM_WIDE = SMEM + 3 * 32 * NW_WIDE * CfgS<D>::ROWB;
     const int64_t wide_tiles = (p.Lq + 32 * NW_WIDE - 1) / (32 * NW_WIDE);
-    const bool wide = NW_WIDE > 4 && bp.dq_nsplit <= 1 && wide_tiles * p.H * p.B >= 256;
+    // (not for sequences of at most 128 queries, where half of its wavefronts would have none: 4-6 % slower there)
+    const bool wide = NW_WIDE > 4 && bp.dq_nsplit <= 1 && wide_tiles * p.H * p.B >= 256 && p.Lq > 128;
     auto k1 = bp.have_stats ? bwd32s_dq_kernel<D, CAUSAL, true, 4> : bwd32s_dq_kernel<D, CAUSAL, false, 4>;
     auto k1w = bp.have_stats ? bwd32s_dq_kernel<D, CAUSAL, true, NW_WIDE> : bwd32s_dq_kernel<D, CAUSAL, false, NW_WIDE>;
     auto k2 = bwd32s_dkdv_kernel<D, CAUSAL, BWD_DV>;
