@@ -890,12 +890,14 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs
     const AttnParams &p = a.p;
     extern __shared__ __attribute__((aligned(16))) unsigned char flash_smem[];
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)flash_smem;
-    // K tiles (later the partial outputs), V tiles, weight staging, exchanged statistics
-    const unsigned Kp = lds0, Vp = lds0 + 2 * TILEB;
-    float *xstat = (float *)(flash_smem + 4 * TILEB + 4 * FLASH_WSTAGE_BYTES);   // [4 wavefronts][32 rows][2]
-    float *xout = (float *)flash_smem;                                           // [4 wavefronts][D / 2 registers][64 lanes]
+    // K tiles (later the partial outputs), V tiles, weight staging, exchanged statistics, the query block's planes.
+    // Calls with at most 64 keys have one tile per tensor (69 KiB in all: two workgroups per compute unit)
+    const unsigned kt = p.Lkv <= BN ? 1u : 2u;
+    const unsigned Kp = lds0, Vp = lds0 + kt * TILEB, behind = 2 * kt * TILEB;
+    float *xstat = (float *)(flash_smem + behind + 4 * FLASH_WSTAGE_BYTES);   // [4 wavefronts][32 rows][2]
+    float *xout = (float *)flash_smem;                                        // [2 kt wavefronts with a key block][D / 2 registers][64 lanes]
     constexpr int QPLANEB = 32 * ROWB, QCHUNKS = 32 * D / 4 / 256;
-    const unsigned Qp = lds0 + 4 * TILEB + 4 * FLASH_WSTAGE_BYTES + 4 * 32 * 2 * (unsigned)sizeof(float);   // the query block's planes
+    const unsigned Qp = lds0 + behind + 4 * FLASH_WSTAGE_BYTES + 4 * 32 * 2 * (unsigned)sizeof(float);
     typedef __attribute__((address_space(3))) const plane8 *lds_plane8_t;
     typedef __attribute__((address_space(3))) u32x2_t *lds8_t;
 
@@ -1039,7 +1041,7 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs
     }
 
     // ---- weights and the wavefront's share of the output
-    const unsigned wlds = lds0 + 4u * TILEB + wave * FLASH_WSTAGE_BYTES;
+    const unsigned wlds = lds0 + behind + wave * FLASH_WSTAGE_BYTES;
     if (active) {
         flash_softmax_tile<T, 1, D / 32, CAUSAL, XT, PHASE_FINAL, float, 1>(a, keep, f.o, f.m, f.l, b, h, iw, j0, FlashStaged<1>(), 0, wlds, nullptr, p.Lkv);
         if (do_pv) weights_times_values32s<D, 1, 1>(f, Vp + blk, keep);
@@ -1051,10 +1053,12 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs
     // the partial outputs go through LDS (the K planes' region: nobody reads them any more); each wavefront adds up
     // and writes a quarter of the row
     if (!do_pv) return;
+    if (wave < (int)(2 * kt)) {
 #pragma unroll
-    for (int dvb = 0; dvb < D / 32; dvb++)
+        for (int dvb = 0; dvb < D / 32; dvb++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) xout[(wave * (D / 2) + 16 * dvb + v) * 64 + lane] = f.o[0][dvb][v];
+            for (int v = 0; v < 16; v++) xout[(wave * (D / 2) + 16 * dvb + v) * 64 + lane] = f.o[0][dvb][v];
+    }
     __syncthreads();
     if (qi < p.Lq) {
         float *orow = (float *)p.out + p.Ev * (qi + p.Lq * b) + p.Dv * h;
@@ -1065,8 +1069,10 @@ __global__ __launch_bounds__(256, 1) void flash32_resident_quad_kernel(FlashArgs
             floatx4_t o4 = (floatx4_t){0};
 #pragma unroll
             for (int w = 0; w < 4; w++)
+                if (w < (int)(2 * kt)) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) o4[e] += xout[(w * (D / 2) + 16 * dvb + 4 * g + e) * 64 + lane];
+                    for (int e = 0; e < 4; e++) o4[e] += xout[(w * (D / 2) + 16 * dvb + 4 * g + e) * 64 + lane];
+                }
             if (32 * dvb + 8 * g + 4 * hh < p.Dv) *(floatx4_t *)(orow + 32 * dvb + 8 * g + 4 * hh) = o4;
         }
     }
@@ -1331,10 +1337,13 @@ int32_t launch_resident(const FlashArgs &a, hipStream_t st, bool extras) {
     static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;   // the workgroup of eight, for comparisons
     // at most one workgroup per compute unit: a wavefront per 32-key block (with two or four workgroups per unit the
     // workgroups below are faster: 16.7 against 15.0 us at 512, 31.8 against 15.4 us at 1024)
-    if (total_quad <= RESIDENT_QUAD_MAX_BLOCKS && !no_quad) {
+    // (with at most 64 keys two of these workgroups fit a compute unit and it wins at any number of blocks: 2048 pairs of
+    // 32 x 32 with the weights 73 -> 33 us, 1024 pairs of 64 x 64 40.6 -> 36.2)
+    if ((total_quad <= RESIDENT_QUAD_MAX_BLOCKS || a.p.Lkv <= BN) && !no_quad) {
         auto kern = a.p.causal ? (extras ? flash32_resident_quad_kernel<D, true, true> : flash32_resident_quad_kernel<D, true, false>)
                                : (extras ? flash32_resident_quad_kernel<D, false, true> : flash32_resident_quad_kernel<D, false, false>);
-        hipLaunchKernelGGL(kern, dim3((unsigned)total_quad), dim3(256), smem_quad, st, a);
+        const size_t smem_q = a.p.Lkv <= BN ? smem_quad - 2 * CfgS<D>::TILEB : smem_quad;   // one tile per tensor
+        hipLaunchKernelGGL(kern, dim3((unsigned)total_quad), dim3(256), smem_q, st, a);
     } else if (a.p.Lkv > BN) {   // two key tiles: a wavefront per tile and query block
         auto kern = a.p.causal ? (extras ? flash32_resident_pair_kernel<D, true, true> : flash32_resident_pair_kernel<D, true, false>)
                                : (extras ? flash32_resident_pair_kernel<D, false, true> : flash32_resident_pair_kernel<D, false, false>);
@@ -1443,7 +1452,12 @@ int32_t launch_attention_flash32(const AttnParams &p, hipStream_t st) {
     // few keys and the weights returned: everything resident, one pass (flash32_resident_kernel); without the weights
     // when the call leaves most of the chip idle (the workgroup per 32-query block)
     const bool few_blocks = (p.Lq + 31) / 32 * p.H * p.B <= RESIDENT_QUAD_MAX_BLOCKS;
-    const bool resident = narrow && (p.weights || few_blocks) && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted();
+    // at most 64 keys: the workgroup per query block needs 69 KiB of LDS, two fit a compute unit, and it beats the
+    // two-pass kernel on any number of pairs up to 1024 blocks, or when a sequence is one block (2048 pairs of 32 x 32:
+    // 48 -> 31 us; 512 pairs of 48 x 48: 18.4 -> 15.7; 1024 pairs of 64 x 64 are 25.6 on the two-pass kernel against 32.1)
+    const int64_t q_blocks = (p.Lq + 31) / 32 * p.H * p.B;
+    const bool short_keys = p.Lkv <= BN && (q_blocks <= 1024 || p.Lq <= 32);
+    const bool resident = narrow && (p.weights || few_blocks || short_keys) && p.Lkv <= RES_TILES * BN && !exact_instruction_wanted();
     static const bool no_quad = getenv("MI355ATTN_NO_QUAD") != nullptr;
     // against the two-pass kernel the workgroup per query block still wins at two workgroups per compute unit when the
     // weights are written or the mask is causal (512 blocks of 512 keys: 43 against 58 us with weights, causal 36 against

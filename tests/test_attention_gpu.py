@@ -309,7 +309,7 @@ SMALL_F32_CASES = [
     (256, 97, 97, 17, 4, dict(causal=True)),
     (128, 1100, 100, 4, 2, dict(bias_shape=(100, 1100, 2, 1), mask_shape=(100, 1100))),
     (256, 128, 128, 17, 4, dict(causal=True, mask_shape=(128, 128, 1, 17))),
-    (512, 160, 64, 8, 8, {}),                                            # the same with at most 64 keys: four wavefronts, one per query block
+    (512, 160, 64, 8, 8, {}),                                            # at most 64 keys and many blocks: two workgroups per compute unit
     (256, 60, 60, 33, 4, dict(causal=True)),
     (128, 1100, 50, 4, 2, dict(bias_shape=(50, 1100, 2, 1), mask_shape=(50, 1100))),
 ]
