@@ -1361,8 +1361,10 @@ int32_t launch_set_planes(const FlashArgs &a, const AttnBwdParams &bp, hipStream
         // kernel reads the statistics it is given; the dK / dV kernel reads what the dQ kernel before it left in
         // bp.stats, whichever that was
         const bool can = !a.kv_len && !no_small;
-        small_q = can && bp.have_stats && bp.dq_nsplit <= 1 && q_blocks <= 512;
-        small_k = can && k_blocks <= 512;
+        // (sequences of one block take them at any number of pairs: 2048 pairs of 32 x 32 176 -> 150 us; two blocks per
+        // sequence lose beyond the limit: 1024 pairs of 64 x 64 98 against 153)
+        small_q = can && bp.have_stats && bp.dq_nsplit <= 1 && (q_blocks <= 512 || p.Lq <= 32);
+        small_k = can && (k_blocks <= 512 || p.Lkv <= 32);
         // no statistics from the caller: where the forward kernels of this shape of call apply (a workgroup per 32
         // queries, at most 512 keys), their statistics-only run (no values, no output) fills bp.stats first
         if (can && !bp.have_stats && bp.dq_nsplit <= 1 && q_blocks <= 256 && p.Lkv <= 512 && p.scale_D == 0 && !exact_instruction_wanted()) {

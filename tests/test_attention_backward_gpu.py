@@ -191,6 +191,8 @@ F32_CASES = [
     (64, 2, 100, 200, (2,), "random", True),
     (32, 4, 257, 129, (1,), "random", True),
     (64, 2, 130, 600, (1,), "random", False),
+    (64, 8, 32, 32, (80,), None, True),                  # 640 sequences of one block: those kernels at any number of pairs
+    (64, 8, 30, 90, (70,), None, True),                  # ... the dQ kernel only
     # more blocks than that: the workgroups of 128 queries / keys with saved statistics
     (64, 4, 128, 128, (40,), None, True),
     (64, 4, 100, 100, (40,), "causal", True),
